@@ -1,0 +1,84 @@
+/*
+ * mi355_serving.h -- C ABI of libmi355_serving.so: the fp16 GEMM and the fused multi-head-attention forward
+ * for AMD Instinct MI355X (gfx950), as plain pointers and sizes. No torch types, no C++ types.
+ *
+ * This layer is what the PyTorch operators `gemm_unified::finegemm_N` and `fmha_unified::finefmha_N` call
+ * after validating their tensors; it can equally be bound from C, C++ or ctypes.
+ *
+ * Conventions
+ *   - every pointer is a DEVICE pointer owned by the caller; nothing is allocated, freed or retained;
+ *   - `stream` is a hipStream_t passed as void* (NULL = the null stream); calls are asynchronous;
+ *   - fp16 data is IEEE binary16 (`_Float16` / `__half` / torch.float16);
+ *   - return value 0 = launched; non-zero = a hipError_t value or MI355_ERR_* below, nothing was launched.
+ *     mi355_last_error() returns a thread-local description of the last failure.
+ *   - calls are re-entrant and thread-safe; the library keeps no mutable global state besides one-time
+ *     kernel attribute initialisation.
+ */
+#ifndef MI355_SERVING_H
+#define MI355_SERVING_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MI355_SERVING_VERSION 100
+
+/* argument errors (distinct from hipError_t values, which are < 10000) */
+#define MI355_ERR_BAD_ARGUMENT 10001
+#define MI355_ERR_UNSUPPORTED 10002
+
+/* operand layouts of mi355_hgemm */
+#define MI355_GEMM_NN 0 /* A is [M,K] row-major, B is [K,N] row-major           */
+#define MI355_GEMM_NT 1 /* A is [M,K] row-major, B is stored [N,K] (C = A * B^T) */
+#define MI355_GEMM_TN 2 /* A is stored [K,M] (C = A^T * B), B is [K,N]           */
+
+/*
+ * C[M,N] (fp16, row-major, leading dimension ldc) = op(A) * op(B), fp32 accumulation, one rounding to fp16.
+ *
+ * Replaces the device side of the reference's host wrappers `at::Tensor finegemm_N(const at::Tensor& a,
+ * const at::Tensor& b)`:
+ *   layout NN  <- finegemm_0..11  (kernels/gemm/pkg/gemm_unified/csrc/auto/gemm_7.cu:111-151,
+ *                                  semi/gemm_11_amd.cpp:129-154)
+ *   layout TN  <- finegemm_12, 16 (manual/gemm_12_amd.cpp:294-316, manual/gemm_16_amd.cpp:345-367)
+ *   layout NT  <- finegemm_13..15 (manual/gemm_13_amd.cpp:248-270, gemm_14_amd.cpp:268-290,
+ *                                  gemm_15_amd.cpp:291-313)
+ * lda/ldb/ldc are in elements and refer to the stored matrices (e.g. lda >= M for layout TN).
+ * Any M, N, K >= 1 is accepted; shapes that are multiples of the kernel tiles take the fast paths.
+ */
+int mi355_hgemm(const void* A, const void* B, void* C, int M, int N, int K, int64_t lda, int64_t ldb,
+                int64_t ldc, int layout, void* stream);
+
+/*
+ * Fused attention forward, O = softmax(scale * Q K^T + mask) V, online softmax with fp32 statistics.
+ *
+ * Replaces the device side of `torch::Tensor finefmha_N(Q, K, V, causal, is_decode, decode_length)`
+ * (kernels/fmha/pkg/fmha_unified/csrc/semi/fmha_2_amd.cpp:311-359, auto/fmha_0.cu:301-330).
+ *
+ *   Q, O : [B, Hq,  Sq, D] fp16 contiguous ("BHSD")          K, V : [B, Hkv, Sk, D] fp16 contiguous
+ *   LSE  : [B, Hq, Sq] fp32, natural-log log-sum-exp of the scaled, masked scores; may be NULL
+ *   Hq % Hkv == 0; query head h reads kv head h / (Hq / Hkv)   (fmha_2_amd.cpp:33-42)
+ *   D must be 128                                               (fmha_2_amd.cpp:329)
+ *   kv_valid_len : keys with index >= kv_valid_len are masked (1 <= kv_valid_len <= Sk); this is the
+ *                  `decode_length` argument of the reference with its off-by-one (`>`,
+ *                  fmha_2_amd.cpp:191) corrected. Pass Sk for "all keys valid".
+ *   causal != 0  : key j is visible to query i iff j <= i + (Sk - Sq), i.e. the mask is aligned to the
+ *                  bottom-right corner; with Sq == Sk this is the reference's `q_pos < k_pos => masked`
+ *                  rule (fmha_2_amd.cpp:187-190).
+ *   Sq and Sk are arbitrary (>= 1); ragged tails are masked inside the kernel, no padding is needed.
+ *   A query row with no visible key yields O = 0 and LSE = -inf.
+ */
+int mi355_fmha_fwd(const void* Q, const void* K, const void* V, void* O, float* LSE, int B, int Hq, int Hkv,
+                   int Sq, int Sk, int D, float scale, int causal, int kv_valid_len, void* stream);
+
+/* Thread-local text for the last non-zero return of this thread ("" if none). */
+const char* mi355_last_error(void);
+
+/* MI355_SERVING_VERSION of the loaded library. */
+int mi355_serving_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MI355_SERVING_H */

@@ -1,0 +1,367 @@
+// fp16 GEMM for gfx950 (MI355X): C[M,N] = op(A) * op(B), fp16 operands, fp32 accumulation in the MFMA
+// accumulators, one rounding to fp16 on the store.
+//
+// Replaces the reference's GEMM ladder (kernels/gemm/pkg/gemm_unified/csrc/{auto,semi,manual}/gemm_*.{cu,cpp});
+// the three operand layouts are the ones the reference's op indices use
+// (kernels/gemm/test/correct.py:9-15): NN for finegemm_0..11, TN (a stored [K,M]) for 12/16 and NT (b stored
+// [N,K]) for 13..15.
+//
+// Main kernel: one workgroup of 8 waves computes a 256x256 tile of C, K is walked in steps of 64.
+//   * global -> LDS staging uses 16-byte direct-to-LDS copies (no VGPR bounce), double buffered; every
+//     wave-instruction writes 1 KiB of contiguous LDS, the XOR swizzle is applied on the global-address side.
+//   * an operand whose K index is contiguous in memory is read from LDS with ds_read_b128; an operand whose
+//     M/N index is contiguous (B in the NN case) is read with the transposing ds_read_b64_tr_b16, so no
+//     transpose pass over B is ever made.
+//   * each wave owns a 128x64 sub-tile = 4x2 MFMA 32x32x16 blocks (128 fp32 accumulators per lane).
+//     The MFMA is issued with the B fragment as first operand, i.e. it produces the transposed block, so a
+//     lane ends up with 4 consecutive N of one row of C and can store 8 bytes at a time.
+#include "mi355_common.h"
+#include "mi355_serving_internal.h"
+
+namespace mi355 {
+
+// ---------------------------------------------------------------------------------------------------------
+// LDS tile descriptions
+// ---------------------------------------------------------------------------------------------------------
+
+// Operand tile whose K index is contiguous in memory: LDS holds [ROWS][BK] halfs, row = M (or N) index.
+// 16-byte chunk c of row r lives at chunk position c ^ swz(r).
+template <int ROWS, int BK, int NWAVES>
+struct KContigTile {
+    static constexpr int kChunksPerRow = BK / 8;
+    static constexpr int kRowBytes = BK * 2;
+    static constexpr int kRowsPerInst = 64 / kChunksPerRow;
+    static constexpr int kRowsPerPass = kRowsPerInst * NWAVES;
+    static constexpr int kInsts = ROWS / kRowsPerPass;
+    static constexpr int kBytes = ROWS * kRowBytes;
+    static_assert(ROWS % kRowsPerPass == 0, "tile rows must be a multiple of one pass of the workgroup");
+    static_assert(BK == 64, "swizzle below is written for 128-byte rows");
+
+    __device__ static __forceinline__ int swz(int row) { return (row & 7) ^ ((row >> 3) & 1); }
+
+    // element offset (in halfs, relative to the tile origin in global memory) of this lane's first copy
+    __device__ static __forceinline__ long first_copy_offset(int wave, int lane, long ld) {
+        int row = wave * kRowsPerInst + lane / kChunksPerRow;
+        int chunk = (lane % kChunksPerRow) ^ swz(row);
+        return (long)row * ld + chunk * 8;
+    }
+    __device__ static __forceinline__ long copy_stride(long ld) { return (long)kRowsPerPass * ld; }
+    __device__ static __forceinline__ long ktile_stride(long /*ld*/) { return BK; }
+    __device__ static __forceinline__ int lds_inst_offset(int inst, int wave) { return (inst * NWAVES + wave) * 1024; }
+
+    // byte offset inside the tile of the fragment (32 rows x 16 k) for k-substep kk, first row row0
+    __device__ static __forceinline__ int frag_offset(int row0, int kk, int lane) {
+        int row = row0 + (lane & 31);
+        int chunk = (kk * 2 + (lane >> 5)) ^ swz(row);
+        return row * kRowBytes + chunk * 16;
+    }
+};
+
+// Operand tile whose M/N index is contiguous in memory: LDS holds [BK][COLS] halfs, row = K index.
+template <int COLS, int BK, int NWAVES>
+struct MNContigTile {
+    static constexpr int kChunksPerRow = COLS / 8;
+    static constexpr int kRowBytes = COLS * 2;
+    static constexpr int kRowsPerInst = 64 / kChunksPerRow;
+    static constexpr int kRowsPerPass = kRowsPerInst * NWAVES;
+    static constexpr int kInsts = BK / kRowsPerPass;
+    static constexpr int kBytes = BK * kRowBytes;
+    static_assert(COLS == 256, "swizzle below is written for 512-byte rows");
+    static_assert(BK % kRowsPerPass == 0, "tile depth must be a multiple of one pass of the workgroup");
+
+    // depends on (row % 4) only; keeps the 16 lanes of one transposing read on distinct banks
+    __device__ static __forceinline__ int swz(int row) {
+        int r = row & 3;
+        return (r << 1) | ((r & 1) << 3);  // 0, 10, 4, 14
+    }
+    __device__ static __forceinline__ long first_copy_offset(int wave, int lane, long ld) {
+        int row = wave * kRowsPerInst + lane / kChunksPerRow;
+        int chunk = (lane % kChunksPerRow) ^ swz(row);
+        return (long)row * ld + chunk * 8;
+    }
+    __device__ static __forceinline__ long copy_stride(long ld) { return (long)kRowsPerPass * ld; }
+    __device__ static __forceinline__ long ktile_stride(long ld) { return (long)BK * ld; }
+    __device__ static __forceinline__ int lds_inst_offset(int inst, int wave) { return (inst * NWAVES + wave) * 1024; }
+
+    // byte offset of this lane's transposing read for the fragment (16 k x 32 cols) whose first column is
+    // col0, at k rows [8*(lane/32) .. +3]; add (kk*16 + 4*t) * kRowBytes for substep kk and half t.
+    __device__ static __forceinline__ int frag_offset(int col0, int lane) {
+        int row = 8 * (lane >> 5) + ((lane & 15) >> 2);
+        int chunk = (col0 >> 3) + 2 * ((lane >> 4) & 1) + ((lane & 3) >> 1);
+        return row * kRowBytes + ((chunk ^ swz(row)) << 4) + (lane & 1) * 8;
+    }
+};
+
+// ---------------------------------------------------------------------------------------------------------
+// 256x256x64 main kernel
+// ---------------------------------------------------------------------------------------------------------
+
+template <bool A_KC, bool B_KC>
+struct MainCfg {
+    static constexpr int BM = 256, BN = 256, BK = 64;
+    static constexpr int WM = 2, WN = 4, NWAVES = 8, NTHREADS = 512;
+    static constexpr int TM = BM / WM / 32;  // 4 MFMA blocks along M per wave
+    static constexpr int TN = BN / WN / 32;  // 2 along N
+    using ATileK = KContigTile<BM, BK, NWAVES>;
+    using ATileM = MNContigTile<BM, BK, NWAVES>;
+    using BTileK = KContigTile<BN, BK, NWAVES>;
+    using BTileN = MNContigTile<BN, BK, NWAVES>;
+    static constexpr int A_BYTES = BM * BK * 2;
+    static constexpr int B_BYTES = BN * BK * 2;
+    static constexpr int STAGE_BYTES = A_BYTES + B_BYTES;
+    static constexpr int NSTAGE = 2;
+    static constexpr int LDS_BYTES = STAGE_BYTES * NSTAGE;
+    static constexpr int A_INSTS = 4, B_INSTS = 4;
+};
+
+// Map the linear workgroup id to a C tile so that the workgroups resident on one XCD (ids congruent mod 8)
+// cover a compact rectangle of tiles: they then share A row-panels and B column-panels in that XCD's L2.
+__device__ __forceinline__ void tile_of_block(int bid, int tiles_m, int tiles_n, int& tm, int& tn) {
+    const int total = tiles_m * tiles_n;
+    constexpr int kXcd = 8;
+    int t = bid;
+    if (total % kXcd == 0) {
+        int per = total / kXcd;
+        t = (bid % kXcd) * per + bid / kXcd;
+    }
+    // grouped ordering: walk down GROUP rows of tiles before moving to the next column
+    constexpr int GROUP = 8;
+    int group_size = GROUP * tiles_n;
+    int g = t / group_size;
+    int first_m = g * GROUP;
+    int rows = min(GROUP, tiles_m - first_m);
+    int in_g = t - g * group_size;
+    tm = first_m + in_g % rows;
+    tn = in_g / rows;
+}
+
+template <bool A_KC, bool B_KC>
+__global__ __launch_bounds__(512) void hgemm_main_kernel(const half_t* __restrict__ A, const half_t* __restrict__ B,
+                                                         half_t* __restrict__ C, int M, int N, int K, long lda,
+                                                         long ldb, long ldc) {
+    using Cfg = MainCfg<A_KC, B_KC>;
+    using ATK = typename Cfg::ATileK;
+    using ATM = typename Cfg::ATileM;
+    using BTK = typename Cfg::BTileK;
+    using BTN = typename Cfg::BTileN;
+    constexpr int TM = Cfg::TM, TN = Cfg::TN, BK = Cfg::BK;
+
+    extern __shared__ __attribute__((aligned(1024))) char smem_raw[];
+    MI355_LDS char* smem = (MI355_LDS char*)smem_raw;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave / Cfg::WN;
+    const int wn = wave % Cfg::WN;
+
+    int tile_m, tile_n;
+    tile_of_block(blockIdx.x, M / Cfg::BM, N / Cfg::BN, tile_m, tile_n);
+    const long m0 = (long)tile_m * Cfg::BM;
+    const long n0 = (long)tile_n * Cfg::BN;
+
+    // ---- global -> LDS copy descriptors --------------------------------------------------------------
+    const half_t* a_src;
+    long a_copy_stride, a_k_stride;
+    if constexpr (A_KC) {  // A stored [M,K]
+        a_src = A + m0 * lda + ATK::first_copy_offset(wave, lane, lda);
+        a_copy_stride = ATK::copy_stride(lda);
+        a_k_stride = ATK::ktile_stride(lda);
+    } else {  // A stored [K,M]
+        a_src = A + m0 + ATM::first_copy_offset(wave, lane, lda);
+        a_copy_stride = ATM::copy_stride(lda);
+        a_k_stride = ATM::ktile_stride(lda);
+    }
+    const half_t* b_src;
+    long b_copy_stride, b_k_stride;
+    if constexpr (B_KC) {  // B stored [N,K]
+        b_src = B + n0 * ldb + BTK::first_copy_offset(wave, lane, ldb);
+        b_copy_stride = BTK::copy_stride(ldb);
+        b_k_stride = BTK::ktile_stride(ldb);
+    } else {  // B stored [K,N]
+        b_src = B + n0 + BTN::first_copy_offset(wave, lane, ldb);
+        b_copy_stride = BTN::copy_stride(ldb);
+        b_k_stride = BTN::ktile_stride(ldb);
+    }
+
+    auto issue_copies = [&](int stage) {
+        MI355_LDS char* sa = smem + stage * Cfg::STAGE_BYTES;
+        MI355_LDS char* sb = sa + Cfg::A_BYTES;
+#pragma unroll
+        for (int i = 0; i < Cfg::A_INSTS; ++i)
+            copy16_global_to_lds(a_src + i * a_copy_stride, sa + (i * Cfg::NWAVES + wave) * 1024);
+#pragma unroll
+        for (int i = 0; i < Cfg::B_INSTS; ++i)
+            copy16_global_to_lds(b_src + i * b_copy_stride, sb + (i * Cfg::NWAVES + wave) * 1024);
+        a_src += a_k_stride;
+        b_src += b_k_stride;
+    };
+
+    // ---- LDS fragment read offsets (bytes inside one stage) -------------------------------------------
+    // A fragments: TM blocks of 32 rows; B fragments: TN blocks of 32 columns.
+    int a_off[4];  // K-contiguous: per k-substep; M-contiguous: per block pair (only [0..TM) used)
+    int b_off[4];
+    if constexpr (A_KC) {
+#pragma unroll
+        for (int kk = 0; kk < 4; ++kk) a_off[kk] = ATK::frag_offset(wm * TM * 32, kk, lane);
+    } else {
+#pragma unroll
+        for (int i = 0; i < TM; ++i) a_off[i] = ATM::frag_offset(wm * TM * 32 + i * 32, lane);
+    }
+    if constexpr (B_KC) {
+#pragma unroll
+        for (int kk = 0; kk < 4; ++kk) b_off[kk] = Cfg::A_BYTES + BTK::frag_offset(wn * TN * 32, kk, lane);
+    } else {
+#pragma unroll
+        for (int j = 0; j < TN; ++j) b_off[j] = Cfg::A_BYTES + BTN::frag_offset(wn * TN * 32 + j * 32, lane);
+    }
+
+    float16v acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+
+    const int ktiles = K / BK;
+    issue_copies(0);
+
+    for (int kt = 0; kt < ktiles; ++kt) {
+        wait_vmcnt<0>();
+        __syncthreads();
+        if (kt + 1 < ktiles) issue_copies((kt + 1) & 1);
+
+        MI355_LDS char* st = smem + (kt & 1) * Cfg::STAGE_BYTES;
+#pragma unroll
+        for (int kk = 0; kk < BK / 16; ++kk) {
+            half8 af[TM], bf[TN];
+#pragma unroll
+            for (int i = 0; i < TM; ++i) {
+                if constexpr (A_KC) {
+                    af[i] = lds_read_b128(st + a_off[kk] + i * 32 * ATK::kRowBytes);
+                } else {
+                    half4 lo = lds_read_tr16_b64(st + a_off[i] + (kk * 16) * ATM::kRowBytes);
+                    half4 hi = lds_read_tr16_b64(st + a_off[i] + (kk * 16 + 4) * ATM::kRowBytes);
+                    af[i] = concat(lo, hi);
+                }
+            }
+#pragma unroll
+            for (int j = 0; j < TN; ++j) {
+                if constexpr (B_KC) {
+                    bf[j] = lds_read_b128(st + b_off[kk] + j * 32 * BTK::kRowBytes);
+                } else {
+                    half4 lo = lds_read_tr16_b64(st + b_off[j] + (kk * 16) * BTN::kRowBytes);
+                    half4 hi = lds_read_tr16_b64(st + b_off[j] + (kk * 16 + 4) * BTN::kRowBytes);
+                    bf[j] = concat(lo, hi);
+                }
+            }
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bf[j], af[i], acc[i][j], 0, 0, 0);
+        }
+    }
+
+    // ---- epilogue: lane holds C[m][n .. n+3] for m = l%32, n = 8p + 4*(l/32) ----------------------------
+    const long row_base = m0 + wm * TM * 32 + (lane & 31);
+    const long col_base = n0 + wn * TN * 32 + 4 * (lane >> 5);
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+        half_t* crow = C + (row_base + i * 32) * ldc + col_base;
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+#pragma unroll
+            for (int p = 0; p < 4; ++p) {
+                half4 v;
+                v[0] = (half_t)acc[i][j][4 * p + 0];
+                v[1] = (half_t)acc[i][j][4 * p + 1];
+                v[2] = (half_t)acc[i][j][4 * p + 2];
+                v[3] = (half_t)acc[i][j][4 * p + 3];
+                *(half4*)(crow + j * 32 + 8 * p) = v;
+            }
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------------------
+// Bounds-checked kernel for any shape: 64x64 tile per wave-quad, operands gathered with guarded scalar loads
+// into the MFMA layout. Used for shapes the tiled kernels do not cover; correctness first.
+// ---------------------------------------------------------------------------------------------------------
+template <bool A_KC, bool B_KC>
+__global__ __launch_bounds__(256) void hgemm_edge_kernel(const half_t* __restrict__ A, const half_t* __restrict__ B,
+                                                         half_t* __restrict__ C, int M, int N, int K, long lda,
+                                                         long ldb, long ldc) {
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const long m = (long)blockIdx.y * 64 + (wave >> 1) * 32 + (lane & 31);
+    const long n = (long)blockIdx.x * 64 + (wave & 1) * 32 + (lane & 31);
+    const int kh = 8 * (lane >> 5);
+    float16v acc;
+#pragma unroll
+    for (int e = 0; e < 16; ++e) acc[e] = 0.f;
+    for (int k0 = 0; k0 < K; k0 += 16) {
+        half8 a, b;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            int k = k0 + kh + j;
+            bool kin = k < K;
+            half_t av = (half_t)0.f, bv = (half_t)0.f;
+            if (kin && m < M) av = A_KC ? A[m * lda + k] : A[(long)k * lda + m];
+            if (kin && n < N) bv = B_KC ? B[n * ldb + k] : B[(long)k * ldb + n];
+            a[j] = av;
+            b[j] = bv;
+        }
+        acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, acc, 0, 0, 0);
+    }
+    // acc element 4p+q is C[row 8p + 4*(lane/32) + q][col lane%32] of this wave's 32x32 block
+    const long rb = (long)blockIdx.y * 64 + (wave >> 1) * 32 + 4 * (lane >> 5);
+#pragma unroll
+    for (int p = 0; p < 4; ++p)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            long r = rb + 8 * p + q;
+            if (r < M && n < N) C[r * ldc + n] = (half_t)acc[4 * p + q];
+        }
+}
+
+template <bool A_KC, bool B_KC>
+static hipError_t launch_layout(const half_t* A, const half_t* B, half_t* C, int M, int N, int K, long lda, long ldb,
+                                long ldc, hipStream_t stream) {
+    using Cfg = MainCfg<A_KC, B_KC>;
+    const bool aligned = (reinterpret_cast<uintptr_t>(A) % 16 == 0) && (reinterpret_cast<uintptr_t>(B) % 16 == 0) &&
+                         (reinterpret_cast<uintptr_t>(C) % 8 == 0) && (lda % 8 == 0) && (ldb % 8 == 0) &&
+                         (ldc % 4 == 0);
+    if (aligned && M % Cfg::BM == 0 && N % Cfg::BN == 0 && K % Cfg::BK == 0 && K >= Cfg::BK) {
+        static bool attr_set = false;
+        auto kern = hgemm_main_kernel<A_KC, B_KC>;
+        if (!attr_set) {
+            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::LDS_BYTES);
+            if (e != hipSuccess) return e;
+            attr_set = true;
+        }
+        int blocks = (M / Cfg::BM) * (N / Cfg::BN);
+        kern<<<dim3(blocks), dim3(Cfg::NTHREADS), Cfg::LDS_BYTES, stream>>>(A, B, C, M, N, K, lda, ldb, ldc);
+        return hipGetLastError();
+    }
+    dim3 grid((N + 63) / 64, (M + 63) / 64);
+    hgemm_edge_kernel<A_KC, B_KC><<<grid, dim3(256), 0, stream>>>(A, B, C, M, N, K, lda, ldb, ldc);
+    return hipGetLastError();
+}
+
+hipError_t hgemm_dispatch(const void* A, const void* B, void* C, int M, int N, int K, long lda, long ldb, long ldc,
+                          int layout, hipStream_t stream) {
+    const half_t* a = static_cast<const half_t*>(A);
+    const half_t* b = static_cast<const half_t*>(B);
+    half_t* c = static_cast<half_t*>(C);
+    switch (layout) {
+        case MI355_GEMM_NN: return launch_layout<true, false>(a, b, c, M, N, K, lda, ldb, ldc, stream);
+        case MI355_GEMM_NT: return launch_layout<true, true>(a, b, c, M, N, K, lda, ldb, ldc, stream);
+        case MI355_GEMM_TN: return launch_layout<false, false>(a, b, c, M, N, K, lda, ldb, ldc, stream);
+        default: return hipErrorInvalidValue;
+    }
+}
+
+}  // namespace mi355

@@ -1,0 +1,75 @@
+// Shared device-side helpers for the gfx950 (MI355X, CDNA4) serving kernels.
+//
+// Everything here is written for wave64 and for the gfx950 instruction set only:
+//   * v_mfma_f32_32x32x16_f16 / v_mfma_f32_16x16x32_f16 (fp16 in, fp32 accumulate)
+//   * global_load_lds_dwordx4 (16-byte global -> LDS copies that bypass the VGPRs)
+//   * ds_read_b64_tr_b16 (LDS read that transposes a 4x16 block of 16-bit values)
+//
+// Register layouts (checked on hardware):
+//   mfma 32x32x16: operand lane l holds 8 consecutive k (k = 8*(l/32) .. +7) of row/col l%32;
+//                  accumulator element 4p+q of lane l is D[8p + 4*(l/32) + q][l%32].
+//   mfma 16x16x32: operand lane l holds k = 8*(l/16) .. +7 of row/col l%16;
+//                  accumulator element q of lane l is D[4*(l/16) + q][l%16].
+//   ds_read_b64_tr_b16: inside each group of 16 lanes, input lane j supplies the four 16-bit values
+//                  X[j/4][4*(j%4) .. +3] of a 4x16 block X; output lane i receives X[0..3][i].
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace mi355 {
+
+typedef _Float16 half_t;
+typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+typedef _Float16 half4 __attribute__((ext_vector_type(4)));
+typedef _Float16 half2v __attribute__((ext_vector_type(2)));
+typedef float float16v __attribute__((ext_vector_type(16)));
+typedef float float4v __attribute__((ext_vector_type(4)));
+typedef short short4v __attribute__((ext_vector_type(4)));
+typedef int int4v __attribute__((ext_vector_type(4)));
+typedef int int2v __attribute__((ext_vector_type(2)));
+
+#define MI355_LDS __attribute__((address_space(3)))
+#define MI355_GLOBAL __attribute__((address_space(1)))
+
+// s_waitcnt immediates (gfx9 encoding): vmcnt = bits [3:0] and [15:14], expcnt [6:4], lgkmcnt [11:8].
+__device__ __forceinline__ constexpr int waitcnt_imm(int vm, int lgkm) {
+    return (vm & 0xF) | ((vm >> 4) << 14) | (0x7 << 4) | ((lgkm & 0xF) << 8);
+}
+template <int VM>
+__device__ __forceinline__ void wait_vmcnt() {
+    __builtin_amdgcn_s_waitcnt(waitcnt_imm(VM, 0xF));
+}
+template <int LGKM>
+__device__ __forceinline__ void wait_lgkmcnt() {
+    __builtin_amdgcn_s_waitcnt(waitcnt_imm(0x3F, LGKM));
+}
+
+// 16-byte global -> LDS copy (global_load_lds_dwordx4). Lane l of the wave writes LDS bytes
+// [lds_wave_base + 16*l, +16); lds_wave_base must be wave-uniform (it travels in M0).
+// Written as inline assembly on purpose: the compiler then does not treat the copy as an LDS store, so it
+// does not put a full "s_waitcnt vmcnt(0)" in front of every later LDS read. The caller orders the copy
+// against LDS reads itself: wait_vmcnt<N>() followed by a workgroup barrier before the data is read.
+__device__ __forceinline__ void copy16_global_to_lds(const void* gptr, MI355_LDS void* lds_wave_base) {
+    asm volatile(
+        "s_mov_b32 m0, %1\n\t"
+        "s_nop 0\n\t"
+        "global_load_lds_dwordx4 %0, off"
+        :
+        : "v"(gptr), "s"((uint32_t)(uintptr_t)lds_wave_base)
+        : "memory", "m0");
+}
+
+__device__ __forceinline__ half4 lds_read_tr16_b64(MI355_LDS const void* p) {
+    short4v t = __builtin_amdgcn_ds_read_tr16_b64_v4i16((MI355_LDS short4v*)p);
+    return __builtin_bit_cast(half4, t);
+}
+
+__device__ __forceinline__ half8 lds_read_b128(MI355_LDS const void* p) {
+    return *(MI355_LDS const half8*)p;
+}
+
+__device__ __forceinline__ half8 concat(half4 lo, half4 hi) {
+    return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+}
+
+}  // namespace mi355

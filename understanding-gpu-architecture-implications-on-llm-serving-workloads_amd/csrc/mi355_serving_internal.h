@@ -1,0 +1,16 @@
+// Internal C++ entry points behind the C ABI of include/mi355_serving.h.
+#pragma once
+#include <hip/hip_runtime.h>
+#include "../../include/mi355_serving.h"
+
+namespace mi355 {
+
+// Launches the GEMM kernels; arguments as mi355_hgemm after validation.
+hipError_t hgemm_dispatch(const void* A, const void* B, void* C, int M, int N, int K, long lda, long ldb, long ldc,
+                          int layout, hipStream_t stream);
+
+// Launches the attention forward kernels; arguments as mi355_fmha_fwd after validation.
+hipError_t fmha_fwd_dispatch(const void* Q, const void* K, const void* V, void* O, float* LSE, int B, int Hq, int Hkv,
+                             int Sq, int Sk, float scale, int causal, int kv_valid_len, hipStream_t stream);
+
+}  // namespace mi355
