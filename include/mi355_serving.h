@@ -66,6 +66,7 @@ int mi355_hgemm(const void* A, const void* B, void* C, int M, int N, int K, int6
  *   causal != 0  : key j is visible to query i iff j <= i + (Sk - Sq), i.e. the mask is aligned to the
  *                  bottom-right corner; with Sq == Sk this is the reference's `q_pos < k_pos => masked`
  *                  rule (fmha_2_amd.cpp:187-190).
+ *   scale        : softmax scale, positive and finite (the operators pass 1/sqrt(D), fmha_2_amd.cpp:320).
  *   Sq and Sk are arbitrary (>= 1); ragged tails are masked inside the kernel, no padding is needed.
  *   A query row with no visible key yields O = 0 and LSE = -inf.
  */

@@ -1,0 +1,261 @@
+"""CPU oracle for the two serving kernels: fp16 GEMM and fused attention forward.
+
+TEST INFRASTRUCTURE ONLY. Nothing in the product (the HIP library, the torch operators, their python shims)
+imports this module; it is used by tests/, by __graft_entry__.smoke() and by bench.py's cpu_baseline leg, as
+the checker and as the timed CPU baseline, never as the implementation.
+
+What it restates. The reference's path is CUDA/HIP device code with no CPU implementation, and none of it can be
+compiled or run without a GPU; every function on the path is a realisation of one of two textbook results, so the
+oracle states those results directly in fp32 (torch) and, for small inputs, again in fp64 with explicit loops:
+
+  gemm_ref            C = op(a) op(b) in fp32 over the fp16-rounded operands. Layout per operator index follows
+                      kernels/gemm/test/correct.py:9-15 (a.T @ b for a_format 'N', a @ b.T for b_format 'N') and
+                      the loads in manual/gemm_12_amd.cpp:52-57, gemm_13_amd.cpp:58-60, gemm_16_amd.cpp:55-57.
+  attention_ref       O = softmax(scale q k^T + mask) v and LSE, fp32. GQA head mapping follows
+                      kernels/fmha/test/perf.py:10-24 (repeat_kv == repeat_interleave on the head axis) and
+                      semi/fmha_2_amd.cpp:33-42; causal rule "masked iff q_pos < k_pos" follows fmha_2_amd.cpp:187-190
+                      generalised to the bottom-right alignment (identical when Sq == Sk); keys at or beyond
+                      kv_valid_len are masked (fmha_2_amd.cpp:191 with its off-by-one corrected); scale 1/sqrt(d)
+                      follows fmha_2_amd.cpp:320.
+  fine_fmha_ref       the pad-to-64 / decode_length / slice shim of kernels/fmha/pkg/fmha_unified/ops.py:8-29
+                      expressed on top of attention_ref (padding rows are masked, so it reduces to attention_ref).
+  llama_layer_ref     the Llama-3-8B-shaped prefill chain of the benchmark configuration (QKV GEMM -> causal GQA
+                      attention -> O projection -> gate/up GEMM -> SiLU(gate)*up -> down GEMM), fp32.
+
+Reference-specific numerical behaviour (fp16 accumulation in finegemm_0..11, fp16 softmax statistics in
+finefmha_0..3) is deliberately NOT restated: the parity target is the fp32 result.
+
+Pinning. The reference's tests hold no stored vectors (only seeded generators: correct.py seeds 0 / 42), so the
+oracle is pinned by what the mathematics fixes; tests/test_oracle.py checks every function below against closed
+forms (identity, one-hot, all-ones, exact power-of-two sums; uniform-softmax running means, single visible key,
+V = ones, dominant key, key-permutation invariance, GQA head sharing), against fp64 brute force written with
+explicit loops (gemm_bruteforce_f64, attention_bruteforce_f64), and against torch's own
+scaled_dot_product_attention as a second opinion. No function here is "parity unpinned".
+"""
+import math
+
+import numpy as np
+import torch
+
+GEMM_LAYOUT_OF_INDEX = {i: "NN" for i in range(12)}
+GEMM_LAYOUT_OF_INDEX.update({12: "TN", 16: "TN", 13: "NT", 14: "NT", 15: "NT"})
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# GEMM
+# ---------------------------------------------------------------------------------------------------------------
+def gemm_ref(a: torch.Tensor, b: torch.Tensor, layout: str = "NN") -> torch.Tensor:
+    """fp32 product of the (fp16-valued) operands. layout NN: a[M,K] b[K,N]; TN: a[K,M]; NT: b[N,K]."""
+    a32 = a.detach().to("cpu", torch.float32)
+    b32 = b.detach().to("cpu", torch.float32)
+    if layout == "TN":
+        a32 = a32.t()
+    elif layout == "NT":
+        b32 = b32.t()
+    elif layout != "NN":
+        raise ValueError(layout)
+    return a32 @ b32
+
+
+def fine_gemm_ref(a, b, kernel_index: int) -> torch.Tensor:
+    """What gemm_unified.ops.fine_gemm(a, b, kernel_index) must return, in fp32."""
+    return gemm_ref(a, b, GEMM_LAYOUT_OF_INDEX[int(kernel_index)])
+
+
+def gemm_bruteforce_f64(a, b, layout: str = "NN") -> np.ndarray:
+    """Triple loop in fp64 (small inputs only)."""
+    a = np.asarray(a, dtype=np.float64)
+    b = np.asarray(b, dtype=np.float64)
+    if layout == "TN":
+        a = a.T
+    if layout == "NT":
+        b = b.T
+    M, K = a.shape
+    K2, N = b.shape
+    assert K == K2
+    c = np.zeros((M, N), dtype=np.float64)
+    for i in range(M):
+        for j in range(N):
+            s = 0.0
+            for k in range(K):
+                s += a[i, k] * b[k, j]
+            c[i, j] = s
+    return c
+
+
+def gemm_tolerance_ok(c, ref, K: int):
+    """Element-wise |err| <= 2e-2*sqrt(K/1024) + 1e-2*|ref| and max|err|/max|ref| <= 1e-2. Returns (ok, stats)."""
+    c32 = c.detach().to("cpu", torch.float32)
+    r32 = ref.detach().to("cpu", torch.float32)
+    err = (c32 - r32).abs()
+    bound = 2e-2 * math.sqrt(K / 1024.0) + 1e-2 * r32.abs()
+    elem_ok = bool((err <= bound).all())
+    max_ref = float(r32.abs().max())
+    rel = float(err.max()) / max_ref if max_ref > 0 else float(err.max())
+    return elem_ok and rel <= 1e-2, {"max_abs_err": float(err.max()), "max_rel_to_max": rel,
+                                     "violations": int((err > bound).sum())}
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# attention
+# ---------------------------------------------------------------------------------------------------------------
+def visible_mask(Sq: int, Sk: int, causal: bool, kv_valid_len=None) -> torch.Tensor:
+    """Boolean [Sq, Sk]: True where key j is visible to query i."""
+    if kv_valid_len is None:
+        kv_valid_len = Sk
+    j = torch.arange(Sk)[None, :]
+    i = torch.arange(Sq)[:, None]
+    vis = (j < kv_valid_len).expand(Sq, Sk).clone()
+    if causal:
+        vis &= j <= i + (Sk - Sq)
+    return vis
+
+
+def attention_ref(q, k, v, causal: bool = False, kv_valid_len=None, scale=None):
+    """fp32 softmax attention. q [B,Hq,Sq,D], k, v [B,Hkv,Sk,D]. Returns (O [B,Hq,Sq,D], LSE [B,Hq,Sq]) fp32.
+
+    Rows with no visible key give O = 0 and LSE = -inf.
+    """
+    q32 = q.detach().to("cpu", torch.float32)
+    k32 = k.detach().to("cpu", torch.float32)
+    v32 = v.detach().to("cpu", torch.float32)
+    B, Hq, Sq, D = q32.shape
+    Hkv, Sk = k32.shape[1], k32.shape[2]
+    assert Hq % Hkv == 0
+    rep = Hq // Hkv
+    if rep > 1:
+        k32 = k32.repeat_interleave(rep, dim=1)
+        v32 = v32.repeat_interleave(rep, dim=1)
+    if scale is None:
+        scale = 1.0 / math.sqrt(D)
+    vis = visible_mask(Sq, Sk, causal, kv_valid_len)
+    out = torch.empty_like(q32)
+    lse = torch.empty((B, Hq, Sq), dtype=torch.float32)
+    for b in range(B):  # head by head keeps the score matrix small
+        for h in range(Hq):
+            s = (q32[b, h] @ k32[b, h].t()) * scale
+            s = s.masked_fill(~vis, float("-inf"))
+            l = torch.logsumexp(s, dim=-1)
+            p = torch.exp(s - torch.where(torch.isinf(l), torch.zeros_like(l), l)[:, None])
+            p = torch.where(vis, p, torch.zeros_like(p))
+            out[b, h] = p @ v32[b, h]
+            lse[b, h] = l
+    return out, lse
+
+
+def fine_fmha_ref(q, k, v, causal: bool, is_decode: bool):
+    """What fmha_unified.ops.fine_fmha must return (fp32): ops.py:8-29 pads to 64, passes decode_length =
+    un-padded key count, slices the padded query rows off. Padded keys are masked, padded queries are dropped,
+    so this equals attention over the un-padded tensors."""
+    if is_decode and causal:
+        raise ValueError("causal is not supported in decode mode")  # semi/fmha_2_amd.cpp:331-333
+    return attention_ref(q, k, v, causal=causal, kv_valid_len=k.shape[2])[0]
+
+
+def attention_bruteforce_f64(q, k, v, causal=False, kv_valid_len=None, scale=None):
+    """Explicit-loop fp64 attention (tiny inputs only). Returns (O, LSE) as numpy arrays."""
+    q = np.asarray(q, dtype=np.float64)
+    k = np.asarray(k, dtype=np.float64)
+    v = np.asarray(v, dtype=np.float64)
+    B, Hq, Sq, D = q.shape
+    Hkv, Sk = k.shape[1], k.shape[2]
+    rep = Hq // Hkv
+    if scale is None:
+        scale = 1.0 / math.sqrt(D)
+    if kv_valid_len is None:
+        kv_valid_len = Sk
+    O = np.zeros((B, Hq, Sq, D))
+    L = np.full((B, Hq, Sq), -np.inf)
+    for b in range(B):
+        for h in range(Hq):
+            hk = h // rep
+            for i in range(Sq):
+                scores = []
+                for j in range(Sk):
+                    if j >= kv_valid_len or (causal and j > i + (Sk - Sq)):
+                        continue
+                    scores.append((j, scale * float(np.dot(q[b, h, i], k[b, hk, j]))))
+                if not scores:
+                    continue
+                m = max(s for _, s in scores)
+                den = sum(math.exp(s - m) for _, s in scores)
+                acc = np.zeros(D)
+                for j, s in scores:
+                    acc += math.exp(s - m) / den * v[b, hk, j]
+                O[b, h, i] = acc
+                L[b, h, i] = m + math.log(den)
+    return O, L
+
+
+def fmha_tolerance_ok(o, lse, o_ref, lse_ref):
+    """max|O - O_ref| <= 2e-3 and max|LSE - LSE_ref| <= 1e-3 (rows with -inf LSE must match exactly)."""
+    o32 = o.detach().to("cpu", torch.float32)
+    eo = float((o32 - o_ref).abs().max())
+    stats = {"max_abs_err_o": eo}
+    ok = eo <= 2e-3
+    if lse is not None:
+        l32 = lse.detach().to("cpu", torch.float32)
+        inf_ref = torch.isinf(lse_ref)
+        same_inf = bool((torch.isinf(l32) == inf_ref).all())
+        fin = ~inf_ref
+        el = float((l32[fin] - lse_ref[fin]).abs().max()) if fin.any() else 0.0
+        stats["max_abs_err_lse"] = el
+        ok = ok and same_inf and el <= 1e-3
+    return ok, stats
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# Llama-3-8B-shaped prefill layer (benchmark configuration 5): hidden 4096, 32 q / 8 kv heads, d 128, FFN 14336
+# ---------------------------------------------------------------------------------------------------------------
+def llama_layer_ref(x, w_qkv, w_o, w_gu, w_d, n_q=32, n_kv=8, d=128, stage_inputs=None):
+    """fp32 chain. x [S, H]; weights stored [K, N]. Returns dict of every stage's fp32 output.
+
+    stage_inputs, when given, maps a stage name to the tensor to feed INTO that stage instead of the oracle's own
+    previous output (used to check each GPU stage against an oracle fed the GPU's previous-stage result)."""
+    si = stage_inputs or {}
+    f = lambda t: t.detach().to("cpu", torch.float32)
+    S = x.shape[0]
+    out = {}
+    qkv = f(si.get("qkv_in", x)) @ f(w_qkv)
+    out["qkv"] = qkv
+    qkv_used = f(si.get("attn_in", qkv.half()))
+    q = qkv_used[:, : n_q * d].reshape(S, n_q, d).permute(1, 0, 2)[None]
+    k = qkv_used[:, n_q * d: (n_q + n_kv) * d].reshape(S, n_kv, d).permute(1, 0, 2)[None]
+    v = qkv_used[:, (n_q + n_kv) * d:].reshape(S, n_kv, d).permute(1, 0, 2)[None]
+    o, lse = attention_ref(q, k, v, causal=True)
+    out["attn"] = o
+    out["attn_lse"] = lse
+    attn_used = f(si.get("oproj_in", o.half()))
+    a2 = attn_used[0].permute(1, 0, 2).reshape(S, n_q * d)
+    out["oproj"] = a2 @ f(w_o)
+    gu = f(si.get("gu_in", out["oproj"].half())) @ f(w_gu)
+    out["gate_up"] = gu
+    gu_used = f(si.get("act_in", gu.half()))
+    ffn = w_gu.shape[1] // 2
+    act = torch.nn.functional.silu(gu_used[:, :ffn]) * gu_used[:, ffn:]
+    out["act"] = act
+    out["down"] = f(si.get("down_in", act.half())) @ f(w_d)
+    return out
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# seeded synthetic inputs of the benchmark configurations (generated on the CPU, rounded to fp16)
+# ---------------------------------------------------------------------------------------------------------------
+def randn_fp16(shape, seed, std=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(shape, generator=g, dtype=torch.float32) * std).to(torch.float16)
+
+
+def gemm_inputs(M, N, K, seed=0, a_std=1.0, b_std=1.0):
+    g = torch.Generator().manual_seed(seed)
+    a = (torch.randn((M, K), generator=g, dtype=torch.float32) * a_std).to(torch.float16)
+    b = (torch.randn((K, N), generator=g, dtype=torch.float32) * b_std).to(torch.float16)
+    return a, b
+
+
+def fmha_inputs(B, Hq, Hkv, Sq, Sk, D=128, seed=42, std=1.0):
+    g = torch.Generator().manual_seed(seed)
+    q = (torch.randn((B, Hq, Sq, D), generator=g, dtype=torch.float32) * std).to(torch.float16)
+    k = (torch.randn((B, Hkv, Sk, D), generator=g, dtype=torch.float32) * std).to(torch.float16)
+    v = (torch.randn((B, Hkv, Sk, D), generator=g, dtype=torch.float32) * std).to(torch.float16)
+    return q, k, v

@@ -1,0 +1,105 @@
+"""CPU-only checks of the drop-in boundary: the C-ABI library loads and exports every symbol the header declares,
+argument validation rejects bad calls before any device work, and the torch operator surface (schemas, python
+shims, error behaviour) matches the reference's (kernels/*/pkg/*_unified/csrc/*_kernel.cpp, ops.py)."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "mi355_serving.h")
+
+
+def declared_functions():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(mi355_\w+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol(lib):
+    names = declared_functions()
+    assert names == sorted(lib.EXPORTED_SYMBOLS)
+    cdll = lib.load()
+    for n in names:
+        assert getattr(cdll, n) is not None
+    assert cdll.mi355_serving_version() == 100
+
+
+def test_capi_rejects_bad_arguments_without_a_gpu(lib):
+    cdll = lib.load()
+    assert cdll.mi355_hgemm(None, None, None, 4, 4, 4, 4, 4, 4, 0, None) == 10001
+    assert b"null pointer" in cdll.mi355_last_error()
+    p = ctypes.c_void_p(0x1000)
+    assert cdll.mi355_hgemm(p, p, p, 0, 4, 4, 4, 4, 4, 0, None) == 10001
+    assert cdll.mi355_hgemm(p, p, p, 4, 4, 4, 4, 4, 4, 7, None) == 10001
+    assert b"layout" in cdll.mi355_last_error()
+    assert cdll.mi355_hgemm(p, p, p, 4, 8, 4, 4, 4, 4, 0, None) == 10001  # ldb < N
+    assert cdll.mi355_fmha_fwd(p, p, p, p, None, 1, 4, 1, 8, 8, 64, 0.1, 0, 8, None) == 10002  # head_dim != 128
+    assert b"128" in cdll.mi355_last_error()
+    assert cdll.mi355_fmha_fwd(p, p, p, p, None, 1, 5, 2, 8, 8, 128, 0.1, 0, 8, None) == 10001  # Hq % Hkv
+    assert cdll.mi355_fmha_fwd(p, p, p, p, None, 1, 4, 2, 8, 8, 128, 0.1, 0, 9, None) == 10001  # kv_valid > Sk
+    assert cdll.mi355_fmha_fwd(p, p, p, p, None, 1, 4, 2, 8, 8, 128, -1.0, 0, 8, None) == 10001  # scale <= 0
+    with pytest.raises(lib.Mi355Error):
+        lib.hgemm_raw(0, 0, 0, 4, 4, 4, 4, 4, 4, 0)
+
+
+def test_operator_schemas_match_reference():
+    import fmha_unified  # noqa: F401
+    import gemm_unified  # noqa: F401
+    for i in range(17):  # gemm_kernel.cpp:10-26
+        op = getattr(torch.ops.gemm_unified, f"finegemm_{i}").default
+        assert str(op._schema) == f"gemm_unified::finegemm_{i}(Tensor a, Tensor b) -> Tensor"
+    for i in range(8):  # fmha_kernel.cpp:10-17
+        op = getattr(torch.ops.fmha_unified, f"finefmha_{i}").default
+        assert str(op._schema) == (f"fmha_unified::finefmha_{i}(Tensor q, Tensor k, Tensor v, bool causal, "
+                                   "bool is_decode, int decode_length) -> Tensor")
+    assert "-> (Tensor, Tensor)" in str(torch.ops.fmha_unified.finefmha_fwd_lse.default._schema)
+
+
+def test_gemm_operator_validation_errors():
+    import gemm_unified
+    a = torch.randn(8, 8).half()
+    with pytest.raises(RuntimeError, match="GPU tensors"):
+        gemm_unified.ops.fine_gemm(a, a, 0)
+    with pytest.raises(RuntimeError, match="float16"):
+        gemm_unified.ops.fine_gemm(a.float(), a, 0)
+    with pytest.raises(RuntimeError, match="inner dimensions"):
+        gemm_unified.ops.fine_gemm(a[:, :4], a, 0)
+    with pytest.raises(RuntimeError, match="inner dimensions"):  # index 13 reads b as [N, K]
+        gemm_unified.ops.fine_gemm(a, a[:, :4], 13)
+    with pytest.raises(RuntimeError, match="2-D"):
+        gemm_unified.ops.fine_gemm(a[None], a, 0)
+    with pytest.raises(AttributeError):
+        gemm_unified.ops.fine_gemm(a, a, 17)
+    assert gemm_unified.ops.LAYOUT_OF_INDEX[16] == "TN" and gemm_unified.ops.LAYOUT_OF_INDEX[14] == "NT"
+
+
+def test_fmha_operator_validation_errors():
+    import fmha_unified
+    q = torch.randn(1, 4, 8, 128).half()
+    kv = torch.randn(1, 2, 8, 128).half()
+    with pytest.raises(RuntimeError, match="GPU tensors"):
+        fmha_unified.ops.fine_fmha(q, kv, kv, True, False, 2)
+    with pytest.raises(RuntimeError, match="128"):
+        fmha_unified.ops.fine_fmha(q[..., :64], kv[..., :64], kv[..., :64], True, False, 2)
+    with pytest.raises(RuntimeError, match="float16"):
+        fmha_unified.ops.fine_fmha(q.float(), kv, kv, True, False, 2)
+    with pytest.raises(RuntimeError, match="decode"):  # semi/fmha_2_amd.cpp:331-333
+        fmha_unified.ops.fine_fmha(q, kv, kv, True, True, 2)
+    with pytest.raises(RuntimeError, match="multiple of kv heads"):
+        fmha_unified.ops.fine_fmha(q[:, :3], kv, kv, False, False, 2)
+    with pytest.raises(RuntimeError, match="decode_length"):
+        torch.ops.fmha_unified.finefmha_2.default(q, kv, kv, False, False, 9)
+    with pytest.raises(RuntimeError, match="v shape"):
+        fmha_unified.ops.fine_fmha(q, kv, kv[:, :, :4], False, False, 2)
+
+
+def test_product_code_does_not_touch_the_oracle():
+    pkg = os.path.join(ROOT, "understanding-gpu-architecture-implications-on-llm-serving-workloads_amd")
+    for dirpath, _, files in os.walk(pkg):
+        for f in files:
+            if f.endswith((".py", ".cpp", ".hip", ".h")):
+                text = open(os.path.join(dirpath, f)).read()
+                assert "serving_oracle" not in text and "oracle/" not in text, os.path.join(dirpath, f)

@@ -1,0 +1,193 @@
+"""GPU parity tests of the fused attention forward: the HIP kernel called through the C ABI (ctypes) and through
+the torch operators, against the CPU oracle on the same seeded inputs. Tolerance (benchmark definition):
+max|O - O_ref| <= 2e-3 and max|LSE - LSE_ref| <= 1e-3 against fp32 softmax attention."""
+import math
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import serving_oracle as so
+
+pytestmark = pytest.mark.gpu
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+
+
+def run(lib, gpu, q, k, v, causal=False, kv_valid_len=None):
+    o, lse = lib.fmha_fwd(q.to(gpu), k.to(gpu), v.to(gpu), causal=causal, kv_valid_len=kv_valid_len)
+    torch.cuda.synchronize()
+    return o.cpu(), lse.cpu()
+
+
+def check(lib, gpu, q, k, v, causal=False, kv_valid_len=None):
+    o, lse = run(lib, gpu, q, k, v, causal, kv_valid_len)
+    o_ref, lse_ref = so.attention_ref(q, k, v, causal=causal, kv_valid_len=kv_valid_len)
+    ok, st = so.fmha_tolerance_ok(o, lse, o_ref, lse_ref)
+    assert ok, (tuple(q.shape), tuple(k.shape), causal, kv_valid_len, st)
+    return o, lse
+
+
+# ---- benchmark configurations ------------------------------------------------------------------------------------
+def test_config_f3_noncausal_mha(lib, gpu):
+    q, k, v = so.fmha_inputs(4, 32, 32, 1024, 1024, seed=42)
+    check(lib, gpu, q, k, v, causal=False)
+
+
+def test_config_f4_causal_gqa_with_lse(lib, gpu):
+    q, k, v = so.fmha_inputs(1, 32, 8, 4096, 4096, seed=42)
+    o, lse = check(lib, gpu, q, k, v, causal=True)
+    assert lse.shape == (1, 32, 4096) and lse.dtype == torch.float32
+
+
+# ---- closed forms ---------------------------------------------------------------------------------------------------
+def test_equal_keys_running_mean(lib, gpu):
+    B, H, S = 1, 2, 333
+    q = so.randn_fp16((B, H, S, 128), 1)
+    k = so.randn_fp16((B, H, 1, 128), 2).expand(B, H, S, 128).contiguous()
+    v = so.randn_fp16((B, H, S, 128), 3)
+    o, lse = run(lib, gpu, q, k, v, causal=True)
+    vm = v.float().cumsum(2) / torch.arange(1, S + 1)[None, None, :, None]
+    s0 = (q.float() * k.float()).sum(-1) / math.sqrt(128)
+    assert (o.float() - vm).abs().max() <= 2e-3
+    assert (lse - (s0 + torch.log(torch.arange(1, S + 1).float()))).abs().max() <= 1e-3
+
+
+def test_first_causal_row_is_first_value_exactly(lib, gpu):
+    q, k, v = so.fmha_inputs(2, 4, 2, 200, 200, seed=5)
+    o, lse = run(lib, gpu, q, k, v, causal=True)
+    assert torch.equal(o[:, :, 0], v.repeat_interleave(2, 1)[:, :, 0])
+    s00 = (q.float()[:, :, 0] * k.float().repeat_interleave(2, 1)[:, :, 0]).sum(-1) / math.sqrt(128)
+    assert (lse[:, :, 0] - s00).abs().max() <= 1e-4
+
+
+def test_ones_value_rows_sum_to_one_and_zero_query_lse(lib, gpu):
+    q, k, _ = so.fmha_inputs(1, 2, 2, 150, 777, seed=6)
+    v = torch.ones(1, 2, 777, 128).half()
+    o, _ = run(lib, gpu, q, k, v, causal=False)
+    assert (o.float() - 1).abs().max() <= 1e-3
+    o, lse = run(lib, gpu, torch.zeros_like(q), k, v, causal=True)  # Sq=150 < Sk=777: query i sees 628+i keys
+    assert (lse[0, 0] - torch.log(torch.arange(628, 778).float())).abs().max() <= 1e-4
+
+
+def test_dominant_key_selects_its_value(lib, gpu):
+    _, k, v = so.fmha_inputs(1, 1, 1, 64, 500, seed=7)
+    q = (k[:, :, 321:322] * 8).expand(1, 1, 64, 128).contiguous()
+    o, _ = run(lib, gpu, q, k, v)
+    assert (o.float() - v.float()[:, :, 321:322]).abs().max() <= 2e-3
+
+
+def test_key_permutation_invariance_across_tiles(lib, gpu):
+    q, k, v = so.fmha_inputs(1, 2, 1, 96, 1000, seed=8)
+    perm = torch.randperm(1000, generator=torch.Generator().manual_seed(1))
+    o1, l1 = run(lib, gpu, q, k, v)
+    o2, l2 = run(lib, gpu, q, k[:, :, perm].contiguous(), v[:, :, perm].contiguous())
+    assert (o1.float() - o2.float()).abs().max() <= 2e-3 and (l1 - l2).abs().max() <= 1e-4
+
+
+def test_gqa_heads_sharing_kv_with_identical_queries_agree(lib, gpu):
+    q1 = so.randn_fp16((1, 1, 130, 128), 9)
+    q = q1.expand(1, 8, 130, 128).contiguous()
+    _, k, v = so.fmha_inputs(1, 8, 2, 130, 130, seed=10)
+    o, lse = run(lib, gpu, q, k, v, causal=True)
+    for g in range(2):
+        for h in range(1, 4):
+            assert torch.equal(o[:, 4 * g + h], o[:, 4 * g]) and torch.equal(lse[:, 4 * g + h], lse[:, 4 * g])
+    assert not torch.equal(o[:, 0], o[:, 4])
+
+
+# ---- ragged shapes, masks, decode -----------------------------------------------------------------------------------
+@pytest.mark.parametrize("B,Hq,Hkv,Sq,Sk,causal,kvv", [
+    (1, 1, 1, 128, 128, False, None), (1, 1, 1, 128, 128, True, None), (1, 4, 1, 128, 128, True, None),
+    (2, 4, 2, 100, 77, False, None), (2, 4, 2, 100, 177, True, None), (1, 2, 1, 300, 300, True, 290),
+    (1, 2, 2, 70, 40, True, None),      # Sq > Sk, causal: the first 30 queries see no key
+    (1, 2, 2, 1, 333, False, None),     # decode step: one query
+    (3, 6, 3, 1, 64, False, 50), (1, 2, 1, 65, 129, True, None), (1, 1, 1, 8, 8, True, None),
+    (1, 2, 2, 257, 63, False, 1), (1, 3, 1, 511, 513, True, 512), (2, 2, 2, 64, 1024, True, None),
+])
+def test_ragged_shapes_and_masks(lib, gpu, B, Hq, Hkv, Sq, Sk, causal, kvv):
+    q, k, v = so.fmha_inputs(B, Hq, Hkv, Sq, Sk, seed=Sq * 7 + Sk)
+    o, lse = check(lib, gpu, q, k, v, causal, kvv)
+    if causal and Sq > Sk:
+        n = Sq - Sk
+        assert bool((o[:, :, :n] == 0).all()) and bool(torch.isinf(lse[:, :, :n]).all()) and bool((lse[:, :, :n] < 0).all())
+
+
+def test_masked_keys_may_hold_garbage(lib, gpu):
+    # keys at or beyond kv_valid_len must not influence the result, whatever they contain
+    q, k, v = so.fmha_inputs(1, 2, 2, 90, 200, seed=11)
+    k2, v2 = k.clone(), v.clone()
+    k2[:, :, 150:] = float("nan")
+    v2[:, :, 150:] = float("inf")
+    o1, l1 = run(lib, gpu, q, k, v, False, 150)
+    o2, l2 = run(lib, gpu, q, k2, v2, False, 150)
+    assert torch.equal(o1, o2) and torch.equal(l1, l2)
+
+
+def test_lse_pointer_is_optional(lib, gpu):
+    q, k, v = (t.to(gpu) for t in so.fmha_inputs(1, 2, 1, 100, 100, seed=12))
+    o1 = lib.fmha_fwd(q, k, v, causal=True, return_lse=False)
+    o2, _ = lib.fmha_fwd(q, k, v, causal=True)
+    assert torch.equal(o1, o2)
+
+
+def test_reference_seeded_case_from_golden_fixture(lib, gpu):
+    z = np.load(os.path.join(GOLDEN, "fmha_seed42_128.npz"))
+    q, k, v = (torch.from_numpy(z[n]) for n in ("q", "k", "v"))
+    rows = z["qrows"]
+    for tag, causal in (("full", False), ("causal", True)):
+        o, lse = run(lib, gpu, q, k, v, causal)
+        assert np.abs(o.float().numpy()[:, :, rows] - z["o_" + tag]).max() <= 2e-3
+        assert np.abs(lse.numpy() - z["lse_" + tag]).max() <= 1e-3
+
+
+# ---- size-independent properties at the benchmark size --------------------------------------------------------------
+def test_full_size_split_kv_merge_with_lse(lib, gpu):
+    # attention over all keys == LSE-weighted merge of attention over two halves of the keys (non-causal)
+    q, k, v = (t.to(gpu) for t in so.fmha_inputs(1, 32, 8, 4096, 4096, seed=42))
+    o, lse = lib.fmha_fwd(q, k, v)
+    o1, l1 = lib.fmha_fwd(q, k[:, :, :2048].contiguous(), v[:, :, :2048].contiguous())
+    o2, l2 = lib.fmha_fwd(q, k[:, :, 2048:].contiguous(), v[:, :, 2048:].contiguous())
+    lm = torch.logaddexp(l1, l2)
+    merged = torch.exp(l1 - lm)[..., None] * o1.float() + torch.exp(l2 - lm)[..., None] * o2.float()
+    assert (lm - lse).abs().max() <= 1e-3
+    assert (merged - o.float()).abs().max() <= 3e-3  # two fp16 roundings of the halves
+    # causal: rows of the last tile against kv_valid_len truncation of the non-causal kernel
+    oc, lc = lib.fmha_fwd(q, k, v, causal=True)
+    ot, lt = lib.fmha_fwd(q[:, :, 2047:2048].contiguous(), k, v, causal=False, kv_valid_len=2048)
+    assert (oc[:, :, 2047:2048].float() - ot.float()).abs().max() <= 2e-3 and (lc[:, :, 2047:2048] - lt).abs().max() <= 1e-3
+
+
+# ---- torch operator path ----------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("index", list(range(8)))
+def test_torch_operator_every_index(gpu, index):
+    import fmha_unified
+    q, k, v = so.fmha_inputs(1, 8, 2, 200, 200, seed=index)
+    o = fmha_unified.ops.fine_fmha(q.to(gpu), k.to(gpu), v.to(gpu), True, False, index)
+    assert o.dtype == torch.float16 and o.shape == q.shape
+    ok, st = so.fmha_tolerance_ok(o, None, so.fine_fmha_ref(q, k, v, True, False), None)
+    assert ok, (index, st)
+
+
+def test_torch_operator_decode_and_lse(gpu):
+    import fmha_unified
+    q, k, v = so.fmha_inputs(2, 8, 2, 1, 301, seed=3)
+    o = fmha_unified.ops.fine_fmha(q.to(gpu), k.to(gpu), v.to(gpu), False, True, 2)
+    ok, st = so.fmha_tolerance_ok(o, None, so.fine_fmha_ref(q, k, v, False, True), None)
+    assert ok, st
+    o2, lse = fmha_unified.ops.fine_fmha_with_lse(q.to(gpu), k.to(gpu), v.to(gpu), False)
+    o_ref, lse_ref = so.attention_ref(q, k, v)
+    ok, st = so.fmha_tolerance_ok(o2, lse, o_ref, lse_ref)
+    assert ok, st
+
+
+def test_torch_operator_accepts_reference_style_padded_call(gpu):
+    # the reference's ops.py pads q, k, v to a multiple of 64 and passes the un-padded key count as decode_length;
+    # calling the operator that way must give the un-padded result in the first Sq rows
+    import torch.nn.functional as F
+    import fmha_unified  # noqa: F401
+    q, k, v = so.fmha_inputs(1, 4, 1, 100, 100, seed=4)
+    pad = lambda t: F.pad(t, (0, 0, 0, 28)).contiguous().to(gpu)
+    o = torch.ops.fmha_unified.finefmha_2.default(pad(q), pad(k), pad(v), True, False, 100)[:, :, :100]
+    ok, st = so.fmha_tolerance_ok(o, None, so.fine_fmha_ref(q, k, v, True, False), None)
+    assert ok, st

@@ -1,0 +1,162 @@
+"""GPU parity tests of the fp16 GEMM: the HIP kernels called through the C ABI (ctypes) and through the torch
+operators, compared with the CPU oracle on the same seeded inputs. Tolerance (stated by the benchmark definition):
+|err| <= 2e-2*sqrt(K/1024) + 1e-2*|ref| element-wise and max|err| / max|ref| <= 1e-2; cases whose exact answer is
+representable are compared bit-exactly."""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import serving_oracle as so
+
+pytestmark = pytest.mark.gpu
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+
+
+def run(lib, gpu, a, b, layout="NN"):
+    c = lib.hgemm(a.to(gpu), b.to(gpu), layout)
+    torch.cuda.synchronize()
+    return c.cpu()
+
+
+def check(lib, gpu, a, b, layout, K):
+    c = run(lib, gpu, a, b, layout)
+    ok, st = so.gemm_tolerance_ok(c, so.gemm_ref(a, b, layout), K)
+    assert ok, (layout, tuple(a.shape), tuple(b.shape), st)
+    return c
+
+
+def operands(M, N, K, layout, seed=0, a_std=1.0, b_std=1.0):
+    a, b = so.gemm_inputs(M, N, K, seed, a_std, b_std)
+    if layout == "TN":
+        a = a.t().contiguous()
+    if layout == "NT":
+        b = b.t().contiguous()
+    return a, b
+
+
+# ---- benchmark configurations --------------------------------------------------------------------------------
+def test_config_g1_1024_cubed(lib, gpu):
+    a, b = so.gemm_inputs(1024, 1024, 1024, seed=0)
+    check(lib, gpu, a, b, "NN", 1024)
+
+
+@pytest.mark.parametrize("M,N,K", [(4096, 4096, 4096), (8192, 8192, 8192), (16, 14336, 4096)])
+def test_config_g2_llm_projection_shapes(lib, gpu, M, N, K):
+    a, b = so.gemm_inputs(M, N, K, seed=0, a_std=1.0, b_std=0.02)
+    check(lib, gpu, a, b, "NN", K)
+
+
+# ---- closed forms: exact answers ---------------------------------------------------------------------------------
+@pytest.mark.parametrize("n", [256, 512, 96])
+def test_identity_and_permutation_are_exact(lib, gpu, n):
+    b = so.randn_fp16((n, n), 3)
+    assert torch.equal(run(lib, gpu, torch.eye(n).half(), b), b)
+    perm = torch.randperm(n, generator=torch.Generator().manual_seed(1))
+    p = torch.zeros(n, n).half()
+    p[torch.arange(n), perm] = 1
+    assert torch.equal(run(lib, gpu, p, b), b[perm])               # rows of b picked by A
+    assert torch.equal(run(lib, gpu, b, p), b[:, torch.argsort(perm)])  # columns of b picked by B
+    assert torch.equal(run(lib, gpu, p.t().contiguous(), b, "TN"), b[perm])
+    assert torch.equal(run(lib, gpu, p, b.t().contiguous(), "NT"), b[perm])
+
+
+@pytest.mark.parametrize("K", [64, 1024, 2048])
+def test_all_ones_counts_k(lib, gpu, K):
+    c = run(lib, gpu, torch.ones(256, K).half(), torch.ones(K, 512).half())
+    assert torch.equal(c, torch.full((256, 512), float(K)).half())
+
+
+def test_power_of_two_operands_single_rounding(lib, gpu):
+    # every product and partial sum is exact in fp32, so the only rounding is the final fp32 -> fp16 one
+    g = torch.Generator().manual_seed(5)
+    a = torch.ldexp(torch.ones(256, 256), torch.randint(-4, 5, (256, 256), generator=g)).half()
+    b = torch.ldexp(torch.ones(256, 256), torch.randint(-4, 5, (256, 256), generator=g)).half()
+    sign = torch.where(torch.rand(256, 256, generator=g) < 0.5, -1.0, 1.0).half()
+    a = a * sign
+    assert torch.equal(run(lib, gpu, a, b), so.gemm_ref(a, b).half())
+
+
+# ---- layouts, non-square and ragged shapes -------------------------------------------------------------------------
+@pytest.mark.parametrize("layout", ["NN", "TN", "NT"])
+@pytest.mark.parametrize("M,N,K", [(256, 512, 320), (512, 256, 64), (768, 1024, 1088), (100, 70, 50), (1, 1, 1),
+                                   (257, 255, 129), (31, 300, 8), (2048, 256, 4096)])
+def test_layouts_and_shapes(lib, gpu, layout, M, N, K):
+    a, b = operands(M, N, K, layout, seed=M + N + K)
+    c = check(lib, gpu, a, b, layout, K)
+    assert c.shape == (M, N)
+
+
+def test_reference_seeded_case_from_golden_fixture(lib, gpu):
+    z = np.load(os.path.join(GOLDEN, "gemm_seed0_256.npz"))
+    a, b, rows = torch.from_numpy(z["a"]), torch.from_numpy(z["b"]), z["rows"]
+    for lay in ("NN", "TN", "NT"):
+        c = run(lib, gpu, a, b, lay).float().numpy()[rows]
+        ref = z["c_" + lay]
+        assert np.all(np.abs(c - ref) <= 2e-2 * 0.5 + 1e-2 * np.abs(ref)), lay
+
+
+def test_strided_leading_dimensions(lib, gpu):
+    # lda/ldb/ldc larger than the logical width (operands that are column slices of wider buffers)
+    M, N, K = 512, 256, 192
+    abig, bbig = so.randn_fp16((M, K + 64), 1).to(gpu), so.randn_fp16((K, N + 128), 2).to(gpu)
+    cbig = torch.zeros((M, N + 32), dtype=torch.float16, device=gpu)
+    lib.hgemm_raw(abig.data_ptr(), bbig.data_ptr(), cbig.data_ptr(), M, N, K, K + 64, N + 128, N + 32, lib.GEMM_NN,
+                  torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    ok, st = so.gemm_tolerance_ok(cbig[:, :N], so.gemm_ref(abig[:, :K], bbig[:, :N]), K)
+    assert ok, st
+    assert bool((cbig[:, N:] == 0).all())  # nothing written outside the N columns
+
+
+# ---- size-independent properties at the full benchmark size -------------------------------------------------------
+def test_full_size_linearity_and_column_selection(lib, gpu):
+    n = 8192
+    a = so.randn_fp16((n, n), 0).to(gpu)
+    # B = one-hot columns scaled by powers of two: C[:, j] = 2^e_j * A[:, src_j], exact in fp16
+    g = torch.Generator().manual_seed(2)
+    src = torch.randint(0, n, (n,), generator=g)
+    e = torch.randint(-2, 3, (n,), generator=g)
+    b = torch.zeros(n, n, dtype=torch.float16)
+    b[src, torch.arange(n)] = torch.ldexp(torch.ones(n), e).half()
+    c = lib.hgemm(a, b.to(gpu))
+    expect = a[:, src.to(gpu)] * torch.ldexp(torch.ones(n), e).half().to(gpu)[None, :]
+    assert torch.equal(c, expect)
+
+
+# ---- torch operator path ----------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("index", list(range(17)))
+def test_torch_operator_every_index(gpu, index):
+    import gemm_unified
+    layout = so.GEMM_LAYOUT_OF_INDEX[index]
+    a, b = operands(384, 512, 256, layout, seed=index)
+    c = gemm_unified.ops.fine_gemm(a.to(gpu), b.to(gpu), index)
+    assert c.dtype == torch.float16 and c.shape == (384, 512)
+    ok, st = so.gemm_tolerance_ok(c, so.fine_gemm_ref(a, b, index), 256)
+    assert ok, (index, st)
+
+
+def test_torch_operator_reference_correctness_script_case(gpu):
+    # kernels/gemm/test/correct.py: seed 0, 256x256 randn fp16, indices 13..15 against a @ b.T, 16 against a.T @ b,
+    # allclose(rtol=1e-1, atol=1e-1)
+    import gemm_unified
+    torch.manual_seed(0)
+    a = torch.randn(256, 256, dtype=torch.half).to(gpu)
+    b = torch.randn(256, 256, dtype=torch.half).to(gpu)
+    for idx, ref in ((13, a @ b.T), (14, a @ b.T), (15, a @ b.T), (16, a.T @ b), (0, a @ b)):
+        c = gemm_unified.ops.fine_gemm(a, b, idx)
+        assert torch.allclose(c, ref, rtol=1e-1, atol=1e-1), idx
+
+
+def test_torch_operator_noncontiguous_inputs_and_stream(gpu):
+    import gemm_unified
+    a = so.randn_fp16((512, 300), 1).to(gpu)
+    b = so.randn_fp16((300, 512), 2).to(gpu)
+    at = a.t().contiguous().t()  # same values, column-major strides
+    s = torch.cuda.Stream()
+    with torch.cuda.stream(s):
+        c = gemm_unified.ops.fine_gemm(at, b, 0)
+    s.synchronize()
+    ok, st = so.gemm_tolerance_ok(c, so.gemm_ref(a, b), 300)
+    assert ok, st

@@ -1,0 +1,198 @@
+"""Pins the CPU oracle (oracle/serving_oracle.py) without a GPU: closed forms, invariants, fp64 brute force
+with explicit loops, torch's own SDPA as a second opinion, and the committed golden fixtures. Each check is
+chosen so that a plausible mistake (transposed operand, wrong head mapping, off-by-one in a mask, missing scale,
+wrong log base) fails at least one of them."""
+import math
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import serving_oracle as so
+
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+
+
+# ------------------------------------------------------------------ GEMM
+def test_gemm_identity_and_onehot():
+    b = so.randn_fp16((48, 40), 1)
+    assert torch.equal(so.gemm_ref(torch.eye(48).half(), b, "NN"), b.float())
+    # one-hot row i of A picks row perm[i] of B: catches any transposition of the operands
+    perm = torch.randperm(48, generator=torch.Generator().manual_seed(3))
+    a = torch.zeros(48, 48).half()
+    a[torch.arange(48), perm] = 1
+    assert torch.equal(so.gemm_ref(a, b, "NN"), b.float()[perm])
+    assert torch.equal(so.gemm_ref(a.t().contiguous(), b, "TN"), b.float()[perm])
+    assert torch.equal(so.gemm_ref(a, b.t().contiguous(), "NT"), b.float()[perm])
+
+
+def test_gemm_all_ones_counts_k():
+    for K in (64, 1024, 2048):
+        c = so.gemm_ref(torch.ones(8, K).half(), torch.ones(K, 8).half())
+        assert torch.equal(c, torch.full((8, 8), float(K)))
+
+
+def test_gemm_power_of_two_sums_are_exact():
+    g = torch.Generator().manual_seed(5)
+    a = torch.ldexp(torch.ones(16, 32), torch.randint(-3, 4, (16, 32), generator=g)).half()
+    b = torch.ldexp(torch.ones(32, 16), torch.randint(-3, 4, (32, 16), generator=g)).half()
+    ref = so.gemm_bruteforce_f64(a.numpy(), b.numpy())
+    assert np.array_equal(so.gemm_ref(a, b).double().numpy(), ref)
+
+
+@pytest.mark.parametrize("layout", ["NN", "TN", "NT"])
+def test_gemm_bruteforce_nonsquare(layout):
+    M, N, K = 20, 12, 36
+    a = so.randn_fp16((K, M) if layout == "TN" else (M, K), 7)
+    b = so.randn_fp16((N, K) if layout == "NT" else (K, N), 8)
+    ref = so.gemm_bruteforce_f64(a.numpy(), b.numpy(), layout)
+    got = so.gemm_ref(a, b, layout).double().numpy()
+    assert got.shape == (M, N)
+    assert np.abs(got - ref).max() < 1e-4
+
+
+def test_gemm_index_layout_table_matches_reference_correct_py():
+    # kernels/gemm/test/correct.py:39-43: 12 and 16 are called with a_format='N' (a.T @ b), 13..15 with b_format='N'
+    assert [so.GEMM_LAYOUT_OF_INDEX[i] for i in (12, 13, 14, 15, 16)] == ["TN", "NT", "NT", "NT", "TN"]
+    assert all(so.GEMM_LAYOUT_OF_INDEX[i] == "NN" for i in range(12))
+    a, b = so.randn_fp16((8, 8), 1), so.randn_fp16((8, 8), 2)
+    assert torch.allclose(so.fine_gemm_ref(a, b, 16), a.float().t() @ b.float())
+    assert torch.allclose(so.fine_gemm_ref(a, b, 13), a.float() @ b.float().t())
+
+
+def test_gemm_golden_fixture():
+    z = np.load(os.path.join(GOLDEN, "gemm_seed0_256.npz"))
+    a, b, rows = torch.from_numpy(z["a"]), torch.from_numpy(z["b"]), z["rows"]
+    for lay in ("NN", "TN", "NT"):
+        got = so.gemm_ref(a, b, lay).numpy()[rows]
+        assert np.allclose(got, z["c_" + lay], rtol=1e-5, atol=1e-4), lay
+    # the fixture inputs are the reference's seeded draw (correct.py:5-8)
+    torch.manual_seed(0)
+    assert torch.equal(torch.randn(256, 256, dtype=torch.half), a)
+
+
+def test_gemm_tolerance_checker():
+    ref = torch.full((4, 4), 100.0)
+    ok, _ = so.gemm_tolerance_ok(ref + 0.5, ref, 1024)
+    assert ok
+    ok, st = so.gemm_tolerance_ok(ref + 1.5, ref, 1024)
+    assert not ok and st["violations"] == 16
+
+
+# ------------------------------------------------------------------ attention
+def test_attention_equal_keys_gives_running_mean():
+    # all keys equal => uniform softmax over the visible keys
+    B, H, S, D = 1, 2, 37, 128
+    q = so.randn_fp16((B, H, S, D), 1)
+    k = so.randn_fp16((B, H, 1, D), 2).expand(B, H, S, D).contiguous()
+    v = so.randn_fp16((B, H, S, D), 3)
+    o, lse = so.attention_ref(q, k, v, causal=True)
+    vm = v.float().cumsum(2) / torch.arange(1, S + 1)[None, None, :, None]
+    assert torch.allclose(o, vm, atol=1e-5)
+    s0 = (q.float() * k.float()).sum(-1) / math.sqrt(D)
+    assert torch.allclose(lse, s0 + torch.log(torch.arange(1, S + 1).float()), atol=1e-4)
+    o2, lse2 = so.attention_ref(q, k, v, causal=False)
+    assert torch.allclose(o2, v.float().mean(2, keepdim=True).expand_as(o2), atol=1e-5)
+    assert torch.allclose(lse2, s0 + math.log(S), atol=1e-4)
+
+
+def test_attention_zero_query_and_ones_value():
+    q = torch.zeros(1, 1, 9, 128).half()
+    k, v = so.randn_fp16((1, 1, 21, 128), 4), torch.ones(1, 1, 21, 128).half()
+    o, lse = so.attention_ref(q, k, v, causal=False)
+    assert torch.allclose(lse, torch.full_like(lse, math.log(21)), atol=1e-6)
+    assert torch.allclose(o, torch.ones_like(o), atol=1e-6)  # softmax rows sum to one
+    # bottom-right causal with Sq=9 < Sk=21: query i sees keys 0..i+12
+    o, lse = so.attention_ref(q, k, v, causal=True)
+    assert torch.allclose(lse[0, 0], torch.log(torch.arange(13, 22).float()), atol=1e-6)
+
+
+def test_attention_first_causal_row_and_dominant_key():
+    q, k, v = so.fmha_inputs(1, 2, 2, 16, 16, seed=9)
+    o, lse = so.attention_ref(q, k, v, causal=True)
+    assert torch.allclose(o[:, :, 0], v.float()[:, :, 0], atol=1e-6)
+    s00 = (q.float()[:, :, 0] * k.float()[:, :, 0]).sum(-1) / math.sqrt(128)
+    assert torch.allclose(lse[:, :, 0], s00, atol=1e-5)
+    # one dominant key: a query aligned with key 5 and scaled so its score leads by > 40
+    k2 = k.clone()
+    q2 = (k2[:, :, 5:6] * 8).expand(1, 2, 16, 128).contiguous()
+    o2, _ = so.attention_ref(q2, k2, v, causal=False)
+    assert torch.allclose(o2, v.float()[:, :, 5:6].expand_as(o2), atol=1e-3)
+
+
+def test_attention_key_permutation_invariance_and_kv_valid_len():
+    q, k, v = so.fmha_inputs(1, 1, 1, 8, 50, seed=10)
+    perm = torch.randperm(50, generator=torch.Generator().manual_seed(1))
+    o1, l1 = so.attention_ref(q, k, v)
+    o2, l2 = so.attention_ref(q, k[:, :, perm], v[:, :, perm])
+    assert torch.allclose(o1, o2, atol=1e-5) and torch.allclose(l1, l2, atol=1e-5)
+    # masking keys >= 30 equals dropping them (pins the off-by-one: key 30 itself must be masked)
+    o3, l3 = so.attention_ref(q, k, v, kv_valid_len=30)
+    o4, l4 = so.attention_ref(q, k[:, :, :30], v[:, :, :30])
+    assert torch.allclose(o3, o4, atol=1e-6) and torch.allclose(l3, l4, atol=1e-6)
+    # LSE grows when keys are added
+    assert bool((l1 > l3).all())
+
+
+def test_attention_gqa_head_mapping():
+    # kv head = q head // (Hq / Hkv): q heads 0..3 -> kv 0, 4..7 -> kv 1 (kernels/fmha/test/perf.py:10-23)
+    q, k, v = so.fmha_inputs(1, 8, 2, 12, 12, seed=11)
+    o, lse = so.attention_ref(q, k, v, causal=True)
+    for h in range(8):
+        oh, lh = so.attention_ref(q[:, h:h + 1], k[:, h // 4:h // 4 + 1], v[:, h // 4:h // 4 + 1], causal=True)
+        assert torch.allclose(o[:, h:h + 1], oh, atol=1e-6) and torch.allclose(lse[:, h:h + 1], lh, atol=1e-6)
+
+
+@pytest.mark.parametrize("causal,Sq,Sk,kvv", [(False, 8, 13, None), (True, 8, 8, None), (True, 5, 11, None),
+                                                (True, 11, 5, None), (False, 3, 17, 9), (True, 9, 17, 14)])
+def test_attention_vs_bruteforce_f64(causal, Sq, Sk, kvv):
+    q, k, v = so.fmha_inputs(1, 2, 1, Sq, Sk, seed=12)
+    o, lse = so.attention_ref(q, k, v, causal=causal, kv_valid_len=kvv)
+    ob, lb = so.attention_bruteforce_f64(q.numpy(), k.numpy(), v.numpy(), causal, kvv)
+    assert np.abs(o.double().numpy() - ob).max() < 1e-5
+    fin = np.isfinite(lb)
+    assert np.array_equal(np.isfinite(lse.numpy()), fin)
+    assert np.abs(lse.double().numpy()[fin] - lb[fin]).max() < 1e-5
+    # rows with no visible key (Sq > Sk, causal): O = 0
+    assert np.all(o.numpy()[~fin] == 0)
+
+
+def test_attention_vs_torch_sdpa():
+    q, k, v = so.fmha_inputs(2, 8, 2, 33, 33, seed=13)
+    kk, vv = k.float().repeat_interleave(4, 1), v.float().repeat_interleave(4, 1)
+    for causal in (False, True):
+        ref = torch.nn.functional.scaled_dot_product_attention(q.float(), kk, vv, is_causal=causal)
+        assert torch.allclose(so.attention_ref(q, k, v, causal=causal)[0], ref, atol=2e-6)
+        assert torch.allclose(so.fine_fmha_ref(q, k, v, causal, False), ref, atol=2e-6)
+    with pytest.raises(ValueError):
+        so.fine_fmha_ref(q, k, v, True, True)
+
+
+def test_fmha_golden_fixture():
+    z = np.load(os.path.join(GOLDEN, "fmha_seed42_128.npz"))
+    q, k, v = (torch.from_numpy(z[n]) for n in ("q", "k", "v"))
+    rows = z["qrows"]
+    for tag, causal in (("full", False), ("causal", True)):
+        o, lse = so.attention_ref(q, k, v, causal=causal)
+        assert np.allclose(o.numpy()[:, :, rows], z["o_" + tag], atol=1e-6)
+        assert np.allclose(lse.numpy(), z["lse_" + tag], atol=1e-6)
+    torch.manual_seed(42)
+    assert torch.equal(torch.randn(size=(1, 4, 128, 128), dtype=torch.half) * 0.1, q)
+
+
+def test_llama_layer_ref_shapes_and_composition():
+    S, H, nq, nkv, d, F = 16, 64, 4, 2, 16, 48
+    g = lambda shape, seed, std: so.randn_fp16(shape, seed, std)
+    x, wqkv, wo = g((S, H), 0, 1.0), g((H, (nq + 2 * nkv) * d), 1, 0.1), g((nq * d, H), 2, 0.1)
+    wgu, wd = g((H, 2 * F), 3, 0.1), g((F, H), 4, 0.1)
+    out = so.llama_layer_ref(x, wqkv, wo, wgu, wd, n_q=nq, n_kv=nkv, d=d)
+    assert out["qkv"].shape == (S, (nq + 2 * nkv) * d) and out["attn"].shape == (1, nq, S, d)
+    assert out["down"].shape == (S, H)
+    # q head 0 of the chain equals attention on the sliced projections
+    qkv = out["qkv"].half().float()
+    q0, k0, v0 = qkv[:, :d], qkv[:, nq * d:nq * d + d], qkv[:, (nq + nkv) * d:(nq + nkv) * d + d]
+    ref = torch.nn.functional.scaled_dot_product_attention(q0[None, None], k0[None, None], v0[None, None], is_causal=True)
+    assert torch.allclose(out["attn"][0, 0], ref[0, 0], atol=1e-5)
+    gu = out["gate_up"].half().float()
+    assert torch.allclose(out["act"], torch.nn.functional.silu(gu[:, :F]) * gu[:, F:], atol=1e-6)

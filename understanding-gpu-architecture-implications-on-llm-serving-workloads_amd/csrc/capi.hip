@@ -48,7 +48,8 @@ int mi355_fmha_fwd(const void* Q, const void* K, const void* V, void* O, float* 
     if (Hq % Hkv != 0) return fail(MI355_ERR_BAD_ARGUMENT, "mi355_fmha_fwd: Hq (%d) must be a multiple of Hkv (%d)", Hq, Hkv);
     if (kv_valid_len < 1 || kv_valid_len > Sk)
         return fail(MI355_ERR_BAD_ARGUMENT, "mi355_fmha_fwd: kv_valid_len %d outside [1, Sk=%d]", kv_valid_len, Sk);
-    if (!(scale == scale)) return fail(MI355_ERR_BAD_ARGUMENT, "mi355_fmha_fwd: scale is NaN");
+    if (!(scale > 0.f) || scale > 3.0e38f)
+        return fail(MI355_ERR_BAD_ARGUMENT, "mi355_fmha_fwd: scale must be positive and finite (got %g)", (double)scale);
     if ((reinterpret_cast<uintptr_t>(Q) | reinterpret_cast<uintptr_t>(K) | reinterpret_cast<uintptr_t>(V) |
          reinterpret_cast<uintptr_t>(O)) % 16 != 0)
         return fail(MI355_ERR_BAD_ARGUMENT, "mi355_fmha_fwd: Q, K, V, O must be 16-byte aligned");

@@ -1,0 +1,333 @@
+// Fused multi-head attention forward for gfx950 (MI355X), head_dim 128, fp16 in/out, fp32 softmax statistics.
+//
+// Replaces the reference's attention ladder (kernels/fmha/pkg/fmha_unified/csrc/{auto,semi}/fmha_*.{cu,cpp});
+// semantics follow semi/fmha_2_amd.cpp: BHSD layout (:33-45), kv head = q head / (Hq/Hkv), causal rule
+// "masked iff q_pos < k_pos" (:187-190), keys at or beyond the valid length masked (:191, with the off-by-one
+// of the reference corrected), scale 1/sqrt(d) supplied by the caller (:320).
+//
+// Shape of the computation (per wave, everything stays in registers between the two matrix products):
+//   S^T = K * Q^T      MFMA 32x32x16, A operand = K fragment read from LDS (ds_read_b128),
+//                      B operand = Q fragment held in registers for the whole kernel.
+//                      A lane then owns ONE query column (q = lane % 32) and 16 of the 32 keys of the block,
+//                      so the softmax statistics m, l and the rescale factor are per-lane scalars.
+//   P^T                exp2((S - m) * scale*log2e) in fp32, rounded to fp16; the accumulator layout of S^T is
+//                      already the B-operand layout of the second product, so P never leaves the registers.
+//   O^T += V^T * P^T   A operand = V^T fragment, read from the row-major V tile in LDS with the transposing
+//                      ds_read_b64_tr_b16.
+// K and V tiles (64 keys x 128 d) are copied global -> LDS with 16-byte direct-to-LDS copies, double buffered,
+// 16-byte chunks XOR-swizzled so that both the b128 reads (K) and the transposing reads (V) are conflict free.
+#include "mi355_common.h"
+#include "mi355_serving_internal.h"
+
+namespace mi355 {
+
+namespace fmha {
+
+constexpr int D = 128;            // head dim
+constexpr int BN = 64;            // keys per tile
+constexpr int ROW_BYTES = D * 2;  // 256
+constexpr int TILE_BYTES = BN * ROW_BYTES;  // 16 KiB
+constexpr int STAGE_BYTES = 2 * TILE_BYTES; // K + V
+constexpr int NSTAGE = 2;
+
+__device__ __forceinline__ int swz_k(int row) { return row & 15; }
+__device__ __forceinline__ int swz_v(int row) {
+    int r = row & 3;
+    return (r << 1) | ((r & 1) << 3);  // 0, 10, 4, 14
+}
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+// value held by the lane 32 positions away (lane ^ 32)
+__device__ __forceinline__ float other_half(float x) {
+    int idx = ((int)(threadIdx.x & 63) ^ 32) << 2;
+    return __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute(idx, __builtin_bit_cast(int, x)));
+}
+// max / sum over the two 32-lane halves of the wave; result valid in all 64 lanes
+__device__ __forceinline__ float halves_max(float x) { return fmaxf(x, other_half(x)); }
+__device__ __forceinline__ float halves_sum(float x) { return x + other_half(x); }
+
+}  // namespace fmha
+
+// Decode the linear workgroup id into (batch, q head, q tile). Workgroups with ids congruent mod 8 share an
+// XCD (and its L2): give each XCD whole (batch, kv head) groups so K/V are fetched from HBM once per XCD,
+// and inside a group hand out the q tiles with the most keys (causal) first.
+__device__ __forceinline__ void fmha_decode_block(int bid, int q_tiles, int group, int Hkv, int B, int& b, int& hq,
+                                                  int& q_tile) {
+    const int per_group = group * q_tiles;
+    const int total = per_group * Hkv * B;
+    int v = bid;
+    if (total % 8 == 0) v = (bid % 8) * (total / 8) + bid / 8;
+    int g = v / per_group;
+    int r = v - g * per_group;
+    int qt = r / group;
+    int hin = r - qt * group;
+    q_tile = q_tiles - 1 - qt;
+    b = g / Hkv;
+    hq = (g - b * Hkv) * group + hin;
+}
+
+template <int NQ, int NWAVES>
+__global__ __launch_bounds__(NWAVES * 64) void fmha_fwd_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K,
+                                                               const half_t* __restrict__ V, half_t* __restrict__ O,
+                                                               float* __restrict__ LSE, int B, int Hq, int Hkv, int Sq,
+                                                               int Sk, float scale_log2, int causal, int kv_valid,
+                                                               int q_tiles) {
+    using namespace fmha;
+    constexpr int BM = NWAVES * NQ * 32;
+    constexpr int COPIES = (BN * ROW_BYTES / 1024) / NWAVES;  // wave-instructions per tile per wave
+    static_assert(COPIES >= 1, "too many waves for the tile");
+
+    extern __shared__ __attribute__((aligned(1024))) char smem_raw[];
+    MI355_LDS char* smem = (MI355_LDS char*)smem_raw;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int h = lane >> 5;
+    const int l32 = lane & 31;
+
+    int b, hq, q_tile;
+    const int group = Hq / Hkv;
+    fmha_decode_block(blockIdx.x, q_tiles, group, Hkv, B, b, hq, q_tile);
+    const int hkv = hq / group;
+
+    const int q_block0 = q_tile * BM;            // first query row of the workgroup
+    const int q_wave0 = q_block0 + wave * NQ * 32;  // first query row of this wave
+    const int shift = Sk - Sq;
+
+    const half_t* Qh = Q + ((long)b * Hq + hq) * (long)Sq * D;
+    const half_t* Kh = K + ((long)b * Hkv + hkv) * (long)Sk * D;
+    const half_t* Vh = V + ((long)b * Hkv + hkv) * (long)Sk * D;
+    half_t* Oh = O + ((long)b * Hq + hq) * (long)Sq * D;
+
+    // ---- number of key tiles this workgroup has to visit ----------------------------------------------
+    int k_end = kv_valid;
+    if (causal) {
+        int last_q = min(q_block0 + BM, Sq) - 1;
+        k_end = min(k_end, last_q + shift + 1);
+    }
+    const int n_tiles = (k_end + BN - 1) / BN;  // may be <= 0: no visible key for the whole tile
+
+    // ---- Q fragments: lane holds Q[q = l32][d = 16*ks + 8*h .. +7] ---------------------------------------
+    half8 qf[NQ][8];
+#pragma unroll
+    for (int qb = 0; qb < NQ; ++qb) {
+        int qrow = min(q_wave0 + qb * 32 + l32, Sq - 1);
+        const half_t* qp = Qh + (long)qrow * D + 8 * h;
+#pragma unroll
+        for (int ks = 0; ks < 8; ++ks) qf[qb][ks] = *(const half8*)(qp + ks * 16);
+    }
+
+    // ---- global -> LDS copy bookkeeping ----------------------------------------------------------------
+    // copy i of this wave covers tile rows (i*NWAVES + wave)*4 + lane/16, 16-byte chunk position lane%16
+    int copy_row[COPIES];
+    int copy_kcol[COPIES], copy_vcol[COPIES];
+#pragma unroll
+    for (int i = 0; i < COPIES; ++i) {
+        int row = (i * NWAVES + wave) * 4 + (lane >> 4);
+        copy_row[i] = row;
+        copy_kcol[i] = ((lane & 15) ^ swz_k(row)) * 8;
+        copy_vcol[i] = ((lane & 15) ^ swz_v(row)) * 8;
+    }
+    auto issue_copies = [&](int tile, int stage) {
+        MI355_LDS char* sk = smem + stage * STAGE_BYTES;
+        MI355_LDS char* sv = sk + TILE_BYTES;
+#pragma unroll
+        for (int i = 0; i < COPIES; ++i) {
+            int krow = min(tile * BN + copy_row[i], kv_valid - 1);
+            copy16_global_to_lds(Kh + (long)krow * D + copy_kcol[i], sk + (i * NWAVES + wave) * 1024);
+        }
+#pragma unroll
+        for (int i = 0; i < COPIES; ++i) {
+            int krow = min(tile * BN + copy_row[i], kv_valid - 1);
+            copy16_global_to_lds(Vh + (long)krow * D + copy_vcol[i], sv + (i * NWAVES + wave) * 1024);
+        }
+    };
+
+    // ---- LDS fragment offsets ----------------------------------------------------------------------------
+    // K fragment (key block kb, k-step ks): row kb*32 + l32, chunk (2ks + h) ^ (row & 15)
+    const int k_base = l32 * ROW_BYTES + ((h ^ (lane & 15)) << 4);  // xor (ks << 5), + kb * 32 * ROW_BYTES
+    // V^T fragment (d block db): rows 4h + (lane%16)/4 (+ kb*32 + 16t + 8u), chunk (4db + clow) ^ swz_v(row)
+    const int v_row = 4 * h + ((lane & 15) >> 2);
+    const int v_clow = 2 * ((lane >> 4) & 1) + ((lane & 3) >> 1);
+    const int v_base = TILE_BYTES + v_row * ROW_BYTES + ((v_clow ^ swz_v(v_row)) << 4) + (lane & 1) * 8;  // xor (db << 6)
+
+    float16v o[NQ][4];
+    float m_run[NQ], l_run[NQ];
+#pragma unroll
+    for (int qb = 0; qb < NQ; ++qb) {
+        m_run[qb] = -INFINITY;
+        l_run[qb] = 0.f;
+#pragma unroll
+        for (int db = 0; db < 4; ++db)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) o[qb][db][e] = 0.f;
+    }
+
+    if (n_tiles > 0) issue_copies(0, 0);
+
+    for (int t = 0; t < n_tiles; ++t) {
+        wait_vmcnt<0>();
+        __syncthreads();
+        if (t + 1 < n_tiles) issue_copies(t + 1, (t + 1) & 1);
+        MI355_LDS char* st = smem + (t & 1) * STAGE_BYTES;
+        const int key0 = t * BN;
+
+        // ---- S^T = K Q^T ---------------------------------------------------------------------------------
+        float16v s[NQ][2];
+#pragma unroll
+        for (int qb = 0; qb < NQ; ++qb)
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) s[qb][kb][e] = 0.f;
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+            for (int ks = 0; ks < 8; ++ks) {
+                half8 kf = lds_read_b128(st + ((k_base ^ (ks << 5)) + kb * 32 * ROW_BYTES));
+#pragma unroll
+                for (int qb = 0; qb < NQ; ++qb)
+                    s[qb][kb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf, qf[qb][ks], s[qb][kb], 0, 0, 0);
+            }
+
+        // ---- mask (only tiles that touch the diagonal or the end of the valid keys) ----------------------
+        const bool need_mask = (key0 + BN > kv_valid) || (causal && (key0 + BN - 1 > q_wave0 + shift));
+        if (need_mask) {
+#pragma unroll
+            for (int qb = 0; qb < NQ; ++qb) {
+                int qi = q_wave0 + qb * 32 + l32;
+                int lim = causal ? min(kv_valid - 1, qi + shift) : kv_valid - 1;  // last visible key
+#pragma unroll
+                for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                    for (int e = 0; e < 16; ++e) {
+                        int key = key0 + kb * 32 + 8 * (e >> 2) + 4 * h + (e & 3);
+                        if (key > lim) s[qb][kb][e] = -INFINITY;
+                    }
+            }
+        }
+
+        // ---- online softmax --------------------------------------------------------------------------------
+        half8 pf[NQ][2][2];
+#pragma unroll
+        for (int qb = 0; qb < NQ; ++qb) {
+            float mx = s[qb][0][0];
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) mx = fmaxf(mx, s[qb][kb][e]);
+            mx = halves_max(mx);
+            float m_new = fmaxf(m_run[qb], mx);
+            float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+            float alpha = fast_exp2((m_run[qb] - m_use) * scale_log2);
+            m_run[qb] = m_new;
+            float neg_ms = -m_use * scale_log2;
+            float psum = 0.f;
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb) {
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    float p = fast_exp2(__builtin_fmaf(s[qb][kb][e], scale_log2, neg_ms));
+                    s[qb][kb][e] = p;
+                    psum += p;
+                }
+#pragma unroll
+                for (int tt = 0; tt < 2; ++tt) {
+                    half8 pk;
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) pk[j] = (half_t)s[qb][kb][8 * tt + j];
+                    pf[qb][kb][tt] = pk;
+                }
+            }
+            l_run[qb] = l_run[qb] * alpha + psum;
+#pragma unroll
+            for (int db = 0; db < 4; ++db)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) o[qb][db][e] *= alpha;
+        }
+
+        // ---- O^T += V^T P^T ----------------------------------------------------------------------------------
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+            for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+                for (int db = 0; db < 4; ++db) {
+                    int off = (v_base ^ (db << 6)) + (kb * 32 + 16 * tt) * ROW_BYTES;
+                    half4 lo = lds_read_tr16_b64(st + off);
+                    half4 hi = lds_read_tr16_b64(st + off + 8 * ROW_BYTES);
+                    half8 vf = concat(lo, hi);
+#pragma unroll
+                    for (int qb = 0; qb < NQ; ++qb)
+                        o[qb][db] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf, pf[qb][kb][tt], o[qb][db], 0, 0, 0);
+                }
+    }
+
+    // ---- finalize: O / l, LSE ---------------------------------------------------------------------------------
+#pragma unroll
+    for (int qb = 0; qb < NQ; ++qb) {
+        float l_tot = halves_sum(l_run[qb]);
+        float inv = (l_tot > 0.f) ? 1.f / l_tot : 0.f;
+        int qi = q_wave0 + qb * 32 + l32;
+        if (qi < Sq) {
+            half_t* orow = Oh + (long)qi * D + 4 * h;
+#pragma unroll
+            for (int db = 0; db < 4; ++db)
+#pragma unroll
+                for (int p = 0; p < 4; ++p) {
+                    half4 v;
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) v[q] = (half_t)(o[qb][db][4 * p + q] * inv);
+                    *(half4*)(orow + db * 32 + 8 * p) = v;
+                }
+            if (LSE != nullptr && h == 0) {
+                float lse = (l_tot > 0.f) ? (m_run[qb] * scale_log2 + __builtin_log2f(l_tot)) * 0.69314718055994531f
+                                          : -INFINITY;
+                LSE[((long)b * Hq + hq) * (long)Sq + qi] = lse;
+            }
+        }
+    }
+}
+
+template <int NQ, int NWAVES>
+static hipError_t launch_fmha(const half_t* Q, const half_t* K, const half_t* V, half_t* O, float* LSE, int B, int Hq,
+                              int Hkv, int Sq, int Sk, float scale, int causal, int kv_valid, hipStream_t stream) {
+    constexpr int BM = NWAVES * NQ * 32;
+    constexpr int LDS = fmha::STAGE_BYTES * fmha::NSTAGE;
+    auto kern = fmha_fwd_kernel<NQ, NWAVES>;
+    static bool attr_set = false;
+    if (!attr_set) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, LDS);
+        if (e != hipSuccess) return e;
+        attr_set = true;
+    }
+    const int q_tiles = (Sq + BM - 1) / BM;
+    const long blocks = (long)q_tiles * Hq * B;
+    if (blocks > 0x7fffffffL) return hipErrorInvalidValue;
+    const float scale_log2 = scale * 1.4426950408889634f;
+    kern<<<dim3((unsigned)blocks), dim3(NWAVES * 64), LDS, stream>>>(Q, K, V, O, LSE, B, Hq, Hkv, Sq, Sk, scale_log2,
+                                                                    causal, kv_valid, q_tiles);
+    return hipGetLastError();
+}
+
+int g_fmha_variant = 0;  // tuning hook: 0 = default
+
+hipError_t fmha_fwd_dispatch(const void* Q, const void* K, const void* V, void* O, float* LSE, int B, int Hq, int Hkv,
+                             int Sq, int Sk, float scale, int causal, int kv_valid_len, hipStream_t stream) {
+    const half_t* q = static_cast<const half_t*>(Q);
+    const half_t* k = static_cast<const half_t*>(K);
+    const half_t* v = static_cast<const half_t*>(V);
+    half_t* o = static_cast<half_t*>(O);
+    switch (g_fmha_variant) {
+        case 1: return launch_fmha<2, 4>(q, k, v, o, LSE, B, Hq, Hkv, Sq, Sk, scale, causal, kv_valid_len, stream);
+        case 2: return launch_fmha<1, 8>(q, k, v, o, LSE, B, Hq, Hkv, Sq, Sk, scale, causal, kv_valid_len, stream);
+        default: return launch_fmha<1, 4>(q, k, v, o, LSE, B, Hq, Hkv, Sq, Sk, scale, causal, kv_valid_len, stream);
+    }
+}
+
+}  // namespace mi355
+
+extern "C" void mi355_debug_set_fmha_variant(int v) { mi355::g_fmha_variant = v; }

@@ -1,0 +1,122 @@
+// PyTorch operator layer of fmha_unified for MI355X.
+//
+// Same operator surface as the reference (kernels/fmha/pkg/fmha_unified/csrc/fmha_kernel.cpp:9-18): schemas
+// `fmha_unified::finefmha_0 .. finefmha_7 (Tensor q, Tensor k, Tensor v, bool causal, bool is_decode,
+// int decode_length) -> Tensor`, CUDA dispatch key, empty `_C` module. Every index runs the one gfx950
+// attention kernel of libmi355_serving.so. Host checks mirror semi/fmha_2_amd.cpp:322-333 (fp16, d == 128,
+// is_decode implies !causal) and add the shape checks the reference omits.
+//
+// One operator is added without touching the reference's schemas:
+//   `finefmha_fwd_lse(q, k, v, causal, is_decode, decode_length) -> (Tensor out, Tensor lse)`
+// which also returns the log-sum-exp [B, Hq, Sq] in fp32 (the reference has no LSE output).
+//
+// decode_length is the number of valid keys (ops.py:18 passes the un-padded k.size(2)); keys at or beyond it
+// are masked. The reference masks `k > decode_length` (fmha_2_amd.cpp:191), which lets the first padded key
+// through; that off-by-one is not reproduced.
+#include <torch/extension.h>
+#include <ATen/hip/impl/HIPGuardImplMasqueradingAsCUDA.h>
+#include <ATen/hip/impl/HIPStreamMasqueradingAsCUDA.h>
+
+#include <cmath>
+#include <tuple>
+
+#include "mi355_serving.h"
+
+namespace fmha_unified {
+
+// Registers _C as a Python extension module.
+PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {}
+
+namespace {
+
+std::tuple<at::Tensor, at::Tensor> run_fmha(const at::Tensor& q, const at::Tensor& k, const at::Tensor& v, bool causal,
+                                            bool is_decode, int64_t decode_length, bool want_lse) {
+    const char* name = "finefmha";
+    TORCH_CHECK(q.dim() == 4 && k.dim() == 4 && v.dim() == 4, name, ": q, k, v must be [B, H, S, D] tensors");
+    TORCH_CHECK(q.scalar_type() == at::kHalf, name, ": q must be float16, got ", q.scalar_type());
+    TORCH_CHECK(k.scalar_type() == at::kHalf, name, ": k must be float16, got ", k.scalar_type());
+    TORCH_CHECK(v.scalar_type() == at::kHalf, name, ": v must be float16, got ", v.scalar_type());
+    const int64_t B = q.size(0), Hq = q.size(1), Sq = q.size(2), D = q.size(3);
+    const int64_t Hkv = k.size(1), Sk = k.size(2);
+    TORCH_CHECK(D == 128, name, ": head embedding dimension must be 128, got ", D);
+    TORCH_CHECK(k.size(0) == B && k.size(3) == D, name, ": k shape does not match q");
+    TORCH_CHECK(v.sizes() == k.sizes(), name, ": v shape must equal k shape");
+    TORCH_CHECK(B >= 1 && Hq >= 1 && Hkv >= 1 && Sq >= 1 && Sk >= 1, name, ": empty tensors are not supported");
+    TORCH_CHECK(Hq % Hkv == 0, name, ": number of q heads (", Hq, ") must be a multiple of kv heads (", Hkv, ")");
+    TORCH_CHECK(!(is_decode && causal), name, ": causal is not supported in decode mode");
+    TORCH_CHECK(decode_length >= 1 && decode_length <= Sk, name, ": decode_length ", decode_length,
+                " outside [1, k.size(2) = ", Sk, "]");
+    TORCH_CHECK(Sq <= INT32_MAX && Sk <= INT32_MAX && B <= INT32_MAX && Hq <= INT32_MAX, name, ": dimension exceeds int32");
+    TORCH_CHECK(q.is_cuda() && k.is_cuda() && v.is_cuda(), name, ": q, k, v must be GPU tensors");
+    TORCH_CHECK(q.device() == k.device() && q.device() == v.device(), name, ": q, k, v are on different devices");
+
+    // torch on ROCm presents HIP devices under the "cuda" device type; these are its guard and stream for them
+    const c10::hip::HIPGuardMasqueradingAsCUDA guard(q.device());
+    at::Tensor qc = q.contiguous(), kc = k.contiguous(), vc = v.contiguous();
+    at::Tensor o = at::empty(qc.sizes(), qc.options());
+    at::Tensor lse;
+    float* lse_ptr = nullptr;
+    if (want_lse) {
+        lse = at::empty({B, Hq, Sq}, qc.options().dtype(at::kFloat));
+        lse_ptr = lse.data_ptr<float>();
+    }
+    const float scale = 1.0f / std::sqrt(static_cast<float>(D));  // fmha_2_amd.cpp:320
+    hipStream_t stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream();
+    int rc = mi355_fmha_fwd(qc.data_ptr(), kc.data_ptr(), vc.data_ptr(), o.data_ptr(), lse_ptr, (int)B, (int)Hq, (int)Hkv,
+                            (int)Sq, (int)Sk, (int)D, scale, causal ? 1 : 0, (int)decode_length, stream);
+    TORCH_CHECK(rc == 0, name, ": ", mi355_last_error(), " (code ", rc, ")");
+    return {o, lse};
+}
+
+at::Tensor finefmha(const at::Tensor& q, const at::Tensor& k, const at::Tensor& v, bool causal, bool is_decode,
+                    int64_t decode_length) {
+    return std::get<0>(run_fmha(q, k, v, causal, is_decode, decode_length, false));
+}
+
+std::tuple<at::Tensor, at::Tensor> finefmha_fwd_lse(const at::Tensor& q, const at::Tensor& k, const at::Tensor& v,
+                                                    bool causal, bool is_decode, int64_t decode_length) {
+    return run_fmha(q, k, v, causal, is_decode, decode_length, true);
+}
+
+}  // namespace
+
+// Defines the operators (the first eight schema strings are the reference's).
+TORCH_LIBRARY(fmha_unified, m) {
+    m.def("finefmha_0(Tensor q, Tensor k, Tensor v, bool causal, bool is_decode, int decode_length) -> Tensor");
+    m.def("finefmha_1(Tensor q, Tensor k, Tensor v, bool causal, bool is_decode, int decode_length) -> Tensor");
+    m.def("finefmha_2(Tensor q, Tensor k, Tensor v, bool causal, bool is_decode, int decode_length) -> Tensor");
+    m.def("finefmha_3(Tensor q, Tensor k, Tensor v, bool causal, bool is_decode, int decode_length) -> Tensor");
+    m.def("finefmha_4(Tensor q, Tensor k, Tensor v, bool causal, bool is_decode, int decode_length) -> Tensor");
+    m.def("finefmha_5(Tensor q, Tensor k, Tensor v, bool causal, bool is_decode, int decode_length) -> Tensor");
+    m.def("finefmha_6(Tensor q, Tensor k, Tensor v, bool causal, bool is_decode, int decode_length) -> Tensor");
+    m.def("finefmha_7(Tensor q, Tensor k, Tensor v, bool causal, bool is_decode, int decode_length) -> Tensor");
+    m.def("finefmha_fwd_lse(Tensor q, Tensor k, Tensor v, bool causal, bool is_decode, int decode_length) -> (Tensor, Tensor)");
+}
+
+TORCH_LIBRARY_IMPL(fmha_unified, CUDA, m) {
+    m.impl("finefmha_0", &finefmha);
+    m.impl("finefmha_1", &finefmha);
+    m.impl("finefmha_2", &finefmha);
+    m.impl("finefmha_3", &finefmha);
+    m.impl("finefmha_4", &finefmha);
+    m.impl("finefmha_5", &finefmha);
+    m.impl("finefmha_6", &finefmha);
+    m.impl("finefmha_7", &finefmha);
+    m.impl("finefmha_fwd_lse", &finefmha_fwd_lse);
+}
+
+// The same functions under the CPU key: CPU tensors then reach the argument validation above and are
+// rejected with its message ("must be GPU tensors") instead of a dispatcher error. Nothing is computed on the CPU.
+TORCH_LIBRARY_IMPL(fmha_unified, CPU, m) {
+    m.impl("finefmha_0", &finefmha);
+    m.impl("finefmha_1", &finefmha);
+    m.impl("finefmha_2", &finefmha);
+    m.impl("finefmha_3", &finefmha);
+    m.impl("finefmha_4", &finefmha);
+    m.impl("finefmha_5", &finefmha);
+    m.impl("finefmha_6", &finefmha);
+    m.impl("finefmha_7", &finefmha);
+    m.impl("finefmha_fwd_lse", &finefmha_fwd_lse);
+}
+
+}  // namespace fmha_unified

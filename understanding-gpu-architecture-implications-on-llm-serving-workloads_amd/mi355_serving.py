@@ -1,0 +1,110 @@
+"""ctypes binding of libmi355_serving.so (the C ABI declared in include/mi355_serving.h).
+
+This is the torch-free boundary: plain device pointers and sizes. Tensors are used here only as a convenient way
+to own device memory and a stream; ``hgemm`` / ``fmha_fwd`` take anything with ``data_ptr()``.
+There is no fallback: if the shared library has not been built, loading raises.
+"""
+import ctypes
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libmi355_serving.so")
+
+GEMM_NN, GEMM_NT, GEMM_TN = 0, 1, 2
+LAYOUTS = {"NN": GEMM_NN, "NT": GEMM_NT, "TN": GEMM_TN}
+
+EXPORTED_SYMBOLS = ("mi355_hgemm", "mi355_fmha_fwd", "mi355_last_error", "mi355_serving_version")
+
+_lib = None
+
+
+class Mi355Error(RuntimeError):
+    def __init__(self, code, text):
+        super().__init__("%s (code %d)" % (text, code))
+        self.code = code
+
+
+def load():
+    """Load the shared library (once) and declare the argument types of its entry points."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise FileNotFoundError(
+            "%s is missing: build it with `python build.py` in %s (there is no CPU fallback)" % (LIB_PATH, _HERE))
+    import torch  # noqa: F401  loads the HIP runtime the library binds to
+    lib = ctypes.CDLL(LIB_PATH, mode=ctypes.RTLD_GLOBAL)
+    vp, i32, i64, f32 = ctypes.c_void_p, ctypes.c_int, ctypes.c_int64, ctypes.c_float
+    lib.mi355_hgemm.argtypes = [vp, vp, vp, i32, i32, i32, i64, i64, i64, i32, vp]
+    lib.mi355_hgemm.restype = i32
+    lib.mi355_fmha_fwd.argtypes = [vp, vp, vp, vp, vp, i32, i32, i32, i32, i32, i32, f32, i32, i32, vp]
+    lib.mi355_fmha_fwd.restype = i32
+    lib.mi355_last_error.argtypes = []
+    lib.mi355_last_error.restype = ctypes.c_char_p
+    lib.mi355_serving_version.argtypes = []
+    lib.mi355_serving_version.restype = i32
+    _lib = lib
+    return lib
+
+
+def _ptr(x):
+    if x is None:
+        return None
+    return x.data_ptr() if hasattr(x, "data_ptr") else int(x)
+
+
+def _check(rc):
+    if rc != 0:
+        raise Mi355Error(rc, load().mi355_last_error().decode())
+
+
+def hgemm_raw(a_ptr, b_ptr, c_ptr, M, N, K, lda, ldb, ldc, layout, stream=0):
+    """Direct call of mi355_hgemm with integer device addresses."""
+    _check(load().mi355_hgemm(a_ptr, b_ptr, c_ptr, M, N, K, lda, ldb, ldc, layout, stream))
+
+
+def fmha_fwd_raw(q_ptr, k_ptr, v_ptr, o_ptr, lse_ptr, B, Hq, Hkv, Sq, Sk, D, scale, causal, kv_valid_len, stream=0):
+    """Direct call of mi355_fmha_fwd with integer device addresses."""
+    _check(load().mi355_fmha_fwd(q_ptr, k_ptr, v_ptr, o_ptr, lse_ptr, B, Hq, Hkv, Sq, Sk, D, scale, causal,
+                                 kv_valid_len, stream))
+
+
+def hgemm(a, b, layout="NN", out=None):
+    """C = op(a) op(b) through the C ABI on torch's current stream. a, b: contiguous fp16 GPU tensors."""
+    import torch
+    lay = LAYOUTS[layout] if isinstance(layout, str) else int(layout)
+    assert a.dtype == torch.float16 and b.dtype == torch.float16 and a.is_cuda and b.is_cuda
+    assert a.is_contiguous() and b.is_contiguous()
+    if lay == GEMM_TN:
+        K, M = a.shape
+    else:
+        M, K = a.shape
+    if lay == GEMM_NT:
+        N, Kb = b.shape
+    else:
+        Kb, N = b.shape
+    if K != Kb:
+        raise ValueError("inner dimensions differ: %d vs %d" % (K, Kb))
+    if out is None:
+        out = torch.empty((M, N), dtype=torch.float16, device=a.device)
+    stream = torch.cuda.current_stream(a.device).cuda_stream
+    hgemm_raw(_ptr(a), _ptr(b), _ptr(out), M, N, K, a.stride(0), b.stride(0), out.stride(0), lay, stream)
+    return out
+
+
+def fmha_fwd(q, k, v, causal=False, kv_valid_len=None, scale=None, return_lse=True):
+    """Attention forward through the C ABI on torch's current stream. Returns (O, LSE) or O."""
+    import torch
+    assert q.dtype == torch.float16 and q.is_cuda and q.is_contiguous() and k.is_contiguous() and v.is_contiguous()
+    B, Hq, Sq, D = q.shape
+    _, Hkv, Sk, _ = k.shape
+    if scale is None:
+        scale = 1.0 / (D ** 0.5)
+    if kv_valid_len is None:
+        kv_valid_len = Sk
+    o = torch.empty_like(q)
+    lse = torch.empty((B, Hq, Sq), dtype=torch.float32, device=q.device) if return_lse else None
+    stream = torch.cuda.current_stream(q.device).cuda_stream
+    fmha_fwd_raw(_ptr(q), _ptr(k), _ptr(v), _ptr(o), _ptr(lse), B, Hq, Hkv, Sq, Sk, D, float(scale), int(bool(causal)),
+                 int(kv_valid_len), stream)
+    return (o, lse) if return_lse else o
