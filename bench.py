@@ -1,0 +1,250 @@
+#!/usr/bin/env python3
+"""Benchmark of the MI355X serving kernels on the benchmark's headline configurations.
+
+One "step" = one pass of the hot path over one batch of synthetic input, resident in HBM before timing starts:
+    1. fp16 GEMM  C = A B, M = N = K = 8192, A ~ N(0,1), B ~ N(0, 0.02^2), fp32 accumulate        (configuration G2b)
+    2. attention forward, causal GQA, b = 1, 32 q / 8 kv heads, s = 4096, d = 128, fp16, + LSE   (configuration F4)
+both called through the C ABI of libmi355_serving.so on torch's current stream.
+
+`value` is the whole-step throughput: (GEMM flops 2MNK + attention flops 4*B*Hq*d*#unmasked(q,k) pairs) / time,
+in TFLOP/s. Per-kernel figures (TFLOP/s, % of the 2.5 PFLOP/s dense fp16 MFMA peak, average launch duration
+measured with HIP events on the launch stream) are in `kernels`; `roofline` describes the dominant kernel (the
+GEMM); `cpu_baseline` is the same step on the host cores with torch fp32 (reported, not a target);
+`other_configs` lists the remaining benchmark configurations (parity cases, quick timings).
+
+Output: ONE JSON line on stdout.
+"""
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+PKG = os.path.join(ROOT, "understanding-gpu-architecture-implications-on-llm-serving-workloads_amd")
+sys.path.insert(0, PKG)
+sys.path.insert(0, os.path.join(ROOT, "oracle"))
+
+PEAK_FP16_TFLOPS = 2500.0   # MI355X dense fp16 MFMA
+PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
+
+# HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (see profiles/);
+# None until measured for the current kernel.
+MEASURED_TRAFFIC_BYTES = None
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def time_launches(fn, iters, warmup):
+    """Average duration (ms) of `iters` back-to-back launches, HIP events on the current stream."""
+    import torch
+    for _ in range(warmup):
+        fn()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    e0.record()
+    for _ in range(iters):
+        fn()
+    e1.record()
+    e1.synchronize()
+    return e0.elapsed_time(e1) / iters
+
+
+def causal_pairs(Sq, Sk):
+    shift = Sk - Sq
+    return sum(max(0, min(Sk, i + shift + 1)) for i in range(Sq))
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-other-configs", action="store_true")
+    ap.add_argument("--no-check", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build measures one GPU only (--gpus 1); multi-GPU sharding is described in "
+                 "the design notes and not implemented")
+
+    import torch
+    import mi355_serving as lib
+    import serving_oracle as so
+
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU visible; the kernels have no CPU fallback")
+    lib.load()
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+
+    # ---- synthetic inputs, resident in HBM -------------------------------------------------------------------
+    M = N = K = 8192
+    a_h, b_h = so.gemm_inputs(M, N, K, seed=0, a_std=1.0, b_std=0.02)
+    a, b = a_h.to(dev), b_h.to(dev)
+    c = torch.empty((M, N), dtype=torch.float16, device=dev)
+    B_, Hq, Hkv, S, D = 1, 32, 8, 4096, 128
+    q_h, k_h, v_h = so.fmha_inputs(B_, Hq, Hkv, S, S, seed=42)
+    q, k, v = q_h.to(dev), k_h.to(dev), v_h.to(dev)
+    o = torch.empty_like(q)
+    lse = torch.empty((B_, Hq, S), dtype=torch.float32, device=dev)
+    scale = 1.0 / math.sqrt(D)
+    stream = torch.cuda.current_stream().cuda_stream
+
+    def gemm():
+        lib.hgemm_raw(a.data_ptr(), b.data_ptr(), c.data_ptr(), M, N, K, K, N, N, lib.GEMM_NN, stream)
+
+    def fmha():
+        lib.fmha_fwd_raw(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), lse.data_ptr(), B_, Hq, Hkv, S, S, D,
+                         scale, 1, S, stream)
+
+    gemm_flops = 2.0 * M * N * K
+    fmha_flops = 4.0 * B_ * Hq * D * causal_pairs(S, S)       # causal-discounted (algorithmic)
+    fmha_flops_ref_convention = 4.0 * S * S * D * Hq          # kernels/fmha/test/perf.py:89 (no causal discount)
+
+    # ---- correctness of what is being timed (sampled rows against the oracle) ----------------------------------
+    checks = {}
+    if not args.no_check:
+        gemm(); fmha(); torch.cuda.synchronize()
+        rows = torch.arange(0, M, 127)
+        ok_g, st_g = so.gemm_tolerance_ok(c[rows.to(dev)], so.gemm_ref(a_h[rows], b_h), K)
+        heads = [0, 13, 31]
+        oks, stf = True, {}
+        for h in heads:
+            orf, lrf = so.attention_ref(q_h[:, h:h + 1], k_h[:, h // 4:h // 4 + 1], v_h[:, h // 4:h // 4 + 1], causal=True)
+            okh, sth = so.fmha_tolerance_ok(o[:, h:h + 1], lse[:, h:h + 1], orf, lrf)
+            oks = oks and okh
+            stf = {kk: max(stf.get(kk, 0.0), vv) for kk, vv in sth.items()}
+        checks = {"gemm_within_tolerance": bool(ok_g), "gemm": st_g, "fmha_within_tolerance": bool(oks), "fmha": stf}
+        log("[bench] parity of the timed configuration:", checks)
+        if not (ok_g and oks):
+            sys.exit("bench.py: timed configuration is outside tolerance: %s" % checks)
+
+    # ---- timed region: exactly K steps between device synchronisations -------------------------------------------
+    for _ in range(args.warmup):
+        gemm(); fmha()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        gemm(); fmha()
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+    value = (gemm_flops + fmha_flops) / (ms_per_step * 1e-3) / 1e12
+
+    # ---- per-kernel launch durations (HIP events on the launch stream) --------------------------------------------
+    gemm_ms = time_launches(gemm, args.steps, 2)
+    fmha_ms = time_launches(fmha, args.steps, 2)
+    gemm_tf = gemm_flops / (gemm_ms * 1e-3) / 1e12
+    fmha_tf = fmha_flops / (fmha_ms * 1e-3) / 1e12
+    kernels = {
+        "hgemm_8192x8192x8192_nn": {"ms": gemm_ms, "tflops": gemm_tf, "pct_of_fp16_mfma_peak": 100 * gemm_tf / PEAK_FP16_TFLOPS},
+        "fmha_fwd_causal_gqa_b1_h32_8_s4096_d128": {
+            "ms": fmha_ms, "tflops": fmha_tf, "pct_of_fp16_mfma_peak": 100 * fmha_tf / PEAK_FP16_TFLOPS,
+            "tflops_reference_convention_4s2dh": fmha_flops_ref_convention / (fmha_ms * 1e-3) / 1e12},
+    }
+    roofline = {"kernel": "hgemm_main_kernel (8192^3, NN)", "bound": "mfma", "achieved": gemm_tf, "peak": PEAK_FP16_TFLOPS,
+                "unit": "TFLOP/s", "frac": gemm_tf / PEAK_FP16_TFLOPS, "traffic": MEASURED_TRAFFIC_BYTES}
+    roofline_fmha = {"kernel": "fmha_fwd_kernel (F4)", "bound": "mfma", "achieved": fmha_tf, "peak": PEAK_FP16_TFLOPS,
+                     "unit": "TFLOP/s", "frac": fmha_tf / PEAK_FP16_TFLOPS, "traffic": None}
+
+    # ---- the other benchmark configurations (quick timings) ----------------------------------------------------------
+    other = {}
+    if not args.no_other_configs:
+        def t_gemm(m, n, kk, iters=20):
+            x = so.randn_fp16((m, kk), 1).to(dev)
+            w = so.randn_fp16((kk, n), 2, 0.02).to(dev)
+            out = torch.empty((m, n), dtype=torch.float16, device=dev)
+            ms = time_launches(lambda: lib.hgemm_raw(x.data_ptr(), w.data_ptr(), out.data_ptr(), m, n, kk, kk, n, n,
+                                                     lib.GEMM_NN, stream), iters, 3)
+            fl, by = 2.0 * m * n * kk, 2.0 * (m * kk + kk * n + m * n)
+            return {"ms": ms, "tflops": fl / ms / 1e9, "pct_of_fp16_mfma_peak": 100 * fl / ms / 1e9 / PEAK_FP16_TFLOPS,
+                    "gbs": by / ms / 1e6, "pct_of_hbm_peak": 100 * by / ms / 1e6 / PEAK_HBM_GBS}
+        other["G1_gemm_1024"] = t_gemm(1024, 1024, 1024)
+        other["G2a_gemm_4096"] = t_gemm(4096, 4096, 4096)
+        other["G2c_gemm_decode_16x14336x4096"] = t_gemm(16, 14336, 4096)
+        q3, k3, v3 = (t.to(dev) for t in so.fmha_inputs(4, 32, 32, 1024, 1024, seed=42))
+        o3 = torch.empty_like(q3)
+        ms3 = time_launches(lambda: lib.fmha_fwd_raw(q3.data_ptr(), k3.data_ptr(), v3.data_ptr(), o3.data_ptr(), None, 4, 32,
+                                                     32, 1024, 1024, 128, scale, 0, 1024, stream), 20, 3)
+        fl3 = 4.0 * 4 * 32 * 128 * 1024 * 1024
+        other["F3_fmha_noncausal_b4_h32_s1024"] = {"ms": ms3, "tflops": fl3 / ms3 / 1e9,
+                                                   "pct_of_fp16_mfma_peak": 100 * fl3 / ms3 / 1e9 / PEAK_FP16_TFLOPS}
+        del q3, k3, v3, o3
+        # L5: Llama-3-8B-shaped prefill layer at s = 8192, per stage
+        S5, H5, F5 = 8192, 4096, 14336
+        x5 = so.randn_fp16((S5, H5), 0).to(dev)
+        wqkv, wo = so.randn_fp16((H5, 6144), 1, 0.02).to(dev), so.randn_fp16((H5, H5), 2, 0.02).to(dev)
+        wgu, wd = so.randn_fp16((H5, 2 * F5), 3, 0.02).to(dev), so.randn_fp16((F5, H5), 4, 0.02).to(dev)
+        st = {}
+        def stage(name, fn, flops, iters=5):
+            ms = time_launches(fn, iters, 1)
+            st[name] = {"ms": ms, "tflops": flops / ms / 1e9}
+        qkv5 = torch.empty((S5, 6144), dtype=torch.float16, device=dev)
+        stage("qkv_gemm", lambda: lib.hgemm(x5, wqkv, out=qkv5), 2.0 * S5 * H5 * 6144)
+        q5 = qkv5[:, :4096].reshape(S5, 32, 128).permute(1, 0, 2)[None].contiguous()
+        k5 = qkv5[:, 4096:5120].reshape(S5, 8, 128).permute(1, 0, 2)[None].contiguous()
+        v5 = qkv5[:, 5120:].reshape(S5, 8, 128).permute(1, 0, 2)[None].contiguous()
+        o5 = torch.empty_like(q5)
+        stage("fmha_causal_gqa_s8192", lambda: lib.fmha_fwd_raw(q5.data_ptr(), k5.data_ptr(), v5.data_ptr(), o5.data_ptr(),
+                                                                 None, 1, 32, 8, S5, S5, 128, scale, 1, S5, stream),
+              4.0 * 32 * 128 * causal_pairs(S5, S5))
+        a5 = o5[0].permute(1, 0, 2).reshape(S5, H5).contiguous()
+        op5 = torch.empty((S5, H5), dtype=torch.float16, device=dev)
+        stage("oproj_gemm", lambda: lib.hgemm(a5, wo, out=op5), 2.0 * S5 * H5 * H5)
+        gu5 = torch.empty((S5, 2 * F5), dtype=torch.float16, device=dev)
+        stage("gate_up_gemm", lambda: lib.hgemm(op5, wgu, out=gu5), 2.0 * S5 * H5 * 2 * F5)
+        act5 = (torch.nn.functional.silu(gu5[:, :F5].float()) * gu5[:, F5:].float()).half()
+        dn5 = torch.empty((S5, H5), dtype=torch.float16, device=dev)
+        stage("down_gemm", lambda: lib.hgemm(act5, wd, out=dn5), 2.0 * S5 * F5 * H5)
+        tot_ms = sum(s["ms"] for s in st.values())
+        tot_fl = 2.0 * S5 * H5 * 6144 + 4.0 * 32 * 128 * causal_pairs(S5, S5) + 2.0 * S5 * H5 * H5 + 2.0 * S5 * H5 * 2 * F5 + 2.0 * S5 * F5 * H5
+        other["L5_llama3_8b_layer_s8192"] = {"stages": st, "kernel_ms_total": tot_ms, "tflops_total": tot_fl / tot_ms / 1e9,
+                                             "note": "GEMM and attention stages only; reshapes and SiLU*up run in torch and are not timed; no RoPE/norm/residual"}
+
+    # ---- CPU baseline: the same step with torch fp32 on the host cores -------------------------------------------------
+    cpu_baseline = None
+    if not args.no_cpu_baseline:
+        cores = torch.get_num_threads()
+        a32, b32 = a_h.float(), b_h.float()
+        so.attention_sdpa_ref(q_h[:, :2], k_h[:, :1], v_h[:, :1], True)  # warm up the SDPA path on a small slice
+        t0 = time.perf_counter()
+        torch.matmul(a32, b32)
+        t_g = time.perf_counter() - t0
+        t0 = time.perf_counter()
+        so.attention_sdpa_ref(q_h, k_h, v_h, True)
+        t_f = time.perf_counter() - t0
+        cpu_baseline = {"value": (gemm_flops + fmha_flops) / (t_g + t_f) / 1e12, "unit": "TFLOP/s", "cores": cores,
+                        "kind": "port",
+                        "sample": "one full step on the host: torch.matmul fp32 8192^3 (%.2f s, %.3f TFLOP/s) + torch SDPA fp32 "
+                                  "causal GQA F4 with repeat_kv (%.2f s, %.3f TFLOP/s algorithmic); single run, no warm-up of the GEMM"
+                                  % (t_g, gemm_flops / t_g / 1e12, t_f, fmha_flops / t_f / 1e12),
+                        "cpu": _cpu_model()}
+
+    out = {
+        "metric": "TFLOP/s + % fp16 MFMA peak: GEMM 8192^3 and causal GQA FMHA s=4096 d=128",
+        "value": value, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "fp16 (fp32 accumulate)", "data": "synthetic",
+        "config": {"workload": "one step = hgemm 8192x8192x8192 NN (G2b) + fmha fwd causal GQA b1 h32/8 s4096 d128 with LSE (F4)",
+                   "flops_per_step": gemm_flops + fmha_flops, "pct_of_fp16_mfma_peak": 100 * value / PEAK_FP16_TFLOPS},
+        "kernels": kernels, "roofline": roofline, "roofline_fmha": roofline_fmha, "cpu_baseline": cpu_baseline,
+        "other_configs": other, "parity": checks,
+    }
+    print(json.dumps(out))
+
+
+def _cpu_model():
+    try:
+        for line in open("/proc/cpuinfo"):
+            if line.startswith("model name"):
+                return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
+if __name__ == "__main__":
+    main()

@@ -17,6 +17,8 @@ oracle states those results directly in fp32 (torch) and, for small inputs, agai
                       generalised to the bottom-right alignment (identical when Sq == Sk); keys at or beyond
                       kv_valid_len are masked (fmha_2_amd.cpp:191 with its off-by-one corrected); scale 1/sqrt(d)
                       follows fmha_2_amd.cpp:320.
+  attention_sdpa_ref  the reference's test-side baseline torch_attn (kernels/fmha/test/perf.py:10-24): repeat_kv +
+                      torch SDPA; checked against attention_ref, used as the timed CPU baseline.
   fine_fmha_ref       the pad-to-64 / decode_length / slice shim of kernels/fmha/pkg/fmha_unified/ops.py:8-29
                       expressed on top of attention_ref (padding rows are masked, so it reduces to attention_ref).
   llama_layer_ref     the Llama-3-8B-shaped prefill chain of the benchmark configuration (QKV GEMM -> causal GQA
@@ -150,6 +152,20 @@ def fine_fmha_ref(q, k, v, causal: bool, is_decode: bool):
     if is_decode and causal:
         raise ValueError("causal is not supported in decode mode")  # semi/fmha_2_amd.cpp:331-333
     return attention_ref(q, k, v, causal=causal, kv_valid_len=k.shape[2])[0]
+
+
+def attention_sdpa_ref(q, k, v, causal: bool = False):
+    """The reference's own test baseline (kernels/fmha/test/perf.py:10-24, correct.py:9-23): repeat the kv heads
+    (repeat_kv == repeat_interleave on dim 1) and call torch's scaled_dot_product_attention, here in fp32 on the
+    CPU. Top-left causal alignment, so only meaningful for Sq == Sk when causal. Used as the timed CPU baseline."""
+    q32 = q.detach().to("cpu", torch.float32)
+    k32 = k.detach().to("cpu", torch.float32)
+    v32 = v.detach().to("cpu", torch.float32)
+    rep = q32.shape[1] // k32.shape[1]
+    if rep > 1:
+        k32 = k32.repeat_interleave(rep, dim=1)
+        v32 = v32.repeat_interleave(rep, dim=1)
+    return torch.nn.functional.scaled_dot_product_attention(q32, k32, v32, is_causal=causal)
 
 
 def attention_bruteforce_f64(q, k, v, causal=False, kv_valid_len=None, scale=None):

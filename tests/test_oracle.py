@@ -165,6 +165,7 @@ def test_attention_vs_torch_sdpa():
         ref = torch.nn.functional.scaled_dot_product_attention(q.float(), kk, vv, is_causal=causal)
         assert torch.allclose(so.attention_ref(q, k, v, causal=causal)[0], ref, atol=2e-6)
         assert torch.allclose(so.fine_fmha_ref(q, k, v, causal, False), ref, atol=2e-6)
+        assert torch.allclose(so.attention_sdpa_ref(q, k, v, causal), ref, atol=1e-6)
     with pytest.raises(ValueError):
         so.fine_fmha_ref(q, k, v, True, True)
 
