@@ -114,6 +114,20 @@ struct MainCfg {
     static constexpr int A_INSTS = 4, B_INSTS = 4;
 };
 
+// Scheduling hint: alternate NMFMA matrix instructions with NDS LDS reads, spreading the reads evenly
+// (sched_group_barrier wants literal counts, hence the recursion over the MFMA index).
+template <int M, int NMFMA, int NDS>
+struct InterleaveMfmaWithLdsReads {
+    __device__ static __forceinline__ void emit() {
+        if constexpr (M < NMFMA) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // one MFMA
+            constexpr int nds = NDS * (M + 1) / NMFMA - NDS * M / NMFMA;
+            if constexpr (nds > 0) __builtin_amdgcn_sched_group_barrier(0x100, nds, 0);  // LDS reads
+            InterleaveMfmaWithLdsReads<M + 1, NMFMA, NDS>::emit();
+        }
+    }
+};
+
 // Map the linear workgroup id to a C tile so that the workgroups resident on one XCD (ids congruent mod 8)
 // cover a compact rectangle of tiles: they then share A row-panels and B column-panels in that XCD's L2.
 __device__ __forceinline__ void tile_of_block(int bid, int tiles_m, int tiles_n, int& tm, int& tn) {
@@ -224,44 +238,92 @@ __global__ __launch_bounds__(512) void hgemm_main_kernel(const half_t* __restric
 #pragma unroll
             for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 
-    const int ktiles = K / BK;
-    issue_copies(0);
+    // fragment loads of one k-substep (16 deep) from stage `st`
+    auto load_frags = [&](MI355_LDS char* st, int kk, half8(&af)[TM], half8(&bf)[TN]) {
+#pragma unroll
+        for (int i = 0; i < TM; ++i) {
+            if constexpr (A_KC) {
+                af[i] = lds_read_b128(st + a_off[kk] + i * 32 * ATK::kRowBytes);
+            } else {
+                half4 lo = lds_read_tr16_b64(st + a_off[i] + (kk * 16) * ATM::kRowBytes);
+                half4 hi = lds_read_tr16_b64(st + a_off[i] + (kk * 16 + 4) * ATM::kRowBytes);
+                af[i] = concat(lo, hi);
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+            if constexpr (B_KC) {
+                bf[j] = lds_read_b128(st + b_off[kk] + j * 32 * BTK::kRowBytes);
+            } else {
+                half4 lo = lds_read_tr16_b64(st + b_off[j] + (kk * 16) * BTN::kRowBytes);
+                half4 hi = lds_read_tr16_b64(st + b_off[j] + (kk * 16 + 4) * BTN::kRowBytes);
+                bf[j] = concat(lo, hi);
+            }
+        }
+    };
+    auto mma = [&](const half8(&af)[TM], const half8(&bf)[TN]) {
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bf[j], af[i], acc[i][j], 0, 0, 0);
+    };
+    // ask the scheduler to alternate the TM*TN MFMAs of one substep with the LDS reads of the next one
+    constexpr int kDsReads = (A_KC ? TM : 2 * TM) + (B_KC ? TN : 2 * TN);
+    auto interleave = [&]() {
+#ifndef EXP_NOSCHED
+        InterleaveMfmaWithLdsReads<0, TM * TN, kDsReads>::emit();
+#endif
+    };
 
-    for (int kt = 0; kt < ktiles; ++kt) {
+    // Software pipeline: the fragments of substep kk+1 are read from LDS while the MFMAs of substep kk run;
+    // the barrier that hands over the next K tile sits in front of the LAST substep of the current tile, so
+    // the first fragments of the next tile are read under that substep's MFMAs and no wave starts a tile
+    // with an exposed LDS round trip.
+    const int ktiles = K / BK;
+    half8 af[2][TM], bf[2][TN];
+    issue_copies(0);
+    wait_vmcnt<0>();
+    __syncthreads();
+    if (ktiles > 1) issue_copies(1);
+    load_frags(smem, 0, af[0], bf[0]);
+
+    for (int kt = 0; kt + 1 < ktiles; ++kt) {
+        MI355_LDS char* st = smem + (kt & 1) * Cfg::STAGE_BYTES;
+        MI355_LDS char* stn = smem + ((kt + 1) & 1) * Cfg::STAGE_BYTES;
+        load_frags(st, 1, af[1], bf[1]);
+        mma(af[0], bf[0]);
+        interleave();
+        load_frags(st, 2, af[0], bf[0]);
+        mma(af[1], bf[1]);
+        interleave();
+        load_frags(st, 3, af[1], bf[1]);
+        mma(af[0], bf[0]);
+        interleave();
+        // my copies of tile kt+1 have landed and my reads of this stage are complete; after the barrier that
+        // holds for every wave, so this stage may be refilled and the next one may be read
+#ifndef EXP_NOBARRIER
         wait_vmcnt<0>();
         __syncthreads();
-        if (kt + 1 < ktiles) issue_copies((kt + 1) & 1);
-
-        MI355_LDS char* st = smem + (kt & 1) * Cfg::STAGE_BYTES;
-#pragma unroll
-        for (int kk = 0; kk < BK / 16; ++kk) {
-            half8 af[TM], bf[TN];
-#pragma unroll
-            for (int i = 0; i < TM; ++i) {
-                if constexpr (A_KC) {
-                    af[i] = lds_read_b128(st + a_off[kk] + i * 32 * ATK::kRowBytes);
-                } else {
-                    half4 lo = lds_read_tr16_b64(st + a_off[i] + (kk * 16) * ATM::kRowBytes);
-                    half4 hi = lds_read_tr16_b64(st + a_off[i] + (kk * 16 + 4) * ATM::kRowBytes);
-                    af[i] = concat(lo, hi);
-                }
-            }
-#pragma unroll
-            for (int j = 0; j < TN; ++j) {
-                if constexpr (B_KC) {
-                    bf[j] = lds_read_b128(st + b_off[kk] + j * 32 * BTK::kRowBytes);
-                } else {
-                    half4 lo = lds_read_tr16_b64(st + b_off[j] + (kk * 16) * BTN::kRowBytes);
-                    half4 hi = lds_read_tr16_b64(st + b_off[j] + (kk * 16 + 4) * BTN::kRowBytes);
-                    bf[j] = concat(lo, hi);
-                }
-            }
-#pragma unroll
-            for (int i = 0; i < TM; ++i)
-#pragma unroll
-                for (int j = 0; j < TN; ++j)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bf[j], af[i], acc[i][j], 0, 0, 0);
-        }
+#endif
+#ifndef EXP_NOLOAD
+        if (kt + 2 < ktiles) issue_copies(kt & 1);
+#endif
+        load_frags(stn, 0, af[0], bf[0]);
+        mma(af[1], bf[1]);
+        interleave();
+    }
+    {  // last tile: nothing left to fetch
+        MI355_LDS char* st = smem + ((ktiles - 1) & 1) * Cfg::STAGE_BYTES;
+        load_frags(st, 1, af[1], bf[1]);
+        mma(af[0], bf[0]);
+        interleave();
+        load_frags(st, 2, af[0], bf[0]);
+        mma(af[1], bf[1]);
+        interleave();
+        load_frags(st, 3, af[1], bf[1]);
+        mma(af[0], bf[0]);
+        mma(af[1], bf[1]);
     }
 
     // ---- epilogue: lane holds C[m][n .. n+3] for m = l%32, n = 8p + 4*(l/32) ----------------------------
@@ -326,6 +388,152 @@ __global__ __launch_bounds__(256) void hgemm_edge_kernel(const half_t* __restric
         }
 }
 
+// ---------------------------------------------------------------------------------------------------------
+// Small-M kernel (decode-shaped GEMM, M <= 16 rows per workgroup row), layout NN. HBM-bound: B is streamed once.
+//   * a workgroup owns 64 columns of C; its 8 waves split K between them (in-workgroup split-K, reduced
+//     through LDS at the end, so no global workspace and no atomics);
+//   * every wave runs its own copy pipeline, without workgroup barriers: per 32-deep k-step it copies a
+//     32x64 slab of B (4 KiB) and a 16x32 slab of A (1 KiB) global -> LDS with 16-byte direct-to-LDS copies,
+//     keeps kSmallMStages-1 steps in flight, and waits for the oldest with s_waitcnt vmcnt;
+//   * B fragments are read with the transposing LDS read, the product is MFMA 16x16x32.
+// ---------------------------------------------------------------------------------------------------------
+constexpr int kSmallMStages = 3;
+constexpr int kSmallMStageBytes = 5 * 1024;  // 4 KiB of B + 1 KiB of A
+constexpr int kSmallMWaveBytes = kSmallMStages * kSmallMStageBytes;
+constexpr int kSmallMLdsBytes = 8 * kSmallMWaveBytes;
+
+__global__ __launch_bounds__(512) void hgemm_smallm_nn_kernel(const half_t* __restrict__ A, const half_t* __restrict__ B,
+                                                              half_t* __restrict__ C, int M, int N, int K, long lda,
+                                                              long ldb, long ldc, int n_tiles) {
+    extern __shared__ __attribute__((aligned(1024))) char smem_raw[];
+    MI355_LDS char* smem = (MI355_LDS char*)smem_raw;
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+
+    // consecutive column tiles stay on one XCD so neighbouring 128-byte row segments meet in the same L2
+    int tile = blockIdx.x;
+    if (n_tiles % 8 == 0) tile = (blockIdx.x % 8) * (n_tiles / 8) + blockIdx.x / 8;
+    const int n0 = tile * 64;
+    const int m0 = blockIdx.y * 16;
+
+    const int ksteps = K / 32;
+    const int s_begin = (int)((long)wave * ksteps / 8);
+    const int s_end = (int)((long)(wave + 1) * ksteps / 8);
+
+    MI355_LDS char* wbase = smem + wave * kSmallMWaveBytes;
+
+    // ---- copy descriptors -------------------------------------------------------------------------------
+    // B slab: 32 rows (k) x 128 bytes; copy i covers rows 8i .. 8i+7, chunk position lane%8, chunk c of row r
+    // is stored at position c ^ 2*(r%4) (keeps the 16 lanes of a transposing read on distinct banks)
+    const int b_row = lane >> 3;                                  // + 8*i
+    const int b_chunk = (lane & 7) ^ (2 * (b_row & 3));           // (8i + b_row) % 4 == b_row % 4
+    const int n_chunk_max = N / 8 - 1;
+    const int b_col = min(n0 / 8 + b_chunk, n_chunk_max) * 8;     // clamp: columns past N are never stored
+    const half_t* b_src = B + (long)(s_begin * 32 + b_row) * ldb + b_col;
+    // A slab: 16 rows (m) x 64 bytes; row lane/4, chunk position lane%4, chunk c of row r at c ^ ((r>>1)&3)
+    const int a_row = lane >> 2;
+    const int a_chunk = (lane & 3) ^ ((a_row >> 1) & 3);
+    const half_t* a_src = A + (long)min(m0 + a_row, M - 1) * lda + (long)s_begin * 32 + a_chunk * 8;
+
+    auto issue_stage = [&](int slot) {
+        MI355_LDS char* st = wbase + slot * kSmallMStageBytes;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) copy16_global_to_lds(b_src + (long)(8 * i) * ldb, st + i * 1024);
+        copy16_global_to_lds(a_src, st + 4096);
+        b_src += 32 * ldb;
+        a_src += 32;
+    };
+
+    // ---- fragment read offsets inside a stage ---------------------------------------------------------------
+    // A fragment: lane holds A[m = lane%16][k = 8*(lane/16) .. +7]
+    const int a_off = 4096 + (lane & 15) * 64 + (((lane >> 4) ^ (((lane & 15) >> 1) & 3)) << 4);
+    // B fragment of column block j: rows 8*(lane/16) + 4t + (lane%16)/4, columns 16j + 4*(lane%4) .. +3
+    const int bt_row = 8 * (lane >> 4) + ((lane & 15) >> 2);
+    const int bt_swz = 2 * (bt_row & 3);
+    int b_off[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        int chunk = (2 * j + ((lane & 3) >> 1)) ^ bt_swz;
+        b_off[j] = bt_row * 128 + chunk * 16 + (lane & 1) * 8;
+    }
+
+    float4v acc[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc[j] = float4v{0.f, 0.f, 0.f, 0.f};
+
+    // ---- pipeline ---------------------------------------------------------------------------------------------
+    int issued = s_begin;
+#pragma unroll
+    for (int i = 0; i < kSmallMStages - 1; ++i)
+        if (issued < s_end) {
+            issue_stage(i);
+            ++issued;
+        }
+    int slot = 0, fill = kSmallMStages - 1;
+    for (int s = s_begin; s < s_end; ++s) {
+        if (issued < s_end) {
+            issue_stage(fill);
+            ++issued;
+            fill = (fill + 1 == kSmallMStages) ? 0 : fill + 1;
+            wait_vmcnt<5 * (kSmallMStages - 1)>();  // everything but the newest kSmallMStages-1 steps has landed
+        } else {
+            wait_vmcnt<0>();
+        }
+        MI355_LDS char* st = wbase + slot * kSmallMStageBytes;
+        slot = (slot + 1 == kSmallMStages) ? 0 : slot + 1;
+        half8 af = lds_read_b128(st + a_off);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            half4 lo = lds_read_tr16_b64(st + b_off[j]);
+            half4 hi = lds_read_tr16_b64(st + b_off[j] + 4 * 128);
+            acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(af, concat(lo, hi), acc[j], 0, 0, 0);
+        }
+        // the reads of this slot must be complete before a later copy refills it
+        wait_lgkmcnt<0>();
+    }
+
+    // ---- reduce the 8 partial tiles through LDS ---------------------------------------------------------------
+    // acc[j][q] is D[m = 4*(lane/16) + q][n = 16j + lane%16]
+    __syncthreads();  // every wave is done with its staging memory
+    MI355_LDS float* red = (MI355_LDS float*)smem;
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) red[wave * 1024 + (4 * (lane >> 4) + q) * 64 + 16 * j + (lane & 15)] = acc[j][q];
+    __syncthreads();
+    const int o = tid * 2;  // two neighbouring columns of one row
+    float s0 = 0.f, s1 = 0.f;
+#pragma unroll
+    for (int w = 0; w < 8; ++w) {
+        s0 += red[w * 1024 + o];
+        s1 += red[w * 1024 + o + 1];
+    }
+    const int m = m0 + (o >> 6);
+    const int n = n0 + (o & 63);
+    if (m < M && n < N) {
+        half2v v;
+        v[0] = (half_t)s0;
+        v[1] = (half_t)s1;
+        *(half2v*)(C + (long)m * ldc + n) = v;
+    }
+}
+
+static hipError_t launch_smallm_nn(const half_t* A, const half_t* B, half_t* C, int M, int N, int K, long lda, long ldb,
+                                   long ldc, hipStream_t stream) {
+    static bool attr_set = false;
+    if (!attr_set) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(hgemm_smallm_nn_kernel),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, kSmallMLdsBytes);
+        if (e != hipSuccess) return e;
+        attr_set = true;
+    }
+    const int n_tiles = (N + 63) / 64;
+    dim3 grid(n_tiles, (M + 15) / 16);
+    hgemm_smallm_nn_kernel<<<grid, dim3(512), kSmallMLdsBytes, stream>>>(A, B, C, M, N, K, lda, ldb, ldc, n_tiles);
+    return hipGetLastError();
+}
+
 template <bool A_KC, bool B_KC>
 static hipError_t launch_layout(const half_t* A, const half_t* B, half_t* C, int M, int N, int K, long lda, long ldb,
                                 long ldc, hipStream_t stream) {
@@ -345,6 +553,10 @@ static hipError_t launch_layout(const half_t* A, const half_t* B, half_t* C, int
         int blocks = (M / Cfg::BM) * (N / Cfg::BN);
         kern<<<dim3(blocks), dim3(Cfg::NTHREADS), Cfg::LDS_BYTES, stream>>>(A, B, C, M, N, K, lda, ldb, ldc);
         return hipGetLastError();
+    }
+    if constexpr (A_KC && !B_KC) {
+        if (aligned && M <= 64 && K % 32 == 0 && K >= 32 && N % 8 == 0 && ldc % 2 == 0)
+            return launch_smallm_nn(A, B, C, M, N, K, lda, ldb, ldc, stream);
     }
     dim3 grid((N + 63) / 64, (M + 63) / 64);
     hgemm_edge_kernel<A_KC, B_KC><<<grid, dim3(256), 0, stream>>>(A, B, C, M, N, K, lda, ldb, ldc);
