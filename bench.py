@@ -66,6 +66,9 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-other-configs", action="store_true")
     ap.add_argument("--no-check", action="store_true")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also launch one 1 GiB device-to-device copy, so FETCH_SIZE / WRITE_SIZE read under rocprofv3 "
+                         "--pmc can be scaled by what the same counter reports for a transfer of known size")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU only (--gpus 1); multi-GPU sharding is described in "
@@ -122,6 +125,13 @@ def main():
         log("[bench] parity of the timed configuration:", checks)
         if not (ok_g and oks):
             sys.exit("bench.py: timed configuration is outside tolerance: %s" % checks)
+
+    if args.calibrate_copy:
+        src = torch.empty(1 << 30, dtype=torch.uint8, device=dev).fill_(1)
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
 
     # ---- timed region: exactly K steps between device synchronisations -------------------------------------------
     for _ in range(args.warmup):

@@ -29,6 +29,7 @@ constexpr int ROW_BYTES = D * 2;  // 256
 constexpr int TILE_BYTES = BN * ROW_BYTES;  // 16 KiB
 constexpr int STAGE_BYTES = 2 * TILE_BYTES; // K + V
 constexpr int NSTAGE = 2;
+constexpr float kLazyLog2 = 8.f;  // rescale only when a row maximum grows by more than 2^8
 
 __device__ __forceinline__ int swz_k(int row) { return row & 15; }
 __device__ __forceinline__ int swz_v(int row) {
@@ -68,7 +69,7 @@ __device__ __forceinline__ void fmha_decode_block(int bid, int q_tiles, int grou
 }
 
 template <int NQ, int NWAVES>
-__global__ __launch_bounds__(NWAVES * 64) void fmha_fwd_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K,
+__global__ __launch_bounds__(NWAVES * 64, (NQ == 1 ? 2 : 1)) void fmha_fwd_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K,
                                                                const half_t* __restrict__ V, half_t* __restrict__ O,
                                                                float* __restrict__ LSE, int B, int Hq, int Hkv, int Sq,
                                                                int Sk, float scale_log2, int causal, int kv_valid,
@@ -209,7 +210,11 @@ __global__ __launch_bounds__(NWAVES * 64) void fmha_fwd_kernel(const half_t* __r
             }
         }
 
-        // ---- online softmax --------------------------------------------------------------------------------
+        // ---- online softmax with lazy rescaling --------------------------------------------------------------
+        // m_run is the exponent reference of the running sums, not necessarily the running maximum: it is only
+        // raised (and O, l rescaled) when some row of the wave exceeds it by more than 2^kLazyLog2, which after the
+        // first tiles almost never happens; until then P = exp2((S - m_run) * c) is at most 2^kLazyLog2, exact in
+        // fp16/fp32 terms, and the final O / l and LSE do not depend on the choice of reference.
         half8 pf[NQ][2][2];
 #pragma unroll
         for (int qb = 0; qb < NQ; ++qb) {
@@ -219,11 +224,19 @@ __global__ __launch_bounds__(NWAVES * 64) void fmha_fwd_kernel(const half_t* __r
 #pragma unroll
                 for (int e = 0; e < 16; ++e) mx = fmaxf(mx, s[qb][kb][e]);
             mx = halves_max(mx);
-            float m_new = fmaxf(m_run[qb], mx);
-            float m_use = (m_new == -INFINITY) ? 0.f : m_new;
-            float alpha = fast_exp2((m_run[qb] - m_use) * scale_log2);
-            m_run[qb] = m_new;
-            float neg_ms = -m_use * scale_log2;
+            const bool raise = (mx - m_run[qb]) * scale_log2 > kLazyLog2;  // -inf - -inf = NaN compares false
+            if (__builtin_amdgcn_ballot_w64(raise) != 0) {
+                float m_new = fmaxf(m_run[qb], mx);
+                float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+                float alpha = fast_exp2((m_run[qb] - m_use) * scale_log2);
+                m_run[qb] = m_new;
+                l_run[qb] *= alpha;
+#pragma unroll
+                for (int db = 0; db < 4; ++db)
+#pragma unroll
+                    for (int e = 0; e < 16; ++e) o[qb][db][e] *= alpha;
+            }
+            const float neg_ms = (m_run[qb] == -INFINITY) ? 0.f : -m_run[qb] * scale_log2;
             float psum = 0.f;
 #pragma unroll
             for (int kb = 0; kb < 2; ++kb) {
@@ -241,11 +254,7 @@ __global__ __launch_bounds__(NWAVES * 64) void fmha_fwd_kernel(const half_t* __r
                     pf[qb][kb][tt] = pk;
                 }
             }
-            l_run[qb] = l_run[qb] * alpha + psum;
-#pragma unroll
-            for (int db = 0; db < 4; ++db)
-#pragma unroll
-                for (int e = 0; e < 16; ++e) o[qb][db][e] *= alpha;
+            l_run[qb] += psum;
         }
 
         // ---- O^T += V^T P^T ----------------------------------------------------------------------------------
