@@ -300,6 +300,309 @@ __global__ __launch_bounds__(NWAVES * 64, (NQ == 1 ? 2 : 1)) void fmha_fwd_kerne
     }
 }
 
+// ---------------------------------------------------------------------------------------------------------
+// Ping-pong kernel: 8 waves x 32 queries per workgroup, two waves per SIMD that alternate roles.
+// Same mathematics and LDS layouts as fmha_fwd_kernel. A wave alternates between
+//     an M phase: 16 MFMAs of S(j+1) = K(j+1) Q^T and 16 MFMAs of O += V(j)^T P(j)   (matrix pipe + LDS reads)
+//     a  V phase: softmax of S(j+1) -> P(j+1)                                          (VALU only)
+// separated by workgroup barriers. Waves 4..7 run one phase behind waves 0..3, so on every SIMD one wave is in
+// its M phase while the other is in its V phase: the matrix pipe and the VALU are busy at the same time without
+// relying on the instruction scheduler to interleave them inside one wave. The phases of the workgroup are
+// numbered P0, P1, ...; waves 0..3 run M in the even ones, waves 4..7 in the odd ones.
+// K and V have separate double buffers: tile j lives in Kbuf[j&1] / Vbuf[j&1], is copied by all 8 waves at the
+// start of an even phase (K(i+1) and V(i) at P(2i)) and has two phases to land (waited for at the end of P(2i+1)).
+// ---------------------------------------------------------------------------------------------------------
+template <int NMFMA, int NDS>
+struct InterleaveMfmaLds {
+    template <int M>
+    __device__ static __forceinline__ void emit() {
+        if constexpr (M < NMFMA) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);    // one MFMA
+            __builtin_amdgcn_sched_group_barrier(0x100, NDS, 0);  // LDS reads of a later MFMA
+            emit<M + 1>();
+        }
+    }
+};
+
+__global__ __launch_bounds__(512, 2) void fmha_fwd_pingpong_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K,
+                                                                   const half_t* __restrict__ V, half_t* __restrict__ O,
+                                                                   float* __restrict__ LSE, int B, int Hq, int Hkv, int Sq,
+                                                                   int Sk, float scale_log2, int causal, int kv_valid,
+                                                                   int q_tiles) {
+    using namespace fmha;
+    constexpr int NWAVES = 8;
+    constexpr int BM = NWAVES * 32;
+    constexpr int COPIES = (BN * ROW_BYTES / 1024) / NWAVES;  // 2 wave-instructions per tile per wave
+
+    extern __shared__ __attribute__((aligned(1024))) char smem_raw[];
+    MI355_LDS char* smem = (MI355_LDS char*)smem_raw;
+    MI355_LDS char* kbuf = smem;                   // 2 x TILE_BYTES
+    MI355_LDS char* vbuf = smem + 2 * TILE_BYTES;  // 2 x TILE_BYTES
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int late = wave >> 2;  // 0: waves 0..3 (M in even phases), 1: waves 4..7 (one phase behind)
+    const int h = lane >> 5;
+    const int l32 = lane & 31;
+
+    int b, hq, q_tile;
+    const int group = Hq / Hkv;
+    fmha_decode_block(blockIdx.x, q_tiles, group, Hkv, B, b, hq, q_tile);
+    const int hkv = hq / group;
+    const int q_block0 = q_tile * BM;
+    const int q_wave0 = q_block0 + wave * 32;
+    const int shift = Sk - Sq;
+
+    const half_t* Qh = Q + ((long)b * Hq + hq) * (long)Sq * D;
+    const half_t* Kh = K + ((long)b * Hkv + hkv) * (long)Sk * D;
+    const half_t* Vh = V + ((long)b * Hkv + hkv) * (long)Sk * D;
+    half_t* Oh = O + ((long)b * Hq + hq) * (long)Sq * D;
+
+    int k_end = kv_valid;
+    if (causal) k_end = min(k_end, min(q_block0 + BM, Sq) - 1 + shift + 1);
+    const int n_tiles = (k_end + BN - 1) / BN;  // may be <= 0: no visible key for the whole workgroup
+
+    half8 qf[8];
+    {
+        int qrow = min(q_wave0 + l32, Sq - 1);
+        const half_t* qp = Qh + (long)qrow * D + 8 * h;
+#pragma unroll
+        for (int ks = 0; ks < 8; ++ks) qf[ks] = *(const half8*)(qp + ks * 16);
+    }
+
+    // copy i of this wave covers tile rows (i*NWAVES + wave)*4 + lane/16, 16-byte chunk position lane%16
+    int copy_row[COPIES], copy_kcol[COPIES], copy_vcol[COPIES];
+#pragma unroll
+    for (int i = 0; i < COPIES; ++i) {
+        int row = (i * NWAVES + wave) * 4 + (lane >> 4);
+        copy_row[i] = row;
+        copy_kcol[i] = ((lane & 15) ^ swz_k(row)) * 8;
+        copy_vcol[i] = ((lane & 15) ^ swz_v(row)) * 8;
+    }
+    auto issue_k = [&](int tile) {
+#pragma unroll
+        for (int i = 0; i < COPIES; ++i) {
+            int krow = min(tile * BN + copy_row[i], kv_valid - 1);
+            copy16_global_to_lds(Kh + (long)krow * D + copy_kcol[i], kbuf + (tile & 1) * TILE_BYTES + (i * NWAVES + wave) * 1024);
+        }
+    };
+    auto issue_v = [&](int tile) {
+#pragma unroll
+        for (int i = 0; i < COPIES; ++i) {
+            int krow = min(tile * BN + copy_row[i], kv_valid - 1);
+            copy16_global_to_lds(Vh + (long)krow * D + copy_vcol[i], vbuf + (tile & 1) * TILE_BYTES + (i * NWAVES + wave) * 1024);
+        }
+    };
+
+    const int k_base = l32 * ROW_BYTES + ((h ^ (lane & 15)) << 4);  // xor (ks << 5), + kb * 32 * ROW_BYTES
+    const int v_row = 4 * h + ((lane & 15) >> 2);
+    const int v_clow = 2 * ((lane >> 4) & 1) + ((lane & 3) >> 1);
+    const int v_base = v_row * ROW_BYTES + ((v_clow ^ swz_v(v_row)) << 4) + (lane & 1) * 8;  // xor (db << 6)
+
+    float16v o[4];
+#pragma unroll
+    for (int db = 0; db < 4; ++db)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) o[db][e] = 0.f;
+    float m_run = -INFINITY, l_run = 0.f;
+
+    // The compiler is free to move register-only work across s_barrier; these empty asm statements make a value
+    // "used" at a program point, which keeps the softmax in the V phase and the MFMAs in the M phase.
+    auto pin_s = [](float16v(&s)[2]) { asm volatile("" : "+v"(s[0]), "+v"(s[1])); };
+    auto pin_p = [](half8(&pf)[2][2]) { asm volatile("" : "+v"(pf[0][0]), "+v"(pf[0][1]), "+v"(pf[1][0]), "+v"(pf[1][1])); };
+    auto pin_o = [&]() { asm volatile("" : "+v"(o[0]), "+v"(o[1]), "+v"(o[2]), "+v"(o[3])); };
+
+    // ---- phase bookkeeping -------------------------------------------------------------------------------------
+    int phase = 0;  // index of the workgroup phase this wave is in
+    // ends the current phase and starts the next one
+    auto next_phase = [&]() {
+        if (phase & 1) wait_vmcnt<0>();  // copies issued at the start of the previous (even) phase have landed
+        __syncthreads();
+        ++phase;
+        if (!(phase & 1)) {
+            const int i = phase >> 1;
+            if (i + 1 < n_tiles) issue_k(i + 1);
+            if (i < n_tiles) issue_v(i);
+        }
+    };
+
+    // ---- building blocks ----------------------------------------------------------------------------------------
+    auto qk_tile = [&](int tile, float16v(&s)[2]) {
+        MI355_LDS char* kst = kbuf + (tile & 1) * TILE_BYTES;
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb) {
+#pragma unroll
+            for (int e = 0; e < 16; ++e) s[kb][e] = 0.f;
+#pragma unroll
+            for (int ks = 0; ks < 8; ++ks) {
+                half8 kf = lds_read_b128(kst + ((k_base ^ (ks << 5)) + kb * 32 * ROW_BYTES));
+#ifndef EXP_PP_NOMFMA
+                s[kb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf, qf[ks], s[kb], 0, 0, 0);
+#else
+                s[kb][ks] += (float)kf[0];
+#endif
+            }
+        }
+    };
+    auto pv_tile = [&](int tile, const half8(&pf)[2][2]) {
+        MI355_LDS char* vst = vbuf + (tile & 1) * TILE_BYTES;
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+            for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+                for (int db = 0; db < 4; ++db) {
+                    int off = (v_base ^ (db << 6)) + (kb * 32 + 16 * tt) * ROW_BYTES;
+                    half4 lo = lds_read_tr16_b64(vst + off);
+                    half4 hi = lds_read_tr16_b64(vst + off + 8 * ROW_BYTES);
+#ifndef EXP_PP_NOMFMA
+                    o[db] = __builtin_amdgcn_mfma_f32_32x32x16_f16(concat(lo, hi), pf[kb][tt], o[db], 0, 0, 0);
+#else
+                    o[db][tt] += (float)lo[0] + (float)hi[1] + (float)pf[kb][tt][0];
+#endif
+                }
+    };
+    auto softmax_tile = [&](float16v(&s)[2], int tile, half8(&pf)[2][2]) {
+#ifdef EXP_PP_NOSOFTMAX
+        for (int kb = 0; kb < 2; ++kb) for (int tt = 0; tt < 2; ++tt) for (int j = 0; j < 8; ++j) pf[kb][tt][j] = (half_t)s[kb][8 * tt + j];
+        return;
+#endif
+        const int key0 = tile * BN;
+        const bool need_mask = (key0 + BN > kv_valid) || (causal && (key0 + BN - 1 > q_wave0 + shift));
+        if (need_mask) {
+            int qi = q_wave0 + l32;
+            int lim = causal ? min(kv_valid - 1, qi + shift) : kv_valid - 1;  // last visible key
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    int key = key0 + kb * 32 + 8 * (e >> 2) + 4 * h + (e & 3);
+                    if (key > lim) s[kb][e] = -INFINITY;
+                }
+        }
+        float mx = s[0][0];
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) mx = fmaxf(mx, s[kb][e]);
+        mx = halves_max(mx);
+        const bool raise = (mx - m_run) * scale_log2 > kLazyLog2;  // lazy rescaling, see fmha_fwd_kernel
+        if (__builtin_amdgcn_ballot_w64(raise) != 0) {
+            float m_new = fmaxf(m_run, mx);
+            float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+            float alpha = fast_exp2((m_run - m_use) * scale_log2);
+            m_run = m_new;
+            l_run *= alpha;
+#pragma unroll
+            for (int db = 0; db < 4; ++db)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) o[db][e] *= alpha;
+        }
+        const float neg_ms = (m_run == -INFINITY) ? 0.f : -m_run * scale_log2;
+        float psum = 0.f;
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+            for (int tt = 0; tt < 2; ++tt) {
+                half8 pk;
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    float p = fast_exp2(__builtin_fmaf(s[kb][8 * tt + j], scale_log2, neg_ms));
+                    psum += p;
+                    pk[j] = (half_t)p;
+                }
+                pf[kb][tt] = pk;
+            }
+        l_run += psum;
+    };
+
+    if (n_tiles > 0) {
+        // before P0: K(0) must be in LDS
+        issue_k(0);
+        wait_vmcnt<0>();
+        __syncthreads();
+        if (1 < n_tiles) issue_k(1);  // start of P0
+        issue_v(0);
+        if (late) next_phase();  // waves 4..7 idle during P0
+
+        float16v s[2];
+        half8 pf[2][2];
+        __builtin_amdgcn_s_setprio(1);
+        qk_tile(0, s);
+        __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
+        InterleaveMfmaLds<16, 1>::emit<0>();
+        __builtin_amdgcn_s_setprio(0);
+        pin_s(s);
+        next_phase();
+        for (int j = 0; j + 1 < n_tiles; ++j) {
+            softmax_tile(s, j, pf);  // V phase
+            pin_p(pf);
+            next_phase();
+            __builtin_amdgcn_s_setprio(1);
+            qk_tile(j + 1, s);       // M phase
+            pv_tile(j, pf);
+            __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
+            InterleaveMfmaLds<16, 1>::emit<0>();
+            __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
+            InterleaveMfmaLds<16, 2>::emit<0>();
+            __builtin_amdgcn_s_setprio(0);
+            pin_s(s);
+            pin_o();
+            next_phase();
+        }
+        softmax_tile(s, n_tiles - 1, pf);
+        pin_p(pf);
+        next_phase();
+        pv_tile(n_tiles - 1, pf);
+        __builtin_amdgcn_sched_group_barrier(0x100, 8, 0);
+        InterleaveMfmaLds<16, 2>::emit<0>();
+        next_phase();
+        if (!late) next_phase();  // waves 0..3 idle while waves 4..7 finish
+    }
+
+    // ---- finalize: O / l, LSE ---------------------------------------------------------------------------------
+    float l_tot = halves_sum(l_run);
+    float inv = (l_tot > 0.f) ? 1.f / l_tot : 0.f;
+    int qi = q_wave0 + l32;
+    if (qi < Sq) {
+        half_t* orow = Oh + (long)qi * D + 4 * h;
+#pragma unroll
+        for (int db = 0; db < 4; ++db)
+#pragma unroll
+            for (int p = 0; p < 4; ++p) {
+                half4 v;
+#pragma unroll
+                for (int q = 0; q < 4; ++q) v[q] = (half_t)(o[db][4 * p + q] * inv);
+                *(half4*)(orow + db * 32 + 8 * p) = v;
+            }
+        if (LSE != nullptr && h == 0) {
+            float lse = (l_tot > 0.f) ? (m_run * scale_log2 + __builtin_log2f(l_tot)) * 0.69314718055994531f : -INFINITY;
+            LSE[((long)b * Hq + hq) * (long)Sq + qi] = lse;
+        }
+    }
+}
+
+static hipError_t launch_fmha_pingpong(const half_t* Q, const half_t* K, const half_t* V, half_t* O, float* LSE, int B, int Hq,
+                                       int Hkv, int Sq, int Sk, float scale, int causal, int kv_valid, hipStream_t stream) {
+    constexpr int BM = 256;
+    constexpr int LDS = 4 * fmha::TILE_BYTES;
+    static bool attr_set = false;
+    if (!attr_set) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(fmha_fwd_pingpong_kernel),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, LDS);
+        if (e != hipSuccess) return e;
+        attr_set = true;
+    }
+    const int q_tiles = (Sq + BM - 1) / BM;
+    const long blocks = (long)q_tiles * Hq * B;
+    if (blocks > 0x7fffffffL) return hipErrorInvalidValue;
+    const float scale_log2 = scale * 1.4426950408889634f;
+    fmha_fwd_pingpong_kernel<<<dim3((unsigned)blocks), dim3(512), LDS, stream>>>(Q, K, V, O, LSE, B, Hq, Hkv, Sq, Sk, scale_log2,
+                                                                                causal, kv_valid, q_tiles);
+    return hipGetLastError();
+}
+
 template <int NQ, int NWAVES>
 static hipError_t launch_fmha(const half_t* Q, const half_t* K, const half_t* V, half_t* O, float* LSE, int B, int Hq,
                               int Hkv, int Sq, int Sk, float scale, int causal, int kv_valid, hipStream_t stream) {
@@ -333,6 +636,7 @@ hipError_t fmha_fwd_dispatch(const void* Q, const void* K, const void* V, void* 
     switch (g_fmha_variant) {
         case 1: return launch_fmha<2, 4>(q, k, v, o, LSE, B, Hq, Hkv, Sq, Sk, scale, causal, kv_valid_len, stream);
         case 2: return launch_fmha<1, 8>(q, k, v, o, LSE, B, Hq, Hkv, Sq, Sk, scale, causal, kv_valid_len, stream);
+        case 3: return launch_fmha_pingpong(q, k, v, o, LSE, B, Hq, Hkv, Sq, Sk, scale, causal, kv_valid_len, stream);
         default: return launch_fmha<1, 4>(q, k, v, o, LSE, B, Hq, Hkv, Sq, Sk, scale, causal, kv_valid_len, stream);
     }
 }

@@ -66,7 +66,7 @@ struct MNContigTile {
     static constexpr int kRowsPerPass = kRowsPerInst * NWAVES;
     static constexpr int kInsts = BK / kRowsPerPass;
     static constexpr int kBytes = BK * kRowBytes;
-    static_assert(COLS == 256, "swizzle below is written for 512-byte rows");
+    static_assert(COLS == 256 || COLS == 128, "swizzle below needs at least 16 chunks per row");
     static_assert(BK % kRowsPerPass == 0, "tile depth must be a multiple of one pass of the workgroup");
 
     // depends on (row % 4) only; keeps the 16 lanes of one transposing read on distinct banks
@@ -96,12 +96,12 @@ struct MNContigTile {
 // 256x256x64 main kernel
 // ---------------------------------------------------------------------------------------------------------
 
-template <bool A_KC, bool B_KC>
+template <bool A_KC, bool B_KC, int BM_, int BN_, int WM_, int WN_>
 struct MainCfg {
-    static constexpr int BM = 256, BN = 256, BK = 64;
-    static constexpr int WM = 2, WN = 4, NWAVES = 8, NTHREADS = 512;
-    static constexpr int TM = BM / WM / 32;  // 4 MFMA blocks along M per wave
-    static constexpr int TN = BN / WN / 32;  // 2 along N
+    static constexpr int BM = BM_, BN = BN_, BK = 64;
+    static constexpr int WM = WM_, WN = WN_, NWAVES = WM_ * WN_, NTHREADS = NWAVES * 64;
+    static constexpr int TM = BM / WM / 32;  // MFMA blocks along M per wave
+    static constexpr int TN = BN / WN / 32;  // along N
     using ATileK = KContigTile<BM, BK, NWAVES>;
     using ATileM = MNContigTile<BM, BK, NWAVES>;
     using BTileK = KContigTile<BN, BK, NWAVES>;
@@ -111,7 +111,9 @@ struct MainCfg {
     static constexpr int STAGE_BYTES = A_BYTES + B_BYTES;
     static constexpr int NSTAGE = 2;
     static constexpr int LDS_BYTES = STAGE_BYTES * NSTAGE;
-    static constexpr int A_INSTS = 4, B_INSTS = 4;
+    static constexpr int A_INSTS = A_BYTES / (NWAVES * 1024);  // 16-byte copies per lane per K tile
+    static constexpr int B_INSTS = B_BYTES / (NWAVES * 1024);
+    static constexpr int FRAG_SLOTS = (TM > TN ? TM : TN) > 4 ? (TM > TN ? TM : TN) : 4;
 };
 
 // Scheduling hint: alternate NMFMA matrix instructions with NDS LDS reads, spreading the reads evenly
@@ -149,11 +151,11 @@ __device__ __forceinline__ void tile_of_block(int bid, int tiles_m, int tiles_n,
     tn = in_g / rows;
 }
 
-template <bool A_KC, bool B_KC>
-__global__ __launch_bounds__(512) void hgemm_main_kernel(const half_t* __restrict__ A, const half_t* __restrict__ B,
+template <bool A_KC, bool B_KC, int BM, int BN, int WM, int WN>
+__global__ __launch_bounds__(WM * WN * 64) void hgemm_main_kernel(const half_t* __restrict__ A, const half_t* __restrict__ B,
                                                          half_t* __restrict__ C, int M, int N, int K, long lda,
                                                          long ldb, long ldc) {
-    using Cfg = MainCfg<A_KC, B_KC>;
+    using Cfg = MainCfg<A_KC, B_KC, BM, BN, WM, WN>;
     using ATK = typename Cfg::ATileK;
     using ATM = typename Cfg::ATileM;
     using BTK = typename Cfg::BTileK;
@@ -204,17 +206,19 @@ __global__ __launch_bounds__(512) void hgemm_main_kernel(const half_t* __restric
 #pragma unroll
         for (int i = 0; i < Cfg::A_INSTS; ++i)
             copy16_global_to_lds(a_src + i * a_copy_stride, sa + (i * Cfg::NWAVES + wave) * 1024);
+#ifndef EXP_HALFLOAD
 #pragma unroll
         for (int i = 0; i < Cfg::B_INSTS; ++i)
             copy16_global_to_lds(b_src + i * b_copy_stride, sb + (i * Cfg::NWAVES + wave) * 1024);
+#endif
         a_src += a_k_stride;
         b_src += b_k_stride;
     };
 
     // ---- LDS fragment read offsets (bytes inside one stage) -------------------------------------------
     // A fragments: TM blocks of 32 rows; B fragments: TN blocks of 32 columns.
-    int a_off[4];  // K-contiguous: per k-substep; M-contiguous: per block pair (only [0..TM) used)
-    int b_off[4];
+    int a_off[Cfg::FRAG_SLOTS];  // K-contiguous operand: one per k-substep; M/N-contiguous: one per 32-wide block
+    int b_off[Cfg::FRAG_SLOTS];
     if constexpr (A_KC) {
 #pragma unroll
         for (int kk = 0; kk < 4; ++kk) a_off[kk] = ATK::frag_offset(wm * TM * 32, kk, lane);
@@ -534,29 +538,51 @@ static hipError_t launch_smallm_nn(const half_t* A, const half_t* B, half_t* C, 
     return hipGetLastError();
 }
 
+int g_gemm_variant = 0;  // tuning hook: 0 = heuristic
+
+template <bool A_KC, bool B_KC, int BM, int BN, int WM, int WN>
+static hipError_t launch_main(const half_t* A, const half_t* B, half_t* C, int M, int N, int K, long lda, long ldb,
+                              long ldc, hipStream_t stream) {
+    using Cfg = MainCfg<A_KC, B_KC, BM, BN, WM, WN>;
+    static bool attr_set = false;
+    auto kern = hgemm_main_kernel<A_KC, B_KC, BM, BN, WM, WN>;
+    if (!attr_set) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::LDS_BYTES);
+        if (e != hipSuccess) return e;
+        attr_set = true;
+    }
+    int blocks = (M / BM) * (N / BN);
+    kern<<<dim3(blocks), dim3(Cfg::NTHREADS), Cfg::LDS_BYTES, stream>>>(A, B, C, M, N, K, lda, ldb, ldc);
+    return hipGetLastError();
+}
+
 template <bool A_KC, bool B_KC>
 static hipError_t launch_layout(const half_t* A, const half_t* B, half_t* C, int M, int N, int K, long lda, long ldb,
                                 long ldc, hipStream_t stream) {
-    using Cfg = MainCfg<A_KC, B_KC>;
     const bool aligned = (reinterpret_cast<uintptr_t>(A) % 16 == 0) && (reinterpret_cast<uintptr_t>(B) % 16 == 0) &&
                          (reinterpret_cast<uintptr_t>(C) % 8 == 0) && (lda % 8 == 0) && (ldb % 8 == 0) &&
                          (ldc % 4 == 0);
-    if (aligned && M % Cfg::BM == 0 && N % Cfg::BN == 0 && K % Cfg::BK == 0 && K >= Cfg::BK) {
-        static bool attr_set = false;
-        auto kern = hgemm_main_kernel<A_KC, B_KC>;
-        if (!attr_set) {
-            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                               hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::LDS_BYTES);
-            if (e != hipSuccess) return e;
-            attr_set = true;
-        }
-        int blocks = (M / Cfg::BM) * (N / Cfg::BN);
-        kern<<<dim3(blocks), dim3(Cfg::NTHREADS), Cfg::LDS_BYTES, stream>>>(A, B, C, M, N, K, lda, ldb, ldc);
-        return hipGetLastError();
-    }
+    const bool k_ok = aligned && K % 64 == 0 && K >= 64;
+    const bool fits256 = k_ok && M % 256 == 0 && N % 256 == 0;
+    const bool fits128 = k_ok && M % 128 == 0 && N % 128 == 0;
     if constexpr (A_KC && !B_KC) {
         if (aligned && M <= 64 && K % 32 == 0 && K >= 32 && N % 8 == 0 && ldc % 2 == 0)
             return launch_smallm_nn(A, B, C, M, N, K, lda, ldb, ldc, stream);
+    }
+    // 256x256 tiles when they fill the machine (>= ~3/4 of the 256 CUs), 128x128 tiles for smaller problems
+    const long tiles256 = fits256 ? (long)(M / 256) * (N / 256) : 0;
+    int choice = 0;
+    if (fits256 && (tiles256 >= 192 || !fits128)) choice = 1;
+    else if (fits128) choice = 2;
+    if (g_gemm_variant == 1 && fits256) choice = 1;
+    if (g_gemm_variant == 2 && fits128) choice = 2;
+    if (g_gemm_variant == 3 && fits256) choice = 3;
+    switch (choice) {
+        case 1: return launch_main<A_KC, B_KC, 256, 256, 2, 4>(A, B, C, M, N, K, lda, ldb, ldc, stream);
+        case 2: return launch_main<A_KC, B_KC, 128, 128, 2, 2>(A, B, C, M, N, K, lda, ldb, ldc, stream);
+        case 3: return launch_main<A_KC, B_KC, 256, 256, 2, 2>(A, B, C, M, N, K, lda, ldb, ldc, stream);
+        default: break;
     }
     dim3 grid((N + 63) / 64, (M + 63) / 64);
     hgemm_edge_kernel<A_KC, B_KC><<<grid, dim3(256), 0, stream>>>(A, B, C, M, N, K, lda, ldb, ldc);
@@ -577,3 +603,5 @@ hipError_t hgemm_dispatch(const void* A, const void* B, void* C, int M, int N, i
 }
 
 }  // namespace mi355
+
+extern "C" void mi355_debug_set_gemm_variant(int v) { mi355::g_gemm_variant = v; }
