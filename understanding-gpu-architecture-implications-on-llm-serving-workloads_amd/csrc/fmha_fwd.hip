@@ -437,11 +437,7 @@ __global__ __launch_bounds__(512, 2) void fmha_fwd_pingpong_kernel(const half_t*
 #pragma unroll
             for (int ks = 0; ks < 8; ++ks) {
                 half8 kf = lds_read_b128(kst + ((k_base ^ (ks << 5)) + kb * 32 * ROW_BYTES));
-#ifndef EXP_PP_NOMFMA
                 s[kb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf, qf[ks], s[kb], 0, 0, 0);
-#else
-                s[kb][ks] += (float)kf[0];
-#endif
             }
         }
     };
@@ -456,18 +452,10 @@ __global__ __launch_bounds__(512, 2) void fmha_fwd_pingpong_kernel(const half_t*
                     int off = (v_base ^ (db << 6)) + (kb * 32 + 16 * tt) * ROW_BYTES;
                     half4 lo = lds_read_tr16_b64(vst + off);
                     half4 hi = lds_read_tr16_b64(vst + off + 8 * ROW_BYTES);
-#ifndef EXP_PP_NOMFMA
                     o[db] = __builtin_amdgcn_mfma_f32_32x32x16_f16(concat(lo, hi), pf[kb][tt], o[db], 0, 0, 0);
-#else
-                    o[db][tt] += (float)lo[0] + (float)hi[1] + (float)pf[kb][tt][0];
-#endif
                 }
     };
     auto softmax_tile = [&](float16v(&s)[2], int tile, half8(&pf)[2][2]) {
-#ifdef EXP_PP_NOSOFTMAX
-        for (int kb = 0; kb < 2; ++kb) for (int tt = 0; tt < 2; ++tt) for (int j = 0; j < 8; ++j) pf[kb][tt][j] = (half_t)s[kb][8 * tt + j];
-        return;
-#endif
         const int key0 = tile * BN;
         const bool need_mask = (key0 + BN > kv_valid) || (causal && (key0 + BN - 1 > q_wave0 + shift));
         if (need_mask) {

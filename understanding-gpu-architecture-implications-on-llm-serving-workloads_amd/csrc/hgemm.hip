@@ -14,7 +14,8 @@
 //     transpose pass over B is ever made.
 //   * each wave owns a 128x64 sub-tile = 4x2 MFMA 32x32x16 blocks (128 fp32 accumulators per lane).
 //     The MFMA is issued with the B fragment as first operand, i.e. it produces the transposed block, so a
-//     lane ends up with 4 consecutive N of one row of C and can store 8 bytes at a time.
+//     lane ends up with 4 consecutive N of one row of C; the epilogue parks the sub-tile in LDS and stores whole
+//     128-byte lines.
 #include "mi355_common.h"
 #include "mi355_serving_internal.h"
 
@@ -206,11 +207,9 @@ __global__ __launch_bounds__(WM * WN * 64) void hgemm_main_kernel(const half_t* 
 #pragma unroll
         for (int i = 0; i < Cfg::A_INSTS; ++i)
             copy16_global_to_lds(a_src + i * a_copy_stride, sa + (i * Cfg::NWAVES + wave) * 1024);
-#ifndef EXP_HALFLOAD
 #pragma unroll
         for (int i = 0; i < Cfg::B_INSTS; ++i)
             copy16_global_to_lds(b_src + i * b_copy_stride, sb + (i * Cfg::NWAVES + wave) * 1024);
-#endif
         a_src += a_k_stride;
         b_src += b_k_stride;
     };
@@ -275,9 +274,7 @@ __global__ __launch_bounds__(WM * WN * 64) void hgemm_main_kernel(const half_t* 
     // ask the scheduler to alternate the TM*TN MFMAs of one substep with the LDS reads of the next one
     constexpr int kDsReads = (A_KC ? TM : 2 * TM) + (B_KC ? TN : 2 * TN);
     auto interleave = [&]() {
-#ifndef EXP_NOSCHED
         InterleaveMfmaWithLdsReads<0, TM * TN, kDsReads>::emit();
-#endif
     };
 
     // Software pipeline: the fragments of substep kk+1 are read from LDS while the MFMAs of substep kk run;
@@ -306,13 +303,9 @@ __global__ __launch_bounds__(WM * WN * 64) void hgemm_main_kernel(const half_t* 
         interleave();
         // my copies of tile kt+1 have landed and my reads of this stage are complete; after the barrier that
         // holds for every wave, so this stage may be refilled and the next one may be read
-#ifndef EXP_NOBARRIER
         wait_vmcnt<0>();
         __syncthreads();
-#endif
-#ifndef EXP_NOLOAD
         if (kt + 2 < ktiles) issue_copies(kt & 1);
-#endif
         load_frags(stn, 0, af[0], bf[0]);
         mma(af[1], bf[1]);
         interleave();
@@ -330,23 +323,49 @@ __global__ __launch_bounds__(WM * WN * 64) void hgemm_main_kernel(const half_t* 
         mma(af[1], bf[1]);
     }
 
-    // ---- epilogue: lane holds C[m][n .. n+3] for m = l%32, n = 8p + 4*(l/32) ----------------------------
-    const long row_base = m0 + wm * TM * 32 + (lane & 31);
-    const long col_base = n0 + wn * TN * 32 + 4 * (lane >> 5);
+    // ---- epilogue ------------------------------------------------------------------------------------------------
+    // A lane holds C[m][n .. n+3] for m = l%32, n = 8p + 4*(l/32) of every 32x32 block. Storing that directly would
+    // write 8-byte pieces of 32 different rows per instruction (partial cache lines, read-modify-write in the
+    // memory system), so each wave first parks its sub-tile in its own slice of LDS (fp16, 16-byte chunks XOR-
+    // swizzled by row) and then stores whole rows: every store instruction writes complete 128-byte lines.
+    constexpr int kRowHalfs = TN * 32;            // width of the wave sub-tile
+    constexpr int kRowBytesC = kRowHalfs * 2;
+    constexpr int kChunksC = kRowBytesC / 16;     // 16-byte chunks per row (8 or 16)
+    constexpr int kRowsPerStore = 64 / kChunksC;  // rows covered by one store instruction
+    static_assert(Cfg::NWAVES * TM * 32 * kRowBytesC <= Cfg::LDS_BYTES, "epilogue staging does not fit in LDS");
+    __syncthreads();  // every wave has finished reading the operand stages
+    MI355_LDS char* cst = smem + wave * (TM * 32 * kRowBytesC);
+    {
+        const int r = lane & 31;
+        const int hh = lane >> 5;
 #pragma unroll
-    for (int i = 0; i < TM; ++i) {
-        half_t* crow = C + (row_base + i * 32) * ldc + col_base;
+        for (int i = 0; i < TM; ++i) {
+            const int row = i * 32 + r;
 #pragma unroll
-        for (int j = 0; j < TN; ++j) {
+            for (int j = 0; j < TN; ++j) {
 #pragma unroll
-            for (int p = 0; p < 4; ++p) {
-                half4 v;
-                v[0] = (half_t)acc[i][j][4 * p + 0];
-                v[1] = (half_t)acc[i][j][4 * p + 1];
-                v[2] = (half_t)acc[i][j][4 * p + 2];
-                v[3] = (half_t)acc[i][j][4 * p + 3];
-                *(half4*)(crow + j * 32 + 8 * p) = v;
+                for (int p = 0; p < 4; ++p) {
+                    half4 v;
+                    v[0] = (half_t)acc[i][j][4 * p + 0];
+                    v[1] = (half_t)acc[i][j][4 * p + 1];
+                    v[2] = (half_t)acc[i][j][4 * p + 2];
+                    v[3] = (half_t)acc[i][j][4 * p + 3];
+                    const int chunk = (j * 4 + p) ^ (row & 7);
+                    *(MI355_LDS half4*)(cst + row * kRowBytesC + chunk * 16 + hh * 8) = v;
+                }
             }
+        }
+    }
+    // only this wave reads what it wrote: no workgroup barrier needed, the LDS operations of a wave complete in order
+    {
+        const int rr = lane / kChunksC;
+        const int cc = lane % kChunksC;
+        half_t* cbase = C + (m0 + wm * TM * 32) * ldc + n0 + wn * TN * 32 + cc * 8;
+#pragma unroll
+        for (int it = 0; it < TM * 32 / kRowsPerStore; ++it) {
+            const int row = it * kRowsPerStore + rr;
+            half8 v = *(MI355_LDS const half8*)(cst + row * kRowBytesC + ((cc ^ (row & 7)) << 4));
+            *(half8*)(cbase + (long)row * ldc) = v;
         }
     }
 }
@@ -538,7 +557,7 @@ static hipError_t launch_smallm_nn(const half_t* A, const half_t* B, half_t* C, 
     return hipGetLastError();
 }
 
-int g_gemm_variant = 0;  // tuning hook: 0 = heuristic
+int g_gemm_variant = 0;  // tuning hook: 0 = heuristic, 1 = force 256x256 tiles, 2 = force 128x128 tiles
 
 template <bool A_KC, bool B_KC, int BM, int BN, int WM, int WN>
 static hipError_t launch_main(const half_t* A, const half_t* B, half_t* C, int M, int N, int K, long lda, long ldb,
@@ -561,8 +580,8 @@ template <bool A_KC, bool B_KC>
 static hipError_t launch_layout(const half_t* A, const half_t* B, half_t* C, int M, int N, int K, long lda, long ldb,
                                 long ldc, hipStream_t stream) {
     const bool aligned = (reinterpret_cast<uintptr_t>(A) % 16 == 0) && (reinterpret_cast<uintptr_t>(B) % 16 == 0) &&
-                         (reinterpret_cast<uintptr_t>(C) % 8 == 0) && (lda % 8 == 0) && (ldb % 8 == 0) &&
-                         (ldc % 4 == 0);
+                         (reinterpret_cast<uintptr_t>(C) % 16 == 0) && (lda % 8 == 0) && (ldb % 8 == 0) &&
+                         (ldc % 8 == 0);
     const bool k_ok = aligned && K % 64 == 0 && K >= 64;
     const bool fits256 = k_ok && M % 256 == 0 && N % 256 == 0;
     const bool fits128 = k_ok && M % 128 == 0 && N % 128 == 0;
@@ -577,11 +596,9 @@ static hipError_t launch_layout(const half_t* A, const half_t* B, half_t* C, int
     else if (fits128) choice = 2;
     if (g_gemm_variant == 1 && fits256) choice = 1;
     if (g_gemm_variant == 2 && fits128) choice = 2;
-    if (g_gemm_variant == 3 && fits256) choice = 3;
     switch (choice) {
         case 1: return launch_main<A_KC, B_KC, 256, 256, 2, 4>(A, B, C, M, N, K, lda, ldb, ldc, stream);
         case 2: return launch_main<A_KC, B_KC, 128, 128, 2, 2>(A, B, C, M, N, K, lda, ldb, ldc, stream);
-        case 3: return launch_main<A_KC, B_KC, 256, 256, 2, 2>(A, B, C, M, N, K, lda, ldb, ldc, stream);
         default: break;
     }
     dim3 grid((N + 63) / 64, (M + 63) / 64);
