@@ -29,9 +29,10 @@ sys.path.insert(0, os.path.join(ROOT, "oracle"))
 PEAK_FP16_TFLOPS = 2500.0   # MI355X dense fp16 MFMA
 PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 
-# HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (see profiles/);
-# None until measured for the current kernel.
-MEASURED_TRAFFIC_BYTES = None
+# HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (KiB per dispatch), each scaled by what the same
+# counter reads for a 1 GiB device-to-device copy (FETCH_SIZE x2.0, WRITE_SIZE x1.0); see profiles/.
+MEASURED_TRAFFIC_BYTES = (786780 * 2.0 + 131072 * 1.0) * 1024        # hgemm_main_kernel, 8192^3 NN
+MEASURED_TRAFFIC_BYTES_FMHA = (27502 * 2.0 + 33280 * 1.0) * 1024     # fmha_fwd_kernel, F4
 
 
 def log(*a):
@@ -158,7 +159,7 @@ def main():
     roofline = {"kernel": "hgemm_main_kernel (8192^3, NN)", "bound": "mfma", "achieved": gemm_tf, "peak": PEAK_FP16_TFLOPS,
                 "unit": "TFLOP/s", "frac": gemm_tf / PEAK_FP16_TFLOPS, "traffic": MEASURED_TRAFFIC_BYTES}
     roofline_fmha = {"kernel": "fmha_fwd_kernel (F4)", "bound": "mfma", "achieved": fmha_tf, "peak": PEAK_FP16_TFLOPS,
-                     "unit": "TFLOP/s", "frac": fmha_tf / PEAK_FP16_TFLOPS, "traffic": None}
+                     "unit": "TFLOP/s", "frac": fmha_tf / PEAK_FP16_TFLOPS, "traffic": MEASURED_TRAFFIC_BYTES_FMHA}
 
     # ---- the other benchmark configurations (quick timings) ----------------------------------------------------------
     other = {}
