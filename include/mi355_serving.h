@@ -79,6 +79,16 @@ const char* mi355_last_error(void);
 /* MI355_SERVING_VERSION of the loaded library. */
 int mi355_serving_version(void);
 
+/*
+ * Diagnostics (no counterpart in the reference): pin the kernel variant instead of letting the dispatcher choose
+ * by shape, so tests and tuning runs can exercise every variant on every shape. Process-wide; 0 restores the
+ * heuristic. A variant that does not fit the shape (e.g. tile sizes that do not divide it) is ignored.
+ *   gemm: 1 = 256x256 tiles, 2 = 128x128 tiles
+ *   fmha: 1 = 4 waves x 32 queries, 2 = 8 waves x 32 queries, 3 = 8 waves x 32 queries ping-pong
+ */
+void mi355_debug_set_gemm_variant(int variant);
+void mi355_debug_set_fmha_variant(int variant);
+
 #ifdef __cplusplus
 }
 #endif

@@ -113,6 +113,21 @@ def test_ragged_shapes_and_masks(lib, gpu, B, Hq, Hkv, Sq, Sk, causal, kvv):
         assert bool((o[:, :, :n] == 0).all()) and bool(torch.isinf(lse[:, :, :n]).all()) and bool((lse[:, :, :n] < 0).all())
 
 
+@pytest.mark.parametrize("variant", [1, 2, 3])
+@pytest.mark.parametrize("B,Hq,Hkv,Sq,Sk,causal,kvv", [
+    (1, 4, 1, 128, 128, True, None), (2, 4, 2, 100, 177, True, None), (1, 2, 1, 300, 300, True, 290),
+    (1, 2, 2, 70, 40, True, None), (1, 2, 2, 1, 333, False, None), (2, 3, 3, 600, 1000, False, 999),
+    (1, 2, 1, 513, 515, True, None), (1, 1, 1, 700, 64, False, 1), (1, 2, 2, 256, 1024, True, None),
+])
+def test_every_kernel_variant_on_ragged_shapes(lib, gpu, variant, B, Hq, Hkv, Sq, Sk, causal, kvv):
+    q, k, v = so.fmha_inputs(B, Hq, Hkv, Sq, Sk, seed=Sq + 3 * Sk + variant)
+    lib.set_variants(fmha=variant)
+    try:
+        check(lib, gpu, q, k, v, causal, kvv)
+    finally:
+        lib.set_variants()
+
+
 def test_masked_keys_may_hold_garbage(lib, gpu):
     # keys at or beyond kv_valid_len must not influence the result, whatever they contain
     q, k, v = so.fmha_inputs(1, 2, 2, 90, 200, seed=11)

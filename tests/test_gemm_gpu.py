@@ -88,6 +88,17 @@ def test_layouts_and_shapes(lib, gpu, layout, M, N, K):
     assert c.shape == (M, N)
 
 
+@pytest.mark.parametrize("variant", [1, 2])
+@pytest.mark.parametrize("layout", ["NN", "TN", "NT"])
+def test_every_tile_variant(lib, gpu, variant, layout):
+    a, b = operands(512, 768, 448, layout, seed=variant)
+    lib.set_variants(gemm=variant)
+    try:
+        check(lib, gpu, a, b, layout, 448)
+    finally:
+        lib.set_variants()
+
+
 def test_reference_seeded_case_from_golden_fixture(lib, gpu):
     z = np.load(os.path.join(GOLDEN, "gemm_seed0_256.npz"))
     a, b, rows = torch.from_numpy(z["a"]), torch.from_numpy(z["b"]), z["rows"]

@@ -312,18 +312,6 @@ __global__ __launch_bounds__(NWAVES * 64, (NQ == 1 ? 2 : 1)) void fmha_fwd_kerne
 // K and V have separate double buffers: tile j lives in Kbuf[j&1] / Vbuf[j&1], is copied by all 8 waves at the
 // start of an even phase (K(i+1) and V(i) at P(2i)) and has two phases to land (waited for at the end of P(2i+1)).
 // ---------------------------------------------------------------------------------------------------------
-template <int NMFMA, int NDS>
-struct InterleaveMfmaLds {
-    template <int M>
-    __device__ static __forceinline__ void emit() {
-        if constexpr (M < NMFMA) {
-            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);    // one MFMA
-            __builtin_amdgcn_sched_group_barrier(0x100, NDS, 0);  // LDS reads of a later MFMA
-            emit<M + 1>();
-        }
-    }
-};
-
 __global__ __launch_bounds__(512, 2) void fmha_fwd_pingpong_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K,
                                                                    const half_t* __restrict__ V, half_t* __restrict__ O,
                                                                    float* __restrict__ LSE, int B, int Hq, int Hkv, int Sq,
@@ -428,32 +416,82 @@ __global__ __launch_bounds__(512, 2) void fmha_fwd_pingpong_kernel(const half_t*
     };
 
     // ---- building blocks ----------------------------------------------------------------------------------------
-    auto qk_tile = [&](int tile, float16v(&s)[2]) {
+    // LDS fragment reads, named so the M phase below can issue them long before their MFMA
+    auto read_k = [&](MI355_LDS char* kst, int kb, int ks) {
+        return lds_read_b128(kst + ((k_base ^ (ks << 5)) + kb * 32 * ROW_BYTES));
+    };
+    auto read_v = [&](MI355_LDS char* vst, int step) {  // step = (kb*2 + tt)*4 + db, the order the MFMAs consume them
+        const int db = step & 3, tt = (step >> 2) & 1, kb = step >> 3;
+        const int off = (v_base ^ (db << 6)) + (kb * 32 + 16 * tt) * ROW_BYTES;
+        return concat(lds_read_tr16_b64(vst + off), lds_read_tr16_b64(vst + off + 8 * ROW_BYTES));
+    };
+    // The M phase in the exact order it should issue: every fragment is read 8 MFMAs (256 cycles) before the MFMA
+    // that consumes it, into the register its predecessor has just released. sched_barrier pins that order.
+    //   MFMAs  0.. 7: S block 0 (K fragments read up front)        reads issued: K fragments of block 1
+    //   MFMAs  8..15: S block 1                                     reads issued: V fragments 0..7
+    //   MFMAs 16..23: O += V^T P, fragments 0..7                    reads issued: V fragments 8..15
+    //   MFMAs 24..31: O += V^T P, fragments 8..15
+    auto qk_tile = [&](int tile, float16v(&s)[2]) {  // S(tile) alone (first M phase of a wave)
         MI355_LDS char* kst = kbuf + (tile & 1) * TILE_BYTES;
+        half8 kf[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) kf[i] = read_k(kst, 0, i);
 #pragma unroll
         for (int kb = 0; kb < 2; ++kb) {
 #pragma unroll
             for (int e = 0; e < 16; ++e) s[kb][e] = 0.f;
 #pragma unroll
-            for (int ks = 0; ks < 8; ++ks) {
-                half8 kf = lds_read_b128(kst + ((k_base ^ (ks << 5)) + kb * 32 * ROW_BYTES));
-                s[kb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf, qf[ks], s[kb], 0, 0, 0);
+            for (int i = 0; i < 8; ++i) {
+                __builtin_amdgcn_sched_barrier(0);
+                s[kb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf[i], qf[i], s[kb], 0, 0, 0);
+                if (kb == 0) kf[i] = read_k(kst, 1, i);
             }
         }
+        __builtin_amdgcn_sched_barrier(0);
     };
-    auto pv_tile = [&](int tile, const half8(&pf)[2][2]) {
+    auto pv_tile = [&](int tile, const half8(&pf)[2][2]) {  // O += V(tile)^T P alone (last M phase of a wave)
         MI355_LDS char* vst = vbuf + (tile & 1) * TILE_BYTES;
+        half8 vf[8];
 #pragma unroll
-        for (int kb = 0; kb < 2; ++kb)
+        for (int i = 0; i < 8; ++i) vf[i] = read_v(vst, i);
 #pragma unroll
-            for (int tt = 0; tt < 2; ++tt)
+        for (int half = 0; half < 2; ++half)
 #pragma unroll
-                for (int db = 0; db < 4; ++db) {
-                    int off = (v_base ^ (db << 6)) + (kb * 32 + 16 * tt) * ROW_BYTES;
-                    half4 lo = lds_read_tr16_b64(vst + off);
-                    half4 hi = lds_read_tr16_b64(vst + off + 8 * ROW_BYTES);
-                    o[db] = __builtin_amdgcn_mfma_f32_32x32x16_f16(concat(lo, hi), pf[kb][tt], o[db], 0, 0, 0);
-                }
+            for (int i = 0; i < 8; ++i) {
+                __builtin_amdgcn_sched_barrier(0);
+                const int step = half * 8 + i;
+                o[step & 3] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf[i], pf[step >> 3][(step >> 2) & 1], o[step & 3], 0, 0, 0);
+                if (half == 0) vf[i] = read_v(vst, 8 + i);
+            }
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    auto m_phase = [&](int tile_k, float16v(&s)[2], int tile_v, const half8(&pf)[2][2]) {  // S(tile_k) and O += V(tile_v)^T P
+        MI355_LDS char* kst = kbuf + (tile_k & 1) * TILE_BYTES;
+        MI355_LDS char* vst = vbuf + (tile_v & 1) * TILE_BYTES;
+        half8 fr[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) fr[i] = read_k(kst, 0, i);
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb) {
+#pragma unroll
+            for (int e = 0; e < 16; ++e) s[kb][e] = 0.f;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                __builtin_amdgcn_sched_barrier(0);
+                s[kb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fr[i], qf[i], s[kb], 0, 0, 0);
+                fr[i] = (kb == 0) ? read_k(kst, 1, i) : read_v(vst, i);
+            }
+        }
+#pragma unroll
+        for (int half = 0; half < 2; ++half)
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                __builtin_amdgcn_sched_barrier(0);
+                const int step = half * 8 + i;
+                o[step & 3] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fr[i], pf[step >> 3][(step >> 2) & 1], o[step & 3], 0, 0, 0);
+                if (half == 0) fr[i] = read_v(vst, 8 + i);
+            }
+        __builtin_amdgcn_sched_barrier(0);
     };
     auto softmax_tile = [&](float16v(&s)[2], int tile, half8(&pf)[2][2]) {
         const int key0 = tile * BN;
@@ -488,7 +526,19 @@ __global__ __launch_bounds__(512, 2) void fmha_fwd_pingpong_kernel(const half_t*
                 for (int e = 0; e < 16; ++e) o[db][e] *= alpha;
         }
         const float neg_ms = (m_run == -INFINITY) ? 0.f : -m_run * scale_log2;
-        float psum = 0.f;
+        // In this phase the wave is the only one of its SIMD issuing VALU work, so dependent instructions must be
+        // kept apart: all 32 multiply-adds, then all 32 exponentials, then four independent partial sums.
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) s[kb][e] = __builtin_fmaf(s[kb][e], scale_log2, neg_ms);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) s[kb][e] = fast_exp2(s[kb][e]);
+        __builtin_amdgcn_sched_barrier(0);
+        float ps[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
@@ -496,13 +546,12 @@ __global__ __launch_bounds__(512, 2) void fmha_fwd_pingpong_kernel(const half_t*
                 half8 pk;
 #pragma unroll
                 for (int j = 0; j < 8; ++j) {
-                    float p = fast_exp2(__builtin_fmaf(s[kb][8 * tt + j], scale_log2, neg_ms));
-                    psum += p;
-                    pk[j] = (half_t)p;
+                    ps[j & 3] += s[kb][8 * tt + j];
+                    pk[j] = (half_t)s[kb][8 * tt + j];
                 }
                 pf[kb][tt] = pk;
             }
-        l_run += psum;
+        l_run += (ps[0] + ps[1]) + (ps[2] + ps[3]);
     };
 
     if (n_tiles > 0) {
@@ -518,8 +567,6 @@ __global__ __launch_bounds__(512, 2) void fmha_fwd_pingpong_kernel(const half_t*
         half8 pf[2][2];
         __builtin_amdgcn_s_setprio(1);
         qk_tile(0, s);
-        __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
-        InterleaveMfmaLds<16, 1>::emit<0>();
         __builtin_amdgcn_s_setprio(0);
         pin_s(s);
         next_phase();
@@ -528,12 +575,7 @@ __global__ __launch_bounds__(512, 2) void fmha_fwd_pingpong_kernel(const half_t*
             pin_p(pf);
             next_phase();
             __builtin_amdgcn_s_setprio(1);
-            qk_tile(j + 1, s);       // M phase
-            pv_tile(j, pf);
-            __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
-            InterleaveMfmaLds<16, 1>::emit<0>();
-            __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
-            InterleaveMfmaLds<16, 2>::emit<0>();
+            m_phase(j + 1, s, j, pf);
             __builtin_amdgcn_s_setprio(0);
             pin_s(s);
             pin_o();
@@ -543,8 +585,6 @@ __global__ __launch_bounds__(512, 2) void fmha_fwd_pingpong_kernel(const half_t*
         pin_p(pf);
         next_phase();
         pv_tile(n_tiles - 1, pf);
-        __builtin_amdgcn_sched_group_barrier(0x100, 8, 0);
-        InterleaveMfmaLds<16, 2>::emit<0>();
         next_phase();
         if (!late) next_phase();  // waves 0..3 idle while waves 4..7 finish
     }
@@ -613,7 +653,7 @@ static hipError_t launch_fmha(const half_t* Q, const half_t* K, const half_t* V,
     return hipGetLastError();
 }
 
-int g_fmha_variant = 0;  // tuning hook: 0 = default
+int g_fmha_variant = 0;  // tuning hook: 0 = heuristic, 1 = 4 waves x 32 queries, 2 = 8 waves x 32 queries, 3 = ping-pong
 
 hipError_t fmha_fwd_dispatch(const void* Q, const void* K, const void* V, void* O, float* LSE, int B, int Hq, int Hkv,
                              int Sq, int Sk, float scale, int causal, int kv_valid_len, hipStream_t stream) {
@@ -621,8 +661,13 @@ hipError_t fmha_fwd_dispatch(const void* Q, const void* K, const void* V, void* 
     const half_t* k = static_cast<const half_t*>(K);
     const half_t* v = static_cast<const half_t*>(V);
     half_t* o = static_cast<half_t*>(O);
-    switch (g_fmha_variant) {
-        case 1: return launch_fmha<2, 4>(q, k, v, o, LSE, B, Hq, Hkv, Sq, Sk, scale, causal, kv_valid_len, stream);
+    int variant = g_fmha_variant;
+    if (variant == 0) {
+        // 256-query ping-pong workgroups once there are enough of them to fill the 256 CUs, otherwise 128-query ones
+        const long wg256 = (long)((Sq + 255) / 256) * Hq * B;
+        variant = (wg256 >= 256) ? 3 : 1;
+    }
+    switch (variant) {
         case 2: return launch_fmha<1, 8>(q, k, v, o, LSE, B, Hq, Hkv, Sq, Sk, scale, causal, kv_valid_len, stream);
         case 3: return launch_fmha_pingpong(q, k, v, o, LSE, B, Hq, Hkv, Sq, Sk, scale, causal, kv_valid_len, stream);
         default: return launch_fmha<1, 4>(q, k, v, o, LSE, B, Hq, Hkv, Sq, Sk, scale, causal, kv_valid_len, stream);

@@ -13,7 +13,8 @@ LIB_PATH = os.path.join(_HERE, "libmi355_serving.so")
 GEMM_NN, GEMM_NT, GEMM_TN = 0, 1, 2
 LAYOUTS = {"NN": GEMM_NN, "NT": GEMM_NT, "TN": GEMM_TN}
 
-EXPORTED_SYMBOLS = ("mi355_hgemm", "mi355_fmha_fwd", "mi355_last_error", "mi355_serving_version")
+EXPORTED_SYMBOLS = ("mi355_hgemm", "mi355_fmha_fwd", "mi355_last_error", "mi355_serving_version",
+                    "mi355_debug_set_gemm_variant", "mi355_debug_set_fmha_variant")
 
 _lib = None
 
@@ -43,8 +44,19 @@ def load():
     lib.mi355_last_error.restype = ctypes.c_char_p
     lib.mi355_serving_version.argtypes = []
     lib.mi355_serving_version.restype = i32
+    lib.mi355_debug_set_gemm_variant.argtypes = [i32]
+    lib.mi355_debug_set_gemm_variant.restype = None
+    lib.mi355_debug_set_fmha_variant.argtypes = [i32]
+    lib.mi355_debug_set_fmha_variant.restype = None
     _lib = lib
     return lib
+
+
+def set_variants(gemm=0, fmha=0):
+    """Pin kernel variants (diagnostics; 0 = let the dispatcher choose by shape)."""
+    lib = load()
+    lib.mi355_debug_set_gemm_variant(int(gemm))
+    lib.mi355_debug_set_fmha_variant(int(fmha))
 
 
 def _ptr(x):
