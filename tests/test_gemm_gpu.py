@@ -99,6 +99,13 @@ def test_every_tile_variant(lib, gpu, variant, layout):
         lib.set_variants()
 
 
+@pytest.mark.parametrize("layout", ["NN", "NT", "TN"])
+@pytest.mark.parametrize("M,N,K", [(16, 4096, 4096), (1, 1000, 512), (64, 304, 128), (33, 24, 192), (7, 72, 96), (16, 64, 4096)])
+def test_decode_shaped_small_m(lib, gpu, layout, M, N, K):
+    a, b = operands(M, N, K, layout, seed=M * 3 + N, b_std=0.05)
+    check(lib, gpu, a, b, layout, K)
+
+
 def test_reference_seeded_case_from_golden_fixture(lib, gpu):
     z = np.load(os.path.join(GOLDEN, "gemm_seed0_256.npz"))
     a, b, rows = torch.from_numpy(z["a"]), torch.from_numpy(z["b"]), z["rows"]

@@ -557,6 +557,125 @@ static hipError_t launch_smallm_nn(const half_t* A, const half_t* B, half_t* C, 
     return hipGetLastError();
 }
 
+// ---------------------------------------------------------------------------------------------------------
+// Small-M kernel for layout NT (B stored [N,K]: the nn.Linear weight layout of decode-time projections), M <= 16
+// rows per workgroup row. HBM-bound like hgemm_smallm_nn_kernel and built the same way: a workgroup owns 16
+// columns of C (16 rows of B), its 8 waves split K and are reduced through LDS; every wave runs a private,
+// barrier-free copy pipeline of 64-deep k-steps (16x64 of B and 16x64 of A, 2 KiB each, direct-to-LDS), both
+// operands are K-contiguous so both fragments are plain ds_read_b128, the product is MFMA 16x16x32.
+// ---------------------------------------------------------------------------------------------------------
+constexpr int kSmallMNtStages = 4;
+constexpr int kSmallMNtStageBytes = 4 * 1024;  // 2 KiB of B + 2 KiB of A
+constexpr int kSmallMNtWaveBytes = kSmallMNtStages * kSmallMNtStageBytes;
+constexpr int kSmallMNtLdsBytes = 8 * kSmallMNtWaveBytes;
+
+__global__ __launch_bounds__(512) void hgemm_smallm_nt_kernel(const half_t* __restrict__ A, const half_t* __restrict__ B,
+                                                              half_t* __restrict__ C, int M, int N, int K, long lda,
+                                                              long ldb, long ldc, int n_tiles) {
+    extern __shared__ __attribute__((aligned(1024))) char smem_raw[];
+    MI355_LDS char* smem = (MI355_LDS char*)smem_raw;
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+
+    int tile = blockIdx.x;
+    if (n_tiles % 8 == 0) tile = (blockIdx.x % 8) * (n_tiles / 8) + blockIdx.x / 8;
+    const int n0 = tile * 16;
+    const int m0 = blockIdx.y * 16;
+
+    const int ksteps = K / 64;
+    const int s_begin = (int)((long)wave * ksteps / 8);
+    const int s_end = (int)((long)(wave + 1) * ksteps / 8);
+    MI355_LDS char* wbase = smem + wave * kSmallMNtWaveBytes;
+
+    // slab = 16 rows x 128 bytes; a copy instruction covers 8 rows (row lane/8, chunk position lane%8);
+    // chunk c of row r is stored at position c ^ (r & 7)
+    const int c_row = lane >> 3;  // + 8*i
+    const int c_chunk = (lane & 7) ^ (c_row & 7);
+    const half_t* b_src0 = B + (long)min(n0 + c_row, N - 1) * ldb + (long)s_begin * 64 + c_chunk * 8;
+    const half_t* b_src1 = B + (long)min(n0 + c_row + 8, N - 1) * ldb + (long)s_begin * 64 + c_chunk * 8;
+    const half_t* a_src0 = A + (long)min(m0 + c_row, M - 1) * lda + (long)s_begin * 64 + c_chunk * 8;
+    const half_t* a_src1 = A + (long)min(m0 + c_row + 8, M - 1) * lda + (long)s_begin * 64 + c_chunk * 8;
+
+    auto issue_stage = [&](int slot) {
+        MI355_LDS char* st = wbase + slot * kSmallMNtStageBytes;
+        copy16_global_to_lds(b_src0, st);
+        copy16_global_to_lds(b_src1, st + 1024);
+        copy16_global_to_lds(a_src0, st + 2048);
+        copy16_global_to_lds(a_src1, st + 3072);
+        b_src0 += 64;
+        b_src1 += 64;
+        a_src0 += 64;
+        a_src1 += 64;
+    };
+
+    // fragment of k-substep sub (32 deep): lane holds X[row = lane%16][k = 32*sub + 8*(lane/16) .. +7]
+    const int f_row = lane & 15;
+    int f_off[2];
+#pragma unroll
+    for (int sub = 0; sub < 2; ++sub) f_off[sub] = f_row * 128 + (((4 * sub + (lane >> 4)) ^ (f_row & 7)) << 4);
+
+    float4v acc = float4v{0.f, 0.f, 0.f, 0.f};
+
+    int issued = s_begin;
+#pragma unroll
+    for (int i = 0; i < kSmallMNtStages - 1; ++i)
+        if (issued < s_end) {
+            issue_stage(i);
+            ++issued;
+        }
+    int slot = 0, fill = kSmallMNtStages - 1;
+    for (int s = s_begin; s < s_end; ++s) {
+        if (issued < s_end) {
+            issue_stage(fill);
+            ++issued;
+            fill = (fill + 1 == kSmallMNtStages) ? 0 : fill + 1;
+            wait_vmcnt<4 * (kSmallMNtStages - 1)>();  // everything but the newest kSmallMNtStages-1 steps has landed
+        } else {
+            wait_vmcnt<0>();
+        }
+        MI355_LDS char* st = wbase + slot * kSmallMNtStageBytes;
+        slot = (slot + 1 == kSmallMNtStages) ? 0 : slot + 1;
+#pragma unroll
+        for (int sub = 0; sub < 2; ++sub) {
+            half8 bf = lds_read_b128(st + f_off[sub]);
+            half8 af = lds_read_b128(st + 2048 + f_off[sub]);
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(af, bf, acc, 0, 0, 0);
+        }
+        wait_lgkmcnt<0>();  // the reads of this slot are complete before a later copy refills it
+    }
+
+    // acc[q] is D[m = 4*(lane/16) + q][n = lane%16]; reduce the 8 partial tiles through LDS
+    __syncthreads();
+    MI355_LDS float* red = (MI355_LDS float*)smem;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) red[wave * 256 + (4 * (lane >> 4) + q) * 16 + (lane & 15)] = acc[q];
+    __syncthreads();
+    if (tid < 256) {
+        float sum = 0.f;
+#pragma unroll
+        for (int w = 0; w < 8; ++w) sum += red[w * 256 + tid];
+        const int m = m0 + (tid >> 4);
+        const int n = n0 + (tid & 15);
+        if (m < M && n < N) C[(long)m * ldc + n] = (half_t)sum;
+    }
+}
+
+static hipError_t launch_smallm_nt(const half_t* A, const half_t* B, half_t* C, int M, int N, int K, long lda, long ldb,
+                                   long ldc, hipStream_t stream) {
+    static bool attr_set = false;
+    if (!attr_set) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(hgemm_smallm_nt_kernel),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, kSmallMNtLdsBytes);
+        if (e != hipSuccess) return e;
+        attr_set = true;
+    }
+    const int n_tiles = (N + 15) / 16;
+    dim3 grid(n_tiles, (M + 15) / 16);
+    hgemm_smallm_nt_kernel<<<grid, dim3(512), kSmallMNtLdsBytes, stream>>>(A, B, C, M, N, K, lda, ldb, ldc, n_tiles);
+    return hipGetLastError();
+}
+
 int g_gemm_variant = 0;  // tuning hook: 0 = heuristic, 1 = force 256x256 tiles, 2 = force 128x128 tiles
 
 template <bool A_KC, bool B_KC, int BM, int BN, int WM, int WN>
@@ -588,6 +707,9 @@ static hipError_t launch_layout(const half_t* A, const half_t* B, half_t* C, int
     if constexpr (A_KC && !B_KC) {
         if (aligned && M <= 64 && K % 32 == 0 && K >= 32 && N % 8 == 0 && ldc % 2 == 0)
             return launch_smallm_nn(A, B, C, M, N, K, lda, ldb, ldc, stream);
+    }
+    if constexpr (A_KC && B_KC) {
+        if (aligned && M <= 64 && K % 64 == 0 && K >= 64) return launch_smallm_nt(A, B, C, M, N, K, lda, ldb, ldc, stream);
     }
     // 256x256 tiles when they fill the machine (>= ~3/4 of the 256 CUs), 128x128 tiles for smaller problems
     const long tiles256 = fits256 ? (long)(M / 256) * (N / 256) : 0;
