@@ -6,13 +6,17 @@
  * after validating their tensors; it can equally be bound from C, C++ or ctypes.
  *
  * Conventions
- *   - every pointer is a DEVICE pointer owned by the caller; nothing is allocated, freed or retained;
+ *   - every pointer is a DEVICE pointer owned by the caller; none is retained. The only memory the library ever
+ *     allocates is a workspace for the partial results of the split-KV attention path (taken when
+ *     Hq/Hkv * Sq <= 32 and kv_valid_len >= 512, i.e. generation steps): one buffer per (device, stream), obtained
+ *     with hipMallocAsync on that stream at first use (>= 4 MiB, regrown when a call needs more, kept until the
+ *     process ends), so steady-state calls allocate nothing and calls on different streams never share it;
  *   - `stream` is a hipStream_t passed as void* (NULL = the null stream); calls are asynchronous;
  *   - fp16 data is IEEE binary16 (`_Float16` / `__half` / torch.float16);
  *   - return value 0 = launched; non-zero = a hipError_t value or MI355_ERR_* below, nothing was launched.
  *     mi355_last_error() returns a thread-local description of the last failure.
- *   - calls are re-entrant and thread-safe; the library keeps no mutable global state besides one-time
- *     kernel attribute initialisation.
+ *   - calls are re-entrant and thread-safe; the only mutable global state is one-time kernel attribute
+ *     initialisation and the mutex-protected table of those workspaces.
  */
 #ifndef MI355_SERVING_H
 #define MI355_SERVING_H
@@ -84,7 +88,8 @@ int mi355_serving_version(void);
  * by shape, so tests and tuning runs can exercise every variant on every shape. Process-wide; 0 restores the
  * heuristic. A variant that does not fit the shape (e.g. tile sizes that do not divide it) is ignored.
  *   gemm: 1 = 256x256 tiles, 2 = 128x128 tiles
- *   fmha: 1 = 4 waves x 32 queries, 2 = 8 waves x 32 queries, 3 = 8 waves x 32 queries ping-pong
+ *   fmha: 1 = 4 waves x 32 queries, 2 = 8 waves x 32 queries, 3 = 8 waves x 32 queries ping-pong (1..3 also
+ *         keep generation-step shapes off the split-KV path)
  */
 void mi355_debug_set_gemm_variant(int variant);
 void mi355_debug_set_fmha_variant(int variant);

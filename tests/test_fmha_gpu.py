@@ -128,6 +128,42 @@ def test_every_kernel_variant_on_ragged_shapes(lib, gpu, variant, B, Hq, Hkv, Sq
         lib.set_variants()
 
 
+@pytest.mark.parametrize("B,Hq,Hkv,Sq,Sk,causal,kvv", [
+    (1, 32, 8, 1, 8192, False, None),    # Llama-3-8B generation step
+    (2, 8, 2, 1, 1000, False, 999), (1, 32, 8, 4, 2048, True, None), (1, 4, 4, 1, 600, False, None),
+    (3, 16, 2, 3, 777, True, 700), (1, 1, 1, 1, 70000, False, None), (1, 32, 1, 1, 513, False, 512),
+])
+def test_generation_step_split_kv_path(lib, gpu, B, Hq, Hkv, Sq, Sk, causal, kvv):
+    # Hq/Hkv * Sq <= 32 and >= 512 valid keys: the split-KV kernels; compared with the oracle and with the
+    # prefill kernel on the same inputs
+    q, k, v = so.fmha_inputs(B, Hq, Hkv, Sq, Sk, seed=Sk + Hq)
+    o, lse = check(lib, gpu, q, k, v, causal, kvv)
+    lib.set_variants(fmha=1)
+    try:
+        o1, lse1 = run(lib, gpu, q, k, v, causal, kvv)
+    finally:
+        lib.set_variants()
+    assert (o.float() - o1.float()).abs().max() <= 2e-3 and (lse - lse1).abs().max() <= 1e-3
+
+
+def test_generation_step_on_two_streams(lib, gpu):
+    # the split-KV workspace is per stream: interleaved calls on two streams must not disturb each other
+    qa, ka, va = (t.to(gpu) for t in so.fmha_inputs(1, 32, 8, 1, 4096, seed=1))
+    qb, kb, vb = (t.to(gpu) for t in so.fmha_inputs(2, 16, 4, 1, 3000, seed=2))
+    ref_a = lib.fmha_fwd(qa, ka, va)[0].clone()
+    ref_b = lib.fmha_fwd(qb, kb, vb)[0].clone()
+    torch.cuda.synchronize()
+    s1, s2 = torch.cuda.Stream(), torch.cuda.Stream()
+    outs_a, outs_b = [], []
+    for _ in range(5):
+        with torch.cuda.stream(s1):
+            outs_a.append(lib.fmha_fwd(qa, ka, va)[0])
+        with torch.cuda.stream(s2):
+            outs_b.append(lib.fmha_fwd(qb, kb, vb)[0])
+    torch.cuda.synchronize()
+    assert all(torch.equal(o, ref_a) for o in outs_a) and all(torch.equal(o, ref_b) for o in outs_b)
+
+
 def test_masked_keys_may_hold_garbage(lib, gpu):
     # keys at or beyond kv_valid_len must not influence the result, whatever they contain
     q, k, v = so.fmha_inputs(1, 2, 2, 90, 200, seed=11)

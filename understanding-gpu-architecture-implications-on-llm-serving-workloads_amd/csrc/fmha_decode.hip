@@ -1,0 +1,347 @@
+// Decode-shaped attention forward for gfx950 (MI355X): few query rows per kv head, long key sequence.
+//
+// The reference runs its generation step (`is_decode`, one query row padded to 64 by ops.py:19-25) through the
+// prefill kernel, one workgroup per (batch, q head) walking all keys (semi/fmha_2_amd.cpp:341-356); that leaves
+// almost the whole GPU idle and is bound by one workgroup's memory rate. Here the step is a split-KV
+// ("flash-decoding") pass, HBM-bound by the single read of K and V:
+//
+//   pass 1  fmha_decode_split_kernel: a work unit is one wave = (batch, kv head, key range). The query rows of all
+//           q heads that share the kv head are packed side by side as the (up to 32) columns of the S^T = K Q^T
+//           product, so K and V are read once per kv head, not once per q head. The wave streams its key range in
+//           tiles of 32 keys through its own LDS pipeline (direct-to-LDS copies, no workgroup barriers), runs the
+//           same register-resident online softmax as the prefill kernel and writes unnormalised partial results
+//           (O~ [128], m, l per column, fp32) to a workspace.
+//   pass 2  fmha_decode_merge_kernel: one workgroup per query row combines the partials of all key ranges,
+//           O = sum_s 2^((m_s - m) c) O~_s / sum_s 2^((m_s - m) c) l_s, and writes O (fp16) and LSE.
+//
+// Mask semantics are those of the prefill kernel (keys >= kv_valid_len masked; causal: key j visible to query i
+// iff j <= i + Sk - Sq).
+#include <map>
+#include <mutex>
+#include <utility>
+
+#include "mi355_common.h"
+#include "mi355_serving_internal.h"
+
+namespace mi355 {
+
+namespace dec {
+constexpr int D = 128;
+constexpr int TK = 32;                       // keys per tile
+constexpr int ROW_BYTES = D * 2;             // 256
+constexpr int TILE_BYTES = TK * ROW_BYTES;   // 8 KiB
+constexpr int STAGE_BYTES = 2 * TILE_BYTES;  // K + V
+constexpr int NSTAGE = 3;
+constexpr int WAVES = 2;                     // work units per workgroup
+constexpr int WAVE_BYTES = NSTAGE * STAGE_BYTES;
+constexpr int LDS_BYTES = WAVES * WAVE_BYTES;  // 96 KiB
+constexpr int COPIES = 2 * (TILE_BYTES / 1024);  // 16 copy instructions per stage
+constexpr int PART_STRIDE = D + 4;           // floats per (unit, column): O~[128], m, l, 2 pad (keeps rows 16-byte aligned)
+
+__device__ __forceinline__ int swz_k(int row) { return row & 15; }
+__device__ __forceinline__ int swz_v(int row) {
+    int r = row & 3;
+    return (r << 1) | ((r & 1) << 3);
+}
+__device__ __forceinline__ float other_half(float x) {
+    int idx = ((int)(threadIdx.x & 63) ^ 32) << 2;
+    return __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute(idx, __builtin_bit_cast(int, x)));
+}
+}  // namespace dec
+
+// units = B * Hkv * splits, unit u = (b * Hkv + hkv) * splits + s covers key tiles [s * tiles_per_split, ...)
+__global__ __launch_bounds__(dec::WAVES * 64) void fmha_decode_split_kernel(
+    const half_t* __restrict__ Q, const half_t* __restrict__ K, const half_t* __restrict__ V, float* __restrict__ part, int B,
+    int Hq, int Hkv, int Sq, int Sk, float scale_log2, int causal, int kv_valid, int splits, int tiles_per_split, int units) {
+    using namespace dec;
+    extern __shared__ __attribute__((aligned(1024))) char smem_raw[];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int unit = blockIdx.x * WAVES + wave;
+    if (unit >= units) return;  // no workgroup barrier is used anywhere in this kernel
+    MI355_LDS char* wbase = (MI355_LDS char*)smem_raw + wave * WAVE_BYTES;
+
+    const int h = lane >> 5;
+    const int l32 = lane & 31;
+    const int s_idx = unit % splits;
+    const int bh = unit / splits;
+    const int hkv = bh % Hkv;
+    const int b = bh / Hkv;
+    const int group = Hq / Hkv;
+    const int ncols = group * Sq;  // <= 32
+    const int shift = Sk - Sq;
+
+    // column c of the packed query block = (q head hkv*group + c / Sq, query row c % Sq)
+    const int col = min(l32, ncols - 1);
+    const int hq = hkv * group + col / Sq;
+    const int qi = col % Sq;
+    const half_t* qp = Q + (((long)b * Hq + hq) * Sq + qi) * D + 8 * h;
+    half8 qf[8];
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks) qf[ks] = *(const half8*)(qp + ks * 16);
+    const int lim = causal ? min(kv_valid - 1, qi + shift) : kv_valid - 1;  // last visible key of this column
+
+    const half_t* Kh = K + ((long)b * Hkv + hkv) * (long)Sk * D;
+    const half_t* Vh = V + ((long)b * Hkv + hkv) * (long)Sk * D;
+
+    const int tiles = (kv_valid + TK - 1) / TK;
+    const int t_begin = s_idx * tiles_per_split;
+    const int t_end = min(t_begin + tiles_per_split, tiles);
+
+    // copy i (0..7) of a tile covers rows 4i + lane/16, chunk position lane%16
+    const int c_row = lane >> 4;
+    auto issue_stage = [&](int tile, int slot) {
+        MI355_LDS char* st = wbase + slot * STAGE_BYTES;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            int row = 4 * i + c_row;
+            int grow = min(tile * TK + row, kv_valid - 1);
+            copy16_global_to_lds(Kh + (long)grow * D + ((lane & 15) ^ swz_k(row)) * 8, st + i * 1024);
+        }
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            int row = 4 * i + c_row;
+            int grow = min(tile * TK + row, kv_valid - 1);
+            copy16_global_to_lds(Vh + (long)grow * D + ((lane & 15) ^ swz_v(row)) * 8, st + TILE_BYTES + i * 1024);
+        }
+    };
+
+    const int k_base = l32 * ROW_BYTES + ((h ^ (lane & 15)) << 4);  // xor (ks << 5)
+    const int v_row = 4 * h + ((lane & 15) >> 2);
+    const int v_clow = 2 * ((lane >> 4) & 1) + ((lane & 3) >> 1);
+    const int v_base = TILE_BYTES + v_row * ROW_BYTES + ((v_clow ^ swz_v(v_row)) << 4) + (lane & 1) * 8;  // xor (db << 6)
+
+    float16v o[4];
+#pragma unroll
+    for (int db = 0; db < 4; ++db)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) o[db][e] = 0.f;
+    float m_run = -INFINITY, l_run = 0.f;
+
+    int issued = t_begin;
+#pragma unroll
+    for (int i = 0; i < NSTAGE - 1; ++i)
+        if (issued < t_end) {
+            issue_stage(issued, i);
+            ++issued;
+        }
+    int slot = 0, fill = NSTAGE - 1;
+    for (int t = t_begin; t < t_end; ++t) {
+        if (issued < t_end) {
+            issue_stage(issued, fill);
+            ++issued;
+            fill = (fill + 1 == NSTAGE) ? 0 : fill + 1;
+            wait_vmcnt<COPIES*(NSTAGE - 1)>();  // everything but the newest NSTAGE-1 tiles has landed
+        } else {
+            wait_vmcnt<0>();
+        }
+        MI355_LDS char* st = wbase + slot * STAGE_BYTES;
+        slot = (slot + 1 == NSTAGE) ? 0 : slot + 1;
+
+        // S^T = K Q^T : lane holds keys 8p + 4h + q of column l32
+        float16v s;
+#pragma unroll
+        for (int e = 0; e < 16; ++e) s[e] = 0.f;
+#pragma unroll
+        for (int ks = 0; ks < 8; ++ks) {
+            half8 kf = lds_read_b128(st + (k_base ^ (ks << 5)));
+            s = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf, qf[ks], s, 0, 0, 0);
+        }
+        const int key0 = t * TK;
+        float mx = -INFINITY;
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+            int key = key0 + 8 * (e >> 2) + 4 * h + (e & 3);
+            if (key > lim) s[e] = -INFINITY;
+            mx = fmaxf(mx, s[e]);
+        }
+        mx = fmaxf(mx, other_half(mx));
+        float m_new = fmaxf(m_run, mx);
+        float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+        float alpha = __builtin_amdgcn_exp2f((m_run - m_use) * scale_log2);
+        m_run = m_new;
+        const float neg_ms = -m_use * scale_log2;
+        float psum = 0.f;
+        half8 pf[2];
+#pragma unroll
+        for (int tt = 0; tt < 2; ++tt) {
+            half8 pk;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                float p = __builtin_amdgcn_exp2f(__builtin_fmaf(s[8 * tt + j], scale_log2, neg_ms));
+                psum += p;
+                pk[j] = (half_t)p;
+            }
+            pf[tt] = pk;
+        }
+        l_run = l_run * alpha + psum;
+#pragma unroll
+        for (int db = 0; db < 4; ++db)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) o[db][e] *= alpha;
+        // O^T += V^T P^T
+#pragma unroll
+        for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+            for (int db = 0; db < 4; ++db) {
+                int off = (v_base ^ (db << 6)) + (16 * tt) * ROW_BYTES;
+                half8 vf = concat(lds_read_tr16_b64(st + off), lds_read_tr16_b64(st + off + 8 * ROW_BYTES));
+                o[db] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf, pf[tt], o[db], 0, 0, 0);
+            }
+        wait_lgkmcnt<0>();  // the reads of this slot are complete before a later copy refills it
+    }
+
+    // partial result of this unit: O~ (unnormalised), m (raw score units), l
+    const float l_tot = l_run + other_half(l_run);
+    if (l32 < ncols) {
+        float* pp = part + ((long)unit * ncols + l32) * PART_STRIDE;
+#pragma unroll
+        for (int db = 0; db < 4; ++db)
+#pragma unroll
+            for (int p = 0; p < 4; ++p) {
+                float4v v;
+#pragma unroll
+                for (int q = 0; q < 4; ++q) v[q] = o[db][4 * p + q];
+                *(float4v*)(pp + db * 32 + 8 * p + 4 * h) = v;
+            }
+        if (h == 0) {
+            pp[D] = m_run;
+            pp[D + 1] = l_tot;
+        }
+    }
+}
+
+// one workgroup of 128 threads per query row (b, hq, qi). The statistics of the key ranges are combined with the
+// ranges spread over the threads (so their loads are independent), then thread d merges element d of O.
+constexpr int kMaxSplits = 512;
+
+__global__ __launch_bounds__(128) void fmha_decode_merge_kernel(const float* __restrict__ part, half_t* __restrict__ O,
+                                                                float* __restrict__ LSE, int Hq, int Hkv, int Sq,
+                                                                float scale_log2, int splits) {
+    using namespace dec;
+    __shared__ float w_sh[kMaxSplits];
+    __shared__ float red[128];
+    const int tid = threadIdx.x;
+    const int row = blockIdx.x;  // (b * Hq + hq) * Sq + qi
+    const int qi = row % Sq;
+    const int hq = (row / Sq) % Hq;
+    const int b = row / (Sq * Hq);
+    const int group = Hq / Hkv;
+    const int hkv = hq / group;
+    const int ncols = group * Sq;
+    const int col = (hq - hkv * group) * Sq + qi;
+    const float* base = part + (((long)(b * Hkv + hkv) * splits) * ncols + col) * PART_STRIDE;
+    const long unit_stride = (long)ncols * PART_STRIDE;
+
+    // m = max over ranges
+    float m_loc = -INFINITY;
+    for (int s = tid; s < splits; s += 128) {
+        float ms = base[s * unit_stride + D];
+        w_sh[s] = ms;
+        m_loc = fmaxf(m_loc, ms);
+    }
+    red[tid] = m_loc;
+    __syncthreads();
+    float m = -INFINITY;
+#pragma unroll 8
+    for (int t = 0; t < 128; ++t) m = fmaxf(m, red[t]);
+    __syncthreads();
+    // weights 2^((m_s - m) c) (0 for ranges without a visible key) and l = sum_s w_s l_s
+    float l_loc = 0.f;
+    for (int s = tid; s < splits; s += 128) {
+        float w = (m == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f((w_sh[s] - m) * scale_log2);
+        w_sh[s] = w;
+        l_loc += w * base[s * unit_stride + D + 1];
+    }
+    red[tid] = l_loc;
+    __syncthreads();
+    float l = 0.f;
+#pragma unroll 8
+    for (int t = 0; t < 128; ++t) l += red[t];
+    // O[d] = sum_s w_s O~_s[d] / l
+    float acc = 0.f;
+#pragma unroll 8
+    for (int s = 0; s < splits; ++s) acc += w_sh[s] * base[s * unit_stride + tid];
+    O[(long)row * D + tid] = (half_t)((l > 0.f) ? acc / l : 0.f);
+    if (LSE != nullptr && tid == 0)
+        LSE[row] = (l > 0.f) ? (m * scale_log2 + __builtin_log2f(l)) * 0.69314718055994531f : -INFINITY;
+}
+
+bool fmha_decode_applicable(int B, int Hq, int Hkv, int Sq, int Sk, int kv_valid_len) {
+    const int group = Hq / Hkv;
+    return (long)group * Sq <= 32 && kv_valid_len >= 512 && Sk >= kv_valid_len && B >= 1;
+}
+
+// Workspace for the partial results: one buffer per (device, stream), allocated stream-ordered on first use and
+// regrown (never shrunk) when a call needs more. Calls on one stream are ordered, so they can share it; calls on
+// different streams get different buffers. Steady-state calls allocate nothing.
+static hipError_t decode_workspace(size_t bytes, hipStream_t stream, float** out) {
+    struct Buf {
+        void* ptr = nullptr;
+        size_t size = 0;
+    };
+    static std::mutex mu;
+    static std::map<std::pair<int, hipStream_t>, Buf> bufs;
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    std::lock_guard<std::mutex> lock(mu);
+    Buf& b = bufs[std::make_pair(dev, stream)];
+    if (b.size < bytes) {
+        if (b.ptr != nullptr) {
+            e = hipFreeAsync(b.ptr, stream);  // ordered after the kernels already queued on this stream
+            b.ptr = nullptr;
+            b.size = 0;
+            if (e != hipSuccess) return e;
+        }
+        size_t want = bytes < (size_t(4) << 20) ? (size_t(4) << 20) : bytes + bytes / 2;
+        e = hipMallocAsync(&b.ptr, want, stream);
+        if (e != hipSuccess) {
+            b.ptr = nullptr;
+            return e;
+        }
+        b.size = want;
+    }
+    *out = static_cast<float*>(b.ptr);
+    return hipSuccess;
+}
+
+hipError_t fmha_decode_dispatch(const half_t* Q, const half_t* K, const half_t* V, half_t* O, float* LSE, int B, int Hq,
+                                int Hkv, int Sq, int Sk, float scale, int causal, int kv_valid, hipStream_t stream) {
+    using namespace dec;
+    static bool attr_set = false;
+    if (!attr_set) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(fmha_decode_split_kernel),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
+        if (e != hipSuccess) return e;
+        attr_set = true;
+    }
+    const int group = Hq / Hkv;
+    const int ncols = group * Sq;
+    const int tiles = (kv_valid + TK - 1) / TK;
+    // about two waves per CU in flight, at least 4 key tiles (128 keys) per wave
+    int splits = 512 / (B * Hkv);
+    splits = splits < 1 ? 1 : splits;
+    int max_splits = (tiles + 3) / 4;
+    if (splits > max_splits) splits = max_splits;
+    if (splits > kMaxSplits) splits = kMaxSplits;
+    const int tiles_per_split = (tiles + splits - 1) / splits;
+    splits = (tiles + tiles_per_split - 1) / tiles_per_split;
+    const long units = (long)B * Hkv * splits;
+    const size_t bytes = (size_t)units * ncols * PART_STRIDE * sizeof(float);
+
+    float* part = nullptr;
+    hipError_t e = decode_workspace(bytes, stream, &part);
+    if (e != hipSuccess) return e;
+    const float scale_log2 = scale * 1.4426950408889634f;
+    const unsigned blocks = (unsigned)((units + WAVES - 1) / WAVES);
+    fmha_decode_split_kernel<<<dim3(blocks), dim3(WAVES * 64), LDS_BYTES, stream>>>(
+        Q, K, V, part, B, Hq, Hkv, Sq, Sk, scale_log2, causal, kv_valid, splits, tiles_per_split, (int)units);
+    e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    fmha_decode_merge_kernel<<<dim3((unsigned)((long)B * Hq * Sq)), dim3(128), 0, stream>>>(part, O, LSE, Hq, Hkv, Sq,
+                                                                                          scale_log2, splits);
+    return hipGetLastError();
+}
+
+}  // namespace mi355

@@ -662,7 +662,9 @@ hipError_t fmha_fwd_dispatch(const void* Q, const void* K, const void* V, void* 
     const half_t* v = static_cast<const half_t*>(V);
     half_t* o = static_cast<half_t*>(O);
     int variant = g_fmha_variant;
-    if (variant == 0) {
+    if ((variant == 0 || variant == 4) && fmha_decode_applicable(B, Hq, Hkv, Sq, Sk, kv_valid_len))
+        return fmha_decode_dispatch(q, k, v, o, LSE, B, Hq, Hkv, Sq, Sk, scale, causal, kv_valid_len, stream);
+    if (variant == 0 || variant == 4) {
         // 256-query ping-pong workgroups once there are enough of them to fill the 256 CUs, otherwise 128-query ones
         const long wg256 = (long)((Sq + 255) / 256) * Hq * B;
         variant = (wg256 >= 256) ? 3 : 1;

@@ -13,4 +13,9 @@ hipError_t hgemm_dispatch(const void* A, const void* B, void* C, int M, int N, i
 hipError_t fmha_fwd_dispatch(const void* Q, const void* K, const void* V, void* O, float* LSE, int B, int Hq, int Hkv,
                              int Sq, int Sk, float scale, int causal, int kv_valid_len, hipStream_t stream);
 
+// Split-KV path for few query rows per kv head (generation step); see fmha_decode.hip.
+bool fmha_decode_applicable(int B, int Hq, int Hkv, int Sq, int Sk, int kv_valid_len);
+hipError_t fmha_decode_dispatch(const _Float16* Q, const _Float16* K, const _Float16* V, _Float16* O, float* LSE, int B, int Hq,
+                                int Hkv, int Sq, int Sk, float scale, int causal, int kv_valid_len, hipStream_t stream);
+
 }  // namespace mi355
