@@ -31,8 +31,8 @@ PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 
 # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (KiB per dispatch), each scaled by what the same
 # counter reads for a 1 GiB device-to-device copy (FETCH_SIZE x2.0, WRITE_SIZE x1.0); see profiles/.
-MEASURED_TRAFFIC_BYTES = (786780 * 2.0 + 131072 * 1.0) * 1024        # hgemm_main_kernel, 8192^3 NN
-MEASURED_TRAFFIC_BYTES_FMHA = (27502 * 2.0 + 33280 * 1.0) * 1024     # fmha_fwd_kernel, F4
+MEASURED_TRAFFIC_BYTES = (786882 * 2.0 + 131072 * 1.0) * 1024        # hgemm_main_kernel, 8192^3 NN
+MEASURED_TRAFFIC_BYTES_FMHA = (26371 * 2.0 + 33280 * 1.0) * 1024     # fmha_fwd_pingpong_kernel, F4
 
 
 def log(*a):
@@ -158,7 +158,7 @@ def main():
     }
     roofline = {"kernel": "hgemm_main_kernel (8192^3, NN)", "bound": "mfma", "achieved": gemm_tf, "peak": PEAK_FP16_TFLOPS,
                 "unit": "TFLOP/s", "frac": gemm_tf / PEAK_FP16_TFLOPS, "traffic": MEASURED_TRAFFIC_BYTES}
-    roofline_fmha = {"kernel": "fmha_fwd_kernel (F4)", "bound": "mfma", "achieved": fmha_tf, "peak": PEAK_FP16_TFLOPS,
+    roofline_fmha = {"kernel": "fmha_fwd_pingpong_kernel (F4)", "bound": "mfma", "achieved": fmha_tf, "peak": PEAK_FP16_TFLOPS,
                      "unit": "TFLOP/s", "frac": fmha_tf / PEAK_FP16_TFLOPS, "traffic": MEASURED_TRAFFIC_BYTES_FMHA}
 
     # ---- the other benchmark configurations (quick timings) ----------------------------------------------------------
@@ -184,6 +184,23 @@ def main():
         other["F3_fmha_noncausal_b4_h32_s1024"] = {"ms": ms3, "tflops": fl3 / ms3 / 1e9,
                                                    "pct_of_fp16_mfma_peak": 100 * fl3 / ms3 / 1e9 / PEAK_FP16_TFLOPS}
         del q3, k3, v3, o3
+        # generation-step shapes (HBM bound): nn.Linear-layout weight GEMM and attention over a long KV cache
+        xd = so.randn_fp16((16, 4096), 1).to(dev)
+        wd_nt = so.randn_fp16((14336, 4096), 2, 0.02).to(dev)
+        od = torch.empty((16, 14336), dtype=torch.float16, device=dev)
+        msd = time_launches(lambda: lib.hgemm_raw(xd.data_ptr(), wd_nt.data_ptr(), od.data_ptr(), 16, 14336, 4096, 4096, 4096,
+                                                  14336, lib.GEMM_NT, stream), 20, 3)
+        byd = 2.0 * (16 * 4096 + 4096 * 14336 + 16 * 14336)
+        other["gemm_decode_nt_16x14336x4096"] = {"ms": msd, "gbs": byd / msd / 1e6, "pct_of_hbm_peak": 100 * byd / msd / 1e6 / PEAK_HBM_GBS}
+        for bd, skd in ((1, 8192), (8, 8192), (1, 32768)):
+            qd, kd, vd = (t.to(dev) for t in so.fmha_inputs(bd, 32, 8, 1, skd, seed=7))
+            o_d = torch.empty_like(qd)
+            ms_d = time_launches(lambda: lib.fmha_fwd_raw(qd.data_ptr(), kd.data_ptr(), vd.data_ptr(), o_d.data_ptr(), None, bd,
+                                                          32, 8, 1, skd, 128, scale, 0, skd, stream), 20, 3)
+            by_d = 2.0 * (2 * bd * 8 * skd * 128 + 2 * bd * 32 * 128)
+            other["fmha_decode_b%d_h32_8_sk%d" % (bd, skd)] = {"ms": ms_d, "gbs": by_d / ms_d / 1e6,
+                                                               "pct_of_hbm_peak": 100 * by_d / ms_d / 1e6 / PEAK_HBM_GBS}
+        del xd, wd_nt, od, qd, kd, vd, o_d
         # L5: Llama-3-8B-shaped prefill layer at s = 8192, per stage
         S5, H5, F5 = 8192, 4096, 14336
         x5 = so.randn_fp16((S5, H5), 0).to(dev)
