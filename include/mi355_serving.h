@@ -77,6 +77,22 @@ int mi355_hgemm(const void* A, const void* B, void* C, int M, int N, int K, int6
 int mi355_fmha_fwd(const void* Q, const void* K, const void* V, void* O, float* LSE, int B, int Hq, int Hkv,
                    int Sq, int Sk, int D, float scale, int causal, int kv_valid_len, void* stream);
 
+/*
+ * mi355_fmha_fwd for operands that are not contiguous [B, H, S, D] tensors: element [b][h][s][d] of each operand
+ * lives at b*batch + h*head + s*row + d, with d contiguous. `strides` holds 12 element strides in the order
+ *   q_batch, q_head, q_row,  k_batch, k_head, k_row,  v_batch, v_head, v_row,  o_batch, o_head, o_row
+ * each a non-negative multiple of 8 (16 bytes); rows of O must not overlap. LSE stays [B, Hq, Sq] contiguous.
+ *
+ * Replaces the copies the reference makes before its kernel: its callers hand over transposed views of
+ * [B, S, H, D] projections (benchmarks/flashattn-cuda/modeling_llama.py:658-660) which
+ * kernels/fmha/pkg/fmha_unified/ops.py:23-25 turns into contiguous tensors, and transpose the output back
+ * (modeling_llama.py:700). With strides, Q/K/V can be read straight out of a fused QKV projection
+ * ([B, S, (Hq + 2 Hkv) * D]: row = (Hq + 2 Hkv) * D, head = D) or a KV cache, and O written as [B, S, Hq * D].
+ */
+int mi355_fmha_fwd_strided(const void* Q, const void* K, const void* V, void* O, float* LSE, int B, int Hq, int Hkv,
+                           int Sq, int Sk, int D, float scale, int causal, int kv_valid_len, const int64_t* strides,
+                           void* stream);
+
 /* Thread-local text for the last non-zero return of this thread ("" if none). */
 const char* mi355_last_error(void);
 

@@ -41,6 +41,16 @@ def test_capi_rejects_bad_arguments_without_a_gpu(lib):
     assert cdll.mi355_fmha_fwd(p, p, p, p, None, 1, 5, 2, 8, 8, 128, 0.1, 0, 8, None) == 10001  # Hq % Hkv
     assert cdll.mi355_fmha_fwd(p, p, p, p, None, 1, 4, 2, 8, 8, 128, 0.1, 0, 9, None) == 10001  # kv_valid > Sk
     assert cdll.mi355_fmha_fwd(p, p, p, p, None, 1, 4, 2, 8, 8, 128, -1.0, 0, 8, None) == 10001  # scale <= 0
+    def strided(st):
+        arr = (ctypes.c_int64 * 12)(*st)
+        return cdll.mi355_fmha_fwd_strided(p, p, p, p, None, 2, 4, 2, 8, 8, 128, 0.1, 0, 8, arr, None)
+    good = [4096, 128, 512] * 4
+    assert strided(good[:2] + [516] + good[3:]) == 10001  # q row stride not a multiple of 8 elements
+    assert b"stride 2" in cdll.mi355_last_error()
+    assert strided(good[:5] + [-512] + good[6:]) == 10001  # negative stride
+    assert strided(good[:11] + [64]) == 10001              # rows of O overlap
+    assert b"overlap" in cdll.mi355_last_error()
+    assert cdll.mi355_fmha_fwd_strided(p, p, p, p, None, 2, 4, 2, 8, 8, 128, 0.1, 0, 8, None, None) == 10001
     with pytest.raises(lib.Mi355Error):
         lib.hgemm_raw(0, 0, 0, 4, 4, 4, 4, 4, 4, 0)
 

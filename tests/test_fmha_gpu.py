@@ -164,6 +164,45 @@ def test_generation_step_on_two_streams(lib, gpu):
     assert all(torch.equal(o, ref_a) for o in outs_a) and all(torch.equal(o, ref_b) for o in outs_b)
 
 
+# ---- operands read in place from other layouts ------------------------------------------------------------------------
+@pytest.mark.parametrize("B,Hq,Hkv,Sq,Sk,causal", [
+    (2, 8, 2, 300, 300, True),      # prefill, 128-query workgroups
+    (1, 32, 8, 2048, 2048, True),   # prefill, ping-pong workgroups
+    (2, 8, 2, 1, 1500, False),      # generation step, split-KV kernels
+])
+def test_fused_qkv_projection_layout_read_in_place(lib, gpu, B, Hq, Hkv, Sq, Sk, causal):
+    # q, k, v are slices of one [B, S, (Hq + 2 Hkv) * 128] projection (k, v of a longer cache when Sq < Sk); the output is
+    # written as [B, Sq, Hq * 128]. Same numbers as the contiguous call on copies of the same values.
+    q, k, v = so.fmha_inputs(B, Hq, Hkv, Sq, Sk, seed=11)
+    W = (Hq + 2 * Hkv) * 128
+    fused = torch.zeros((B, Sk, W), dtype=torch.float16)
+    fused[:, :Sq, :Hq * 128] = q.transpose(1, 2).reshape(B, Sq, Hq * 128)
+    fused[:, :, Hq * 128:(Hq + Hkv) * 128] = k.transpose(1, 2).reshape(B, Sk, Hkv * 128)
+    fused[:, :, (Hq + Hkv) * 128:] = v.transpose(1, 2).reshape(B, Sk, Hkv * 128)
+    fused = fused.to(gpu)
+    qv = fused[:, :Sq, :Hq * 128].view(B, Sq, Hq, 128).transpose(1, 2)
+    kv = fused[:, :, Hq * 128:(Hq + Hkv) * 128].view(B, Sk, Hkv, 128).transpose(1, 2)
+    vv = fused[:, :, (Hq + Hkv) * 128:].view(B, Sk, Hkv, 128).transpose(1, 2)
+    assert not qv.is_contiguous() and not kv.is_contiguous()
+    out = torch.full((B, Sq, Hq * 128), float("nan"), dtype=torch.float16, device=gpu)
+    o, lse = lib.fmha_fwd(qv, kv, vv, causal=causal, out=out.view(B, Sq, Hq, 128).transpose(1, 2))
+    o_c, lse_c = lib.fmha_fwd(q.to(gpu), k.to(gpu), v.to(gpu), causal=causal)
+    torch.cuda.synchronize()
+    assert torch.equal(out.view(B, Sq, Hq, 128).transpose(1, 2), o_c) and torch.equal(lse, lse_c)
+    o_ref, lse_ref = so.attention_ref(q, k, v, causal=causal)
+    assert so.fmha_tolerance_ok(o_c.cpu(), lse_c.cpu(), o_ref, lse_ref)[0]
+
+
+def test_broadcast_kv_head_with_zero_stride(lib, gpu):
+    # a kv head stride of 0 shares one K/V head between all kv heads (what expand() produces)
+    q, k, v = so.fmha_inputs(1, 4, 1, 200, 200, seed=3)
+    o1, lse1 = lib.fmha_fwd(q.to(gpu), k.to(gpu), v.to(gpu), causal=True)
+    ke, ve = k.to(gpu).expand(1, 4, 200, 128), v.to(gpu).expand(1, 4, 200, 128)
+    o2, lse2 = lib.fmha_fwd(q.to(gpu), ke, ve, causal=True)
+    torch.cuda.synchronize()
+    assert torch.equal(o1, o2) and torch.equal(lse1, lse2)
+
+
 def test_masked_keys_may_hold_garbage(lib, gpu):
     # keys at or beyond kv_valid_len must not influence the result, whatever they contain
     q, k, v = so.fmha_inputs(1, 2, 2, 90, 200, seed=11)
@@ -242,3 +281,24 @@ def test_torch_operator_accepts_reference_style_padded_call(gpu):
     o = torch.ops.fmha_unified.finefmha_2.default(pad(q), pad(k), pad(v), True, False, 100)[:, :, :100]
     ok, st = so.fmha_tolerance_ok(o, None, so.fine_fmha_ref(q, k, v, True, False), None)
     assert ok, st
+
+
+def test_torch_operator_reads_transposed_views_in_place(gpu):
+    # the in-model call of the reference: [B, S, H, D] projections viewed as [B, H, S, D]
+    # (benchmarks/flashattn-cuda/modeling_llama.py:658-660); the result has q's layout, so transposing it back is free
+    import fmha_unified
+    B, S, Hq, Hkv = 2, 384, 8, 2
+    q, k, v = so.fmha_inputs(B, Hq, Hkv, S, S, seed=21)
+    qp = q.transpose(1, 2).contiguous().to(gpu)   # [B, S, H, D]
+    kp = k.transpose(1, 2).contiguous().to(gpu)
+    vp = v.transpose(1, 2).contiguous().to(gpu)
+    out = fmha_unified.ops.fine_fmha(qp.transpose(1, 2), kp.transpose(1, 2), vp.transpose(1, 2), causal=True,
+                                     is_decode=False, kernel_index=5)
+    assert out.shape == (B, Hq, S, 128) and out.transpose(1, 2).is_contiguous()
+    o_ref, _ = so.attention_ref(q, k, v, causal=True)
+    assert (out.cpu().float() - o_ref).abs().max() <= 2e-3
+    # a view the kernel cannot read in place (last dimension strided) is copied, as the reference does
+    q2 = torch.empty((B, Hq, S, 256), dtype=torch.float16, device=gpu)[..., ::2]
+    q2.copy_(q.to(gpu))
+    out2 = fmha_unified.ops.fine_fmha(q2, k.to(gpu), v.to(gpu), True, False, 2)
+    assert (out2.cpu().float() - o_ref).abs().max() <= 2e-3

@@ -39,24 +39,50 @@ int mi355_hgemm(const void* A, const void* B, void* C, int M, int N, int K, int6
     return 0;
 }
 
-int mi355_fmha_fwd(const void* Q, const void* K, const void* V, void* O, float* LSE, int B, int Hq, int Hkv, int Sq,
-                   int Sk, int D, float scale, int causal, int kv_valid_len, void* stream) {
-    if (!Q || !K || !V || !O) return fail(MI355_ERR_BAD_ARGUMENT, "mi355_fmha_fwd: null pointer");
+static int fmha_checked(const char* fn, const void* Q, const void* K, const void* V, void* O, float* LSE, int B, int Hq, int Hkv,
+                        int Sq, int Sk, int D, float scale, int causal, int kv_valid_len, const mi355::FmhaStrides& sd,
+                        void* stream) {
+    if (!Q || !K || !V || !O) return fail(MI355_ERR_BAD_ARGUMENT, "%s: null pointer", fn);
     if (B < 1 || Hq < 1 || Hkv < 1 || Sq < 1 || Sk < 1)
-        return fail(MI355_ERR_BAD_ARGUMENT, "mi355_fmha_fwd: B, Hq, Hkv, Sq, Sk must be >= 1");
-    if (D != 128) return fail(MI355_ERR_UNSUPPORTED, "mi355_fmha_fwd: head_dim must be 128 (got %d)", D);
-    if (Hq % Hkv != 0) return fail(MI355_ERR_BAD_ARGUMENT, "mi355_fmha_fwd: Hq (%d) must be a multiple of Hkv (%d)", Hq, Hkv);
+        return fail(MI355_ERR_BAD_ARGUMENT, "%s: B, Hq, Hkv, Sq, Sk must be >= 1", fn);
+    if (D != 128) return fail(MI355_ERR_UNSUPPORTED, "%s: head_dim must be 128 (got %d)", fn, D);
+    if (Hq % Hkv != 0) return fail(MI355_ERR_BAD_ARGUMENT, "%s: Hq (%d) must be a multiple of Hkv (%d)", fn, Hq, Hkv);
     if (kv_valid_len < 1 || kv_valid_len > Sk)
-        return fail(MI355_ERR_BAD_ARGUMENT, "mi355_fmha_fwd: kv_valid_len %d outside [1, Sk=%d]", kv_valid_len, Sk);
+        return fail(MI355_ERR_BAD_ARGUMENT, "%s: kv_valid_len %d outside [1, Sk=%d]", fn, kv_valid_len, Sk);
     if (!(scale > 0.f) || scale > 3.0e38f)
-        return fail(MI355_ERR_BAD_ARGUMENT, "mi355_fmha_fwd: scale must be positive and finite (got %g)", (double)scale);
+        return fail(MI355_ERR_BAD_ARGUMENT, "%s: scale must be positive and finite (got %g)", fn, (double)scale);
     if ((reinterpret_cast<uintptr_t>(Q) | reinterpret_cast<uintptr_t>(K) | reinterpret_cast<uintptr_t>(V) |
          reinterpret_cast<uintptr_t>(O)) % 16 != 0)
-        return fail(MI355_ERR_BAD_ARGUMENT, "mi355_fmha_fwd: Q, K, V, O must be 16-byte aligned");
-    hipError_t e = mi355::fmha_fwd_dispatch(Q, K, V, O, LSE, B, Hq, Hkv, Sq, Sk, scale, causal != 0, kv_valid_len,
+        return fail(MI355_ERR_BAD_ARGUMENT, "%s: Q, K, V, O must be 16-byte aligned", fn);
+    const long all[12] = {sd.q_batch, sd.q_head, sd.q_row, sd.k_batch, sd.k_head, sd.k_row,
+                          sd.v_batch, sd.v_head, sd.v_row, sd.o_batch, sd.o_head, sd.o_row};
+    for (int i = 0; i < 12; ++i)
+        if (all[i] < 0 || all[i] % 8 != 0)
+            return fail(MI355_ERR_BAD_ARGUMENT, "%s: stride %d is %ld; strides must be non-negative multiples of 8 elements", fn, i,
+                        all[i]);
+    if (sd.o_row < D || (Hq > 1 && sd.o_head < D) || (B > 1 && sd.o_batch < D))
+        return fail(MI355_ERR_BAD_ARGUMENT, "%s: rows of O overlap (o strides %ld, %ld, %ld)", fn, sd.o_batch, sd.o_head, sd.o_row);
+    hipError_t e = mi355::fmha_fwd_dispatch(Q, K, V, O, LSE, B, Hq, Hkv, Sq, Sk, scale, causal != 0, kv_valid_len, sd,
                                             static_cast<hipStream_t>(stream));
-    if (e != hipSuccess) return hip_fail(e, "mi355_fmha_fwd launch");
+    if (e != hipSuccess) return hip_fail(e, fn);
     return 0;
+}
+
+int mi355_fmha_fwd(const void* Q, const void* K, const void* V, void* O, float* LSE, int B, int Hq, int Hkv, int Sq,
+                   int Sk, int D, float scale, int causal, int kv_valid_len, void* stream) {
+    const long q_head = (long)Sq * D, k_head = (long)Sk * D;
+    const mi355::FmhaStrides sd = {Hq * q_head, q_head, D, Hkv * k_head, k_head, D, Hkv * k_head, k_head, D, Hq * q_head, q_head, D};
+    return fmha_checked("mi355_fmha_fwd", Q, K, V, O, LSE, B, Hq, Hkv, Sq, Sk, D, scale, causal, kv_valid_len, sd, stream);
+}
+
+int mi355_fmha_fwd_strided(const void* Q, const void* K, const void* V, void* O, float* LSE, int B, int Hq, int Hkv, int Sq,
+                           int Sk, int D, float scale, int causal, int kv_valid_len, const int64_t* strides, void* stream) {
+    if (!strides) return fail(MI355_ERR_BAD_ARGUMENT, "mi355_fmha_fwd_strided: null strides");
+    const mi355::FmhaStrides sd = {(long)strides[0], (long)strides[1], (long)strides[2],  (long)strides[3],
+                                   (long)strides[4], (long)strides[5], (long)strides[6],  (long)strides[7],
+                                   (long)strides[8], (long)strides[9], (long)strides[10], (long)strides[11]};
+    return fmha_checked("mi355_fmha_fwd_strided", Q, K, V, O, LSE, B, Hq, Hkv, Sq, Sk, D, scale, causal, kv_valid_len, sd,
+                        stream);
 }
 
 const char* mi355_last_error(void) { return g_err; }

@@ -52,7 +52,8 @@ __device__ __forceinline__ float other_half(float x) {
 // units = B * Hkv * splits, unit u = (b * Hkv + hkv) * splits + s covers key tiles [s * tiles_per_split, ...)
 __global__ __launch_bounds__(dec::WAVES * 64) void fmha_decode_split_kernel(
     const half_t* __restrict__ Q, const half_t* __restrict__ K, const half_t* __restrict__ V, float* __restrict__ part, int B,
-    int Hq, int Hkv, int Sq, int Sk, float scale_log2, int causal, int kv_valid, int splits, int tiles_per_split, int units) {
+    int Hq, int Hkv, int Sq, int Sk, float scale_log2, int causal, int kv_valid, int splits, int tiles_per_split, int units, long q_batch,
+    long q_head, long q_rstride, long k_batch, long k_head, long k_rstride, long v_batch, long v_head, long v_rstride) {
     using namespace dec;
     extern __shared__ __attribute__((aligned(1024))) char smem_raw[];
     const int lane = threadIdx.x & 63;
@@ -75,14 +76,14 @@ __global__ __launch_bounds__(dec::WAVES * 64) void fmha_decode_split_kernel(
     const int col = min(l32, ncols - 1);
     const int hq = hkv * group + col / Sq;
     const int qi = col % Sq;
-    const half_t* qp = Q + (((long)b * Hq + hq) * Sq + qi) * D + 8 * h;
+    const half_t* qp = Q + b * q_batch + hq * q_head + qi * q_rstride + 8 * h;
     half8 qf[8];
 #pragma unroll
     for (int ks = 0; ks < 8; ++ks) qf[ks] = *(const half8*)(qp + ks * 16);
     const int lim = causal ? min(kv_valid - 1, qi + shift) : kv_valid - 1;  // last visible key of this column
 
-    const half_t* Kh = K + ((long)b * Hkv + hkv) * (long)Sk * D;
-    const half_t* Vh = V + ((long)b * Hkv + hkv) * (long)Sk * D;
+    const half_t* Kh = K + b * k_batch + hkv * k_head;
+    const half_t* Vh = V + b * v_batch + hkv * v_head;
 
     const int tiles = (kv_valid + TK - 1) / TK;
     const int t_begin = s_idx * tiles_per_split;
@@ -96,13 +97,13 @@ __global__ __launch_bounds__(dec::WAVES * 64) void fmha_decode_split_kernel(
         for (int i = 0; i < 8; ++i) {
             int row = 4 * i + c_row;
             int grow = min(tile * TK + row, kv_valid - 1);
-            copy16_global_to_lds(Kh + (long)grow * D + ((lane & 15) ^ swz_k(row)) * 8, st + i * 1024);
+            copy16_global_to_lds(Kh + grow * k_rstride + ((lane & 15) ^ swz_k(row)) * 8, st + i * 1024);
         }
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
             int row = 4 * i + c_row;
             int grow = min(tile * TK + row, kv_valid - 1);
-            copy16_global_to_lds(Vh + (long)grow * D + ((lane & 15) ^ swz_v(row)) * 8, st + TILE_BYTES + i * 1024);
+            copy16_global_to_lds(Vh + grow * v_rstride + ((lane & 15) ^ swz_v(row)) * 8, st + TILE_BYTES + i * 1024);
         }
     };
 
@@ -217,7 +218,8 @@ constexpr int kMaxSplits = 512;
 
 __global__ __launch_bounds__(128) void fmha_decode_merge_kernel(const float* __restrict__ part, half_t* __restrict__ O,
                                                                 float* __restrict__ LSE, int Hq, int Hkv, int Sq,
-                                                                float scale_log2, int splits) {
+                                                                float scale_log2, int splits, long o_batch, long o_head,
+                                                                long o_row) {
     using namespace dec;
     __shared__ float w_sh[kMaxSplits];
     __shared__ float red[128];
@@ -262,7 +264,7 @@ __global__ __launch_bounds__(128) void fmha_decode_merge_kernel(const float* __r
     float acc = 0.f;
 #pragma unroll 8
     for (int s = 0; s < splits; ++s) acc += w_sh[s] * base[s * unit_stride + tid];
-    O[(long)row * D + tid] = (half_t)((l > 0.f) ? acc / l : 0.f);
+    O[b * o_batch + hq * o_head + qi * o_row + tid] = (half_t)((l > 0.f) ? acc / l : 0.f);
     if (LSE != nullptr && tid == 0)
         LSE[row] = (l > 0.f) ? (m * scale_log2 + __builtin_log2f(l)) * 0.69314718055994531f : -INFINITY;
 }
@@ -307,7 +309,8 @@ static hipError_t decode_workspace(size_t bytes, hipStream_t stream, float** out
 }
 
 hipError_t fmha_decode_dispatch(const half_t* Q, const half_t* K, const half_t* V, half_t* O, float* LSE, int B, int Hq,
-                                int Hkv, int Sq, int Sk, float scale, int causal, int kv_valid, hipStream_t stream) {
+                                int Hkv, int Sq, int Sk, float scale, int causal, int kv_valid, const FmhaStrides& sd,
+                                hipStream_t stream) {
     using namespace dec;
     static bool attr_set = false;
     if (!attr_set) {
@@ -336,11 +339,12 @@ hipError_t fmha_decode_dispatch(const half_t* Q, const half_t* K, const half_t* 
     const float scale_log2 = scale * 1.4426950408889634f;
     const unsigned blocks = (unsigned)((units + WAVES - 1) / WAVES);
     fmha_decode_split_kernel<<<dim3(blocks), dim3(WAVES * 64), LDS_BYTES, stream>>>(
-        Q, K, V, part, B, Hq, Hkv, Sq, Sk, scale_log2, causal, kv_valid, splits, tiles_per_split, (int)units);
+        Q, K, V, part, B, Hq, Hkv, Sq, Sk, scale_log2, causal, kv_valid, splits, tiles_per_split, (int)units, sd.q_batch,
+        sd.q_head, sd.q_row, sd.k_batch, sd.k_head, sd.k_row, sd.v_batch, sd.v_head, sd.v_row);
     e = hipGetLastError();
     if (e != hipSuccess) return e;
-    fmha_decode_merge_kernel<<<dim3((unsigned)((long)B * Hq * Sq)), dim3(128), 0, stream>>>(part, O, LSE, Hq, Hkv, Sq,
-                                                                                          scale_log2, splits);
+    fmha_decode_merge_kernel<<<dim3((unsigned)((long)B * Hq * Sq)), dim3(128), 0, stream>>>(
+        part, O, LSE, Hq, Hkv, Sq, scale_log2, splits, sd.o_batch, sd.o_head, sd.o_row);
     return hipGetLastError();
 }
 

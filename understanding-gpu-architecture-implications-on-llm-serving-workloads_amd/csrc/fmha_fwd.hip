@@ -73,7 +73,7 @@ __global__ __launch_bounds__(NWAVES * 64, (NQ == 1 ? 2 : 1)) void fmha_fwd_kerne
                                                                const half_t* __restrict__ V, half_t* __restrict__ O,
                                                                float* __restrict__ LSE, int B, int Hq, int Hkv, int Sq,
                                                                int Sk, float scale_log2, int causal, int kv_valid,
-                                                               int q_tiles) {
+                                                               int q_tiles, FmhaStrides sd) {
     using namespace fmha;
     constexpr int BM = NWAVES * NQ * 32;
     constexpr int COPIES = (BN * ROW_BYTES / 1024) / NWAVES;  // wave-instructions per tile per wave
@@ -97,10 +97,10 @@ __global__ __launch_bounds__(NWAVES * 64, (NQ == 1 ? 2 : 1)) void fmha_fwd_kerne
     const int q_wave0 = q_block0 + wave * NQ * 32;  // first query row of this wave
     const int shift = Sk - Sq;
 
-    const half_t* Qh = Q + ((long)b * Hq + hq) * (long)Sq * D;
-    const half_t* Kh = K + ((long)b * Hkv + hkv) * (long)Sk * D;
-    const half_t* Vh = V + ((long)b * Hkv + hkv) * (long)Sk * D;
-    half_t* Oh = O + ((long)b * Hq + hq) * (long)Sq * D;
+    const half_t* Qh = Q + b * sd.q_batch + hq * sd.q_head;
+    const half_t* Kh = K + b * sd.k_batch + hkv * sd.k_head;
+    const half_t* Vh = V + b * sd.v_batch + hkv * sd.v_head;
+    half_t* Oh = O + b * sd.o_batch + hq * sd.o_head;
 
     // ---- number of key tiles this workgroup has to visit ----------------------------------------------
     int k_end = kv_valid;
@@ -115,7 +115,7 @@ __global__ __launch_bounds__(NWAVES * 64, (NQ == 1 ? 2 : 1)) void fmha_fwd_kerne
 #pragma unroll
     for (int qb = 0; qb < NQ; ++qb) {
         int qrow = min(q_wave0 + qb * 32 + l32, Sq - 1);
-        const half_t* qp = Qh + (long)qrow * D + 8 * h;
+        const half_t* qp = Qh + qrow * sd.q_row + 8 * h;
 #pragma unroll
         for (int ks = 0; ks < 8; ++ks) qf[qb][ks] = *(const half8*)(qp + ks * 16);
     }
@@ -137,12 +137,12 @@ __global__ __launch_bounds__(NWAVES * 64, (NQ == 1 ? 2 : 1)) void fmha_fwd_kerne
 #pragma unroll
         for (int i = 0; i < COPIES; ++i) {
             int krow = min(tile * BN + copy_row[i], kv_valid - 1);
-            copy16_global_to_lds(Kh + (long)krow * D + copy_kcol[i], sk + (i * NWAVES + wave) * 1024);
+            copy16_global_to_lds(Kh + krow * sd.k_row + copy_kcol[i], sk + (i * NWAVES + wave) * 1024);
         }
 #pragma unroll
         for (int i = 0; i < COPIES; ++i) {
             int krow = min(tile * BN + copy_row[i], kv_valid - 1);
-            copy16_global_to_lds(Vh + (long)krow * D + copy_vcol[i], sv + (i * NWAVES + wave) * 1024);
+            copy16_global_to_lds(Vh + krow * sd.v_row + copy_vcol[i], sv + (i * NWAVES + wave) * 1024);
         }
     };
 
@@ -281,7 +281,7 @@ __global__ __launch_bounds__(NWAVES * 64, (NQ == 1 ? 2 : 1)) void fmha_fwd_kerne
         float inv = (l_tot > 0.f) ? 1.f / l_tot : 0.f;
         int qi = q_wave0 + qb * 32 + l32;
         if (qi < Sq) {
-            half_t* orow = Oh + (long)qi * D + 4 * h;
+            half_t* orow = Oh + qi * sd.o_row + 4 * h;
 #pragma unroll
             for (int db = 0; db < 4; ++db)
 #pragma unroll
@@ -316,7 +316,7 @@ __global__ __launch_bounds__(512, 2) void fmha_fwd_pingpong_kernel(const half_t*
                                                                    const half_t* __restrict__ V, half_t* __restrict__ O,
                                                                    float* __restrict__ LSE, int B, int Hq, int Hkv, int Sq,
                                                                    int Sk, float scale_log2, int causal, int kv_valid,
-                                                                   int q_tiles) {
+                                                                   int q_tiles, FmhaStrides sd) {
     using namespace fmha;
     constexpr int NWAVES = 8;
     constexpr int BM = NWAVES * 32;
@@ -342,10 +342,10 @@ __global__ __launch_bounds__(512, 2) void fmha_fwd_pingpong_kernel(const half_t*
     const int q_wave0 = q_block0 + wave * 32;
     const int shift = Sk - Sq;
 
-    const half_t* Qh = Q + ((long)b * Hq + hq) * (long)Sq * D;
-    const half_t* Kh = K + ((long)b * Hkv + hkv) * (long)Sk * D;
-    const half_t* Vh = V + ((long)b * Hkv + hkv) * (long)Sk * D;
-    half_t* Oh = O + ((long)b * Hq + hq) * (long)Sq * D;
+    const half_t* Qh = Q + b * sd.q_batch + hq * sd.q_head;
+    const half_t* Kh = K + b * sd.k_batch + hkv * sd.k_head;
+    const half_t* Vh = V + b * sd.v_batch + hkv * sd.v_head;
+    half_t* Oh = O + b * sd.o_batch + hq * sd.o_head;
 
     int k_end = kv_valid;
     if (causal) k_end = min(k_end, min(q_block0 + BM, Sq) - 1 + shift + 1);
@@ -354,7 +354,7 @@ __global__ __launch_bounds__(512, 2) void fmha_fwd_pingpong_kernel(const half_t*
     half8 qf[8];
     {
         int qrow = min(q_wave0 + l32, Sq - 1);
-        const half_t* qp = Qh + (long)qrow * D + 8 * h;
+        const half_t* qp = Qh + qrow * sd.q_row + 8 * h;
 #pragma unroll
         for (int ks = 0; ks < 8; ++ks) qf[ks] = *(const half8*)(qp + ks * 16);
     }
@@ -372,14 +372,14 @@ __global__ __launch_bounds__(512, 2) void fmha_fwd_pingpong_kernel(const half_t*
 #pragma unroll
         for (int i = 0; i < COPIES; ++i) {
             int krow = min(tile * BN + copy_row[i], kv_valid - 1);
-            copy16_global_to_lds(Kh + (long)krow * D + copy_kcol[i], kbuf + (tile & 1) * TILE_BYTES + (i * NWAVES + wave) * 1024);
+            copy16_global_to_lds(Kh + krow * sd.k_row + copy_kcol[i], kbuf + (tile & 1) * TILE_BYTES + (i * NWAVES + wave) * 1024);
         }
     };
     auto issue_v = [&](int tile) {
 #pragma unroll
         for (int i = 0; i < COPIES; ++i) {
             int krow = min(tile * BN + copy_row[i], kv_valid - 1);
-            copy16_global_to_lds(Vh + (long)krow * D + copy_vcol[i], vbuf + (tile & 1) * TILE_BYTES + (i * NWAVES + wave) * 1024);
+            copy16_global_to_lds(Vh + krow * sd.v_row + copy_vcol[i], vbuf + (tile & 1) * TILE_BYTES + (i * NWAVES + wave) * 1024);
         }
     };
 
@@ -594,7 +594,7 @@ __global__ __launch_bounds__(512, 2) void fmha_fwd_pingpong_kernel(const half_t*
     float inv = (l_tot > 0.f) ? 1.f / l_tot : 0.f;
     int qi = q_wave0 + l32;
     if (qi < Sq) {
-        half_t* orow = Oh + (long)qi * D + 4 * h;
+        half_t* orow = Oh + qi * sd.o_row + 4 * h;
 #pragma unroll
         for (int db = 0; db < 4; ++db)
 #pragma unroll
@@ -612,7 +612,8 @@ __global__ __launch_bounds__(512, 2) void fmha_fwd_pingpong_kernel(const half_t*
 }
 
 static hipError_t launch_fmha_pingpong(const half_t* Q, const half_t* K, const half_t* V, half_t* O, float* LSE, int B, int Hq,
-                                       int Hkv, int Sq, int Sk, float scale, int causal, int kv_valid, hipStream_t stream) {
+                                       int Hkv, int Sq, int Sk, float scale, int causal, int kv_valid, const FmhaStrides& sd,
+                                       hipStream_t stream) {
     constexpr int BM = 256;
     constexpr int LDS = 4 * fmha::TILE_BYTES;
     static bool attr_set = false;
@@ -627,13 +628,14 @@ static hipError_t launch_fmha_pingpong(const half_t* Q, const half_t* K, const h
     if (blocks > 0x7fffffffL) return hipErrorInvalidValue;
     const float scale_log2 = scale * 1.4426950408889634f;
     fmha_fwd_pingpong_kernel<<<dim3((unsigned)blocks), dim3(512), LDS, stream>>>(Q, K, V, O, LSE, B, Hq, Hkv, Sq, Sk, scale_log2,
-                                                                                causal, kv_valid, q_tiles);
+                                                                                causal, kv_valid, q_tiles, sd);
     return hipGetLastError();
 }
 
 template <int NQ, int NWAVES>
 static hipError_t launch_fmha(const half_t* Q, const half_t* K, const half_t* V, half_t* O, float* LSE, int B, int Hq,
-                              int Hkv, int Sq, int Sk, float scale, int causal, int kv_valid, hipStream_t stream) {
+                              int Hkv, int Sq, int Sk, float scale, int causal, int kv_valid, const FmhaStrides& sd,
+                                       hipStream_t stream) {
     constexpr int BM = NWAVES * NQ * 32;
     constexpr int LDS = fmha::STAGE_BYTES * fmha::NSTAGE;
     auto kern = fmha_fwd_kernel<NQ, NWAVES>;
@@ -649,30 +651,31 @@ static hipError_t launch_fmha(const half_t* Q, const half_t* K, const half_t* V,
     if (blocks > 0x7fffffffL) return hipErrorInvalidValue;
     const float scale_log2 = scale * 1.4426950408889634f;
     kern<<<dim3((unsigned)blocks), dim3(NWAVES * 64), LDS, stream>>>(Q, K, V, O, LSE, B, Hq, Hkv, Sq, Sk, scale_log2,
-                                                                    causal, kv_valid, q_tiles);
+                                                                    causal, kv_valid, q_tiles, sd);
     return hipGetLastError();
 }
 
 int g_fmha_variant = 0;  // tuning hook: 0 = heuristic, 1 = 4 waves x 32 queries, 2 = 8 waves x 32 queries, 3 = ping-pong
 
 hipError_t fmha_fwd_dispatch(const void* Q, const void* K, const void* V, void* O, float* LSE, int B, int Hq, int Hkv,
-                             int Sq, int Sk, float scale, int causal, int kv_valid_len, hipStream_t stream) {
+                             int Sq, int Sk, float scale, int causal, int kv_valid_len, const FmhaStrides& sd,
+                             hipStream_t stream) {
     const half_t* q = static_cast<const half_t*>(Q);
     const half_t* k = static_cast<const half_t*>(K);
     const half_t* v = static_cast<const half_t*>(V);
     half_t* o = static_cast<half_t*>(O);
     int variant = g_fmha_variant;
     if ((variant == 0 || variant == 4) && fmha_decode_applicable(B, Hq, Hkv, Sq, Sk, kv_valid_len))
-        return fmha_decode_dispatch(q, k, v, o, LSE, B, Hq, Hkv, Sq, Sk, scale, causal, kv_valid_len, stream);
+        return fmha_decode_dispatch(q, k, v, o, LSE, B, Hq, Hkv, Sq, Sk, scale, causal, kv_valid_len, sd, stream);
     if (variant == 0 || variant == 4) {
         // 256-query ping-pong workgroups once there are enough of them to fill the 256 CUs, otherwise 128-query ones
         const long wg256 = (long)((Sq + 255) / 256) * Hq * B;
         variant = (wg256 >= 256) ? 3 : 1;
     }
     switch (variant) {
-        case 2: return launch_fmha<1, 8>(q, k, v, o, LSE, B, Hq, Hkv, Sq, Sk, scale, causal, kv_valid_len, stream);
-        case 3: return launch_fmha_pingpong(q, k, v, o, LSE, B, Hq, Hkv, Sq, Sk, scale, causal, kv_valid_len, stream);
-        default: return launch_fmha<1, 4>(q, k, v, o, LSE, B, Hq, Hkv, Sq, Sk, scale, causal, kv_valid_len, stream);
+        case 2: return launch_fmha<1, 8>(q, k, v, o, LSE, B, Hq, Hkv, Sq, Sk, scale, causal, kv_valid_len, sd, stream);
+        case 3: return launch_fmha_pingpong(q, k, v, o, LSE, B, Hq, Hkv, Sq, Sk, scale, causal, kv_valid_len, sd, stream);
+        default: return launch_fmha<1, 4>(q, k, v, o, LSE, B, Hq, Hkv, Sq, Sk, scale, causal, kv_valid_len, sd, stream);
     }
 }
 

@@ -29,6 +29,17 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {}
 
 namespace {
 
+// A [B, H, S, D] view the kernels can read in place: contiguous last dimension, every other stride a non-negative
+// multiple of 8 elements, 16-byte aligned base. This covers `x.view(B, S, H, D).transpose(1, 2)` and slices of a fused
+// QKV projection, the forms the reference's in-model caller produces (benchmarks/flashattn-cuda/modeling_llama.py:658-660)
+// and which kernels/fmha/pkg/fmha_unified/ops.py:23-25 copies into contiguous tensors first.
+bool readable_in_place(const at::Tensor& t) {
+    if (t.stride(3) != 1 || reinterpret_cast<uintptr_t>(t.data_ptr()) % 16 != 0) return false;
+    for (int i = 0; i < 3; ++i)
+        if (t.stride(i) < 0 || t.stride(i) % 8 != 0) return false;
+    return true;
+}
+
 std::tuple<at::Tensor, at::Tensor> run_fmha(const at::Tensor& q, const at::Tensor& k, const at::Tensor& v, bool causal,
                                             bool is_decode, int64_t decode_length, bool want_lse) {
     const char* name = "finefmha";
@@ -52,8 +63,12 @@ std::tuple<at::Tensor, at::Tensor> run_fmha(const at::Tensor& q, const at::Tenso
 
     // torch on ROCm presents HIP devices under the "cuda" device type; these are its guard and stream for them
     const c10::hip::HIPGuardMasqueradingAsCUDA guard(q.device());
-    at::Tensor qc = q.contiguous(), kc = k.contiguous(), vc = v.contiguous();
-    at::Tensor o = at::empty(qc.sizes(), qc.options());
+    at::Tensor qc = readable_in_place(q) ? q : q.contiguous();
+    at::Tensor kc = readable_in_place(k) ? k : k.contiguous();
+    at::Tensor vc = readable_in_place(v) ? v : v.contiguous();
+    // The output takes q's memory layout when q is a dense permuted view (so `out.transpose(1, 2).contiguous()` in the
+    // caller costs nothing for a [B, S, H, D] projection); otherwise it is a contiguous [B, H, S, D] tensor.
+    at::Tensor o = qc.is_non_overlapping_and_dense() ? at::empty_like(qc) : at::empty(qc.sizes(), qc.options());
     at::Tensor lse;
     float* lse_ptr = nullptr;
     if (want_lse) {
@@ -62,8 +77,11 @@ std::tuple<at::Tensor, at::Tensor> run_fmha(const at::Tensor& q, const at::Tenso
     }
     const float scale = 1.0f / std::sqrt(static_cast<float>(D));  // fmha_2_amd.cpp:320
     hipStream_t stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream();
-    int rc = mi355_fmha_fwd(qc.data_ptr(), kc.data_ptr(), vc.data_ptr(), o.data_ptr(), lse_ptr, (int)B, (int)Hq, (int)Hkv,
-                            (int)Sq, (int)Sk, (int)D, scale, causal ? 1 : 0, (int)decode_length, stream);
+    const int64_t strides[12] = {qc.stride(0), qc.stride(1), qc.stride(2), kc.stride(0), kc.stride(1), kc.stride(2),
+                                 vc.stride(0), vc.stride(1), vc.stride(2), o.stride(0),  o.stride(1),  o.stride(2)};
+    int rc = mi355_fmha_fwd_strided(qc.data_ptr(), kc.data_ptr(), vc.data_ptr(), o.data_ptr(), lse_ptr, (int)B, (int)Hq,
+                                    (int)Hkv, (int)Sq, (int)Sk, (int)D, scale, causal ? 1 : 0, (int)decode_length, strides,
+                                    stream);
     TORCH_CHECK(rc == 0, name, ": ", mi355_last_error(), " (code ", rc, ")");
     return {o, lse};
 }

@@ -13,7 +13,7 @@ LIB_PATH = os.path.join(_HERE, "libmi355_serving.so")
 GEMM_NN, GEMM_NT, GEMM_TN = 0, 1, 2
 LAYOUTS = {"NN": GEMM_NN, "NT": GEMM_NT, "TN": GEMM_TN}
 
-EXPORTED_SYMBOLS = ("mi355_hgemm", "mi355_fmha_fwd", "mi355_last_error", "mi355_serving_version",
+EXPORTED_SYMBOLS = ("mi355_hgemm", "mi355_fmha_fwd", "mi355_fmha_fwd_strided", "mi355_last_error", "mi355_serving_version",
                     "mi355_debug_set_gemm_variant", "mi355_debug_set_fmha_variant")
 
 _lib = None
@@ -40,6 +40,9 @@ def load():
     lib.mi355_hgemm.restype = i32
     lib.mi355_fmha_fwd.argtypes = [vp, vp, vp, vp, vp, i32, i32, i32, i32, i32, i32, f32, i32, i32, vp]
     lib.mi355_fmha_fwd.restype = i32
+    lib.mi355_fmha_fwd_strided.argtypes = [vp, vp, vp, vp, vp, i32, i32, i32, i32, i32, i32, f32, i32, i32,
+                                           ctypes.POINTER(i64), vp]
+    lib.mi355_fmha_fwd_strided.restype = i32
     lib.mi355_last_error.argtypes = []
     lib.mi355_last_error.restype = ctypes.c_char_p
     lib.mi355_serving_version.argtypes = []
@@ -104,19 +107,41 @@ def hgemm(a, b, layout="NN", out=None):
     return out
 
 
-def fmha_fwd(q, k, v, causal=False, kv_valid_len=None, scale=None, return_lse=True):
-    """Attention forward through the C ABI on torch's current stream. Returns (O, LSE) or O."""
+def fmha_fwd_strided_raw(q_ptr, k_ptr, v_ptr, o_ptr, lse_ptr, B, Hq, Hkv, Sq, Sk, D, scale, causal, kv_valid_len, strides,
+                         stream=0):
+    """Direct call of mi355_fmha_fwd_strided; `strides` = 12 element strides (q, k, v, o) x (batch, head, row)."""
+    arr = (ctypes.c_int64 * 12)(*[int(x) for x in strides])
+    _check(load().mi355_fmha_fwd_strided(q_ptr, k_ptr, v_ptr, o_ptr, lse_ptr, B, Hq, Hkv, Sq, Sk, D, scale, causal,
+                                         kv_valid_len, arr, stream))
+
+
+def _bhs_strides(t):
+    return [t.stride(0), t.stride(1), t.stride(2)]
+
+
+def fmha_fwd(q, k, v, causal=False, kv_valid_len=None, scale=None, return_lse=True, out=None):
+    """Attention forward through the C ABI on torch's current stream. Returns (O, LSE) or O.
+
+    q, k, v (and `out`, if given) are [B, H, S, D] fp16 GPU tensors or views with a contiguous last dimension, e.g.
+    `x.view(B, S, H, D).transpose(1, 2)`; contiguous tensors take mi355_fmha_fwd, views mi355_fmha_fwd_strided.
+    """
     import torch
-    assert q.dtype == torch.float16 and q.is_cuda and q.is_contiguous() and k.is_contiguous() and v.is_contiguous()
+    assert q.dtype == torch.float16 and q.is_cuda
     B, Hq, Sq, D = q.shape
     _, Hkv, Sk, _ = k.shape
     if scale is None:
         scale = 1.0 / (D ** 0.5)
     if kv_valid_len is None:
         kv_valid_len = Sk
-    o = torch.empty_like(q)
+    o = torch.empty_like(q) if out is None else out
     lse = torch.empty((B, Hq, Sq), dtype=torch.float32, device=q.device) if return_lse else None
     stream = torch.cuda.current_stream(q.device).cuda_stream
-    fmha_fwd_raw(_ptr(q), _ptr(k), _ptr(v), _ptr(o), _ptr(lse), B, Hq, Hkv, Sq, Sk, D, float(scale), int(bool(causal)),
-                 int(kv_valid_len), stream)
+    if all(t.is_contiguous() for t in (q, k, v, o)):
+        fmha_fwd_raw(_ptr(q), _ptr(k), _ptr(v), _ptr(o), _ptr(lse), B, Hq, Hkv, Sq, Sk, D, float(scale), int(bool(causal)),
+                     int(kv_valid_len), stream)
+    else:
+        assert all(t.stride(3) == 1 for t in (q, k, v, o)), "the last dimension must be contiguous"
+        strides = _bhs_strides(q) + _bhs_strides(k) + _bhs_strides(v) + _bhs_strides(o)
+        fmha_fwd_strided_raw(_ptr(q), _ptr(k), _ptr(v), _ptr(o), _ptr(lse), B, Hq, Hkv, Sq, Sk, D, float(scale),
+                             int(bool(causal)), int(kv_valid_len), strides, stream)
     return (o, lse) if return_lse else o
