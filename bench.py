@@ -232,6 +232,36 @@ def main():
         other["L5_llama3_8b_layer_s8192"] = {"stages": st, "kernel_ms_total": tot_ms, "tflops_total": tot_fl / tot_ms / 1e9,
                                              "note": "GEMM and attention stages only; reshapes and SiLU*up run in torch and are not timed; no RoPE/norm/residual"}
 
+        # the same layer as the in-model adapter runs it: nn.Linear-layout weights, norms, RoPE, residuals, no layout copies
+        del x5, wqkv, wo, wgu, wd, qkv5, q5, k5, v5, o5, a5, op5, gu5, act5, dn5
+        torch.cuda.empty_cache()
+        from llama_layer import FineKVCache, FineLlamaDecoderLayer
+        gw = lambda shape, seed: so.randn_fp16(shape, seed, 0.02).to(dev)
+        wl = dict(q=gw((4096, H5), 11), k=gw((1024, H5), 12), v=gw((1024, H5), 13), o=gw((H5, 4096), 14), gate=gw((F5, H5), 15),
+                  up=gw((F5, H5), 16), down=gw((H5, F5), 17), ln1=torch.ones(H5, dtype=torch.float16, device=dev),
+                  ln2=torch.ones(H5, dtype=torch.float16, device=dev))
+        layer = FineLlamaDecoderLayer(wl, 32, 8, max_positions=S5 + 64)
+        xl = so.randn_fp16((1, S5, H5), 18).to(dev)
+        ms_l = time_launches(lambda: layer(xl), 5, 2)
+        other["L5_decoder_layer_prefill_s8192"] = {
+            "ms": ms_l, "tflops": tot_fl / ms_l / 1e9,
+            "note": "whole FineLlamaDecoderLayer.forward (12 launches: norms, fused QKV GEMM, RoPE, attention on strided operands, "
+                    "O projection, gate/up GEMM, SiLU*up, down GEMM, residual adds), flops of the GEMMs and attention only"}
+        Bd = 8
+        cache = FineKVCache(Bd, S5 + 64, 8, device=dev)
+        cache.k.normal_(0, 1)
+        cache.v.normal_(0, 1)
+        xd1 = so.randn_fp16((Bd, 1, H5), 19).to(dev)
+        def step():
+            cache.length = S5
+            layer(xd1, kv_cache=cache)
+        ms_s = time_launches(step, 20, 3)
+        by_s = 2.0 * (sum(t.numel() for t in (layer.w_qkv, layer.w_o, layer.w_gu, layer.w_d)) + 2 * Bd * S5 * 8 * 128)
+        other["L5_decoder_layer_generation_step_b8_past8192"] = {"ms": ms_s, "gbs": by_s / ms_s / 1e6,
+                                                                 "pct_of_hbm_peak": 100 * by_s / ms_s / 1e6 / PEAK_HBM_GBS,
+                                                                 "note": "bytes = layer weights + KV cache read once"}
+        del layer, cache, wl
+
     # ---- CPU baseline: the same step with torch fp32 on the host cores -------------------------------------------------
     cpu_baseline = None
     if not args.no_cpu_baseline:

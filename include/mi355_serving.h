@@ -93,6 +93,38 @@ int mi355_fmha_fwd_strided(const void* Q, const void* K, const void* V, void* O,
                            int Sq, int Sk, int D, float scale, int causal, int kv_valid_len, const int64_t* strides,
                            void* stream);
 
+/*
+ * Layer glue between the GEMMs and the attention of a Llama decoder layer: memory-bound, fp16 in/out, fp32 arithmetic,
+ * one rounding. They replace the separate PyTorch elementwise kernels of the reference's in-model path
+ * (benchmarks/flashattn-cuda/modeling_llama.py). All pointers 16-byte aligned, all strides in elements and multiples of 8.
+ *
+ * mi355_rmsnorm: out[r] = weight * h[r] * rsqrt(mean(h[r]^2) + eps) over `hidden` columns   (LlamaRMSNorm.forward,
+ *   modeling_llama.py:95-100). residual == NULL (then residual_out == NULL too): h = x. Otherwise h = fp16(residual + x), also
+ *   written to residual_out (the `hidden_states = residual + hidden_states` that precedes each norm,
+ *   modeling_llama.py:776-779); residual_out may be residual itself, and out may alias x.
+ */
+int mi355_rmsnorm(const void* x, const void* residual, void* residual_out, const void* weight, void* out, int64_t rows,
+                  int hidden, int64_t ldx, int64_t ldr, int64_t ldro, int64_t ldo, float eps, void* stream);
+
+/*
+ * mi355_rope: rotary position embedding of `heads` consecutive 128-wide heads of every token (rotate_half convention,
+ *   modeling_llama.py:164-168,193-194): for i < 64, with c = cos_table[p][i], s = sin_table[p][i], p = positions[b*S + t]:
+ *     out[i] = x[i] c - x[i+64] s,   out[i+64] = x[i+64] c + x[i] s.
+ *   Token (b, t) lives at x + b*x_batch + t*x_row (+ head*128), likewise for out, so q and k can be rotated inside a fused
+ *   QKV projection (out == x) or k written straight into a KV cache. cos_table / sin_table: [n_positions][64] fp32, the
+ *   first half of what LlamaRotaryEmbedding.forward builds (modeling_llama.py:119-132); positions outside
+ *   [0, n_positions) are clamped.
+ */
+int mi355_rope(const void* x, void* out, int B, int S, int heads, int D, int64_t x_batch, int64_t x_row, int64_t out_batch,
+               int64_t out_row, const float* cos_table, const float* sin_table, const int32_t* positions, int n_positions,
+               void* stream);
+
+/*
+ * mi355_silu_mul: out[r][j] = silu(g[r][j]) * u[r][j] with g = gate_up[r][0 .. inter), u = gate_up[r][inter .. 2 inter)
+ *   (`act_fn(gate_proj(x)) * up_proj(x)`, modeling_llama.py:230, for gate and up computed by one GEMM).
+ */
+int mi355_silu_mul(const void* gate_up, void* out, int64_t rows, int inter, int64_t ld_in, int64_t ld_out, void* stream);
+
 /* Thread-local text for the last non-zero return of this thread ("" if none). */
 const char* mi355_last_error(void);
 

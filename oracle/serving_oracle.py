@@ -24,6 +24,16 @@ oracle states those results directly in fp32 (torch) and, for small inputs, agai
   llama_layer_ref     the Llama-3-8B-shaped prefill chain of the benchmark configuration (QKV GEMM -> causal GQA
                       attention -> O projection -> gate/up GEMM -> SiLU(gate)*up -> down GEMM), fp32.
 
+  rmsnorm_ref, rope_tables, rope_ref, silu_mul_ref, llama_decoder_layer_ref
+                      the glue of the reference's in-model path in fp32: LlamaRMSNorm.forward
+                      (benchmarks/flashattn-cuda/modeling_llama.py:95-100), LlamaRotaryEmbedding (:113,119-132),
+                      rotate_half / apply_rotary_pos_emb (:164-168,193-194), act_fn(gate) * up (:230) and the
+                      decoder layer that strings them together (LlamaSdpaAttention.forward :652-704 with a KV
+                      cache, LlamaDecoderLayer.forward :755-781). Pinned by closed forms (constant rows, unit
+                      weights, position 0, norm preservation, the relative-position property, d = 2 rotation by
+                      hand, silu(0) / large-argument limits) and against the Llama layer of the installed
+                      `transformers` package as an independent second implementation.
+
 Reference-specific numerical behaviour (fp16 accumulation in finegemm_0..11, fp16 softmax statistics in
 finefmha_0..3) is deliberately NOT restated: the parity target is the fp32 result.
 
@@ -252,6 +262,90 @@ def llama_layer_ref(x, w_qkv, w_o, w_gu, w_d, n_q=32, n_kv=8, d=128, stage_input
     out["act"] = act
     out["down"] = f(si.get("down_in", act.half())) @ f(w_d)
     return out
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# Layer glue of the in-model path (benchmarks/flashattn-cuda/modeling_llama.py)
+# ---------------------------------------------------------------------------------------------------------------
+def _f32(t):
+    return t.detach().to("cpu", torch.float32)
+
+
+def rmsnorm_ref(x, weight, eps=1e-5, residual=None, round_residual=True):
+    """modeling_llama.py:95-100 in fp32: weight * h * rsqrt(mean(h^2) + eps). With `residual`, h = fp16(residual + x)
+    (the fp16 add of :776 / :781; round_residual=False keeps the sum in fp32) and the new residual h is returned too.
+    Returns fp32 (out, h)."""
+    h = _f32(x)
+    if residual is not None:
+        h = h + _f32(residual)
+        if round_residual:
+            h = h.to(torch.float16).float()
+    var = h.pow(2).mean(-1, keepdim=True)
+    return _f32(weight) * (h * torch.rsqrt(var + eps)), h
+
+
+def rope_tables(n_positions, dim=128, base=10000.0):
+    """cos / sin [n_positions, dim/2] fp32: inv_freq = base^(-2i/dim) (:113), angle = position * inv_freq (:128-131).
+    The reference concatenates the table with itself to width dim (:129); both halves are equal, one is kept."""
+    inv_freq = 1.0 / (base ** (torch.arange(0, dim, 2, dtype=torch.int64).float() / dim))
+    ang = torch.arange(n_positions, dtype=torch.float32)[:, None] * inv_freq[None, :]
+    return ang.cos(), ang.sin()
+
+
+def rope_ref(x, cos, sin, positions):
+    """x [B, H, S, D], positions [B, S] -> x * cos + rotate_half(x) * sin in fp32 (:164-168, :193-194)."""
+    x = _f32(x)
+    half = x.shape[-1] // 2
+    c = cos[positions.long()][:, None]          # [B, 1, S, D/2]
+    s_ = sin[positions.long()][:, None]
+    c = torch.cat((c, c), -1)
+    s_ = torch.cat((s_, s_), -1)
+    rot = torch.cat((-x[..., half:], x[..., :half]), -1)
+    return x * c + rot * s_
+
+
+def silu_mul_ref(gate_up):
+    """[rows, 2F] -> silu(gate) * up in fp32 (:230 with gate and up side by side)."""
+    g = _f32(gate_up)
+    F = g.shape[-1] // 2
+    return torch.nn.functional.silu(g[..., :F]) * g[..., F:]
+
+
+def llama_decoder_layer_ref(x, w, positions, n_q, n_kv, eps=1e-5, rope_base=10000.0, past_k=None, past_v=None,
+                            round_stages=True):
+    """One Llama decoder layer in fp32 on the CPU. x [B, S, H]; w: dict with nn.Linear-layout ([out, in]) weights
+    'q', 'k', 'v', 'o', 'gate', 'up', 'down' and norm weights 'ln1', 'ln2'; positions [B, S]; past_k / past_v
+    [B, n_kv, P, D] (already rotated keys). Follows LlamaDecoderLayer.forward (:755-781) and
+    LlamaSdpaAttention.forward (:652-704); attention is causal with the mask aligned bottom-right (prefill: P = 0;
+    generation step: S = 1). round_stages rounds every intermediate to fp16 where an fp16 pipeline stores it, so a
+    kernel chain is compared against the same sequence of roundings. Returns (out fp32 [B,S,H], k, v) with k, v the
+    updated caches [B, n_kv, P+S, D] fp32."""
+    r = (lambda t: t.to(torch.float16).float()) if round_stages else (lambda t: t)
+    x = _f32(x)
+    B, S, H = x.shape
+    D = w["q"].shape[0] // n_q
+    h1, _ = rmsnorm_ref(x, w["ln1"], eps)
+    h1 = r(h1)
+    q = r(h1 @ _f32(w["q"]).T).view(B, S, n_q, D).transpose(1, 2)
+    k = r(h1 @ _f32(w["k"]).T).view(B, S, n_kv, D).transpose(1, 2)
+    v = r(h1 @ _f32(w["v"]).T).view(B, S, n_kv, D).transpose(1, 2)
+    n_pos = int(positions.max()) + 1
+    cos, sin = rope_tables(n_pos, D, rope_base)
+    q = r(rope_ref(q, cos, sin, positions))
+    k = r(rope_ref(k, cos, sin, positions))
+    if past_k is not None:
+        k = torch.cat((_f32(past_k), k), 2)
+        v = torch.cat((_f32(past_v), v), 2)
+    o, _ = attention_ref(q, k, v, causal=True)
+    o = r(o).transpose(1, 2).reshape(B, S, n_q * D)
+    attn = r(o @ _f32(w["o"]).T)
+    h2, res = rmsnorm_ref(attn, w["ln2"], eps, residual=x, round_residual=round_stages)
+    h2 = r(h2)
+    gu = r(torch.cat((h2 @ _f32(w["gate"]).T, h2 @ _f32(w["up"]).T), -1))
+    act = r(silu_mul_ref(gu))
+    down = r(act @ _f32(w["down"]).T)
+    out = (res + down)
+    return (r(out) if round_stages else out), k, v
 
 
 # ---------------------------------------------------------------------------------------------------------------

@@ -1,0 +1,171 @@
+"""GPU parity of the layer glue kernels (RMSNorm, fused residual add + RMSNorm, RoPE, SiLU*up) through the C ABI, and
+of the decoder layer built from them (llama_layer.FineLlamaDecoderLayer) against the CPU oracle.
+
+Tolerances (floating point, fp16 outputs of fp32 arithmetic): a glue kernel rounds once, so
+|out - ref| <= 2^-10 |ref| + 1e-6 against the fp32 oracle; the layer is compared with the oracle that rounds every
+stored intermediate to fp16 like the kernel chain does: relative Frobenius error <= 2e-3 and max |err| <= 2e-2 max|ref|."""
+import pytest
+import torch
+
+import serving_oracle as so
+
+pytestmark = pytest.mark.gpu
+
+
+def close_one_rounding(out, ref):
+    err = (out.float().cpu() - ref).abs()
+    return bool((err <= 2.0 ** -10 * ref.abs() + 1e-6).all()), float(err.max())
+
+
+@pytest.mark.parametrize("rows,hidden", [(1, 8), (7, 4096), (300, 512), (16, 8192), (5, 12288), (3, 1000)])
+def test_rmsnorm(lib, gpu, rows, hidden):
+    x = so.randn_fp16((rows, hidden), 1, 2.0)
+    w = (1 + 0.1 * so.randn_fp16((hidden,), 2).float()).half()
+    ref, _ = so.rmsnorm_ref(x, w, 1e-5)
+    out = lib.rmsnorm(x.to(gpu), w.to(gpu), 1e-5)
+    assert close_one_rounding(out, ref)[0]
+    # closed form: a constant row normalises to sign * weight
+    c = torch.full((2, hidden), -3.0, dtype=torch.float16)
+    outc = lib.rmsnorm(c.to(gpu), w.to(gpu), 0.0)
+    assert close_one_rounding(outc, -w.float().expand(2, hidden))[0]
+
+
+def test_rmsnorm_with_residual_strides_and_in_place(lib, gpu):
+    rows, hidden = 33, 1024
+    x = so.randn_fp16((rows, hidden), 3)
+    r = so.randn_fp16((rows, hidden), 4, 3.0)
+    w = so.randn_fp16((hidden,), 5)
+    ref, h_ref = so.rmsnorm_ref(x, w, 1e-6, residual=r)
+    # x is a column slice of a wider buffer; the residual is updated in place
+    wide = torch.zeros((rows, 3 * hidden), dtype=torch.float16, device=gpu)
+    wide[:, hidden:2 * hidden] = x.to(gpu)
+    rg = r.to(gpu)
+    out, h = lib.rmsnorm(wide[:, hidden:2 * hidden], w.to(gpu), 1e-6, residual=rg, residual_out=rg)
+    assert h.data_ptr() == rg.data_ptr() and torch.equal(h.cpu().float(), h_ref)   # the fp16 sum is exact
+    assert close_one_rounding(out, ref)[0]
+    # out of place: the residual input is left alone
+    rg2 = r.to(gpu)
+    out2, h2 = lib.rmsnorm(x.to(gpu), w.to(gpu), 1e-6, residual=rg2)
+    assert torch.equal(rg2.cpu(), r) and torch.equal(h2, h) and torch.equal(out2, out)
+
+
+@pytest.mark.parametrize("B,S,heads", [(1, 1, 1), (2, 37, 10), (1, 300, 40), (3, 5, 33)])
+def test_rope_in_place_and_into_a_cache(lib, gpu, B, S, heads):
+    cos, sin = so.rope_tables(512, 128, 10000.0)
+    g = torch.Generator().manual_seed(7)
+    pos = torch.randint(0, 512, (B, S), generator=g, dtype=torch.int32)
+    x = so.randn_fp16((B, S, heads + 3, 128), 8)           # the last 3 heads must stay untouched
+    ref = so.rope_ref(x[:, :, :heads].transpose(1, 2), cos, sin, pos).transpose(1, 2)
+    xg = x.to(gpu)
+    lib.rope(xg[:, :, :heads], cos.to(gpu), sin.to(gpu), pos.to(gpu))
+    assert close_one_rounding(xg[:, :, :heads], ref)[0]
+    assert torch.equal(xg[:, :, heads:].cpu(), x[:, :, heads:])
+    # position 0 is the identity, bit for bit
+    x0 = x.to(gpu)
+    lib.rope(x0[:, :, :heads], cos.to(gpu), sin.to(gpu), torch.zeros((B, S), dtype=torch.int32, device=gpu))
+    assert torch.equal(x0.cpu(), x)
+    # out of place into rows [4, 4 + S) of a longer token-major cache
+    cache = torch.zeros((B, S + 9, heads, 128), dtype=torch.float16, device=gpu)
+    src = x.to(gpu)
+    lib.rope(src[:, :, :heads], cos.to(gpu), sin.to(gpu), pos.to(gpu), out=cache[:, 4:4 + S])
+    assert torch.equal(cache[:, 4:4 + S], xg[:, :, :heads]) and torch.equal(src.cpu(), x)
+    assert float(cache[:, :4].abs().max()) == 0.0 and float(cache[:, 4 + S:].abs().max()) == 0.0
+
+
+@pytest.mark.parametrize("rows,inter", [(1, 8), (9, 14336), (70000, 16), (257, 1000)])
+def test_silu_mul(lib, gpu, rows, inter):
+    gu = so.randn_fp16((rows, 2 * inter), 9, 3.0)
+    out = lib.silu_mul(gu.to(gpu))
+    ok, worst = close_one_rounding(out, so.silu_mul_ref(gu))
+    assert ok, worst
+    edge = torch.tensor([[0.0, 30.0, -30.0, 1.0, 0, 0, 0, 0, 3.0, 2.0, 5.0, -4.0, 0, 0, 0, 0]], dtype=torch.float16)
+    oe = lib.silu_mul(edge.to(gpu)).cpu().float()[0]
+    assert oe[0] == 0.0 and oe[1] == 60.0 and abs(oe[2]) < 1e-6 and abs(oe[3] + 4 * 0.7310586) < 4e-3
+
+
+def layer_weights(H, n_q, n_kv, F, seed=0):
+    D = 128
+    g = lambda shape, s, std: so.randn_fp16(shape, seed + s, std)
+    w = dict(q=g((n_q * D, H), 1, 0.03), k=g((n_kv * D, H), 2, 0.03), v=g((n_kv * D, H), 3, 0.03), o=g((H, n_q * D), 4, 0.03),
+             gate=g((F, H), 5, 0.03), up=g((F, H), 6, 0.03), down=g((H, F), 7, 0.03))
+    w["ln1"] = (1 + 0.1 * g((H,), 8, 1.0).float()).half()
+    w["ln2"] = (1 + 0.1 * g((H,), 9, 1.0).float()).half()
+    return w
+
+
+def layer_close(out, ref):
+    out, ref = out.float().cpu(), ref.float()
+    rel = float((out - ref).norm() / ref.norm())
+    worst = float((out - ref).abs().max() / ref.abs().max())
+    return rel <= 2e-3 and worst <= 2e-2, (rel, worst)
+
+
+@pytest.mark.parametrize("B,S,H,n_q,n_kv,F", [(2, 100, 512, 4, 2, 1024), (1, 700, 1024, 8, 2, 2816), (3, 1, 512, 4, 4, 1024)])
+def test_decoder_layer_prefill(lib, gpu, B, S, H, n_q, n_kv, F):
+    from llama_layer import FineLlamaDecoderLayer
+    w = layer_weights(H, n_q, n_kv, F)
+    x = so.randn_fp16((B, S, H), 42)
+    pos = torch.arange(S, dtype=torch.int32)[None].expand(B, S)
+    layer = FineLlamaDecoderLayer({k: v.to(gpu) for k, v in w.items()}, n_q, n_kv, rms_eps=1e-5, max_positions=1024)
+    xg = x.to(gpu)
+    out = layer(xg, pos.to(gpu))
+    torch.cuda.synchronize()
+    assert torch.equal(xg.cpu(), x)  # the input is not modified
+    ref, _, _ = so.llama_decoder_layer_ref(x, w, pos, n_q, n_kv, eps=1e-5)
+    ok, st = layer_close(out, ref)
+    assert ok, st
+
+
+def test_decoder_layer_generation_steps_with_cache(lib, gpu):
+    from llama_layer import FineKVCache, FineLlamaDecoderLayer
+    B, S0, H, n_q, n_kv, F, steps = 2, 600, 512, 8, 2, 1024, 3
+    w = layer_weights(H, n_q, n_kv, F, seed=20)
+    layer = FineLlamaDecoderLayer({k: v.to(gpu) for k, v in w.items()}, n_q, n_kv, max_positions=1024)
+    cache = FineKVCache(B, S0 + steps, n_kv, device=gpu)
+    x = so.randn_fp16((B, S0, H), 1)
+    out = layer(x.to(gpu), kv_cache=cache, time_attention=True)
+    ref, k_ref, v_ref = so.llama_decoder_layer_ref(x, w, torch.arange(S0)[None].expand(B, S0), n_q, n_kv)
+    assert layer_close(out, ref)[0] and cache.length == S0
+    for t in range(steps):
+        xt = so.randn_fp16((B, 1, H), 100 + t)
+        out = layer(xt.to(gpu), kv_cache=cache, time_attention=True)   # 8 query rows per kv head, 600+ keys: split-KV kernels
+        ref, k_ref, v_ref = so.llama_decoder_layer_ref(xt, w, torch.full((B, 1), S0 + t), n_q, n_kv, past_k=k_ref, past_v=v_ref)
+        ok, st = layer_close(out, ref)
+        assert ok, (t, st)
+    assert cache.length == S0 + steps and len(layer.attn_ms["prefill"]) == 1 and len(layer.attn_ms["decode"]) == steps
+    # the cache holds the rotated keys and the values the oracle holds
+    assert (cache.k.transpose(1, 2).float().cpu() - k_ref).abs().max() <= 2e-2
+    assert (cache.v.transpose(1, 2).float().cpu() - v_ref).abs().max() <= 2e-2
+    with pytest.raises(ValueError):
+        layer(xt.to(gpu), kv_cache=cache)
+
+
+def test_decoder_layer_from_transformers_weights(lib, gpu):
+    # weights taken from a transformers LlamaDecoderLayer; compared with that layer run in fp32 on the CPU
+    pytest.importorskip("transformers")
+    from transformers import LlamaConfig
+    from transformers.models.llama import modeling_llama as hf
+    from llama_layer import FineLlamaDecoderLayer
+    cfg = LlamaConfig(hidden_size=512, num_attention_heads=4, num_key_value_heads=2, head_dim=128, intermediate_size=1024,
+                      rms_norm_eps=1e-5, rope_theta=10000.0, vocab_size=32, num_hidden_layers=1)
+    cfg._attn_implementation = "eager"
+    torch.manual_seed(1)
+    ref_layer = hf.LlamaDecoderLayer(cfg, 0).float().eval()
+    for p in ref_layer.parameters():
+        torch.nn.init.normal_(p, std=0.03)
+    ref_layer.input_layernorm.weight.data = 1 + 0.1 * torch.randn(512)
+    ref_layer.post_attention_layernorm.weight.data = 1 + 0.1 * torch.randn(512)
+    for p in ref_layer.parameters():   # the values an fp16 checkpoint would hold
+        p.data = p.data.half().float()
+    B, S = 2, 130
+    x = so.randn_fp16((B, S, 512), 3)
+    pos = torch.arange(S)[None].expand(B, S)
+    cos, sin = hf.LlamaRotaryEmbedding(cfg)(x.float(), pos)
+    mask = torch.full((S, S), float("-inf")).triu(1)[None, None].expand(B, 1, S, S)
+    with torch.no_grad():
+        y = ref_layer(x.float(), attention_mask=mask, position_ids=pos, position_embeddings=(cos, sin))
+    y = y[0] if isinstance(y, tuple) else y
+    layer = FineLlamaDecoderLayer.from_hf(ref_layer, cfg, max_positions=256, device=gpu)
+    out = layer(x.to(gpu))
+    rel = float((out.float().cpu() - y).norm() / y.norm())
+    assert rel <= 3e-3, rel

@@ -197,3 +197,90 @@ def test_llama_layer_ref_shapes_and_composition():
     assert torch.allclose(out["attn"][0, 0], ref[0, 0], atol=1e-5)
     gu = out["gate_up"].half().float()
     assert torch.allclose(out["act"], torch.nn.functional.silu(gu[:, :F]) * gu[:, F:], atol=1e-6)
+
+
+# ---- layer glue of the in-model path ---------------------------------------------------------------------------------
+def test_rmsnorm_closed_forms():
+    # a constant row c normalises to sign(c) * weight (eps = 0); scaling the input leaves the output unchanged
+    w = torch.linspace(0.5, 1.5, 64)
+    out, _ = so.rmsnorm_ref(torch.full((3, 64), -2.5), w, eps=0.0)
+    assert torch.allclose(out, -w.expand(3, 64), atol=1e-6)
+    x = so.randn_fp16((5, 64), 1).float()
+    a, _ = so.rmsnorm_ref(x, w, eps=0.0)
+    b, _ = so.rmsnorm_ref(4 * x, w, eps=0.0)
+    assert torch.allclose(a, b, atol=1e-5)
+    # unit weight: every output row has mean square 1; eps enters as mean(x^2) + eps
+    one, _ = so.rmsnorm_ref(x, torch.ones(64), eps=0.0)
+    assert torch.allclose(one.pow(2).mean(-1), torch.ones(5), atol=1e-5)
+    e, _ = so.rmsnorm_ref(torch.ones(1, 64), torch.ones(64), eps=3.0)
+    assert torch.allclose(e, torch.full((1, 64), 0.5), atol=1e-6)
+    # residual: the sum is rounded to fp16 and returned
+    r = torch.full((1, 64), 1.0)
+    o2, h = so.rmsnorm_ref(torch.full((1, 64), 2.0 ** -12), torch.ones(64), eps=0.0, residual=r)
+    assert torch.equal(h, r)  # 1 + 2^-12 rounds to 1 in fp16
+
+
+def test_rope_closed_forms():
+    cos, sin = so.rope_tables(50, 128, 10000.0)
+    assert cos.shape == (50, 64) and torch.equal(cos[0], torch.ones(64)) and torch.equal(sin[0], torch.zeros(64))
+    # frequency 0 turns by one radian per position, the last one by base^(-126/128)
+    assert abs(cos[7, 0] - math.cos(7.0)) < 1e-6 and abs(sin[3, 63] - math.sin(3.0 * 10000.0 ** (-126 / 128))) < 1e-6
+    x = so.randn_fp16((2, 3, 6, 128), 5).float()
+    pos = torch.tensor([[0, 1, 2, 3, 4, 5], [10, 11, 12, 13, 14, 49]])
+    y = so.rope_ref(x, cos, sin, pos)
+    assert torch.equal(y[0, :, 0], x[0, :, 0])                      # position 0 is the identity
+    assert torch.allclose(y.norm(dim=-1), x.norm(dim=-1), rtol=1e-5)  # a rotation
+    # pair (i, i + 64) turns by the angle pos * inv_freq_i, by hand for one element
+    ang = 12 * 10000.0 ** (-2 * 5 / 128)
+    want = x[1, 2, 2, 5] * math.cos(ang) - x[1, 2, 2, 69] * math.sin(ang)
+    want_hi = x[1, 2, 2, 69] * math.cos(ang) + x[1, 2, 2, 5] * math.sin(ang)
+    assert abs(y[1, 2, 2, 5] - want) < 1e-5 and abs(y[1, 2, 2, 69] - want_hi) < 1e-5
+    # scores depend only on the distance between positions
+    q, k = x[:1, :1, :1], x[:1, 1:2, 1:2]
+    def score(pq, pk):
+        return (so.rope_ref(q, cos, sin, torch.tensor([[pq]])) * so.rope_ref(k, cos, sin, torch.tensor([[pk]]))).sum()
+    assert abs(score(9, 4) - score(30, 25)) < 1e-3 and abs(score(9, 4) - score(9, 5)) > 1e-3
+
+
+def test_silu_mul_closed_forms():
+    gu = torch.tensor([[0.0, 20.0, -20.0, 1.0, 3.0, 2.0, 5.0, -4.0]])
+    out = so.silu_mul_ref(gu)
+    want = torch.tensor([[0.0, 40.0, -20.0 / (1 + math.exp(20.0)) * 5.0, 1.0 / (1 + math.exp(-1.0)) * -4.0]])
+    assert torch.allclose(out, want, atol=1e-6)
+
+
+def test_decoder_layer_against_transformers_llama():
+    # independent second implementation: the Llama layer of the installed transformers package, fp32, eager attention
+    pytest.importorskip("transformers")
+    from transformers import LlamaConfig
+    from transformers.models.llama import modeling_llama as hf
+    cfg = LlamaConfig(hidden_size=512, num_attention_heads=4, num_key_value_heads=2, head_dim=128, intermediate_size=1024,
+                      rms_norm_eps=1e-5, rope_theta=10000.0, vocab_size=32, num_hidden_layers=1, attention_bias=False,
+                      mlp_bias=False)
+    cfg._attn_implementation = "eager"
+    torch.manual_seed(0)
+    layer = hf.LlamaDecoderLayer(cfg, 0).float().eval()
+    for p in layer.parameters():
+        torch.nn.init.normal_(p, std=0.05)
+    layer.input_layernorm.weight.data = 1 + 0.1 * torch.randn(512)
+    layer.post_attention_layernorm.weight.data = 1 + 0.1 * torch.randn(512)
+    B, S = 2, 37
+    x = torch.randn(B, S, 512)
+    pos = torch.arange(S)[None].expand(B, S)
+    cos, sin = hf.LlamaRotaryEmbedding(cfg)(x, pos)
+    mask = torch.full((S, S), float("-inf")).triu(1)[None, None].expand(B, 1, S, S)
+    with torch.no_grad():
+        y = layer(x, attention_mask=mask, position_ids=pos, position_embeddings=(cos, sin))
+    y = y[0] if isinstance(y, tuple) else y
+    a, mlp = layer.self_attn, layer.mlp
+    w = dict(q=a.q_proj.weight, k=a.k_proj.weight, v=a.v_proj.weight, o=a.o_proj.weight, gate=mlp.gate_proj.weight,
+             up=mlp.up_proj.weight, down=mlp.down_proj.weight, ln1=layer.input_layernorm.weight,
+             ln2=layer.post_attention_layernorm.weight)
+    out, k, v = so.llama_decoder_layer_ref(x, w, pos, 4, 2, eps=1e-5, round_stages=False)
+    assert (y - out).abs().max() < 2e-5 * y.abs().max()
+    # generation step with the cache of the prefill == last row of a prefill that is one token longer
+    x1 = torch.randn(B, 1, 512)
+    out1, _, _ = so.llama_decoder_layer_ref(x1, w, torch.full((B, 1), S), 4, 2, past_k=k, past_v=v, round_stages=False)
+    full, _, _ = so.llama_decoder_layer_ref(torch.cat((x, x1), 1), w, torch.arange(S + 1)[None].expand(B, S + 1), 4, 2,
+                                            round_stages=False)
+    assert torch.allclose(out1[:, 0], full[:, -1], atol=1e-4)

@@ -26,7 +26,7 @@ DEVICE_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wno-inline-asm", "-Wno-unused-command-line-argument",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
 ]
-KERNEL_SOURCES = ["csrc/hgemm.hip", "csrc/fmha_fwd.hip", "csrc/fmha_decode.hip", "csrc/capi.hip"]
+KERNEL_SOURCES = ["csrc/hgemm.hip", "csrc/fmha_fwd.hip", "csrc/fmha_decode.hip", "csrc/glue.hip", "csrc/capi.hip"]
 
 
 def _run(cmd, quiet_patterns=("is not a recognized feature for this target",)):

@@ -85,6 +85,58 @@ int mi355_fmha_fwd_strided(const void* Q, const void* K, const void* V, void* O,
                         stream);
 }
 
+static bool aligned16(const void* p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; }
+
+int mi355_rmsnorm(const void* x, const void* residual, void* residual_out, const void* weight, void* out, int64_t rows,
+                  int hidden, int64_t ldx, int64_t ldr, int64_t ldro, int64_t ldo, float eps, void* stream) {
+    if (!x || !weight || !out) return fail(MI355_ERR_BAD_ARGUMENT, "mi355_rmsnorm: null pointer");
+    if ((residual == nullptr) != (residual_out == nullptr))
+        return fail(MI355_ERR_BAD_ARGUMENT, "mi355_rmsnorm: residual and residual_out must both be given or both be NULL");
+    if (rows < 1 || hidden < 8 || hidden % 8 != 0)
+        return fail(MI355_ERR_BAD_ARGUMENT, "mi355_rmsnorm: rows >= 1 and hidden a positive multiple of 8 required (got %lld, %d)",
+                    (long long)rows, hidden);
+    if (ldx < hidden || ldo < hidden || ldx % 8 || ldo % 8 ||
+        (residual && (ldr < hidden || ldro < hidden || ldr % 8 || ldro % 8)))
+        return fail(MI355_ERR_BAD_ARGUMENT, "mi355_rmsnorm: row strides must be multiples of 8 and >= hidden");
+    if (!aligned16(x) || !aligned16(weight) || !aligned16(out) || !aligned16(residual) || !aligned16(residual_out))
+        return fail(MI355_ERR_BAD_ARGUMENT, "mi355_rmsnorm: pointers must be 16-byte aligned");
+    if (!(eps >= 0.f) || eps > 1.f) return fail(MI355_ERR_BAD_ARGUMENT, "mi355_rmsnorm: eps outside [0, 1] (got %g)", (double)eps);
+    hipError_t e = mi355::rmsnorm_dispatch(x, residual, residual_out, weight, out, rows, hidden, ldx, ldr, ldro, ldo, eps,
+                                           static_cast<hipStream_t>(stream));
+    if (e != hipSuccess) return hip_fail(e, "mi355_rmsnorm launch");
+    return 0;
+}
+
+int mi355_rope(const void* x, void* out, int B, int S, int heads, int D, int64_t x_batch, int64_t x_row, int64_t out_batch,
+               int64_t out_row, const float* cos_table, const float* sin_table, const int32_t* positions, int n_positions,
+               void* stream) {
+    if (!x || !out || !cos_table || !sin_table || !positions) return fail(MI355_ERR_BAD_ARGUMENT, "mi355_rope: null pointer");
+    if (D != 128) return fail(MI355_ERR_UNSUPPORTED, "mi355_rope: head_dim must be 128 (got %d)", D);
+    if (B < 1 || S < 1 || heads < 1 || n_positions < 1)
+        return fail(MI355_ERR_BAD_ARGUMENT, "mi355_rope: B, S, heads, n_positions must be >= 1");
+    const int64_t width = (int64_t)heads * D;
+    if (x_row < width || out_row < width || x_row % 8 || out_row % 8 || x_batch % 8 || out_batch % 8 || x_batch < 0 || out_batch < 0)
+        return fail(MI355_ERR_BAD_ARGUMENT, "mi355_rope: strides must be multiples of 8, row strides >= heads * 128");
+    if (!aligned16(x) || !aligned16(out) || !aligned16(cos_table) || !aligned16(sin_table))
+        return fail(MI355_ERR_BAD_ARGUMENT, "mi355_rope: pointers must be 16-byte aligned");
+    hipError_t e = mi355::rope_dispatch(x, out, B, S, heads, x_batch, x_row, out_batch, out_row, cos_table, sin_table, positions,
+                                        n_positions, static_cast<hipStream_t>(stream));
+    if (e != hipSuccess) return hip_fail(e, "mi355_rope launch");
+    return 0;
+}
+
+int mi355_silu_mul(const void* gate_up, void* out, int64_t rows, int inter, int64_t ld_in, int64_t ld_out, void* stream) {
+    if (!gate_up || !out) return fail(MI355_ERR_BAD_ARGUMENT, "mi355_silu_mul: null pointer");
+    if (rows < 1 || inter < 8 || inter % 8 != 0)
+        return fail(MI355_ERR_BAD_ARGUMENT, "mi355_silu_mul: rows >= 1 and inter a positive multiple of 8 required");
+    if (ld_in < 2 * (int64_t)inter || ld_out < inter || ld_in % 8 || ld_out % 8)
+        return fail(MI355_ERR_BAD_ARGUMENT, "mi355_silu_mul: ld_in >= 2 * inter, ld_out >= inter, both multiples of 8 required");
+    if (!aligned16(gate_up) || !aligned16(out)) return fail(MI355_ERR_BAD_ARGUMENT, "mi355_silu_mul: pointers must be 16-byte aligned");
+    hipError_t e = mi355::silu_mul_dispatch(gate_up, out, rows, inter, ld_in, ld_out, static_cast<hipStream_t>(stream));
+    if (e != hipSuccess) return hip_fail(e, "mi355_silu_mul launch");
+    return 0;
+}
+
 const char* mi355_last_error(void) { return g_err; }
 
 int mi355_serving_version(void) { return MI355_SERVING_VERSION; }

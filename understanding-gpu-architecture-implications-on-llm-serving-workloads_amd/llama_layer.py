@@ -1,0 +1,119 @@
+"""A Llama decoder layer on the MI355X kernels: the in-model caller of fine_fmha, rebuilt without its copies.
+
+The reference measures its attention kernels inside a patched Hugging Face layer
+(benchmarks/flashattn-cuda/modeling_llama.py): LlamaSdpaAttention.forward (:652-704) projects with three nn.Linear
+calls, transposes to [B, H, S, D], applies RoPE, expands K/V with repeat_kv (:670-671), calls
+``fmha_unified.ops.fine_fmha`` (:687-690), transposes back with a copy (:700) and projects; LlamaDecoderLayer.forward
+(:755-781) wraps it in RMSNorm, residual adds and the gate/up/down MLP (:227), all as separate PyTorch kernels.
+
+Here one layer is twelve launches with no layout copies:
+    rmsnorm -> QKV GEMM (one fused NT GEMM on the nn.Linear weights) -> RoPE in place on the q and k heads of the
+    projection (k goes straight into the KV cache when there is one) -> attention reading q, k, v where they lie
+    (strided operands, GQA inside the kernel, output written as [B, S, Hq*D]) -> O projection -> residual add fused
+    into the second rmsnorm -> gate/up GEMM (fused) -> SiLU(gate)*up -> down GEMM -> residual add.
+Weights keep the nn.Linear layout ([out_features, in_features]); nothing is transposed or repacked beyond
+concatenating q/k/v and gate/up along the output dimension once at construction.
+"""
+import torch
+
+import mi355_serving as lib
+
+__all__ = ["FineKVCache", "FineLlamaDecoderLayer", "rope_tables"]
+
+
+def rope_tables(n_positions, head_dim=128, base=10000.0, device="cuda"):
+    """cos, sin [n_positions, head_dim / 2] fp32 (LlamaRotaryEmbedding, modeling_llama.py:113,119-132)."""
+    inv_freq = 1.0 / (base ** (torch.arange(0, head_dim, 2, dtype=torch.int64).float() / head_dim))
+    ang = torch.arange(n_positions, dtype=torch.float32)[:, None] * inv_freq[None, :]
+    return ang.cos().contiguous().to(device), ang.sin().contiguous().to(device)
+
+
+class FineKVCache:
+    """Static key/value cache of one layer, [B, max_len, n_kv, 128] fp16 (token-major so a step appends one row)."""
+
+    def __init__(self, batch, max_len, n_kv, head_dim=128, device="cuda"):
+        self.k = torch.empty((batch, max_len, n_kv, head_dim), dtype=torch.float16, device=device)
+        self.v = torch.empty_like(self.k)
+        self.length = 0
+
+    @property
+    def max_len(self):
+        return self.k.shape[1]
+
+
+class FineLlamaDecoderLayer:
+    """forward(hidden_states [B, S, H] fp16, position_ids [B, S]) -> [B, S, H]; causal attention over the cache (if
+    any) plus the new tokens. `weights`: dict of fp16 GPU tensors in nn.Linear layout: q, k, v, o, gate, up, down,
+    and the norm weights ln1, ln2."""
+
+    def __init__(self, weights, n_q_heads, n_kv_heads, rms_eps=1e-5, rope_base=10000.0, max_positions=8192):
+        w = {k: v.detach().to(torch.float16).contiguous() for k, v in weights.items()}
+        self.n_q, self.n_kv = int(n_q_heads), int(n_kv_heads)
+        self.hidden = w["q"].shape[1]
+        self.head_dim = w["q"].shape[0] // self.n_q
+        if self.head_dim != 128:
+            raise ValueError("head_dim must be 128, got %d" % self.head_dim)
+        self.inter = w["gate"].shape[0]
+        self.w_qkv = torch.cat((w["q"], w["k"], w["v"]), 0).contiguous()   # [(Hq + 2 Hkv) * D, H]
+        self.w_o = w["o"]                                                  # [H, Hq * D]
+        self.w_gu = torch.cat((w["gate"], w["up"]), 0).contiguous()        # [2 F, H]
+        self.w_d = w["down"]                                               # [H, F]
+        self.ln1, self.ln2 = w["ln1"], w["ln2"]
+        self.eps = float(rms_eps)
+        self.cos, self.sin = rope_tables(max_positions, self.head_dim, rope_base, device=self.w_o.device)
+        self.attn_ms = {"prefill": [], "decode": []}  # filled when time_attention=True (modeling_llama.py:762-775)
+
+    @classmethod
+    def from_hf(cls, hf_layer, config, max_positions=8192, device="cuda"):
+        """Wrap the weights of a transformers LlamaDecoderLayer."""
+        a, m = hf_layer.self_attn, hf_layer.mlp
+        w = dict(q=a.q_proj.weight, k=a.k_proj.weight, v=a.v_proj.weight, o=a.o_proj.weight, gate=m.gate_proj.weight,
+                 up=m.up_proj.weight, down=m.down_proj.weight, ln1=hf_layer.input_layernorm.weight,
+                 ln2=hf_layer.post_attention_layernorm.weight)
+        w = {k: v.detach().to(device) for k, v in w.items()}
+        base = getattr(config, "rope_theta", None) or (getattr(config, "rope_parameters", None) or {}).get("rope_theta", 10000.0)
+        return cls(w, config.num_attention_heads, config.num_key_value_heads, config.rms_norm_eps, base, max_positions)
+
+    def forward(self, hidden_states, position_ids=None, kv_cache=None, time_attention=False):
+        B, S, H = hidden_states.shape
+        D, Hq, Hkv = self.head_dim, self.n_q, self.n_kv
+        x = hidden_states.reshape(B * S, H)
+        past = kv_cache.length if kv_cache is not None else 0
+        if position_ids is None:
+            position_ids = torch.arange(past, past + S, device=x.device, dtype=torch.int32)[None].expand(B, S)
+        pos = position_ids.to(torch.int32).contiguous()
+
+        h1 = lib.rmsnorm(x, self.ln1, self.eps)
+        if time_attention:
+            torch.cuda.synchronize()
+            t0, t1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            t0.record()
+        qkv = lib.hgemm(h1, self.w_qkv, "NT").view(B, S, Hq + 2 * Hkv, D)
+        q = qkv[:, :, :Hq]
+        if kv_cache is None:
+            lib.rope(qkv[:, :, :Hq + Hkv], self.cos, self.sin, pos)           # q and k heads are adjacent
+            k, v = qkv[:, :, Hq:Hq + Hkv], qkv[:, :, Hq + Hkv:]
+        else:
+            if past + S > kv_cache.max_len:
+                raise ValueError("KV cache of %d tokens cannot take %d more after %d" % (kv_cache.max_len, S, past))
+            lib.rope(q, self.cos, self.sin, pos)
+            lib.rope(qkv[:, :, Hq:Hq + Hkv], self.cos, self.sin, pos, out=kv_cache.k[:, past:past + S])
+            kv_cache.v[:, past:past + S].copy_(qkv[:, :, Hq + Hkv:])
+            kv_cache.length = past + S
+            k, v = kv_cache.k[:, :past + S], kv_cache.v[:, :past + S]
+        attn = torch.empty((B, S, Hq, D), dtype=torch.float16, device=x.device)
+        # [B, S, heads, D] viewed as [B, heads, S, D]: the kernel reads and writes these layouts in place
+        lib.fmha_fwd(q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2), causal=True, return_lse=False,
+                     out=attn.transpose(1, 2))
+        proj = lib.hgemm(attn.view(B * S, Hq * D), self.w_o, "NT")
+        if time_attention:
+            t1.record()
+            torch.cuda.synchronize()
+            self.attn_ms["decode" if (S == 1 and past > 0) else "prefill"].append(t0.elapsed_time(t1))
+        h2, res = lib.rmsnorm(proj, self.ln2, self.eps, residual=x)
+        gu = lib.hgemm(h2, self.w_gu, "NT")
+        act = lib.silu_mul(gu)
+        down = lib.hgemm(act, self.w_d, "NT")
+        return res.add_(down).view(B, S, H)
+
+    __call__ = forward

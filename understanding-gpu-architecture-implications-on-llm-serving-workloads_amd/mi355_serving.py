@@ -13,7 +13,8 @@ LIB_PATH = os.path.join(_HERE, "libmi355_serving.so")
 GEMM_NN, GEMM_NT, GEMM_TN = 0, 1, 2
 LAYOUTS = {"NN": GEMM_NN, "NT": GEMM_NT, "TN": GEMM_TN}
 
-EXPORTED_SYMBOLS = ("mi355_hgemm", "mi355_fmha_fwd", "mi355_fmha_fwd_strided", "mi355_last_error", "mi355_serving_version",
+EXPORTED_SYMBOLS = ("mi355_hgemm", "mi355_fmha_fwd", "mi355_fmha_fwd_strided", "mi355_rmsnorm", "mi355_rope", "mi355_silu_mul",
+                    "mi355_last_error", "mi355_serving_version",
                     "mi355_debug_set_gemm_variant", "mi355_debug_set_fmha_variant")
 
 _lib = None
@@ -43,6 +44,12 @@ def load():
     lib.mi355_fmha_fwd_strided.argtypes = [vp, vp, vp, vp, vp, i32, i32, i32, i32, i32, i32, f32, i32, i32,
                                            ctypes.POINTER(i64), vp]
     lib.mi355_fmha_fwd_strided.restype = i32
+    lib.mi355_rmsnorm.argtypes = [vp, vp, vp, vp, vp, i64, i32, i64, i64, i64, i64, f32, vp]
+    lib.mi355_rmsnorm.restype = i32
+    lib.mi355_rope.argtypes = [vp, vp, i32, i32, i32, i32, i64, i64, i64, i64, vp, vp, vp, i32, vp]
+    lib.mi355_rope.restype = i32
+    lib.mi355_silu_mul.argtypes = [vp, vp, i64, i32, i64, i64, vp]
+    lib.mi355_silu_mul.restype = i32
     lib.mi355_last_error.argtypes = []
     lib.mi355_last_error.restype = ctypes.c_char_p
     lib.mi355_serving_version.argtypes = []
@@ -145,3 +152,51 @@ def fmha_fwd(q, k, v, causal=False, kv_valid_len=None, scale=None, return_lse=Tr
         fmha_fwd_strided_raw(_ptr(q), _ptr(k), _ptr(v), _ptr(o), _ptr(lse), B, Hq, Hkv, Sq, Sk, D, float(scale),
                              int(bool(causal)), int(kv_valid_len), strides, stream)
     return (o, lse) if return_lse else o
+
+
+def _stream_of(t):
+    import torch
+    return torch.cuda.current_stream(t.device).cuda_stream
+
+
+def rmsnorm(x, weight, eps, residual=None, residual_out=None, out=None):
+    """RMSNorm over the last dimension of a [rows, hidden] fp16 tensor (row stride free). With `residual`, normalises
+    h = fp16(residual + x) and writes h to `residual_out` (default: a new tensor). Returns out or (out, h)."""
+    import torch
+    assert x.dim() == 2 and x.stride(1) == 1 and x.dtype == torch.float16 and weight.is_contiguous()
+    rows, hidden = x.shape
+    if out is None:
+        out = torch.empty((rows, hidden), dtype=torch.float16, device=x.device)
+    if residual is not None and residual_out is None:
+        residual_out = torch.empty((rows, hidden), dtype=torch.float16, device=x.device)
+    _check(load().mi355_rmsnorm(_ptr(x), _ptr(residual), _ptr(residual_out), _ptr(weight), _ptr(out), rows, hidden,
+                                x.stride(0), residual.stride(0) if residual is not None else 0,
+                                residual_out.stride(0) if residual_out is not None else 0, out.stride(0), float(eps),
+                                _stream_of(x)))
+    return out if residual is None else (out, residual_out)
+
+
+def rope(x, cos, sin, positions, out=None):
+    """Rotary embedding of x [B, S, heads, 128] (any batch / token stride, heads contiguous), in place unless `out`
+    (same shape, own strides) is given. cos, sin: [n_positions, 64] fp32; positions: [B, S] int32."""
+    import torch
+    B, S, heads, D = x.shape
+    out = x if out is None else out
+    assert x.dtype == torch.float16 and x.stride(3) == 1 and x.stride(2) == D and out.stride(3) == 1 and out.stride(2) == D
+    assert cos.dtype == torch.float32 and cos.is_contiguous() and sin.is_contiguous() and cos.shape == sin.shape
+    assert positions.dtype == torch.int32 and positions.is_contiguous() and positions.numel() == B * S
+    _check(load().mi355_rope(_ptr(x), _ptr(out), B, S, heads, D, x.stride(0), x.stride(1), out.stride(0), out.stride(1),
+                             _ptr(cos), _ptr(sin), _ptr(positions), cos.shape[0], _stream_of(x)))
+    return out
+
+
+def silu_mul(gate_up, out=None):
+    """silu(gate_up[:, :F]) * gate_up[:, F:] for a [rows, 2F] fp16 tensor."""
+    import torch
+    assert gate_up.dim() == 2 and gate_up.stride(1) == 1 and gate_up.dtype == torch.float16
+    rows, two_f = gate_up.shape
+    inter = two_f // 2
+    if out is None:
+        out = torch.empty((rows, inter), dtype=torch.float16, device=gate_up.device)
+    _check(load().mi355_silu_mul(_ptr(gate_up), _ptr(out), rows, inter, gate_up.stride(0), out.stride(0), _stream_of(gate_up)))
+    return out
