@@ -32,9 +32,10 @@ constexpr int ROW_BYTES = D * 2;             // 256
 constexpr int TILE_BYTES = TK * ROW_BYTES;   // 8 KiB
 constexpr int STAGE_BYTES = 2 * TILE_BYTES;  // K + V
 constexpr int NSTAGE = 3;
-constexpr int WAVES = 2;                     // work units per workgroup
+constexpr int WAVES = 3;                     // work units per workgroup
 constexpr int WAVE_BYTES = NSTAGE * STAGE_BYTES;
-constexpr int LDS_BYTES = WAVES * WAVE_BYTES;  // 96 KiB
+constexpr int LDS_BYTES = WAVES * WAVE_BYTES;  // 144 KiB
+constexpr float kLazyLog2 = 8.f;             // rescale only when a column maximum grows by more than 2^8
 constexpr int COPIES = 2 * (TILE_BYTES / 1024);  // 16 copy instructions per stage
 constexpr int PART_STRIDE = D + 4;           // floats per (unit, column): O~[128], m, l, 2 pad (keeps rows 16-byte aligned)
 
@@ -81,6 +82,11 @@ __global__ __launch_bounds__(dec::WAVES * 64) void fmha_decode_split_kernel(
 #pragma unroll
     for (int ks = 0; ks < 8; ++ks) qf[ks] = *(const half8*)(qp + ks * 16);
     const int lim = causal ? min(kv_valid - 1, qi + shift) : kv_valid - 1;  // last visible key of this column
+    // smallest such limit over the wave: tiles that end at or before it need no mask code
+    int lim_min = lim;
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) lim_min = min(lim_min, __shfl_xor(lim_min, off, 64));
+    lim_min = __builtin_amdgcn_readfirstlane(lim_min);
 
     const half_t* Kh = K + b * k_batch + hkv * k_head;
     const half_t* Vh = V + b * v_batch + hkv * v_head;
@@ -119,17 +125,23 @@ __global__ __launch_bounds__(dec::WAVES * 64) void fmha_decode_split_kernel(
         for (int e = 0; e < 16; ++e) o[db][e] = 0.f;
     float m_run = -INFINITY, l_run = 0.f;
 
+    const int n_loc = t_end - t_begin;
+    // each wave starts at a different tile of its range and wraps around (the online softmax does not care about the
+    // order): waves whose ranges lie a large power of two apart then do not walk the same memory channels in step
+    const int rot = n_loc > 0 ? (unit * 5) % n_loc : 0;
+    auto tile_of = [&](int i) { int r = i + rot; return t_begin + (r >= n_loc ? r - n_loc : r); };
     int issued = t_begin;
 #pragma unroll
     for (int i = 0; i < NSTAGE - 1; ++i)
         if (issued < t_end) {
-            issue_stage(issued, i);
+            issue_stage(tile_of(issued - t_begin), i);
             ++issued;
         }
     int slot = 0, fill = NSTAGE - 1;
-    for (int t = t_begin; t < t_end; ++t) {
+    for (int tt0 = t_begin; tt0 < t_end; ++tt0) {
+        const int t = tile_of(tt0 - t_begin);
         if (issued < t_end) {
-            issue_stage(issued, fill);
+            issue_stage(tile_of(issued - t_begin), fill);
             ++issued;
             fill = (fill + 1 == NSTAGE) ? 0 : fill + 1;
             wait_vmcnt<COPIES*(NSTAGE - 1)>();  // everything but the newest NSTAGE-1 tiles has landed
@@ -149,19 +161,32 @@ __global__ __launch_bounds__(dec::WAVES * 64) void fmha_decode_split_kernel(
             s = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf, qf[ks], s, 0, 0, 0);
         }
         const int key0 = t * TK;
-        float mx = -INFINITY;
+        if (key0 + TK - 1 > lim_min) {
 #pragma unroll
-        for (int e = 0; e < 16; ++e) {
-            int key = key0 + 8 * (e >> 2) + 4 * h + (e & 3);
-            if (key > lim) s[e] = -INFINITY;
-            mx = fmaxf(mx, s[e]);
+            for (int e = 0; e < 16; ++e) {
+                int key = key0 + 8 * (e >> 2) + 4 * h + (e & 3);
+                if (key > lim) s[e] = -INFINITY;
+            }
         }
+        float mx = s[0];
+#pragma unroll
+        for (int e = 1; e < 16; ++e) mx = fmaxf(mx, s[e]);
         mx = fmaxf(mx, other_half(mx));
-        float m_new = fmaxf(m_run, mx);
-        float m_use = (m_new == -INFINITY) ? 0.f : m_new;
-        float alpha = __builtin_amdgcn_exp2f((m_run - m_use) * scale_log2);
-        m_run = m_new;
-        const float neg_ms = -m_use * scale_log2;
+        // lazy rescaling as in the prefill kernel: m_run is the exponent reference of the running sums and only moves
+        // (with O and l rescaled) when some column exceeds it by more than 2^kLazyLog2
+        const bool raise = (mx - m_run) * scale_log2 > kLazyLog2;  // -inf - -inf = NaN compares false
+        if (__builtin_amdgcn_ballot_w64(raise) != 0) {
+            float m_new = fmaxf(m_run, mx);
+            float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+            float alpha = __builtin_amdgcn_exp2f((m_run - m_use) * scale_log2);
+            m_run = m_new;
+            l_run *= alpha;
+#pragma unroll
+            for (int db = 0; db < 4; ++db)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) o[db][e] *= alpha;
+        }
+        const float neg_ms = (m_run == -INFINITY) ? 0.f : -m_run * scale_log2;
         float psum = 0.f;
         half8 pf[2];
 #pragma unroll
@@ -175,11 +200,7 @@ __global__ __launch_bounds__(dec::WAVES * 64) void fmha_decode_split_kernel(
             }
             pf[tt] = pk;
         }
-        l_run = l_run * alpha + psum;
-#pragma unroll
-        for (int db = 0; db < 4; ++db)
-#pragma unroll
-            for (int e = 0; e < 16; ++e) o[db][e] *= alpha;
+        l_run += psum;
         // O^T += V^T P^T
 #pragma unroll
         for (int tt = 0; tt < 2; ++tt)
@@ -322,8 +343,8 @@ hipError_t fmha_decode_dispatch(const half_t* Q, const half_t* K, const half_t* 
     const int group = Hq / Hkv;
     const int ncols = group * Sq;
     const int tiles = (kv_valid + TK - 1) / TK;
-    // about two waves per CU in flight, at least 4 key tiles (128 keys) per wave
-    int splits = 512 / (B * Hkv);
+    // about three waves (one workgroup) per CU in flight, at least 4 key tiles (128 keys) per wave
+    int splits = (256 * WAVES) / (B * Hkv);
     splits = splits < 1 ? 1 : splits;
     int max_splits = (tiles + 3) / 4;
     if (splits > max_splits) splits = max_splits;
