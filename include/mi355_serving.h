@@ -33,6 +33,10 @@ extern "C" {
 #define MI355_ERR_BAD_ARGUMENT 10001
 #define MI355_ERR_UNSUPPORTED 10002
 
+/* element types (internal tags of the attention dispatcher; the entry points fix the type by name) */
+#define MI355_DTYPE_FP16 0
+#define MI355_DTYPE_BF16 1
+
 /* operand layouts of mi355_hgemm */
 #define MI355_GEMM_NN 0 /* A is [M,K] row-major, B is [K,N] row-major           */
 #define MI355_GEMM_NT 1 /* A is [M,K] row-major, B is stored [N,K] (C = A * B^T) */
@@ -92,6 +96,15 @@ int mi355_fmha_fwd(const void* Q, const void* K, const void* V, void* O, float* 
 int mi355_fmha_fwd_strided(const void* Q, const void* K, const void* V, void* O, float* LSE, int B, int Hq, int Hkv,
                            int Sq, int Sk, int D, float scale, int causal, int kv_valid_len, const int64_t* strides,
                            void* stream);
+
+/*
+ * The same attention forward for bfloat16 Q, K, V, O (fp32 scores, statistics and accumulation as above; P is rounded to
+ * bfloat16 for the second product). `strides` as in mi355_fmha_fwd_strided, or NULL for contiguous [B, H, S, D] tensors.
+ * For callers of the reference's bf16 operator index (`finefmha_5`: kernels/fmha/pkg/fmha_unified/csrc/manual/fmha_5_nv.cu:148-150,
+ * driven with bf16 tensors by kernels/fmha/test/perf.py:106-108 and the bf16 cases of correct.py:69-72).
+ */
+int mi355_fmha_fwd_bf16(const void* Q, const void* K, const void* V, void* O, float* LSE, int B, int Hq, int Hkv, int Sq,
+                        int Sk, int D, float scale, int causal, int kv_valid_len, const int64_t* strides, void* stream);
 
 /*
  * Layer glue between the GEMMs and the attention of a Llama decoder layer: memory-bound, fp16 in/out, fp32 arithmetic,

@@ -302,3 +302,47 @@ def test_torch_operator_reads_transposed_views_in_place(gpu):
     q2.copy_(q.to(gpu))
     out2 = fmha_unified.ops.fine_fmha(q2, k.to(gpu), v.to(gpu), True, False, 2)
     assert (out2.cpu().float() - o_ref).abs().max() <= 2e-3
+
+
+# ---- bfloat16 -----------------------------------------------------------------------------------------------------------
+# Tolerance for bfloat16 outputs (8 significand bits; the fp16 bound of 2e-3 is below half a bf16 ulp of values near 1):
+# max|O - O_ref| <= 1.6e-2 against fp32 attention over the same bf16-rounded inputs; LSE (fp32 from fp32 scores) keeps 1e-3.
+def bf16_inputs(B, Hq, Hkv, Sq, Sk, seed):
+    q, k, v = so.fmha_inputs(B, Hq, Hkv, Sq, Sk, seed=seed)
+    return q.float().bfloat16(), k.float().bfloat16(), v.float().bfloat16()
+
+
+@pytest.mark.parametrize("B,Hq,Hkv,Sq,Sk,causal,kvv", [
+    (1, 4, 1, 128, 128, True, None),      # the seeded shape of the reference's correct.py
+    (2, 8, 2, 300, 333, True, 320),       # ragged, 128-query workgroups
+    (1, 32, 8, 2048, 2048, True, None),   # ping-pong workgroups
+    (4, 32, 32, 1024, 1024, False, None),  # configuration F3 in bf16
+    (2, 8, 2, 1, 3000, False, 2900),      # generation step, split-KV kernels
+    (1, 16, 2, 3, 700, True, None),
+])
+def test_bfloat16_attention(lib, gpu, B, Hq, Hkv, Sq, Sk, causal, kvv):
+    q, k, v = bf16_inputs(B, Hq, Hkv, Sq, Sk, seed=Sq + Sk)
+    o, lse = lib.fmha_fwd(q.to(gpu), k.to(gpu), v.to(gpu), causal=causal, kv_valid_len=kvv)
+    assert o.dtype == torch.bfloat16 and lse.dtype == torch.float32
+    o_ref, lse_ref = so.attention_ref(q, k, v, causal=causal, kv_valid_len=kvv)
+    assert (o.float().cpu() - o_ref).abs().max() <= 1.6e-2
+    assert (lse.cpu() - lse_ref).abs().max() <= 1e-3
+
+
+def test_bfloat16_closed_forms(lib, gpu):
+    # first causal row returns V[0] exactly; V = ones returns ones exactly (both representable in bf16)
+    q, k, v = bf16_inputs(1, 4, 2, 200, 200, seed=9)
+    o, _ = lib.fmha_fwd(q.to(gpu), k.to(gpu), v.to(gpu), causal=True)
+    assert torch.equal(o[:, :, 0].cpu(), v.repeat_interleave(2, 1)[:, :, 0])
+    o1, _ = lib.fmha_fwd(q.to(gpu), k.to(gpu), torch.ones_like(v).to(gpu), causal=False)
+    assert (o1.float().cpu() - 1).abs().max() <= 2.0 ** -8
+
+
+def test_torch_operator_bfloat16_and_mixed_dtype_rejection(gpu):
+    import fmha_unified
+    q, k, v = bf16_inputs(1, 8, 2, 256, 256, seed=4)
+    out = fmha_unified.ops.fine_fmha(q.to(gpu), k.to(gpu), v.to(gpu), causal=True, is_decode=False, kernel_index=5)
+    o_ref, _ = so.attention_ref(q, k, v, causal=True)
+    assert out.dtype == torch.bfloat16 and (out.float().cpu() - o_ref).abs().max() <= 1.6e-2
+    with pytest.raises(RuntimeError, match="dtype"):
+        fmha_unified.ops.fine_fmha(q.to(gpu), k.half().to(gpu), v.to(gpu), True, False, 5)

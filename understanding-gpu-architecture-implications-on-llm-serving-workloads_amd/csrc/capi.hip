@@ -41,7 +41,7 @@ int mi355_hgemm(const void* A, const void* B, void* C, int M, int N, int K, int6
 
 static int fmha_checked(const char* fn, const void* Q, const void* K, const void* V, void* O, float* LSE, int B, int Hq, int Hkv,
                         int Sq, int Sk, int D, float scale, int causal, int kv_valid_len, const mi355::FmhaStrides& sd,
-                        void* stream) {
+                        int dtype, void* stream) {
     if (!Q || !K || !V || !O) return fail(MI355_ERR_BAD_ARGUMENT, "%s: null pointer", fn);
     if (B < 1 || Hq < 1 || Hkv < 1 || Sq < 1 || Sk < 1)
         return fail(MI355_ERR_BAD_ARGUMENT, "%s: B, Hq, Hkv, Sq, Sk must be >= 1", fn);
@@ -62,7 +62,7 @@ static int fmha_checked(const char* fn, const void* Q, const void* K, const void
                         all[i]);
     if (sd.o_row < D || (Hq > 1 && sd.o_head < D) || (B > 1 && sd.o_batch < D))
         return fail(MI355_ERR_BAD_ARGUMENT, "%s: rows of O overlap (o strides %ld, %ld, %ld)", fn, sd.o_batch, sd.o_head, sd.o_row);
-    hipError_t e = mi355::fmha_fwd_dispatch(Q, K, V, O, LSE, B, Hq, Hkv, Sq, Sk, scale, causal != 0, kv_valid_len, sd,
+    hipError_t e = mi355::fmha_fwd_dispatch(Q, K, V, O, LSE, B, Hq, Hkv, Sq, Sk, scale, causal != 0, kv_valid_len, sd, dtype,
                                             static_cast<hipStream_t>(stream));
     if (e != hipSuccess) return hip_fail(e, fn);
     return 0;
@@ -72,7 +72,8 @@ int mi355_fmha_fwd(const void* Q, const void* K, const void* V, void* O, float* 
                    int Sk, int D, float scale, int causal, int kv_valid_len, void* stream) {
     const long q_head = (long)Sq * D, k_head = (long)Sk * D;
     const mi355::FmhaStrides sd = {Hq * q_head, q_head, D, Hkv * k_head, k_head, D, Hkv * k_head, k_head, D, Hq * q_head, q_head, D};
-    return fmha_checked("mi355_fmha_fwd", Q, K, V, O, LSE, B, Hq, Hkv, Sq, Sk, D, scale, causal, kv_valid_len, sd, stream);
+    return fmha_checked("mi355_fmha_fwd", Q, K, V, O, LSE, B, Hq, Hkv, Sq, Sk, D, scale, causal, kv_valid_len, sd,
+                        MI355_DTYPE_FP16, stream);
 }
 
 int mi355_fmha_fwd_strided(const void* Q, const void* K, const void* V, void* O, float* LSE, int B, int Hq, int Hkv, int Sq,
@@ -82,7 +83,19 @@ int mi355_fmha_fwd_strided(const void* Q, const void* K, const void* V, void* O,
                                    (long)strides[4], (long)strides[5], (long)strides[6],  (long)strides[7],
                                    (long)strides[8], (long)strides[9], (long)strides[10], (long)strides[11]};
     return fmha_checked("mi355_fmha_fwd_strided", Q, K, V, O, LSE, B, Hq, Hkv, Sq, Sk, D, scale, causal, kv_valid_len, sd,
-                        stream);
+                        MI355_DTYPE_FP16, stream);
+}
+
+int mi355_fmha_fwd_bf16(const void* Q, const void* K, const void* V, void* O, float* LSE, int B, int Hq, int Hkv, int Sq,
+                        int Sk, int D, float scale, int causal, int kv_valid_len, const int64_t* strides, void* stream) {
+    const long q_head = (long)Sq * D, k_head = (long)Sk * D;
+    mi355::FmhaStrides sd = {Hq * q_head, q_head, D, Hkv * k_head, k_head, D, Hkv * k_head, k_head, D, Hq * q_head, q_head, D};
+    if (strides)
+        sd = {(long)strides[0], (long)strides[1], (long)strides[2],  (long)strides[3],
+              (long)strides[4], (long)strides[5], (long)strides[6],  (long)strides[7],
+              (long)strides[8], (long)strides[9], (long)strides[10], (long)strides[11]};
+    return fmha_checked("mi355_fmha_fwd_bf16", Q, K, V, O, LSE, B, Hq, Hkv, Sq, Sk, D, scale, causal, kv_valid_len, sd,
+                        MI355_DTYPE_BF16, stream);
 }
 
 static bool aligned16(const void* p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; }

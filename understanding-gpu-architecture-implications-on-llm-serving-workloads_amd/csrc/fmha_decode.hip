@@ -51,11 +51,13 @@ __device__ __forceinline__ float other_half(float x) {
 }  // namespace dec
 
 // units = B * Hkv * splits, unit u = (b * Hkv + hkv) * splits + s covers key tiles [s * tiles_per_split, ...)
+template <typename T>
 __global__ __launch_bounds__(dec::WAVES * 64) void fmha_decode_split_kernel(
-    const half_t* __restrict__ Q, const half_t* __restrict__ K, const half_t* __restrict__ V, float* __restrict__ part, int B,
+    const T* __restrict__ Q, const T* __restrict__ K, const T* __restrict__ V, float* __restrict__ part, int B,
     int Hq, int Hkv, int Sq, int Sk, float scale_log2, int causal, int kv_valid, int splits, int tiles_per_split, int units, long q_batch,
     long q_head, long q_rstride, long k_batch, long k_head, long k_rstride, long v_batch, long v_head, long v_rstride) {
     using namespace dec;
+    using V8 = typename Elem<T>::v8;
     extern __shared__ __attribute__((aligned(1024))) char smem_raw[];
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -77,10 +79,10 @@ __global__ __launch_bounds__(dec::WAVES * 64) void fmha_decode_split_kernel(
     const int col = min(l32, ncols - 1);
     const int hq = hkv * group + col / Sq;
     const int qi = col % Sq;
-    const half_t* qp = Q + b * q_batch + hq * q_head + qi * q_rstride + 8 * h;
-    half8 qf[8];
+    const T* qp = Q + b * q_batch + hq * q_head + qi * q_rstride + 8 * h;
+    V8 qf[8];
 #pragma unroll
-    for (int ks = 0; ks < 8; ++ks) qf[ks] = *(const half8*)(qp + ks * 16);
+    for (int ks = 0; ks < 8; ++ks) qf[ks] = *(const V8*)(qp + ks * 16);
     const int lim = causal ? min(kv_valid - 1, qi + shift) : kv_valid - 1;  // last visible key of this column
     // smallest such limit over the wave: tiles that end at or before it need no mask code
     int lim_min = lim;
@@ -88,8 +90,8 @@ __global__ __launch_bounds__(dec::WAVES * 64) void fmha_decode_split_kernel(
     for (int off = 32; off >= 1; off >>= 1) lim_min = min(lim_min, __shfl_xor(lim_min, off, 64));
     lim_min = __builtin_amdgcn_readfirstlane(lim_min);
 
-    const half_t* Kh = K + b * k_batch + hkv * k_head;
-    const half_t* Vh = V + b * v_batch + hkv * v_head;
+    const T* Kh = K + b * k_batch + hkv * k_head;
+    const T* Vh = V + b * v_batch + hkv * v_head;
 
     const int tiles = (kv_valid + TK - 1) / TK;
     const int t_begin = s_idx * tiles_per_split;
@@ -157,8 +159,8 @@ __global__ __launch_bounds__(dec::WAVES * 64) void fmha_decode_split_kernel(
         for (int e = 0; e < 16; ++e) s[e] = 0.f;
 #pragma unroll
         for (int ks = 0; ks < 8; ++ks) {
-            half8 kf = lds_read_b128(st + (k_base ^ (ks << 5)));
-            s = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf, qf[ks], s, 0, 0, 0);
+            V8 kf = Elem<T>::frag(lds_read_b128(st + (k_base ^ (ks << 5))));
+            s = Elem<T>::mfma32(kf, qf[ks], s);
         }
         const int key0 = t * TK;
         if (key0 + TK - 1 > lim_min) {
@@ -188,15 +190,15 @@ __global__ __launch_bounds__(dec::WAVES * 64) void fmha_decode_split_kernel(
         }
         const float neg_ms = (m_run == -INFINITY) ? 0.f : -m_run * scale_log2;
         float psum = 0.f;
-        half8 pf[2];
+        V8 pf[2];
 #pragma unroll
         for (int tt = 0; tt < 2; ++tt) {
-            half8 pk;
+            V8 pk;
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
                 float p = __builtin_amdgcn_exp2f(__builtin_fmaf(s[8 * tt + j], scale_log2, neg_ms));
                 psum += p;
-                pk[j] = (half_t)p;
+                pk[j] = (T)p;
             }
             pf[tt] = pk;
         }
@@ -207,8 +209,8 @@ __global__ __launch_bounds__(dec::WAVES * 64) void fmha_decode_split_kernel(
 #pragma unroll
             for (int db = 0; db < 4; ++db) {
                 int off = (v_base ^ (db << 6)) + (16 * tt) * ROW_BYTES;
-                half8 vf = concat(lds_read_tr16_b64(st + off), lds_read_tr16_b64(st + off + 8 * ROW_BYTES));
-                o[db] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf, pf[tt], o[db], 0, 0, 0);
+                V8 vf = Elem<T>::frag(concat(lds_read_tr16_b64(st + off), lds_read_tr16_b64(st + off + 8 * ROW_BYTES)));
+                o[db] = Elem<T>::mfma32(vf, pf[tt], o[db]);
             }
         wait_lgkmcnt<0>();  // the reads of this slot are complete before a later copy refills it
     }
@@ -237,11 +239,13 @@ __global__ __launch_bounds__(dec::WAVES * 64) void fmha_decode_split_kernel(
 // ranges spread over the threads (so their loads are independent), then thread d merges element d of O.
 constexpr int kMaxSplits = 512;
 
-__global__ __launch_bounds__(128) void fmha_decode_merge_kernel(const float* __restrict__ part, half_t* __restrict__ O,
+template <typename T>
+__global__ __launch_bounds__(128) void fmha_decode_merge_kernel(const float* __restrict__ part, T* __restrict__ O,
                                                                 float* __restrict__ LSE, int Hq, int Hkv, int Sq,
                                                                 float scale_log2, int splits, long o_batch, long o_head,
                                                                 long o_row) {
     using namespace dec;
+    using V8 = typename Elem<T>::v8;
     __shared__ float w_sh[kMaxSplits];
     __shared__ float red[128];
     const int tid = threadIdx.x;
@@ -285,7 +289,7 @@ __global__ __launch_bounds__(128) void fmha_decode_merge_kernel(const float* __r
     float acc = 0.f;
 #pragma unroll 8
     for (int s = 0; s < splits; ++s) acc += w_sh[s] * base[s * unit_stride + tid];
-    O[b * o_batch + hq * o_head + qi * o_row + tid] = (half_t)((l > 0.f) ? acc / l : 0.f);
+    O[b * o_batch + hq * o_head + qi * o_row + tid] = (T)((l > 0.f) ? acc / l : 0.f);
     if (LSE != nullptr && tid == 0)
         LSE[row] = (l > 0.f) ? (m * scale_log2 + __builtin_log2f(l)) * 0.69314718055994531f : -INFINITY;
 }
@@ -329,13 +333,14 @@ static hipError_t decode_workspace(size_t bytes, hipStream_t stream, float** out
     return hipSuccess;
 }
 
-hipError_t fmha_decode_dispatch(const half_t* Q, const half_t* K, const half_t* V, half_t* O, float* LSE, int B, int Hq,
+template <typename T>
+hipError_t fmha_decode_dispatch(const T* Q, const T* K, const T* V, T* O, float* LSE, int B, int Hq,
                                 int Hkv, int Sq, int Sk, float scale, int causal, int kv_valid, const FmhaStrides& sd,
                                 hipStream_t stream) {
     using namespace dec;
     static bool attr_set = false;
     if (!attr_set) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(fmha_decode_split_kernel),
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(fmha_decode_split_kernel<T>),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
         if (e != hipSuccess) return e;
         attr_set = true;
@@ -359,14 +364,19 @@ hipError_t fmha_decode_dispatch(const half_t* Q, const half_t* K, const half_t* 
     if (e != hipSuccess) return e;
     const float scale_log2 = scale * 1.4426950408889634f;
     const unsigned blocks = (unsigned)((units + WAVES - 1) / WAVES);
-    fmha_decode_split_kernel<<<dim3(blocks), dim3(WAVES * 64), LDS_BYTES, stream>>>(
+    fmha_decode_split_kernel<T><<<dim3(blocks), dim3(WAVES * 64), LDS_BYTES, stream>>>(
         Q, K, V, part, B, Hq, Hkv, Sq, Sk, scale_log2, causal, kv_valid, splits, tiles_per_split, (int)units, sd.q_batch,
         sd.q_head, sd.q_row, sd.k_batch, sd.k_head, sd.k_row, sd.v_batch, sd.v_head, sd.v_row);
     e = hipGetLastError();
     if (e != hipSuccess) return e;
-    fmha_decode_merge_kernel<<<dim3((unsigned)((long)B * Hq * Sq)), dim3(128), 0, stream>>>(
+    fmha_decode_merge_kernel<T><<<dim3((unsigned)((long)B * Hq * Sq)), dim3(128), 0, stream>>>(
         part, O, LSE, Hq, Hkv, Sq, scale_log2, splits, sd.o_batch, sd.o_head, sd.o_row);
     return hipGetLastError();
 }
+
+template hipError_t fmha_decode_dispatch<half_t>(const half_t*, const half_t*, const half_t*, half_t*, float*, int, int, int, int,
+                                                  int, float, int, int, const FmhaStrides&, hipStream_t);
+template hipError_t fmha_decode_dispatch<bf16_t>(const bf16_t*, const bf16_t*, const bf16_t*, bf16_t*, float*, int, int, int, int,
+                                                 int, float, int, int, const FmhaStrides&, hipStream_t);
 
 }  // namespace mi355

@@ -68,13 +68,15 @@ __device__ __forceinline__ void fmha_decode_block(int bid, int q_tiles, int grou
     hq = (g - b * Hkv) * group + hin;
 }
 
-template <int NQ, int NWAVES>
-__global__ __launch_bounds__(NWAVES * 64, (NQ == 1 ? 2 : 1)) void fmha_fwd_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K,
-                                                               const half_t* __restrict__ V, half_t* __restrict__ O,
+template <typename T, int NQ, int NWAVES>
+__global__ __launch_bounds__(NWAVES * 64, (NQ == 1 ? 2 : 1)) void fmha_fwd_kernel(const T* __restrict__ Q, const T* __restrict__ K,
+                                                               const T* __restrict__ V, T* __restrict__ O,
                                                                float* __restrict__ LSE, int B, int Hq, int Hkv, int Sq,
                                                                int Sk, float scale_log2, int causal, int kv_valid,
                                                                int q_tiles, FmhaStrides sd) {
     using namespace fmha;
+    using V8 = typename Elem<T>::v8;
+    using V4 = typename Elem<T>::v4;
     constexpr int BM = NWAVES * NQ * 32;
     constexpr int COPIES = (BN * ROW_BYTES / 1024) / NWAVES;  // wave-instructions per tile per wave
     static_assert(COPIES >= 1, "too many waves for the tile");
@@ -97,10 +99,10 @@ __global__ __launch_bounds__(NWAVES * 64, (NQ == 1 ? 2 : 1)) void fmha_fwd_kerne
     const int q_wave0 = q_block0 + wave * NQ * 32;  // first query row of this wave
     const int shift = Sk - Sq;
 
-    const half_t* Qh = Q + b * sd.q_batch + hq * sd.q_head;
-    const half_t* Kh = K + b * sd.k_batch + hkv * sd.k_head;
-    const half_t* Vh = V + b * sd.v_batch + hkv * sd.v_head;
-    half_t* Oh = O + b * sd.o_batch + hq * sd.o_head;
+    const T* Qh = Q + b * sd.q_batch + hq * sd.q_head;
+    const T* Kh = K + b * sd.k_batch + hkv * sd.k_head;
+    const T* Vh = V + b * sd.v_batch + hkv * sd.v_head;
+    T* Oh = O + b * sd.o_batch + hq * sd.o_head;
 
     // ---- number of key tiles this workgroup has to visit ----------------------------------------------
     int k_end = kv_valid;
@@ -111,13 +113,13 @@ __global__ __launch_bounds__(NWAVES * 64, (NQ == 1 ? 2 : 1)) void fmha_fwd_kerne
     const int n_tiles = (k_end + BN - 1) / BN;  // may be <= 0: no visible key for the whole tile
 
     // ---- Q fragments: lane holds Q[q = l32][d = 16*ks + 8*h .. +7] ---------------------------------------
-    half8 qf[NQ][8];
+    V8 qf[NQ][8];
 #pragma unroll
     for (int qb = 0; qb < NQ; ++qb) {
         int qrow = min(q_wave0 + qb * 32 + l32, Sq - 1);
-        const half_t* qp = Qh + qrow * sd.q_row + 8 * h;
+        const T* qp = Qh + qrow * sd.q_row + 8 * h;
 #pragma unroll
-        for (int ks = 0; ks < 8; ++ks) qf[qb][ks] = *(const half8*)(qp + ks * 16);
+        for (int ks = 0; ks < 8; ++ks) qf[qb][ks] = *(const V8*)(qp + ks * 16);
     }
 
     // ---- global -> LDS copy bookkeeping ----------------------------------------------------------------
@@ -187,10 +189,10 @@ __global__ __launch_bounds__(NWAVES * 64, (NQ == 1 ? 2 : 1)) void fmha_fwd_kerne
         for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
             for (int ks = 0; ks < 8; ++ks) {
-                half8 kf = lds_read_b128(st + ((k_base ^ (ks << 5)) + kb * 32 * ROW_BYTES));
+                V8 kf = Elem<T>::frag(lds_read_b128(st + ((k_base ^ (ks << 5)) + kb * 32 * ROW_BYTES)));
 #pragma unroll
                 for (int qb = 0; qb < NQ; ++qb)
-                    s[qb][kb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf, qf[qb][ks], s[qb][kb], 0, 0, 0);
+                    s[qb][kb] = Elem<T>::mfma32(kf, qf[qb][ks], s[qb][kb]);
             }
 
         // ---- mask (only tiles that touch the diagonal or the end of the valid keys) ----------------------
@@ -215,7 +217,7 @@ __global__ __launch_bounds__(NWAVES * 64, (NQ == 1 ? 2 : 1)) void fmha_fwd_kerne
         // raised (and O, l rescaled) when some row of the wave exceeds it by more than 2^kLazyLog2, which after the
         // first tiles almost never happens; until then P = exp2((S - m_run) * c) is at most 2^kLazyLog2, exact in
         // fp16/fp32 terms, and the final O / l and LSE do not depend on the choice of reference.
-        half8 pf[NQ][2][2];
+        V8 pf[NQ][2][2];
 #pragma unroll
         for (int qb = 0; qb < NQ; ++qb) {
             float mx = s[qb][0][0];
@@ -248,9 +250,9 @@ __global__ __launch_bounds__(NWAVES * 64, (NQ == 1 ? 2 : 1)) void fmha_fwd_kerne
                 }
 #pragma unroll
                 for (int tt = 0; tt < 2; ++tt) {
-                    half8 pk;
+                    V8 pk;
 #pragma unroll
-                    for (int j = 0; j < 8; ++j) pk[j] = (half_t)s[qb][kb][8 * tt + j];
+                    for (int j = 0; j < 8; ++j) pk[j] = (T)s[qb][kb][8 * tt + j];
                     pf[qb][kb][tt] = pk;
                 }
             }
@@ -267,10 +269,10 @@ __global__ __launch_bounds__(NWAVES * 64, (NQ == 1 ? 2 : 1)) void fmha_fwd_kerne
                     int off = (v_base ^ (db << 6)) + (kb * 32 + 16 * tt) * ROW_BYTES;
                     half4 lo = lds_read_tr16_b64(st + off);
                     half4 hi = lds_read_tr16_b64(st + off + 8 * ROW_BYTES);
-                    half8 vf = concat(lo, hi);
+                    V8 vf = Elem<T>::frag(concat(lo, hi));
 #pragma unroll
                     for (int qb = 0; qb < NQ; ++qb)
-                        o[qb][db] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf, pf[qb][kb][tt], o[qb][db], 0, 0, 0);
+                        o[qb][db] = Elem<T>::mfma32(vf, pf[qb][kb][tt], o[qb][db]);
                 }
     }
 
@@ -281,15 +283,15 @@ __global__ __launch_bounds__(NWAVES * 64, (NQ == 1 ? 2 : 1)) void fmha_fwd_kerne
         float inv = (l_tot > 0.f) ? 1.f / l_tot : 0.f;
         int qi = q_wave0 + qb * 32 + l32;
         if (qi < Sq) {
-            half_t* orow = Oh + qi * sd.o_row + 4 * h;
+            T* orow = Oh + qi * sd.o_row + 4 * h;
 #pragma unroll
             for (int db = 0; db < 4; ++db)
 #pragma unroll
                 for (int p = 0; p < 4; ++p) {
-                    half4 v;
+                    V4 v;
 #pragma unroll
-                    for (int q = 0; q < 4; ++q) v[q] = (half_t)(o[qb][db][4 * p + q] * inv);
-                    *(half4*)(orow + db * 32 + 8 * p) = v;
+                    for (int q = 0; q < 4; ++q) v[q] = (T)(o[qb][db][4 * p + q] * inv);
+                    *(V4*)(orow + db * 32 + 8 * p) = v;
                 }
             if (LSE != nullptr && h == 0) {
                 float lse = (l_tot > 0.f) ? (m_run[qb] * scale_log2 + __builtin_log2f(l_tot)) * 0.69314718055994531f
@@ -312,12 +314,15 @@ __global__ __launch_bounds__(NWAVES * 64, (NQ == 1 ? 2 : 1)) void fmha_fwd_kerne
 // K and V have separate double buffers: tile j lives in Kbuf[j&1] / Vbuf[j&1], is copied by all 8 waves at the
 // start of an even phase (K(i+1) and V(i) at P(2i)) and has two phases to land (waited for at the end of P(2i+1)).
 // ---------------------------------------------------------------------------------------------------------
-__global__ __launch_bounds__(512, 2) void fmha_fwd_pingpong_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K,
-                                                                   const half_t* __restrict__ V, half_t* __restrict__ O,
+template <typename T>
+__global__ __launch_bounds__(512, 2) void fmha_fwd_pingpong_kernel(const T* __restrict__ Q, const T* __restrict__ K,
+                                                                   const T* __restrict__ V, T* __restrict__ O,
                                                                    float* __restrict__ LSE, int B, int Hq, int Hkv, int Sq,
                                                                    int Sk, float scale_log2, int causal, int kv_valid,
                                                                    int q_tiles, FmhaStrides sd) {
     using namespace fmha;
+    using V8 = typename Elem<T>::v8;
+    using V4 = typename Elem<T>::v4;
     constexpr int NWAVES = 8;
     constexpr int BM = NWAVES * 32;
     constexpr int COPIES = (BN * ROW_BYTES / 1024) / NWAVES;  // 2 wave-instructions per tile per wave
@@ -342,21 +347,21 @@ __global__ __launch_bounds__(512, 2) void fmha_fwd_pingpong_kernel(const half_t*
     const int q_wave0 = q_block0 + wave * 32;
     const int shift = Sk - Sq;
 
-    const half_t* Qh = Q + b * sd.q_batch + hq * sd.q_head;
-    const half_t* Kh = K + b * sd.k_batch + hkv * sd.k_head;
-    const half_t* Vh = V + b * sd.v_batch + hkv * sd.v_head;
-    half_t* Oh = O + b * sd.o_batch + hq * sd.o_head;
+    const T* Qh = Q + b * sd.q_batch + hq * sd.q_head;
+    const T* Kh = K + b * sd.k_batch + hkv * sd.k_head;
+    const T* Vh = V + b * sd.v_batch + hkv * sd.v_head;
+    T* Oh = O + b * sd.o_batch + hq * sd.o_head;
 
     int k_end = kv_valid;
     if (causal) k_end = min(k_end, min(q_block0 + BM, Sq) - 1 + shift + 1);
     const int n_tiles = (k_end + BN - 1) / BN;  // may be <= 0: no visible key for the whole workgroup
 
-    half8 qf[8];
+    V8 qf[8];
     {
         int qrow = min(q_wave0 + l32, Sq - 1);
-        const half_t* qp = Qh + qrow * sd.q_row + 8 * h;
+        const T* qp = Qh + qrow * sd.q_row + 8 * h;
 #pragma unroll
-        for (int ks = 0; ks < 8; ++ks) qf[ks] = *(const half8*)(qp + ks * 16);
+        for (int ks = 0; ks < 8; ++ks) qf[ks] = *(const V8*)(qp + ks * 16);
     }
 
     // copy i of this wave covers tile rows (i*NWAVES + wave)*4 + lane/16, 16-byte chunk position lane%16
@@ -398,7 +403,7 @@ __global__ __launch_bounds__(512, 2) void fmha_fwd_pingpong_kernel(const half_t*
     // The compiler is free to move register-only work across s_barrier; these empty asm statements make a value
     // "used" at a program point, which keeps the softmax in the V phase and the MFMAs in the M phase.
     auto pin_s = [](float16v(&s)[2]) { asm volatile("" : "+v"(s[0]), "+v"(s[1])); };
-    auto pin_p = [](half8(&pf)[2][2]) { asm volatile("" : "+v"(pf[0][0]), "+v"(pf[0][1]), "+v"(pf[1][0]), "+v"(pf[1][1])); };
+    auto pin_p = [](V8(&pf)[2][2]) { asm volatile("" : "+v"(pf[0][0]), "+v"(pf[0][1]), "+v"(pf[1][0]), "+v"(pf[1][1])); };
     auto pin_o = [&]() { asm volatile("" : "+v"(o[0]), "+v"(o[1]), "+v"(o[2]), "+v"(o[3])); };
 
     // ---- phase bookkeeping -------------------------------------------------------------------------------------
@@ -418,12 +423,12 @@ __global__ __launch_bounds__(512, 2) void fmha_fwd_pingpong_kernel(const half_t*
     // ---- building blocks ----------------------------------------------------------------------------------------
     // LDS fragment reads, named so the M phase below can issue them long before their MFMA
     auto read_k = [&](MI355_LDS char* kst, int kb, int ks) {
-        return lds_read_b128(kst + ((k_base ^ (ks << 5)) + kb * 32 * ROW_BYTES));
+        return Elem<T>::frag(lds_read_b128(kst + ((k_base ^ (ks << 5)) + kb * 32 * ROW_BYTES)));
     };
     auto read_v = [&](MI355_LDS char* vst, int step) {  // step = (kb*2 + tt)*4 + db, the order the MFMAs consume them
         const int db = step & 3, tt = (step >> 2) & 1, kb = step >> 3;
         const int off = (v_base ^ (db << 6)) + (kb * 32 + 16 * tt) * ROW_BYTES;
-        return concat(lds_read_tr16_b64(vst + off), lds_read_tr16_b64(vst + off + 8 * ROW_BYTES));
+        return Elem<T>::frag(concat(lds_read_tr16_b64(vst + off), lds_read_tr16_b64(vst + off + 8 * ROW_BYTES)));
     };
     // The M phase in the exact order it should issue: every fragment is read 8 MFMAs (256 cycles) before the MFMA
     // that consumes it, into the register its predecessor has just released. sched_barrier pins that order.
@@ -433,7 +438,7 @@ __global__ __launch_bounds__(512, 2) void fmha_fwd_pingpong_kernel(const half_t*
     //   MFMAs 24..31: O += V^T P, fragments 8..15
     auto qk_tile = [&](int tile, float16v(&s)[2]) {  // S(tile) alone (first M phase of a wave)
         MI355_LDS char* kst = kbuf + (tile & 1) * TILE_BYTES;
-        half8 kf[8];
+        V8 kf[8];
 #pragma unroll
         for (int i = 0; i < 8; ++i) kf[i] = read_k(kst, 0, i);
 #pragma unroll
@@ -443,15 +448,15 @@ __global__ __launch_bounds__(512, 2) void fmha_fwd_pingpong_kernel(const half_t*
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
                 __builtin_amdgcn_sched_barrier(0);
-                s[kb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf[i], qf[i], s[kb], 0, 0, 0);
+                s[kb] = Elem<T>::mfma32(kf[i], qf[i], s[kb]);
                 if (kb == 0) kf[i] = read_k(kst, 1, i);
             }
         }
         __builtin_amdgcn_sched_barrier(0);
     };
-    auto pv_tile = [&](int tile, const half8(&pf)[2][2]) {  // O += V(tile)^T P alone (last M phase of a wave)
+    auto pv_tile = [&](int tile, const V8(&pf)[2][2]) {  // O += V(tile)^T P alone (last M phase of a wave)
         MI355_LDS char* vst = vbuf + (tile & 1) * TILE_BYTES;
-        half8 vf[8];
+        V8 vf[8];
 #pragma unroll
         for (int i = 0; i < 8; ++i) vf[i] = read_v(vst, i);
 #pragma unroll
@@ -460,15 +465,15 @@ __global__ __launch_bounds__(512, 2) void fmha_fwd_pingpong_kernel(const half_t*
             for (int i = 0; i < 8; ++i) {
                 __builtin_amdgcn_sched_barrier(0);
                 const int step = half * 8 + i;
-                o[step & 3] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf[i], pf[step >> 3][(step >> 2) & 1], o[step & 3], 0, 0, 0);
+                o[step & 3] = Elem<T>::mfma32(vf[i], pf[step >> 3][(step >> 2) & 1], o[step & 3]);
                 if (half == 0) vf[i] = read_v(vst, 8 + i);
             }
         __builtin_amdgcn_sched_barrier(0);
     };
-    auto m_phase = [&](int tile_k, float16v(&s)[2], int tile_v, const half8(&pf)[2][2]) {  // S(tile_k) and O += V(tile_v)^T P
+    auto m_phase = [&](int tile_k, float16v(&s)[2], int tile_v, const V8(&pf)[2][2]) {  // S(tile_k) and O += V(tile_v)^T P
         MI355_LDS char* kst = kbuf + (tile_k & 1) * TILE_BYTES;
         MI355_LDS char* vst = vbuf + (tile_v & 1) * TILE_BYTES;
-        half8 fr[8];
+        V8 fr[8];
 #pragma unroll
         for (int i = 0; i < 8; ++i) fr[i] = read_k(kst, 0, i);
 #pragma unroll
@@ -478,7 +483,7 @@ __global__ __launch_bounds__(512, 2) void fmha_fwd_pingpong_kernel(const half_t*
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
                 __builtin_amdgcn_sched_barrier(0);
-                s[kb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fr[i], qf[i], s[kb], 0, 0, 0);
+                s[kb] = Elem<T>::mfma32(fr[i], qf[i], s[kb]);
                 fr[i] = (kb == 0) ? read_k(kst, 1, i) : read_v(vst, i);
             }
         }
@@ -488,12 +493,12 @@ __global__ __launch_bounds__(512, 2) void fmha_fwd_pingpong_kernel(const half_t*
             for (int i = 0; i < 8; ++i) {
                 __builtin_amdgcn_sched_barrier(0);
                 const int step = half * 8 + i;
-                o[step & 3] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fr[i], pf[step >> 3][(step >> 2) & 1], o[step & 3], 0, 0, 0);
+                o[step & 3] = Elem<T>::mfma32(fr[i], pf[step >> 3][(step >> 2) & 1], o[step & 3]);
                 if (half == 0) fr[i] = read_v(vst, 8 + i);
             }
         __builtin_amdgcn_sched_barrier(0);
     };
-    auto softmax_tile = [&](float16v(&s)[2], int tile, half8(&pf)[2][2]) {
+    auto softmax_tile = [&](float16v(&s)[2], int tile, V8(&pf)[2][2]) {
         const int key0 = tile * BN;
         const bool need_mask = (key0 + BN > kv_valid) || (causal && (key0 + BN - 1 > q_wave0 + shift));
         if (need_mask) {
@@ -543,11 +548,11 @@ __global__ __launch_bounds__(512, 2) void fmha_fwd_pingpong_kernel(const half_t*
         for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
             for (int tt = 0; tt < 2; ++tt) {
-                half8 pk;
+                V8 pk;
 #pragma unroll
                 for (int j = 0; j < 8; ++j) {
                     ps[j & 3] += s[kb][8 * tt + j];
-                    pk[j] = (half_t)s[kb][8 * tt + j];
+                    pk[j] = (T)s[kb][8 * tt + j];
                 }
                 pf[kb][tt] = pk;
             }
@@ -564,7 +569,7 @@ __global__ __launch_bounds__(512, 2) void fmha_fwd_pingpong_kernel(const half_t*
         if (late) next_phase();  // waves 4..7 idle during P0
 
         float16v s[2];
-        half8 pf[2][2];
+        V8 pf[2][2];
         __builtin_amdgcn_s_setprio(1);
         qk_tile(0, s);
         __builtin_amdgcn_s_setprio(0);
@@ -594,15 +599,15 @@ __global__ __launch_bounds__(512, 2) void fmha_fwd_pingpong_kernel(const half_t*
     float inv = (l_tot > 0.f) ? 1.f / l_tot : 0.f;
     int qi = q_wave0 + l32;
     if (qi < Sq) {
-        half_t* orow = Oh + qi * sd.o_row + 4 * h;
+        T* orow = Oh + qi * sd.o_row + 4 * h;
 #pragma unroll
         for (int db = 0; db < 4; ++db)
 #pragma unroll
             for (int p = 0; p < 4; ++p) {
-                half4 v;
+                V4 v;
 #pragma unroll
-                for (int q = 0; q < 4; ++q) v[q] = (half_t)(o[db][4 * p + q] * inv);
-                *(half4*)(orow + db * 32 + 8 * p) = v;
+                for (int q = 0; q < 4; ++q) v[q] = (T)(o[db][4 * p + q] * inv);
+                *(V4*)(orow + db * 32 + 8 * p) = v;
             }
         if (LSE != nullptr && h == 0) {
             float lse = (l_tot > 0.f) ? (m_run * scale_log2 + __builtin_log2f(l_tot)) * 0.69314718055994531f : -INFINITY;
@@ -611,14 +616,15 @@ __global__ __launch_bounds__(512, 2) void fmha_fwd_pingpong_kernel(const half_t*
     }
 }
 
-static hipError_t launch_fmha_pingpong(const half_t* Q, const half_t* K, const half_t* V, half_t* O, float* LSE, int B, int Hq,
+template <typename T>
+static hipError_t launch_fmha_pingpong(const T* Q, const T* K, const T* V, T* O, float* LSE, int B, int Hq,
                                        int Hkv, int Sq, int Sk, float scale, int causal, int kv_valid, const FmhaStrides& sd,
                                        hipStream_t stream) {
     constexpr int BM = 256;
     constexpr int LDS = 4 * fmha::TILE_BYTES;
     static bool attr_set = false;
     if (!attr_set) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(fmha_fwd_pingpong_kernel),
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(fmha_fwd_pingpong_kernel<T>),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, LDS);
         if (e != hipSuccess) return e;
         attr_set = true;
@@ -627,18 +633,18 @@ static hipError_t launch_fmha_pingpong(const half_t* Q, const half_t* K, const h
     const long blocks = (long)q_tiles * Hq * B;
     if (blocks > 0x7fffffffL) return hipErrorInvalidValue;
     const float scale_log2 = scale * 1.4426950408889634f;
-    fmha_fwd_pingpong_kernel<<<dim3((unsigned)blocks), dim3(512), LDS, stream>>>(Q, K, V, O, LSE, B, Hq, Hkv, Sq, Sk, scale_log2,
+    fmha_fwd_pingpong_kernel<T><<<dim3((unsigned)blocks), dim3(512), LDS, stream>>>(Q, K, V, O, LSE, B, Hq, Hkv, Sq, Sk, scale_log2,
                                                                                 causal, kv_valid, q_tiles, sd);
     return hipGetLastError();
 }
 
-template <int NQ, int NWAVES>
-static hipError_t launch_fmha(const half_t* Q, const half_t* K, const half_t* V, half_t* O, float* LSE, int B, int Hq,
+template <typename T, int NQ, int NWAVES>
+static hipError_t launch_fmha(const T* Q, const T* K, const T* V, T* O, float* LSE, int B, int Hq,
                               int Hkv, int Sq, int Sk, float scale, int causal, int kv_valid, const FmhaStrides& sd,
                                        hipStream_t stream) {
     constexpr int BM = NWAVES * NQ * 32;
     constexpr int LDS = fmha::STAGE_BYTES * fmha::NSTAGE;
-    auto kern = fmha_fwd_kernel<NQ, NWAVES>;
+    auto kern = fmha_fwd_kernel<T, NQ, NWAVES>;
     static bool attr_set = false;
     if (!attr_set) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
@@ -657,26 +663,35 @@ static hipError_t launch_fmha(const half_t* Q, const half_t* K, const half_t* V,
 
 int g_fmha_variant = 0;  // tuning hook: 0 = heuristic, 1 = 4 waves x 32 queries, 2 = 8 waves x 32 queries, 3 = ping-pong
 
-hipError_t fmha_fwd_dispatch(const void* Q, const void* K, const void* V, void* O, float* LSE, int B, int Hq, int Hkv,
-                             int Sq, int Sk, float scale, int causal, int kv_valid_len, const FmhaStrides& sd,
-                             hipStream_t stream) {
-    const half_t* q = static_cast<const half_t*>(Q);
-    const half_t* k = static_cast<const half_t*>(K);
-    const half_t* v = static_cast<const half_t*>(V);
-    half_t* o = static_cast<half_t*>(O);
+template <typename T>
+static hipError_t fmha_fwd_dispatch_t(const void* Q, const void* K, const void* V, void* O, float* LSE, int B, int Hq, int Hkv,
+                                      int Sq, int Sk, float scale, int causal, int kv_valid_len, const FmhaStrides& sd,
+                                      hipStream_t stream) {
+    const T* q = static_cast<const T*>(Q);
+    const T* k = static_cast<const T*>(K);
+    const T* v = static_cast<const T*>(V);
+    T* o = static_cast<T*>(O);
     int variant = g_fmha_variant;
     if ((variant == 0 || variant == 4) && fmha_decode_applicable(B, Hq, Hkv, Sq, Sk, kv_valid_len))
-        return fmha_decode_dispatch(q, k, v, o, LSE, B, Hq, Hkv, Sq, Sk, scale, causal, kv_valid_len, sd, stream);
+        return fmha_decode_dispatch<T>(q, k, v, o, LSE, B, Hq, Hkv, Sq, Sk, scale, causal, kv_valid_len, sd, stream);
     if (variant == 0 || variant == 4) {
         // 256-query ping-pong workgroups once there are enough of them to fill the 256 CUs, otherwise 128-query ones
         const long wg256 = (long)((Sq + 255) / 256) * Hq * B;
         variant = (wg256 >= 256) ? 3 : 1;
     }
     switch (variant) {
-        case 2: return launch_fmha<1, 8>(q, k, v, o, LSE, B, Hq, Hkv, Sq, Sk, scale, causal, kv_valid_len, sd, stream);
-        case 3: return launch_fmha_pingpong(q, k, v, o, LSE, B, Hq, Hkv, Sq, Sk, scale, causal, kv_valid_len, sd, stream);
-        default: return launch_fmha<1, 4>(q, k, v, o, LSE, B, Hq, Hkv, Sq, Sk, scale, causal, kv_valid_len, sd, stream);
+        case 2: return launch_fmha<T, 1, 8>(q, k, v, o, LSE, B, Hq, Hkv, Sq, Sk, scale, causal, kv_valid_len, sd, stream);
+        case 3: return launch_fmha_pingpong<T>(q, k, v, o, LSE, B, Hq, Hkv, Sq, Sk, scale, causal, kv_valid_len, sd, stream);
+        default: return launch_fmha<T, 1, 4>(q, k, v, o, LSE, B, Hq, Hkv, Sq, Sk, scale, causal, kv_valid_len, sd, stream);
     }
+}
+
+hipError_t fmha_fwd_dispatch(const void* Q, const void* K, const void* V, void* O, float* LSE, int B, int Hq, int Hkv,
+                             int Sq, int Sk, float scale, int causal, int kv_valid_len, const FmhaStrides& sd, int dtype,
+                             hipStream_t stream) {
+    if (dtype == MI355_DTYPE_BF16)
+        return fmha_fwd_dispatch_t<bf16_t>(Q, K, V, O, LSE, B, Hq, Hkv, Sq, Sk, scale, causal, kv_valid_len, sd, stream);
+    return fmha_fwd_dispatch_t<half_t>(Q, K, V, O, LSE, B, Hq, Hkv, Sq, Sk, scale, causal, kv_valid_len, sd, stream);
 }
 
 }  // namespace mi355

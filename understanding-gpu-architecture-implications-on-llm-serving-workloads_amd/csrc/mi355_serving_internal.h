@@ -20,13 +20,13 @@ struct FmhaStrides {
 // Launches the attention forward kernels; arguments as mi355_fmha_fwd_strided after validation.
 hipError_t fmha_fwd_dispatch(const void* Q, const void* K, const void* V, void* O, float* LSE, int B, int Hq, int Hkv,
                              int Sq, int Sk, float scale, int causal, int kv_valid_len, const FmhaStrides& strides,
-                             hipStream_t stream);
+                             int dtype, hipStream_t stream);
 
 // Split-KV path for few query rows per kv head (generation step); see fmha_decode.hip.
 bool fmha_decode_applicable(int B, int Hq, int Hkv, int Sq, int Sk, int kv_valid_len);
-hipError_t fmha_decode_dispatch(const _Float16* Q, const _Float16* K, const _Float16* V, _Float16* O, float* LSE, int B, int Hq,
-                                int Hkv, int Sq, int Sk, float scale, int causal, int kv_valid_len, const FmhaStrides& strides,
-                                hipStream_t stream);
+template <typename T>
+hipError_t fmha_decode_dispatch(const T* Q, const T* K, const T* V, T* O, float* LSE, int B, int Hq, int Hkv, int Sq, int Sk,
+                                float scale, int causal, int kv_valid_len, const FmhaStrides& strides, hipStream_t stream);
 
 // Layer glue (glue.hip); arguments as the mi355_rmsnorm / mi355_rope / mi355_silu_mul entry points after validation.
 hipError_t rmsnorm_dispatch(const void* x, const void* residual, void* res_out, const void* weight, void* out, long rows,

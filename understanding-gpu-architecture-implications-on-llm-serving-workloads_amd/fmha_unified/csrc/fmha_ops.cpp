@@ -3,7 +3,8 @@
 // Same operator surface as the reference (kernels/fmha/pkg/fmha_unified/csrc/fmha_kernel.cpp:9-18): schemas
 // `fmha_unified::finefmha_0 .. finefmha_7 (Tensor q, Tensor k, Tensor v, bool causal, bool is_decode,
 // int decode_length) -> Tensor`, CUDA dispatch key, empty `_C` module. Every index runs the one gfx950
-// attention kernel of libmi355_serving.so. Host checks mirror semi/fmha_2_amd.cpp:322-333 (fp16, d == 128,
+// attention kernel of libmi355_serving.so, for float16 or bfloat16 tensors. Host checks mirror
+// semi/fmha_2_amd.cpp:322-333 (dtype, d == 128,
 // is_decode implies !causal) and add the shape checks the reference omits.
 //
 // One operator is added without touching the reference's schemas:
@@ -44,9 +45,10 @@ std::tuple<at::Tensor, at::Tensor> run_fmha(const at::Tensor& q, const at::Tenso
                                             bool is_decode, int64_t decode_length, bool want_lse) {
     const char* name = "finefmha";
     TORCH_CHECK(q.dim() == 4 && k.dim() == 4 && v.dim() == 4, name, ": q, k, v must be [B, H, S, D] tensors");
-    TORCH_CHECK(q.scalar_type() == at::kHalf, name, ": q must be float16, got ", q.scalar_type());
-    TORCH_CHECK(k.scalar_type() == at::kHalf, name, ": k must be float16, got ", k.scalar_type());
-    TORCH_CHECK(v.scalar_type() == at::kHalf, name, ": v must be float16, got ", v.scalar_type());
+    const bool bf16 = q.scalar_type() == at::kBFloat16;  // the dtype of the reference's finefmha_5 (manual/fmha_5_nv.cu:148-150)
+    TORCH_CHECK(q.scalar_type() == at::kHalf || bf16, name, ": q must be float16 or bfloat16, got ", q.scalar_type());
+    TORCH_CHECK(k.scalar_type() == q.scalar_type(), name, ": k must have q's dtype ", q.scalar_type(), ", got ", k.scalar_type());
+    TORCH_CHECK(v.scalar_type() == q.scalar_type(), name, ": v must have q's dtype ", q.scalar_type(), ", got ", v.scalar_type());
     const int64_t B = q.size(0), Hq = q.size(1), Sq = q.size(2), D = q.size(3);
     const int64_t Hkv = k.size(1), Sk = k.size(2);
     TORCH_CHECK(D == 128, name, ": head embedding dimension must be 128, got ", D);
@@ -79,9 +81,9 @@ std::tuple<at::Tensor, at::Tensor> run_fmha(const at::Tensor& q, const at::Tenso
     hipStream_t stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream();
     const int64_t strides[12] = {qc.stride(0), qc.stride(1), qc.stride(2), kc.stride(0), kc.stride(1), kc.stride(2),
                                  vc.stride(0), vc.stride(1), vc.stride(2), o.stride(0),  o.stride(1),  o.stride(2)};
-    int rc = mi355_fmha_fwd_strided(qc.data_ptr(), kc.data_ptr(), vc.data_ptr(), o.data_ptr(), lse_ptr, (int)B, (int)Hq,
-                                    (int)Hkv, (int)Sq, (int)Sk, (int)D, scale, causal ? 1 : 0, (int)decode_length, strides,
-                                    stream);
+    auto entry = bf16 ? &mi355_fmha_fwd_bf16 : &mi355_fmha_fwd_strided;
+    int rc = entry(qc.data_ptr(), kc.data_ptr(), vc.data_ptr(), o.data_ptr(), lse_ptr, (int)B, (int)Hq, (int)Hkv, (int)Sq,
+                   (int)Sk, (int)D, scale, causal ? 1 : 0, (int)decode_length, strides, stream);
     TORCH_CHECK(rc == 0, name, ": ", mi355_last_error(), " (code ", rc, ")");
     return {o, lse};
 }

@@ -13,7 +13,7 @@ LIB_PATH = os.path.join(_HERE, "libmi355_serving.so")
 GEMM_NN, GEMM_NT, GEMM_TN = 0, 1, 2
 LAYOUTS = {"NN": GEMM_NN, "NT": GEMM_NT, "TN": GEMM_TN}
 
-EXPORTED_SYMBOLS = ("mi355_hgemm", "mi355_fmha_fwd", "mi355_fmha_fwd_strided", "mi355_rmsnorm", "mi355_rope", "mi355_silu_mul",
+EXPORTED_SYMBOLS = ("mi355_hgemm", "mi355_fmha_fwd", "mi355_fmha_fwd_strided", "mi355_fmha_fwd_bf16", "mi355_rmsnorm", "mi355_rope", "mi355_silu_mul",
                     "mi355_last_error", "mi355_serving_version",
                     "mi355_debug_set_gemm_variant", "mi355_debug_set_fmha_variant")
 
@@ -44,6 +44,8 @@ def load():
     lib.mi355_fmha_fwd_strided.argtypes = [vp, vp, vp, vp, vp, i32, i32, i32, i32, i32, i32, f32, i32, i32,
                                            ctypes.POINTER(i64), vp]
     lib.mi355_fmha_fwd_strided.restype = i32
+    lib.mi355_fmha_fwd_bf16.argtypes = lib.mi355_fmha_fwd_strided.argtypes
+    lib.mi355_fmha_fwd_bf16.restype = i32
     lib.mi355_rmsnorm.argtypes = [vp, vp, vp, vp, vp, i64, i32, i64, i64, i64, i64, f32, vp]
     lib.mi355_rmsnorm.restype = i32
     lib.mi355_rope.argtypes = [vp, vp, i32, i32, i32, i32, i64, i64, i64, i64, vp, vp, vp, i32, vp]
@@ -131,9 +133,10 @@ def fmha_fwd(q, k, v, causal=False, kv_valid_len=None, scale=None, return_lse=Tr
 
     q, k, v (and `out`, if given) are [B, H, S, D] fp16 GPU tensors or views with a contiguous last dimension, e.g.
     `x.view(B, S, H, D).transpose(1, 2)`; contiguous tensors take mi355_fmha_fwd, views mi355_fmha_fwd_strided.
+    bfloat16 tensors take mi355_fmha_fwd_bf16.
     """
     import torch
-    assert q.dtype == torch.float16 and q.is_cuda
+    assert q.dtype in (torch.float16, torch.bfloat16) and q.dtype == k.dtype == v.dtype and q.is_cuda
     B, Hq, Sq, D = q.shape
     _, Hkv, Sk, _ = k.shape
     if scale is None:
@@ -143,7 +146,12 @@ def fmha_fwd(q, k, v, causal=False, kv_valid_len=None, scale=None, return_lse=Tr
     o = torch.empty_like(q) if out is None else out
     lse = torch.empty((B, Hq, Sq), dtype=torch.float32, device=q.device) if return_lse else None
     stream = torch.cuda.current_stream(q.device).cuda_stream
-    if all(t.is_contiguous() for t in (q, k, v, o)):
+    if q.dtype == torch.bfloat16:
+        assert all(t.stride(3) == 1 for t in (q, k, v, o)), "the last dimension must be contiguous"
+        arr = (ctypes.c_int64 * 12)(*(_bhs_strides(q) + _bhs_strides(k) + _bhs_strides(v) + _bhs_strides(o)))
+        _check(load().mi355_fmha_fwd_bf16(_ptr(q), _ptr(k), _ptr(v), _ptr(o), _ptr(lse), B, Hq, Hkv, Sq, Sk, D, float(scale),
+                                          int(bool(causal)), int(kv_valid_len), arr, stream))
+    elif all(t.is_contiguous() for t in (q, k, v, o)):
         fmha_fwd_raw(_ptr(q), _ptr(k), _ptr(v), _ptr(o), _ptr(lse), B, Hq, Hkv, Sq, Sk, D, float(scale), int(bool(causal)),
                      int(kv_valid_len), stream)
     else:
