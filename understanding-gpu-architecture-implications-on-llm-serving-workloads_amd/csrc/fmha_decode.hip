@@ -99,19 +99,26 @@ __global__ __launch_bounds__(dec::WAVES * 64) void fmha_decode_split_kernel(
 
     // copy i (0..7) of a tile covers rows 4i + lane/16, chunk position lane%16
     const int c_row = lane >> 4;
+    // addresses = wave-uniform tile base (scalar registers) + 32-bit lane offset; rows past the last valid key are
+    // clamped onto it (masked later, but V must not feed NaNs into 0 * V)
+    const uint32_t k_row_bytes = (uint32_t)k_rstride * 2, v_row_bytes = (uint32_t)v_rstride * 2;
+    const uint32_t kcol = (lane & 15), c_row4 = c_row;
     auto issue_stage = [&](int tile, int slot) {
         MI355_LDS char* st = wbase + slot * STAGE_BYTES;
+        const int tile_u = __builtin_amdgcn_readfirstlane(tile);
+        const char* kb = (const char*)Kh + (long)tile_u * TK * k_rstride * 2;
+        const char* vb = (const char*)Vh + (long)tile_u * TK * v_rstride * 2;
+        const int last = kv_valid - 1 - tile_u * TK;
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
-            int row = 4 * i + c_row;
-            int grow = min(tile * TK + row, kv_valid - 1);
-            copy16_global_to_lds(Kh + grow * k_rstride + ((lane & 15) ^ swz_k(row)) * 8, st + i * 1024);
+            int row = 4 * i + c_row4;
+            copy16_global_to_lds(kb, (uint32_t)min(row, last) * k_row_bytes + ((kcol ^ swz_k(row)) << 4), st + i * 1024);
         }
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
-            int row = 4 * i + c_row;
-            int grow = min(tile * TK + row, kv_valid - 1);
-            copy16_global_to_lds(Vh + grow * v_rstride + ((lane & 15) ^ swz_v(row)) * 8, st + TILE_BYTES + i * 1024);
+            int row = 4 * i + c_row4;
+            copy16_global_to_lds(vb, (uint32_t)min(row, last) * v_row_bytes + ((kcol ^ swz_v(row)) << 4),
+                                 st + TILE_BYTES + i * 1024);
         }
     };
 

@@ -364,28 +364,34 @@ __global__ __launch_bounds__(512, 2) void fmha_fwd_pingpong_kernel(const T* __re
         for (int ks = 0; ks < 8; ++ks) qf[ks] = *(const V8*)(qp + ks * 16);
     }
 
-    // copy i of this wave covers tile rows (i*NWAVES + wave)*4 + lane/16, 16-byte chunk position lane%16
-    int copy_row[COPIES], copy_kcol[COPIES], copy_vcol[COPIES];
+    // copy i of this wave covers tile rows (i*NWAVES + wave)*4 + lane/16, 16-byte chunk position lane%16.
+    // Addresses = wave-uniform tile base (scalar registers) + 32-bit lane offset; rows past the last valid key are
+    // clamped onto it (they are masked later, but V must not feed NaNs into 0 * V).
+    int copy_row[COPIES];
+    uint32_t copy_kcol[COPIES], copy_vcol[COPIES];
 #pragma unroll
     for (int i = 0; i < COPIES; ++i) {
         int row = (i * NWAVES + wave) * 4 + (lane >> 4);
         copy_row[i] = row;
-        copy_kcol[i] = ((lane & 15) ^ swz_k(row)) * 8;
-        copy_vcol[i] = ((lane & 15) ^ swz_v(row)) * 8;
+        copy_kcol[i] = ((lane & 15) ^ swz_k(row)) * 16;
+        copy_vcol[i] = ((lane & 15) ^ swz_v(row)) * 16;
     }
+    const uint32_t k_row_bytes = (uint32_t)sd.k_row * 2, v_row_bytes = (uint32_t)sd.v_row * 2;
     auto issue_k = [&](int tile) {
+        const char* base = (const char*)Kh + (long)tile * BN * sd.k_row * 2;
+        const int last = kv_valid - 1 - tile * BN;
 #pragma unroll
-        for (int i = 0; i < COPIES; ++i) {
-            int krow = min(tile * BN + copy_row[i], kv_valid - 1);
-            copy16_global_to_lds(Kh + krow * sd.k_row + copy_kcol[i], kbuf + (tile & 1) * TILE_BYTES + (i * NWAVES + wave) * 1024);
-        }
+        for (int i = 0; i < COPIES; ++i)
+            copy16_global_to_lds(base, (uint32_t)min(copy_row[i], last) * k_row_bytes + copy_kcol[i],
+                                 kbuf + (tile & 1) * TILE_BYTES + (i * NWAVES + wave) * 1024);
     };
     auto issue_v = [&](int tile) {
+        const char* base = (const char*)Vh + (long)tile * BN * sd.v_row * 2;
+        const int last = kv_valid - 1 - tile * BN;
 #pragma unroll
-        for (int i = 0; i < COPIES; ++i) {
-            int krow = min(tile * BN + copy_row[i], kv_valid - 1);
-            copy16_global_to_lds(Vh + krow * sd.v_row + copy_vcol[i], vbuf + (tile & 1) * TILE_BYTES + (i * NWAVES + wave) * 1024);
-        }
+        for (int i = 0; i < COPIES; ++i)
+            copy16_global_to_lds(base, (uint32_t)min(copy_row[i], last) * v_row_bytes + copy_vcol[i],
+                                 vbuf + (tile & 1) * TILE_BYTES + (i * NWAVES + wave) * 1024);
     };
 
     const int k_base = l32 * ROW_BYTES + ((h ^ (lane & 15)) << 4);  // xor (ks << 5), + kb * 32 * ROW_BYTES
@@ -672,13 +678,16 @@ static hipError_t fmha_fwd_dispatch_t(const void* Q, const void* K, const void* 
     const T* v = static_cast<const T*>(V);
     T* o = static_cast<T*>(O);
     int variant = g_fmha_variant;
-    if ((variant == 0 || variant == 4) && fmha_decode_applicable(B, Hq, Hkv, Sq, Sk, kv_valid_len))
+    // the split-KV and ping-pong kernels address a K/V tile with 32-bit byte offsets from its first row
+    const bool rows_fit_32bit = sd.k_row < (1L << 24) && sd.v_row < (1L << 24);
+    if ((variant == 0 || variant == 4) && rows_fit_32bit && fmha_decode_applicable(B, Hq, Hkv, Sq, Sk, kv_valid_len))
         return fmha_decode_dispatch<T>(q, k, v, o, LSE, B, Hq, Hkv, Sq, Sk, scale, causal, kv_valid_len, sd, stream);
     if (variant == 0 || variant == 4) {
         // 256-query ping-pong workgroups once there are enough of them to fill the 256 CUs, otherwise 128-query ones
         const long wg256 = (long)((Sq + 255) / 256) * Hq * B;
         variant = (wg256 >= 256) ? 3 : 1;
     }
+    if (variant == 3 && !rows_fit_32bit) variant = 1;
     switch (variant) {
         case 2: return launch_fmha<T, 1, 8>(q, k, v, o, LSE, B, Hq, Hkv, Sq, Sk, scale, causal, kv_valid_len, sd, stream);
         case 3: return launch_fmha_pingpong<T>(q, k, v, o, LSE, B, Hq, Hkv, Sq, Sk, scale, causal, kv_valid_len, sd, stream);

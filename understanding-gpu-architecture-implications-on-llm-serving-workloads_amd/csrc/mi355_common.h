@@ -59,6 +59,19 @@ __device__ __forceinline__ void copy16_global_to_lds(const void* gptr, MI355_LDS
         : "memory", "m0");
 }
 
+// The same copy with the address split into a wave-uniform 64-bit base (kept in scalar registers) and a 32-bit
+// per-lane byte offset: per-tile address arithmetic then runs on the scalar unit and a lane needs one VALU add or none.
+__device__ __forceinline__ void copy16_global_to_lds(const void* uniform_base, uint32_t lane_byte_offset,
+                                                     MI355_LDS void* lds_wave_base) {
+    asm volatile(
+        "s_mov_b32 m0, %2\n\t"
+        "s_nop 0\n\t"
+        "global_load_lds_dwordx4 %0, %1"
+        :
+        : "v"(lane_byte_offset), "s"(uniform_base), "s"((uint32_t)(uintptr_t)lds_wave_base)
+        : "memory", "m0");
+}
+
 __device__ __forceinline__ half4 lds_read_tr16_b64(MI355_LDS const void* p) {
     short4v t = __builtin_amdgcn_ds_read_tr16_b64_v4i16((MI355_LDS short4v*)p);
     return __builtin_bit_cast(half4, t);
