@@ -67,6 +67,9 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-other-configs", action="store_true")
     ap.add_argument("--no-check", action="store_true")
+    ap.add_argument("--layer-only", choices=["prefill", "step"], default=None,
+                    help="run only the Llama-3-8B-shaped decoder layer (prefill at s=8192, or a generation step at batch 8 over "
+                         "8192 cached tokens) for --steps iterations and print its timing; for per-kernel profiles")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also launch one 1 GiB device-to-device copy, so FETCH_SIZE / WRITE_SIZE read under rocprofv3 "
                          "--pmc can be scaled by what the same counter reports for a transfer of known size")
@@ -84,6 +87,24 @@ def main():
     lib.load()
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+
+    if args.layer_only:
+        layer, S5 = llama3_8b_layer(torch, so, dev)
+        from llama_layer import FineKVCache
+        if args.layer_only == "prefill":
+            x = so.randn_fp16((1, S5, 4096), 18).to(dev)
+            fn = lambda: layer(x)
+        else:
+            cache = FineKVCache(8, S5 + 64, 8, device=dev)
+            cache.k.normal_(0, 1)
+            cache.v.normal_(0, 1)
+            x = so.randn_fp16((8, 1, 4096), 19).to(dev)
+            def fn():
+                cache.length = S5
+                layer(x, kv_cache=cache)
+        ms = time_launches(fn, args.steps, args.warmup)
+        print(json.dumps({"layer_only": args.layer_only, "ms": ms, "steps": args.steps, "warmup": args.warmup}))
+        return
 
     # ---- synthetic inputs, resident in HBM -------------------------------------------------------------------
     M = N = K = 8192
@@ -235,12 +256,8 @@ def main():
         # the same layer as the in-model adapter runs it: nn.Linear-layout weights, norms, RoPE, residuals, no layout copies
         del x5, wqkv, wo, wgu, wd, qkv5, q5, k5, v5, o5, a5, op5, gu5, act5, dn5
         torch.cuda.empty_cache()
-        from llama_layer import FineKVCache, FineLlamaDecoderLayer
-        gw = lambda shape, seed: so.randn_fp16(shape, seed, 0.02).to(dev)
-        wl = dict(q=gw((4096, H5), 11), k=gw((1024, H5), 12), v=gw((1024, H5), 13), o=gw((H5, 4096), 14), gate=gw((F5, H5), 15),
-                  up=gw((F5, H5), 16), down=gw((H5, F5), 17), ln1=torch.ones(H5, dtype=torch.float16, device=dev),
-                  ln2=torch.ones(H5, dtype=torch.float16, device=dev))
-        layer = FineLlamaDecoderLayer(wl, 32, 8, max_positions=S5 + 64)
+        from llama_layer import FineKVCache
+        layer, _ = llama3_8b_layer(torch, so, dev)
         xl = so.randn_fp16((1, S5, H5), 18).to(dev)
         ms_l = time_launches(lambda: layer(xl), 5, 2)
         other["L5_decoder_layer_prefill_s8192"] = {
@@ -260,7 +277,7 @@ def main():
         other["L5_decoder_layer_generation_step_b8_past8192"] = {"ms": ms_s, "gbs": by_s / ms_s / 1e6,
                                                                  "pct_of_hbm_peak": 100 * by_s / ms_s / 1e6 / PEAK_HBM_GBS,
                                                                  "note": "bytes = layer weights + KV cache read once"}
-        del layer, cache, wl
+        del layer, cache
 
     # ---- CPU baseline: the same step with torch fp32 on the host cores -------------------------------------------------
     cpu_baseline = None
@@ -292,6 +309,16 @@ def main():
         "other_configs": other, "parity": checks,
     }
     print(json.dumps(out))
+
+
+def llama3_8b_layer(torch, so, dev, S5=8192, H5=4096, F5=14336):
+    """FineLlamaDecoderLayer at Llama-3-8B shapes (32 q / 8 kv heads of 128) with seeded random weights."""
+    from llama_layer import FineLlamaDecoderLayer
+    gw = lambda shape, seed: so.randn_fp16(shape, seed, 0.02).to(dev)
+    wl = dict(q=gw((4096, H5), 11), k=gw((1024, H5), 12), v=gw((1024, H5), 13), o=gw((H5, 4096), 14), gate=gw((F5, H5), 15),
+              up=gw((F5, H5), 16), down=gw((H5, F5), 17), ln1=torch.ones(H5, dtype=torch.float16, device=dev),
+              ln2=torch.ones(H5, dtype=torch.float16, device=dev))
+    return FineLlamaDecoderLayer(wl, 32, 8, max_positions=S5 + 64), S5
 
 
 def _cpu_model():

@@ -121,16 +121,18 @@ int mi355_rmsnorm(const void* x, const void* residual, void* residual_out, const
 
 /*
  * mi355_rope: rotary position embedding of `heads` consecutive 128-wide heads of every token (rotate_half convention,
- *   modeling_llama.py:164-168,193-194): for i < 64, with c = cos_table[p][i], s = sin_table[p][i], p = positions[b*S + t]:
+ *   modeling_llama.py:164-168,193-194): for i < 64, with c = cos_table[p][i], s = sin_table[p][i],
+ *   p = positions[b*pos_batch + t] (pos_batch = S for a [B, S] table, 0 when all batch rows share one [S] table):
  *     out[i] = x[i] c - x[i+64] s,   out[i+64] = x[i+64] c + x[i] s.
  *   Token (b, t) lives at x + b*x_batch + t*x_row (+ head*128), likewise for out, so q and k can be rotated inside a fused
- *   QKV projection (out == x) or k written straight into a KV cache. cos_table / sin_table: [n_positions][64] fp32, the
+ *   QKV projection (out == x) or k written straight into a KV cache. The `copy_heads` heads that follow the rotated ones are
+ *   copied unrotated (the value heads, when k and v go into one cache tensor with a single launch). cos_table / sin_table: [n_positions][64] fp32, the
  *   first half of what LlamaRotaryEmbedding.forward builds (modeling_llama.py:119-132); positions outside
  *   [0, n_positions) are clamped.
  */
-int mi355_rope(const void* x, void* out, int B, int S, int heads, int D, int64_t x_batch, int64_t x_row, int64_t out_batch,
-               int64_t out_row, const float* cos_table, const float* sin_table, const int32_t* positions, int n_positions,
-               void* stream);
+int mi355_rope(const void* x, void* out, int B, int S, int heads, int copy_heads, int D, int64_t x_batch, int64_t x_row,
+               int64_t out_batch, int64_t out_row, const float* cos_table, const float* sin_table, const int32_t* positions,
+               int64_t pos_batch, int n_positions, void* stream);
 
 /*
  * mi355_silu_mul: out[r][j] = silu(g[r][j]) * u[r][j] with g = gate_up[r][0 .. inter), u = gate_up[r][inter .. 2 inter)

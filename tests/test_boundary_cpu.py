@@ -55,9 +55,9 @@ def test_capi_rejects_bad_arguments_without_a_gpu(lib):
     assert cdll.mi355_rmsnorm(p, None, None, p, p, 4, 100, 104, 0, 0, 104, 1e-5, None) == 10001   # hidden % 8
     assert cdll.mi355_rmsnorm(p, p, None, p, p, 4, 128, 128, 128, 128, 128, 1e-5, None) == 10001   # residual without residual_out
     assert cdll.mi355_rmsnorm(p, None, None, p, p, 4, 128, 64, 0, 0, 128, 1e-5, None) == 10001     # ldx < hidden
-    assert cdll.mi355_rope(p, p, 1, 4, 2, 64, 1024, 256, 1024, 256, p, p, p, 16, None) == 10002    # head_dim != 128
-    assert cdll.mi355_rope(p, p, 1, 4, 2, 128, 1024, 128, 1024, 256, p, p, p, 16, None) == 10001   # row stride < heads * 128
-    assert cdll.mi355_rope(p, p, 1, 4, 2, 128, 1024, 256, 1024, 256, p, p, None, 16, None) == 10001
+    assert cdll.mi355_rope(p, p, 1, 4, 2, 0, 64, 1024, 256, 1024, 256, p, p, p, 0, 16, None) == 10002    # head_dim != 128
+    assert cdll.mi355_rope(p, p, 1, 4, 1, 1, 128, 1024, 128, 1024, 256, p, p, p, 0, 16, None) == 10001   # row stride < heads * 128
+    assert cdll.mi355_rope(p, p, 1, 4, 2, 0, 128, 1024, 256, 1024, 256, p, p, None, 0, 16, None) == 10001
     assert cdll.mi355_silu_mul(p, p, 4, 64, 64, 64, None) == 10001                                  # ld_in < 2 * inter
     assert cdll.mi355_silu_mul(p, p, 0, 64, 128, 64, None) == 10001
     with pytest.raises(lib.Mi355Error):

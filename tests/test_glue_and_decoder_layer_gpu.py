@@ -72,6 +72,20 @@ def test_rope_in_place_and_into_a_cache(lib, gpu, B, S, heads):
     assert float(cache[:, :4].abs().max()) == 0.0 and float(cache[:, 4 + S:].abs().max()) == 0.0
 
 
+def test_rope_copies_value_heads_and_shares_one_position_table(lib, gpu):
+    # k heads rotated and v heads copied into a fused K|V cache row by one launch; one [S] position table for all batch rows
+    B, S, n_kv = 3, 17, 5
+    cos, sin = so.rope_tables(64, 128, 10000.0)
+    pos = torch.arange(20, 20 + S, dtype=torch.int32)
+    kv = so.randn_fp16((B, S, 2 * n_kv, 128), 12)
+    ref_k = so.rope_ref(kv[:, :, :n_kv].transpose(1, 2), cos, sin, pos[None].expand(B, S)).transpose(1, 2)
+    cache = torch.zeros((B, 40, 2 * n_kv, 128), dtype=torch.float16, device=gpu)
+    lib.rope(kv.to(gpu), cos.to(gpu), sin.to(gpu), pos.to(gpu), out=cache[:, 20:20 + S], copy_heads=n_kv)
+    assert close_one_rounding(cache[:, 20:20 + S, :n_kv], ref_k)[0]
+    assert torch.equal(cache[:, 20:20 + S, n_kv:].cpu(), kv[:, :, n_kv:])
+    assert float(cache[:, :20].abs().max()) == 0.0 and float(cache[:, 20 + S:].abs().max()) == 0.0
+
+
 @pytest.mark.parametrize("rows,inter", [(1, 8), (9, 14336), (70000, 16), (257, 1000)])
 def test_silu_mul(lib, gpu, rows, inter):
     gu = so.randn_fp16((rows, 2 * inter), 9, 3.0)

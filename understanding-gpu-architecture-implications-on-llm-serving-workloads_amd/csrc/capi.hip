@@ -120,20 +120,20 @@ int mi355_rmsnorm(const void* x, const void* residual, void* residual_out, const
     return 0;
 }
 
-int mi355_rope(const void* x, void* out, int B, int S, int heads, int D, int64_t x_batch, int64_t x_row, int64_t out_batch,
-               int64_t out_row, const float* cos_table, const float* sin_table, const int32_t* positions, int n_positions,
-               void* stream) {
+int mi355_rope(const void* x, void* out, int B, int S, int heads, int copy_heads, int D, int64_t x_batch, int64_t x_row,
+               int64_t out_batch, int64_t out_row, const float* cos_table, const float* sin_table, const int32_t* positions,
+               int64_t pos_batch, int n_positions, void* stream) {
     if (!x || !out || !cos_table || !sin_table || !positions) return fail(MI355_ERR_BAD_ARGUMENT, "mi355_rope: null pointer");
     if (D != 128) return fail(MI355_ERR_UNSUPPORTED, "mi355_rope: head_dim must be 128 (got %d)", D);
-    if (B < 1 || S < 1 || heads < 1 || n_positions < 1)
-        return fail(MI355_ERR_BAD_ARGUMENT, "mi355_rope: B, S, heads, n_positions must be >= 1");
-    const int64_t width = (int64_t)heads * D;
+    if (B < 1 || S < 1 || heads < 0 || copy_heads < 0 || heads + copy_heads < 1 || n_positions < 1 || pos_batch < 0)
+        return fail(MI355_ERR_BAD_ARGUMENT, "mi355_rope: B, S, heads + copy_heads, n_positions must be >= 1, pos_batch >= 0");
+    const int64_t width = (int64_t)(heads + copy_heads) * D;
     if (x_row < width || out_row < width || x_row % 8 || out_row % 8 || x_batch % 8 || out_batch % 8 || x_batch < 0 || out_batch < 0)
-        return fail(MI355_ERR_BAD_ARGUMENT, "mi355_rope: strides must be multiples of 8, row strides >= heads * 128");
+        return fail(MI355_ERR_BAD_ARGUMENT, "mi355_rope: strides must be multiples of 8, row strides >= (heads + copy_heads) * 128");
     if (!aligned16(x) || !aligned16(out) || !aligned16(cos_table) || !aligned16(sin_table))
         return fail(MI355_ERR_BAD_ARGUMENT, "mi355_rope: pointers must be 16-byte aligned");
-    hipError_t e = mi355::rope_dispatch(x, out, B, S, heads, x_batch, x_row, out_batch, out_row, cos_table, sin_table, positions,
-                                        n_positions, static_cast<hipStream_t>(stream));
+    hipError_t e = mi355::rope_dispatch(x, out, B, S, heads, copy_heads, x_batch, x_row, out_batch, out_row, cos_table, sin_table,
+                                        positions, pos_batch, n_positions, static_cast<hipStream_t>(stream));
     if (e != hipSuccess) return hip_fail(e, "mi355_rope launch");
     return 0;
 }

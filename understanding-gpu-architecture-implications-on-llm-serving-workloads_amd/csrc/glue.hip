@@ -71,22 +71,29 @@ __global__ __launch_bounds__(glue::THREADS) void rmsnorm_kernel(const half_t* x,
 //   out[i]      = x[i] * cos[i]      - x[i + 64] * sin[i]
 //   out[i + 64] = x[i + 64] * cos[i] + x[i] * sin[i]
 // (rotate_half convention, modeling_llama.py:164-168,193-194), cos/sin rows of 64 fp32 selected by the token's position.
+// The `copy_heads` heads that follow are moved unrotated (the value heads on their way into a KV cache).
 // A thread owns 8 values of the lower half and their 8 partners; 8 threads per head, 32 heads per workgroup.
 __global__ __launch_bounds__(glue::THREADS) void rope_kernel(const half_t* x, half_t* out, int S,
-                                                             int heads, long x_batch, long x_row, long o_batch, long o_row,
-                                                             const float* __restrict__ cos_t, const float* __restrict__ sin_t,
-                                                             const int* __restrict__ positions, int n_pos) {
+                                                             int heads, int copy_heads, long x_batch, long x_row, long o_batch,
+                                                             long o_row, const float* __restrict__ cos_t,
+                                                             const float* __restrict__ sin_t, const int* __restrict__ positions,
+                                                             long pos_batch, int n_pos) {
     const long token = blockIdx.x;
     const int head = blockIdx.y * 32 + (threadIdx.x >> 3);
-    if (head >= heads) return;
+    if (head >= heads + copy_heads) return;
     const int i0 = (threadIdx.x & 7) * 8;
     const long b = token / S, s = token - b * S;
-    int pos = positions[token];
-    pos = min(max(pos, 0), n_pos - 1);
     const half_t* xp = x + b * x_batch + s * x_row + (long)head * 128 + i0;
     half_t* op = out + b * o_batch + s * o_row + (long)head * 128 + i0;
     const half8 lo = *(const half8*)xp;
     const half8 hi = *(const half8*)(xp + 64);
+    if (head >= heads) {
+        *(half8*)op = lo;
+        *(half8*)(op + 64) = hi;
+        return;
+    }
+    int pos = positions[b * pos_batch + s];
+    pos = min(max(pos, 0), n_pos - 1);
     const float* cp = cos_t + (long)pos * 64 + i0;
     const float* sp = sin_t + (long)pos * 64 + i0;
     const float4v c0 = *(const float4v*)cp, c1 = *(const float4v*)(cp + 4);
@@ -135,12 +142,15 @@ hipError_t rmsnorm_dispatch(const void* x, const void* residual, void* res_out, 
     return hipGetLastError();
 }
 
-hipError_t rope_dispatch(const void* x, void* out, int B, int S, int heads, long x_batch, long x_row, long o_batch, long o_row,
-                         const float* cos_t, const float* sin_t, const int* positions, int n_pos, hipStream_t stream) {
+hipError_t rope_dispatch(const void* x, void* out, int B, int S, int heads, int copy_heads, long x_batch, long x_row,
+                         long o_batch, long o_row, const float* cos_t, const float* sin_t, const int* positions, long pos_batch,
+                         int n_pos, hipStream_t stream) {
     const long tokens = (long)B * S;
-    if (tokens > 0x7fffffffL || (heads + 31) / 32 > 65535) return hipErrorInvalidValue;
-    rope_kernel<<<dim3((unsigned)tokens, (unsigned)((heads + 31) / 32)), dim3(glue::THREADS), 0, stream>>>(
-        (const half_t*)x, (half_t*)out, S, heads, x_batch, x_row, o_batch, o_row, cos_t, sin_t, positions, n_pos);
+    const int groups = (heads + copy_heads + 31) / 32;
+    if (tokens > 0x7fffffffL || groups > 65535) return hipErrorInvalidValue;
+    rope_kernel<<<dim3((unsigned)tokens, (unsigned)groups), dim3(glue::THREADS), 0, stream>>>(
+        (const half_t*)x, (half_t*)out, S, heads, copy_heads, x_batch, x_row, o_batch, o_row, cos_t, sin_t, positions, pos_batch,
+        n_pos);
     return hipGetLastError();
 }
 

@@ -31,8 +31,9 @@ hipError_t fmha_decode_dispatch(const T* Q, const T* K, const T* V, T* O, float*
 // Layer glue (glue.hip); arguments as the mi355_rmsnorm / mi355_rope / mi355_silu_mul entry points after validation.
 hipError_t rmsnorm_dispatch(const void* x, const void* residual, void* res_out, const void* weight, void* out, long rows,
                             int hidden, long ldx, long ldr, long ldro, long ldo, float eps, hipStream_t stream);
-hipError_t rope_dispatch(const void* x, void* out, int B, int S, int heads, long x_batch, long x_row, long o_batch, long o_row,
-                         const float* cos_t, const float* sin_t, const int* positions, int n_pos, hipStream_t stream);
+hipError_t rope_dispatch(const void* x, void* out, int B, int S, int heads, int copy_heads, long x_batch, long x_row,
+                         long o_batch, long o_row, const float* cos_t, const float* sin_t, const int* positions, long pos_batch,
+                         int n_pos, hipStream_t stream);
 hipError_t silu_mul_dispatch(const void* in, void* out, long rows, int inter, long ld_in, long ld_out, hipStream_t stream);
 
 }  // namespace mi355

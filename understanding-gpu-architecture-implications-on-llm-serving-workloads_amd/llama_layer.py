@@ -29,16 +29,19 @@ def rope_tables(n_positions, head_dim=128, base=10000.0, device="cuda"):
 
 
 class FineKVCache:
-    """Static key/value cache of one layer, [B, max_len, n_kv, 128] fp16 (token-major so a step appends one row)."""
+    """Static key/value cache of one layer: one tensor [B, max_len, 2 * n_kv, 128] fp16, token-major (a step appends one
+    row) with the key heads of a token followed by its value heads, so one kernel launch files both. `k` and `v` are the
+    [B, max_len, n_kv, 128] views the attention kernel reads in place."""
 
     def __init__(self, batch, max_len, n_kv, head_dim=128, device="cuda"):
-        self.k = torch.empty((batch, max_len, n_kv, head_dim), dtype=torch.float16, device=device)
-        self.v = torch.empty_like(self.k)
+        self.kv = torch.empty((batch, max_len, 2 * n_kv, head_dim), dtype=torch.float16, device=device)
+        self.k = self.kv[:, :, :n_kv]
+        self.v = self.kv[:, :, n_kv:]
         self.length = 0
 
     @property
     def max_len(self):
-        return self.k.shape[1]
+        return self.kv.shape[1]
 
 
 class FineLlamaDecoderLayer:
@@ -61,6 +64,7 @@ class FineLlamaDecoderLayer:
         self.ln1, self.ln2 = w["ln1"], w["ln2"]
         self.eps = float(rms_eps)
         self.cos, self.sin = rope_tables(max_positions, self.head_dim, rope_base, device=self.w_o.device)
+        self.all_positions = torch.arange(max_positions, dtype=torch.int32, device=self.w_o.device)
         self.attn_ms = {"prefill": [], "decode": []}  # filled when time_attention=True (modeling_llama.py:762-775)
 
     @classmethod
@@ -80,8 +84,9 @@ class FineLlamaDecoderLayer:
         x = hidden_states.reshape(B * S, H)
         past = kv_cache.length if kv_cache is not None else 0
         if position_ids is None:
-            position_ids = torch.arange(past, past + S, device=x.device, dtype=torch.int32)[None].expand(B, S)
-        pos = position_ids.to(torch.int32).contiguous()
+            pos = self.all_positions[past:past + S]   # one [S] table shared by every batch row, no kernel launched
+        else:
+            pos = position_ids.to(torch.int32).contiguous()
 
         h1 = lib.rmsnorm(x, self.ln1, self.eps)
         if time_attention:
@@ -97,8 +102,8 @@ class FineLlamaDecoderLayer:
             if past + S > kv_cache.max_len:
                 raise ValueError("KV cache of %d tokens cannot take %d more after %d" % (kv_cache.max_len, S, past))
             lib.rope(q, self.cos, self.sin, pos)
-            lib.rope(qkv[:, :, Hq:Hq + Hkv], self.cos, self.sin, pos, out=kv_cache.k[:, past:past + S])
-            kv_cache.v[:, past:past + S].copy_(qkv[:, :, Hq + Hkv:])
+            # rotated keys and plain values of the new tokens go into the cache in one launch
+            lib.rope(qkv[:, :, Hq:], self.cos, self.sin, pos, out=kv_cache.kv[:, past:past + S], copy_heads=Hkv)
             kv_cache.length = past + S
             k, v = kv_cache.k[:, :past + S], kv_cache.v[:, :past + S]
         attn = torch.empty((B, S, Hq, D), dtype=torch.float16, device=x.device)

@@ -48,7 +48,7 @@ def load():
     lib.mi355_fmha_fwd_bf16.restype = i32
     lib.mi355_rmsnorm.argtypes = [vp, vp, vp, vp, vp, i64, i32, i64, i64, i64, i64, f32, vp]
     lib.mi355_rmsnorm.restype = i32
-    lib.mi355_rope.argtypes = [vp, vp, i32, i32, i32, i32, i64, i64, i64, i64, vp, vp, vp, i32, vp]
+    lib.mi355_rope.argtypes = [vp, vp, i32, i32, i32, i32, i32, i64, i64, i64, i64, vp, vp, vp, i64, i32, vp]
     lib.mi355_rope.restype = i32
     lib.mi355_silu_mul.argtypes = [vp, vp, i64, i32, i64, i64, vp]
     lib.mi355_silu_mul.restype = i32
@@ -184,17 +184,20 @@ def rmsnorm(x, weight, eps, residual=None, residual_out=None, out=None):
     return out if residual is None else (out, residual_out)
 
 
-def rope(x, cos, sin, positions, out=None):
+def rope(x, cos, sin, positions, out=None, copy_heads=0):
     """Rotary embedding of x [B, S, heads, 128] (any batch / token stride, heads contiguous), in place unless `out`
-    (same shape, own strides) is given. cos, sin: [n_positions, 64] fp32; positions: [B, S] int32."""
+    (same shape, own strides) is given. The last `copy_heads` heads are copied unrotated. cos, sin: [n_positions, 64]
+    fp32; positions: int32, [B, S] or [S] (shared by all batch rows)."""
     import torch
     B, S, heads, D = x.shape
     out = x if out is None else out
     assert x.dtype == torch.float16 and x.stride(3) == 1 and x.stride(2) == D and out.stride(3) == 1 and out.stride(2) == D
     assert cos.dtype == torch.float32 and cos.is_contiguous() and sin.is_contiguous() and cos.shape == sin.shape
-    assert positions.dtype == torch.int32 and positions.is_contiguous() and positions.numel() == B * S
-    _check(load().mi355_rope(_ptr(x), _ptr(out), B, S, heads, D, x.stride(0), x.stride(1), out.stride(0), out.stride(1),
-                             _ptr(cos), _ptr(sin), _ptr(positions), cos.shape[0], _stream_of(x)))
+    assert positions.dtype == torch.int32 and positions.is_contiguous() and positions.numel() in (S, B * S)
+    pos_batch = S if (positions.numel() == B * S and B > 1) else 0
+    _check(load().mi355_rope(_ptr(x), _ptr(out), B, S, heads - copy_heads, copy_heads, D, x.stride(0), x.stride(1),
+                             out.stride(0), out.stride(1), _ptr(cos), _ptr(sin), _ptr(positions), pos_batch, cos.shape[0],
+                             _stream_of(x)))
     return out
 
 
