@@ -205,6 +205,17 @@ def main():
         other["F3_fmha_noncausal_b4_h32_s1024"] = {"ms": ms3, "tflops": fl3 / ms3 / 1e9,
                                                    "pct_of_fp16_mfma_peak": 100 * fl3 / ms3 / 1e9 / PEAK_FP16_TFLOPS}
         del q3, k3, v3, o3
+        # the vendor libraries on the same box, same operands, same timing loop (context for the figures above; not this code)
+        cv = torch.empty_like(c)
+        ms_v = time_launches(lambda: torch.matmul(a, b, out=cv), 20, 3)
+        bt = b.t().contiguous()
+        ms_vt = time_launches(lambda: torch.matmul(a, bt.t(), out=cv), 20, 3)
+        ms_sd = time_launches(lambda: torch.nn.functional.scaled_dot_product_attention(q, k, v, is_causal=True, enable_gqa=True), 20, 3)
+        other["vendor_libraries_same_box"] = {
+            "torch_matmul_hipblaslt_8192_nn": {"ms": ms_v, "tflops": gemm_flops / ms_v / 1e9},
+            "torch_matmul_hipblaslt_8192_nt": {"ms": ms_vt, "tflops": gemm_flops / ms_vt / 1e9},
+            "torch_sdpa_f4_causal_gqa": {"ms": ms_sd, "tflops": fmha_flops / ms_sd / 1e9}}
+        del cv, bt
         # generation-step shapes (HBM bound): nn.Linear-layout weight GEMM and attention over a long KV cache
         xd = so.randn_fp16((16, 4096), 1).to(dev)
         wd_nt = so.randn_fp16((14336, 4096), 2, 0.02).to(dev)
