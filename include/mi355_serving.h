@@ -59,6 +59,19 @@ int mi355_hgemm(const void* A, const void* B, void* C, int M, int N, int K, int6
                 int64_t ldc, int layout, void* stream);
 
 /*
+ * C[M,N] = silu(G) * U, where [G | U] = op(A) * op(B) and op(B) has 2N columns that alternate between 32 columns of G and
+ * the matching 32 columns of U (column 64 b + c is G[:, 32 b + c] for c < 32 and U[:, 32 b + c - 32] for c >= 32): the
+ * gate and up projections of a Llama MLP computed by one GEMM on an interleaved weight matrix, with the activation
+ * applied to the accumulators before the single rounding to fp16. Replaces `self.act_fn(self.gate_proj(x)) * self.up_proj(x)`
+ * (benchmarks/flashattn-cuda/modeling_llama.py:227): two GEMMs, a SiLU kernel and a multiply kernel in the reference.
+ * Layouts NN and NT. Only shapes the tiled kernels cover have the fused form (M and 2N multiples of 128, K a multiple of 64,
+ * 16-byte aligned operands and leading dimensions); others return MI355_ERR_UNSUPPORTED and nothing is launched: run
+ * mi355_hgemm on the same operands followed by mi355_silu_mul with interleave = 32.
+ */
+int mi355_hgemm_silu_mul(const void* A, const void* B, void* C, int M, int N, int K, int64_t lda, int64_t ldb, int64_t ldc,
+                         int layout, void* stream);
+
+/*
  * Fused attention forward, O = softmax(scale * Q K^T + mask) V, online softmax with fp32 statistics.
  *
  * Replaces the device side of `torch::Tensor finefmha_N(Q, K, V, causal, is_decode, decode_length)`
@@ -135,10 +148,13 @@ int mi355_rope(const void* x, void* out, int B, int S, int heads, int copy_heads
                int64_t pos_batch, int n_positions, void* stream);
 
 /*
- * mi355_silu_mul: out[r][j] = silu(g[r][j]) * u[r][j] with g = gate_up[r][0 .. inter), u = gate_up[r][inter .. 2 inter)
- *   (`act_fn(gate_proj(x)) * up_proj(x)`, modeling_llama.py:230, for gate and up computed by one GEMM).
+ * mi355_silu_mul: out[r][j] = silu(g[r][j]) * u[r][j] (`act_fn(gate_proj(x)) * up_proj(x)`, modeling_llama.py:227, for gate
+ *   and up computed by one GEMM). interleave == 0: g = gate_up[r][0 .. inter), u = gate_up[r][inter .. 2 inter).
+ *   interleave == b > 0 (a multiple of 8 dividing inter): g and u alternate in groups of b columns, the layout
+ *   mi355_hgemm_silu_mul consumes (b = 32).
  */
-int mi355_silu_mul(const void* gate_up, void* out, int64_t rows, int inter, int64_t ld_in, int64_t ld_out, void* stream);
+int mi355_silu_mul(const void* gate_up, void* out, int64_t rows, int inter, int interleave, int64_t ld_in, int64_t ld_out,
+                   void* stream);
 
 /* Thread-local text for the last non-zero return of this thread ("" if none). */
 const char* mi355_last_error(void);

@@ -27,7 +27,7 @@ oracle states those results directly in fp32 (torch) and, for small inputs, agai
   rmsnorm_ref, rope_tables, rope_ref, silu_mul_ref, llama_decoder_layer_ref
                       the glue of the reference's in-model path in fp32: LlamaRMSNorm.forward
                       (benchmarks/flashattn-cuda/modeling_llama.py:95-100), LlamaRotaryEmbedding (:113,119-132),
-                      rotate_half / apply_rotary_pos_emb (:164-168,193-194), act_fn(gate) * up (:230) and the
+                      rotate_half / apply_rotary_pos_emb (:164-168,193-194), act_fn(gate) * up (:227) and the
                       decoder layer that strings them together (LlamaSdpaAttention.forward :652-704 with a KV
                       cache, LlamaDecoderLayer.forward :755-781). Pinned by closed forms (constant rows, unit
                       weights, position 0, norm preservation, the relative-position property, d = 2 rotation by
@@ -305,7 +305,7 @@ def rope_ref(x, cos, sin, positions):
 
 
 def silu_mul_ref(gate_up):
-    """[rows, 2F] -> silu(gate) * up in fp32 (:230 with gate and up side by side)."""
+    """[rows, 2F] -> silu(gate) * up in fp32 (:227 with gate and up side by side)."""
     g = _f32(gate_up)
     F = g.shape[-1] // 2
     return torch.nn.functional.silu(g[..., :F]) * g[..., F:]

@@ -97,6 +97,28 @@ def test_silu_mul(lib, gpu, rows, inter):
     assert oe[0] == 0.0 and oe[1] == 60.0 and abs(oe[2]) < 1e-6 and abs(oe[3] + 4 * 0.7310586) < 4e-3
 
 
+@pytest.mark.parametrize("M,F,K,layout", [(256, 256, 128, "NT"), (2048, 4096, 512, "NT"), (1024, 14336, 256, "NT"),
+                                          (384, 192, 64, "NT"), (512, 1024, 256, "NN"), (8, 512, 256, "NT"), (100, 96, 72, "NT")])
+def test_gemm_with_gate_up_epilogue(lib, gpu, M, F, K, layout):
+    # silu(x Wg^T) * (x Wu^T) from one launch on the interleaved weight (tiled shapes) or from the two-step fallback;
+    # compared with the fp32 oracle. One rounding of an fp32 value: |err| <= 2^-10 |ref| + the GEMM's accumulation slack.
+    x = so.randn_fp16((M, K), 1)
+    wg, wu = so.randn_fp16((F, K), 2, 0.05), so.randn_fp16((F, K), 3, 0.05)
+    ref = so.silu_mul_ref(torch.cat((so.gemm_ref(x, wg, "NT"), so.gemm_ref(x, wu, "NT")), 1))
+    if layout == "NT":
+        w = lib.interleave_gate_up(wg.to(gpu), wu.to(gpu), dim=0)
+        assert w.shape == (2 * F, K) and torch.equal(w[:32].cpu(), wg[:32]) and torch.equal(w[32:64].cpu(), wu[:32])
+    else:
+        w = lib.interleave_gate_up(wg.t().contiguous().to(gpu), wu.t().contiguous().to(gpu), dim=1)
+        assert w.shape == (K, 2 * F) and torch.equal(w[:, 32:64].cpu(), wu[:32].t())
+    out = lib.hgemm_silu_mul(x.to(gpu), w, layout)
+    err = (out.float().cpu() - ref).abs()
+    assert bool((err <= 2.0 ** -10 * ref.abs() + 1e-3).all()), float(err.max())
+    # the interleaved silu_mul on the plain product gives the same numbers up to the extra fp16 rounding of the product
+    two_step = lib.silu_mul(lib.hgemm(x.to(gpu), w, layout), interleave=32)
+    assert (two_step.float() - out.float()).abs().max() <= 2e-2 * ref.abs().max()
+
+
 def layer_weights(H, n_q, n_kv, F, seed=0):
     D = 128
     g = lambda shape, s, std: so.randn_fp16(shape, seed + s, std)

@@ -68,6 +68,25 @@ static int fmha_checked(const char* fn, const void* Q, const void* K, const void
     return 0;
 }
 
+int mi355_hgemm_silu_mul(const void* A, const void* B, void* C, int M, int N, int K, int64_t lda, int64_t ldb, int64_t ldc,
+                         int layout, void* stream) {
+    if (!A || !B || !C) return fail(MI355_ERR_BAD_ARGUMENT, "mi355_hgemm_silu_mul: null pointer");
+    if (M < 1 || N < 1 || K < 1) return fail(MI355_ERR_BAD_ARGUMENT, "mi355_hgemm_silu_mul: M, N, K must be >= 1");
+    if (layout != MI355_GEMM_NN && layout != MI355_GEMM_NT)
+        return fail(MI355_ERR_UNSUPPORTED, "mi355_hgemm_silu_mul: layout %d has no fused epilogue (NN and NT do)", layout);
+    const int64_t b_min = (layout == MI355_GEMM_NT) ? K : 2 * (int64_t)N;
+    if (lda < K || ldb < b_min || ldc < N)
+        return fail(MI355_ERR_BAD_ARGUMENT, "mi355_hgemm_silu_mul: leading dimension too small");
+    if (N > 0x3fffffff) return fail(MI355_ERR_BAD_ARGUMENT, "mi355_hgemm_silu_mul: N too large");
+    hipError_t e = mi355::hgemm_silu_mul_dispatch(A, B, C, M, 2 * N, K, lda, ldb, ldc, layout, static_cast<hipStream_t>(stream));
+    if (e == hipErrorNotSupported)
+        return fail(MI355_ERR_UNSUPPORTED,
+                    "mi355_hgemm_silu_mul: needs M and 2N multiples of 128, K a multiple of 64 and 16-byte aligned operands; "
+                    "run mi355_hgemm and mi355_silu_mul(interleave = 32) instead");
+    if (e != hipSuccess) return hip_fail(e, "mi355_hgemm_silu_mul launch");
+    return 0;
+}
+
 int mi355_fmha_fwd(const void* Q, const void* K, const void* V, void* O, float* LSE, int B, int Hq, int Hkv, int Sq,
                    int Sk, int D, float scale, int causal, int kv_valid_len, void* stream) {
     const long q_head = (long)Sq * D, k_head = (long)Sk * D;
@@ -138,14 +157,18 @@ int mi355_rope(const void* x, void* out, int B, int S, int heads, int copy_heads
     return 0;
 }
 
-int mi355_silu_mul(const void* gate_up, void* out, int64_t rows, int inter, int64_t ld_in, int64_t ld_out, void* stream) {
+int mi355_silu_mul(const void* gate_up, void* out, int64_t rows, int inter, int interleave, int64_t ld_in, int64_t ld_out,
+                   void* stream) {
     if (!gate_up || !out) return fail(MI355_ERR_BAD_ARGUMENT, "mi355_silu_mul: null pointer");
     if (rows < 1 || inter < 8 || inter % 8 != 0)
         return fail(MI355_ERR_BAD_ARGUMENT, "mi355_silu_mul: rows >= 1 and inter a positive multiple of 8 required");
+    if (interleave < 0 || interleave % 8 != 0 || (interleave > 0 && inter % interleave != 0))
+        return fail(MI355_ERR_BAD_ARGUMENT, "mi355_silu_mul: interleave must be 0 or a multiple of 8 that divides inter (got %d)",
+                    interleave);
     if (ld_in < 2 * (int64_t)inter || ld_out < inter || ld_in % 8 || ld_out % 8)
         return fail(MI355_ERR_BAD_ARGUMENT, "mi355_silu_mul: ld_in >= 2 * inter, ld_out >= inter, both multiples of 8 required");
     if (!aligned16(gate_up) || !aligned16(out)) return fail(MI355_ERR_BAD_ARGUMENT, "mi355_silu_mul: pointers must be 16-byte aligned");
-    hipError_t e = mi355::silu_mul_dispatch(gate_up, out, rows, inter, ld_in, ld_out, static_cast<hipStream_t>(stream));
+    hipError_t e = mi355::silu_mul_dispatch(gate_up, out, rows, inter, interleave, ld_in, ld_out, static_cast<hipStream_t>(stream));
     if (e != hipSuccess) return hip_fail(e, "mi355_silu_mul launch");
     return 0;
 }

@@ -345,13 +345,8 @@ hipError_t fmha_decode_dispatch(const T* Q, const T* K, const T* V, T* O, float*
                                 int Hkv, int Sq, int Sk, float scale, int causal, int kv_valid, const FmhaStrides& sd,
                                 hipStream_t stream) {
     using namespace dec;
-    static bool attr_set = false;
-    if (!attr_set) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(fmha_decode_split_kernel<T>),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
-        if (e != hipSuccess) return e;
-        attr_set = true;
-    }
+    static DynamicLdsOnce lds_once;
+    if (hipError_t e = lds_once.ensure(reinterpret_cast<const void*>(fmha_decode_split_kernel<T>), LDS_BYTES); e != hipSuccess) return e;
     const int group = Hq / Hkv;
     const int ncols = group * Sq;
     const int tiles = (kv_valid + TK - 1) / TK;

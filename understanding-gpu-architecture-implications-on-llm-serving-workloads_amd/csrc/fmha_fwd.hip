@@ -628,13 +628,8 @@ static hipError_t launch_fmha_pingpong(const T* Q, const T* K, const T* V, T* O,
                                        hipStream_t stream) {
     constexpr int BM = 256;
     constexpr int LDS = 4 * fmha::TILE_BYTES;
-    static bool attr_set = false;
-    if (!attr_set) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(fmha_fwd_pingpong_kernel<T>),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, LDS);
-        if (e != hipSuccess) return e;
-        attr_set = true;
-    }
+    static DynamicLdsOnce lds_once;
+    if (hipError_t e = lds_once.ensure(reinterpret_cast<const void*>(fmha_fwd_pingpong_kernel<T>), LDS); e != hipSuccess) return e;
     const int q_tiles = (Sq + BM - 1) / BM;
     const long blocks = (long)q_tiles * Hq * B;
     if (blocks > 0x7fffffffL) return hipErrorInvalidValue;
@@ -651,13 +646,8 @@ static hipError_t launch_fmha(const T* Q, const T* K, const T* V, T* O, float* L
     constexpr int BM = NWAVES * NQ * 32;
     constexpr int LDS = fmha::STAGE_BYTES * fmha::NSTAGE;
     auto kern = fmha_fwd_kernel<T, NQ, NWAVES>;
-    static bool attr_set = false;
-    if (!attr_set) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, LDS);
-        if (e != hipSuccess) return e;
-        attr_set = true;
-    }
+    static DynamicLdsOnce lds_once;
+    if (hipError_t e = lds_once.ensure(reinterpret_cast<const void*>(kern), LDS); e != hipSuccess) return e;
     const int q_tiles = (Sq + BM - 1) / BM;
     const long blocks = (long)q_tiles * Hq * B;
     if (blocks > 0x7fffffffL) return hipErrorInvalidValue;

@@ -3,7 +3,7 @@
 //
 // These are the operations the reference's in-model path runs as separate PyTorch elementwise kernels between its
 // calls of fine_fmha (benchmarks/flashattn-cuda/modeling_llama.py): LlamaRMSNorm.forward (:95-100), rotate_half /
-// apply_rotary_pos_emb (:164-195), LlamaMLP.forward's act_fn(gate) * up (:230) and the residual adds of
+// apply_rotary_pos_emb (:164-195), LlamaMLP.forward's act_fn(gate) * up (:227) and the residual adds of
 // LlamaDecoderLayer.forward (:776-781). Each kernel moves every byte once with 16-byte accesses.
 #include "mi355_common.h"
 #include "mi355_serving_internal.h"
@@ -111,14 +111,18 @@ __global__ __launch_bounds__(glue::THREADS) void rope_kernel(const half_t* x, ha
     *(half8*)(op + 64) = ohi;
 }
 
-// out[r][j] = silu(gate[r][j]) * up[r][j], gate = in[r][0 .. inter), up = in[r][inter .. 2 inter)
+// out[r][j] = silu(gate[r][j]) * up[r][j]. block == 0: gate = in[r][0 .. inter), up = in[r][inter .. 2 inter);
+// block > 0 (a multiple of 8): gate and up alternate in groups of `block` columns, gate[j] = in[r][(j / block) * 2 block + j % block]
+// and up[j] `block` columns further (the layout the GEMM's gate/up epilogue consumes).
 __global__ __launch_bounds__(glue::THREADS) void silu_mul_kernel(const half_t* __restrict__ in, half_t* __restrict__ out,
-                                                                 int inter, long ld_in, long ld_out) {
+                                                                 int inter, int block, long ld_in, long ld_out) {
     const long row = blockIdx.y;
     const int c = (blockIdx.x * glue::THREADS + threadIdx.x) * 8;
     if (c >= inter) return;
-    const half8 g = *(const half8*)(in + row * ld_in + c);
-    const half8 u = *(const half8*)(in + row * ld_in + inter + c);
+    const long gcol = block ? (long)(c / block) * 2 * block + c % block : c;
+    const long ucol = block ? gcol + block : (long)inter + c;
+    const half8 g = *(const half8*)(in + row * ld_in + gcol);
+    const half8 u = *(const half8*)(in + row * ld_in + ucol);
     half8 o;
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
@@ -154,14 +158,15 @@ hipError_t rope_dispatch(const void* x, void* out, int B, int S, int heads, int 
     return hipGetLastError();
 }
 
-hipError_t silu_mul_dispatch(const void* in, void* out, long rows, int inter, long ld_in, long ld_out, hipStream_t stream) {
+hipError_t silu_mul_dispatch(const void* in, void* out, long rows, int inter, int block, long ld_in, long ld_out,
+                             hipStream_t stream) {
     if (rows > 65535L * 32768L) return hipErrorInvalidValue;
     // grid.y is limited to 65535: fold rows beyond that into several launches
     const unsigned gx = (unsigned)((inter / 8 + glue::THREADS - 1) / glue::THREADS);
     for (long r0 = 0; r0 < rows; r0 += 65535) {
         const long n = rows - r0 < 65535 ? rows - r0 : 65535;
         silu_mul_kernel<<<dim3(gx, (unsigned)n), dim3(glue::THREADS), 0, stream>>>((const half_t*)in + r0 * ld_in,
-                                                                                  (half_t*)out + r0 * ld_out, inter, ld_in, ld_out);
+                                                                                  (half_t*)out + r0 * ld_out, inter, block, ld_in, ld_out);
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) return e;
     }

@@ -152,7 +152,11 @@ __device__ __forceinline__ void tile_of_block(int bid, int tiles_m, int tiles_n,
     tn = in_g / rows;
 }
 
-template <bool A_KC, bool B_KC, int BM, int BN, int WM, int WN>
+// EPI selects what is stored: 0 = the product; 1 = silu(g) * u for a B operand whose columns alternate between 32 gate
+// columns and their 32 up columns (`act_fn(gate_proj(x)) * up_proj(x)`, benchmarks/flashattn-cuda/modeling_llama.py:227,
+// with the two projections interleaved in one weight matrix): a wave then holds g and u of the same outputs in its two
+// column blocks, at the same accumulator positions, and C has N / 2 columns.
+template <bool A_KC, bool B_KC, int BM, int BN, int WM, int WN, int EPI = 0>
 __global__ __launch_bounds__(WM * WN * 64) void hgemm_main_kernel(const half_t* __restrict__ A, const half_t* __restrict__ B,
                                                          half_t* __restrict__ C, int M, int N, int K, long lda,
                                                          long ldb, long ldc) {
@@ -328,7 +332,9 @@ __global__ __launch_bounds__(WM * WN * 64) void hgemm_main_kernel(const half_t* 
     // write 8-byte pieces of 32 different rows per instruction (partial cache lines, read-modify-write in the
     // memory system), so each wave first parks its sub-tile in its own slice of LDS (fp16, 16-byte chunks XOR-
     // swizzled by row) and then stores whole rows: every store instruction writes complete 128-byte lines.
-    constexpr int kRowHalfs = TN * 32;            // width of the wave sub-tile
+    static_assert(EPI == 0 || TN == 2, "the gate/up epilogue pairs the two column blocks of a wave");
+    constexpr int TNO = EPI == 1 ? TN / 2 : TN;   // column blocks a wave stores
+    constexpr int kRowHalfs = TNO * 32;           // width of the stored wave sub-tile
     constexpr int kRowBytesC = kRowHalfs * 2;
     constexpr int kChunksC = kRowBytesC / 16;     // 16-byte chunks per row (8 or 16)
     constexpr int kRowsPerStore = 64 / kChunksC;  // rows covered by one store instruction
@@ -342,15 +348,21 @@ __global__ __launch_bounds__(WM * WN * 64) void hgemm_main_kernel(const half_t* 
         for (int i = 0; i < TM; ++i) {
             const int row = i * 32 + r;
 #pragma unroll
-            for (int j = 0; j < TN; ++j) {
+            for (int j = 0; j < TNO; ++j) {
 #pragma unroll
                 for (int p = 0; p < 4; ++p) {
                     half4 v;
-                    v[0] = (half_t)acc[i][j][4 * p + 0];
-                    v[1] = (half_t)acc[i][j][4 * p + 1];
-                    v[2] = (half_t)acc[i][j][4 * p + 2];
-                    v[3] = (half_t)acc[i][j][4 * p + 3];
-                    const int chunk = (j * 4 + p) ^ (row & 7);
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        if constexpr (EPI == 1) {
+                            const float g = acc[i][2 * j][4 * p + q];
+                            const float sig = __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(-g * 1.4426950408889634f));
+                            v[q] = (half_t)(g * sig * acc[i][2 * j + 1][4 * p + q]);
+                        } else {
+                            v[q] = (half_t)acc[i][j][4 * p + q];
+                        }
+                    }
+                    const int chunk = (j * 4 + p) ^ (row & (kChunksC < 8 ? kChunksC - 1 : 7));
                     *(MI355_LDS half4*)(cst + row * kRowBytesC + chunk * 16 + hh * 8) = v;
                 }
             }
@@ -360,11 +372,11 @@ __global__ __launch_bounds__(WM * WN * 64) void hgemm_main_kernel(const half_t* 
     {
         const int rr = lane / kChunksC;
         const int cc = lane % kChunksC;
-        half_t* cbase = C + (m0 + wm * TM * 32) * ldc + n0 + wn * TN * 32 + cc * 8;
+        half_t* cbase = C + (m0 + wm * TM * 32) * ldc + (EPI == 1 ? n0 / 2 : n0) + wn * TNO * 32 + cc * 8;
 #pragma unroll
         for (int it = 0; it < TM * 32 / kRowsPerStore; ++it) {
             const int row = it * kRowsPerStore + rr;
-            half8 v = *(MI355_LDS const half8*)(cst + row * kRowBytesC + ((cc ^ (row & 7)) << 4));
+            half8 v = *(MI355_LDS const half8*)(cst + row * kRowBytesC + ((cc ^ (row & (kChunksC < 8 ? kChunksC - 1 : 7))) << 4));
             *(half8*)(cbase + (long)row * ldc) = v;
         }
     }
@@ -544,13 +556,8 @@ __global__ __launch_bounds__(512) void hgemm_smallm_nn_kernel(const half_t* __re
 
 static hipError_t launch_smallm_nn(const half_t* A, const half_t* B, half_t* C, int M, int N, int K, long lda, long ldb,
                                    long ldc, hipStream_t stream) {
-    static bool attr_set = false;
-    if (!attr_set) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(hgemm_smallm_nn_kernel),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, kSmallMLdsBytes);
-        if (e != hipSuccess) return e;
-        attr_set = true;
-    }
+    static DynamicLdsOnce lds_once;
+    if (hipError_t e = lds_once.ensure(reinterpret_cast<const void*>(hgemm_smallm_nn_kernel), kSmallMLdsBytes); e != hipSuccess) return e;
     const int n_tiles = (N + 63) / 64;
     dim3 grid(n_tiles, (M + 15) / 16);
     hgemm_smallm_nn_kernel<<<grid, dim3(512), kSmallMLdsBytes, stream>>>(A, B, C, M, N, K, lda, ldb, ldc, n_tiles);
@@ -663,13 +670,8 @@ __global__ __launch_bounds__(512) void hgemm_smallm_nt_kernel(const half_t* __re
 
 static hipError_t launch_smallm_nt(const half_t* A, const half_t* B, half_t* C, int M, int N, int K, long lda, long ldb,
                                    long ldc, hipStream_t stream) {
-    static bool attr_set = false;
-    if (!attr_set) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(hgemm_smallm_nt_kernel),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, kSmallMNtLdsBytes);
-        if (e != hipSuccess) return e;
-        attr_set = true;
-    }
+    static DynamicLdsOnce lds_once;
+    if (hipError_t e = lds_once.ensure(reinterpret_cast<const void*>(hgemm_smallm_nt_kernel), kSmallMNtLdsBytes); e != hipSuccess) return e;
     const int n_tiles = (N + 15) / 16;
     dim3 grid(n_tiles, (M + 15) / 16);
     hgemm_smallm_nt_kernel<<<grid, dim3(512), kSmallMNtLdsBytes, stream>>>(A, B, C, M, N, K, lda, ldb, ldc, n_tiles);
@@ -678,18 +680,13 @@ static hipError_t launch_smallm_nt(const half_t* A, const half_t* B, half_t* C, 
 
 int g_gemm_variant = 0;  // tuning hook: 0 = heuristic, 1 = force 256x256 tiles, 2 = force 128x128 tiles
 
-template <bool A_KC, bool B_KC, int BM, int BN, int WM, int WN>
+template <bool A_KC, bool B_KC, int BM, int BN, int WM, int WN, int EPI = 0>
 static hipError_t launch_main(const half_t* A, const half_t* B, half_t* C, int M, int N, int K, long lda, long ldb,
                               long ldc, hipStream_t stream) {
     using Cfg = MainCfg<A_KC, B_KC, BM, BN, WM, WN>;
-    static bool attr_set = false;
-    auto kern = hgemm_main_kernel<A_KC, B_KC, BM, BN, WM, WN>;
-    if (!attr_set) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::LDS_BYTES);
-        if (e != hipSuccess) return e;
-        attr_set = true;
-    }
+    auto kern = hgemm_main_kernel<A_KC, B_KC, BM, BN, WM, WN, EPI>;
+    static DynamicLdsOnce lds_once;
+    if (hipError_t e = lds_once.ensure(reinterpret_cast<const void*>(kern), Cfg::LDS_BYTES); e != hipSuccess) return e;
     int blocks = (M / BM) * (N / BN);
     kern<<<dim3(blocks), dim3(Cfg::NTHREADS), Cfg::LDS_BYTES, stream>>>(A, B, C, M, N, K, lda, ldb, ldc);
     return hipGetLastError();
@@ -726,6 +723,32 @@ static hipError_t launch_layout(const half_t* A, const half_t* B, half_t* C, int
     dim3 grid((N + 63) / 64, (M + 63) / 64);
     hgemm_edge_kernel<A_KC, B_KC><<<grid, dim3(256), 0, stream>>>(A, B, C, M, N, K, lda, ldb, ldc);
     return hipGetLastError();
+}
+
+// Product with the gate/up epilogue (EPI = 1): N counts the columns of op(B) (twice those of C). Only the tiled kernels
+// have it; other shapes report hipErrorNotSupported and the caller runs the product and mi355_silu_mul separately.
+template <bool A_KC, bool B_KC>
+static hipError_t launch_silu_mul(const half_t* A, const half_t* B, half_t* C, int M, int N, int K, long lda, long ldb,
+                                  long ldc, hipStream_t stream) {
+    const bool aligned = (reinterpret_cast<uintptr_t>(A) % 16 == 0) && (reinterpret_cast<uintptr_t>(B) % 16 == 0) &&
+                         (reinterpret_cast<uintptr_t>(C) % 16 == 0) && (lda % 8 == 0) && (ldb % 8 == 0) && (ldc % 8 == 0);
+    if (!aligned || K % 64 != 0 || K < 64 || M % 128 != 0 || N % 128 != 0) return hipErrorNotSupported;
+    const bool fits256 = M % 256 == 0 && N % 256 == 0;
+    if (fits256 && (long)(M / 256) * (N / 256) >= 192)
+        return launch_main<A_KC, B_KC, 256, 256, 2, 4, 1>(A, B, C, M, N, K, lda, ldb, ldc, stream);
+    return launch_main<A_KC, B_KC, 128, 128, 2, 2, 1>(A, B, C, M, N, K, lda, ldb, ldc, stream);
+}
+
+hipError_t hgemm_silu_mul_dispatch(const void* A, const void* B, void* C, int M, int N2, int K, long lda, long ldb, long ldc,
+                                   int layout, hipStream_t stream) {
+    const half_t* a = static_cast<const half_t*>(A);
+    const half_t* b = static_cast<const half_t*>(B);
+    half_t* c = static_cast<half_t*>(C);
+    switch (layout) {
+        case MI355_GEMM_NN: return launch_silu_mul<true, false>(a, b, c, M, N2, K, lda, ldb, ldc, stream);
+        case MI355_GEMM_NT: return launch_silu_mul<true, true>(a, b, c, M, N2, K, lda, ldb, ldc, stream);
+        default: return hipErrorNotSupported;
+    }
 }
 
 hipError_t hgemm_dispatch(const void* A, const void* B, void* C, int M, int N, int K, long lda, long ldb, long ldc,

@@ -5,6 +5,22 @@
 
 namespace mi355 {
 
+// Raises a kernel's dynamic LDS limit once per device (the attribute belongs to the device the call is made on).
+struct DynamicLdsOnce {
+    static constexpr int kMaxDevices = 64;
+    bool done[kMaxDevices] = {};
+    hipError_t ensure(const void* kernel, int bytes) {
+        int dev = 0;
+        hipError_t e = hipGetDevice(&dev);
+        if (e != hipSuccess) return e;
+        const bool tracked = dev >= 0 && dev < kMaxDevices;
+        if (tracked && done[dev]) return hipSuccess;
+        e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+        if (e == hipSuccess && tracked) done[dev] = true;
+        return e;
+    }
+};
+
 // Launches the GEMM kernels; arguments as mi355_hgemm after validation.
 hipError_t hgemm_dispatch(const void* A, const void* B, void* C, int M, int N, int K, long lda, long ldb, long ldc,
                           int layout, hipStream_t stream);
@@ -16,6 +32,10 @@ struct FmhaStrides {
     long v_batch, v_head, v_row;
     long o_batch, o_head, o_row;
 };
+
+// The product fused with silu(gate) * up (see hgemm_main_kernel's EPI); hipErrorNotSupported for shapes without it.
+hipError_t hgemm_silu_mul_dispatch(const void* A, const void* B, void* C, int M, int N2, int K, long lda, long ldb, long ldc,
+                                   int layout, hipStream_t stream);
 
 // Launches the attention forward kernels; arguments as mi355_fmha_fwd_strided after validation.
 hipError_t fmha_fwd_dispatch(const void* Q, const void* K, const void* V, void* O, float* LSE, int B, int Hq, int Hkv,
@@ -34,6 +54,7 @@ hipError_t rmsnorm_dispatch(const void* x, const void* residual, void* res_out, 
 hipError_t rope_dispatch(const void* x, void* out, int B, int S, int heads, int copy_heads, long x_batch, long x_row,
                          long o_batch, long o_row, const float* cos_t, const float* sin_t, const int* positions, long pos_batch,
                          int n_pos, hipStream_t stream);
-hipError_t silu_mul_dispatch(const void* in, void* out, long rows, int inter, long ld_in, long ld_out, hipStream_t stream);
+hipError_t silu_mul_dispatch(const void* in, void* out, long rows, int inter, int block, long ld_in, long ld_out,
+                             hipStream_t stream);
 
 }  // namespace mi355

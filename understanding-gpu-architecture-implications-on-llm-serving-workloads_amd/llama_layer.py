@@ -6,13 +6,13 @@ calls, transposes to [B, H, S, D], applies RoPE, expands K/V with repeat_kv (:67
 ``fmha_unified.ops.fine_fmha`` (:687-690), transposes back with a copy (:700) and projects; LlamaDecoderLayer.forward
 (:755-781) wraps it in RMSNorm, residual adds and the gate/up/down MLP (:227), all as separate PyTorch kernels.
 
-Here one layer is twelve launches with no layout copies:
+Here one layer is eleven launches (twelve for shapes off the tiled GEMM's grid) with no layout copies:
     rmsnorm -> QKV GEMM (one fused NT GEMM on the nn.Linear weights) -> RoPE in place on the q and k heads of the
     projection (k goes straight into the KV cache when there is one) -> attention reading q, k, v where they lie
     (strided operands, GQA inside the kernel, output written as [B, S, Hq*D]) -> O projection -> residual add fused
-    into the second rmsnorm -> gate/up GEMM (fused) -> SiLU(gate)*up -> down GEMM -> residual add.
+    into the second rmsnorm -> gate/up GEMM with SiLU(gate)*up applied in its epilogue -> down GEMM -> residual add.
 Weights keep the nn.Linear layout ([out_features, in_features]); nothing is transposed or repacked beyond
-concatenating q/k/v and gate/up along the output dimension once at construction.
+concatenating q/k/v and interleaving gate/up along the output dimension once at construction.
 """
 import torch
 
@@ -59,7 +59,10 @@ class FineLlamaDecoderLayer:
         self.inter = w["gate"].shape[0]
         self.w_qkv = torch.cat((w["q"], w["k"], w["v"]), 0).contiguous()   # [(Hq + 2 Hkv) * D, H]
         self.w_o = w["o"]                                                  # [H, Hq * D]
-        self.w_gu = torch.cat((w["gate"], w["up"]), 0).contiguous()        # [2 F, H]
+        # gate and up rows interleaved in groups of 32, so the GEMM epilogue can apply silu(gate) * up to its accumulators
+        self.gu_block = lib.GATE_UP_BLOCK if self.inter % lib.GATE_UP_BLOCK == 0 else 0
+        self.w_gu = (lib.interleave_gate_up(w["gate"], w["up"]) if self.gu_block
+                     else torch.cat((w["gate"], w["up"]), 0).contiguous())   # [2 F, H]
         self.w_d = w["down"]                                               # [H, F]
         self.ln1, self.ln2 = w["ln1"], w["ln2"]
         self.eps = float(rms_eps)
@@ -116,8 +119,7 @@ class FineLlamaDecoderLayer:
             torch.cuda.synchronize()
             self.attn_ms["decode" if (S == 1 and past > 0) else "prefill"].append(t0.elapsed_time(t1))
         h2, res = lib.rmsnorm(proj, self.ln2, self.eps, residual=x)
-        gu = lib.hgemm(h2, self.w_gu, "NT")
-        act = lib.silu_mul(gu)
+        act = lib.hgemm_silu_mul(h2, self.w_gu, "NT") if self.gu_block else lib.silu_mul(lib.hgemm(h2, self.w_gu, "NT"))
         down = lib.hgemm(act, self.w_d, "NT")
         return res.add_(down).view(B, S, H)
 

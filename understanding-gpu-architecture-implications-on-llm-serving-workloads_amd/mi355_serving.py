@@ -12,8 +12,9 @@ LIB_PATH = os.path.join(_HERE, "libmi355_serving.so")
 
 GEMM_NN, GEMM_NT, GEMM_TN = 0, 1, 2
 LAYOUTS = {"NN": GEMM_NN, "NT": GEMM_NT, "TN": GEMM_TN}
+ERR_BAD_ARGUMENT, ERR_UNSUPPORTED = 10001, 10002
 
-EXPORTED_SYMBOLS = ("mi355_hgemm", "mi355_fmha_fwd", "mi355_fmha_fwd_strided", "mi355_fmha_fwd_bf16", "mi355_rmsnorm", "mi355_rope", "mi355_silu_mul",
+EXPORTED_SYMBOLS = ("mi355_hgemm", "mi355_fmha_fwd", "mi355_fmha_fwd_strided", "mi355_fmha_fwd_bf16", "mi355_hgemm_silu_mul", "mi355_rmsnorm", "mi355_rope", "mi355_silu_mul",
                     "mi355_last_error", "mi355_serving_version",
                     "mi355_debug_set_gemm_variant", "mi355_debug_set_fmha_variant")
 
@@ -50,7 +51,9 @@ def load():
     lib.mi355_rmsnorm.restype = i32
     lib.mi355_rope.argtypes = [vp, vp, i32, i32, i32, i32, i32, i64, i64, i64, i64, vp, vp, vp, i64, i32, vp]
     lib.mi355_rope.restype = i32
-    lib.mi355_silu_mul.argtypes = [vp, vp, i64, i32, i64, i64, vp]
+    lib.mi355_silu_mul.argtypes = [vp, vp, i64, i32, i32, i64, i64, vp]
+    lib.mi355_hgemm_silu_mul.argtypes = lib.mi355_hgemm.argtypes
+    lib.mi355_hgemm_silu_mul.restype = i32
     lib.mi355_silu_mul.restype = i32
     lib.mi355_last_error.argtypes = []
     lib.mi355_last_error.restype = ctypes.c_char_p
@@ -201,13 +204,52 @@ def rope(x, cos, sin, positions, out=None, copy_heads=0):
     return out
 
 
-def silu_mul(gate_up, out=None):
-    """silu(gate_up[:, :F]) * gate_up[:, F:] for a [rows, 2F] fp16 tensor."""
+def silu_mul(gate_up, out=None, interleave=0):
+    """silu(gate) * up for a [rows, 2F] fp16 tensor holding gate in its first F columns and up in the rest
+    (interleave=0), or gate and up alternating in groups of `interleave` columns."""
     import torch
     assert gate_up.dim() == 2 and gate_up.stride(1) == 1 and gate_up.dtype == torch.float16
     rows, two_f = gate_up.shape
     inter = two_f // 2
     if out is None:
         out = torch.empty((rows, inter), dtype=torch.float16, device=gate_up.device)
-    _check(load().mi355_silu_mul(_ptr(gate_up), _ptr(out), rows, inter, gate_up.stride(0), out.stride(0), _stream_of(gate_up)))
+    _check(load().mi355_silu_mul(_ptr(gate_up), _ptr(out), rows, inter, int(interleave), gate_up.stride(0), out.stride(0),
+                                 _stream_of(gate_up)))
+    return out
+
+
+GATE_UP_BLOCK = 32  # columns per gate / up group in the operand of mi355_hgemm_silu_mul
+
+
+def interleave_gate_up(gate, up, dim=0):
+    """Weight of mi355_hgemm_silu_mul from the two projection weights: groups of 32 gate outputs alternate with the
+    32 up outputs of the same positions along `dim` (0 for nn.Linear-layout [out, in] weights, 1 for [in, out])."""
+    import torch
+    F = gate.shape[dim]
+    assert gate.shape == up.shape and F % GATE_UP_BLOCK == 0
+    if dim == 0:
+        g = gate.reshape(F // GATE_UP_BLOCK, GATE_UP_BLOCK, -1)
+        u = up.reshape(F // GATE_UP_BLOCK, GATE_UP_BLOCK, -1)
+        return torch.stack((g, u), 1).reshape(2 * F, -1).contiguous()
+    g = gate.reshape(-1, F // GATE_UP_BLOCK, GATE_UP_BLOCK)
+    u = up.reshape(-1, F // GATE_UP_BLOCK, GATE_UP_BLOCK)
+    return torch.stack((g, u), 2).reshape(-1, 2 * F).contiguous()
+
+
+def hgemm_silu_mul(a, w, layout="NT", out=None):
+    """silu(a @ gate) * (a @ up) for a weight built by interleave_gate_up: one launch where the tiled GEMM covers the
+    shape (mi355_hgemm_silu_mul), otherwise the product followed by silu_mul on the interleaved columns."""
+    import torch
+    lay = LAYOUTS[layout] if isinstance(layout, str) else int(layout)
+    assert lay in (GEMM_NN, GEMM_NT) and a.is_contiguous() and w.is_contiguous() and a.dtype == torch.float16
+    M, K = a.shape
+    N2 = w.shape[0] if lay == GEMM_NT else w.shape[1]
+    N = N2 // 2
+    if out is None:
+        out = torch.empty((M, N), dtype=torch.float16, device=a.device)
+    rc = load().mi355_hgemm_silu_mul(_ptr(a), _ptr(w), _ptr(out), M, N, K, a.stride(0), w.stride(0), out.stride(0), lay,
+                                     _stream_of(a))
+    if rc == ERR_UNSUPPORTED:
+        return silu_mul(hgemm(a, w, layout), out=out, interleave=GATE_UP_BLOCK)
+    _check(rc)
     return out
