@@ -53,7 +53,8 @@ extern "C" {
  *   layout NT  <- finegemm_13..15 (manual/gemm_13_amd.cpp:248-270, gemm_14_amd.cpp:268-290,
  *                                  gemm_15_amd.cpp:291-313)
  * lda/ldb/ldc are in elements and refer to the stored matrices (e.g. lda >= M for layout TN).
- * Any M, N, K >= 1 is accepted; shapes that are multiples of the kernel tiles take the fast paths.
+ * Any M, N, K >= 1 is accepted. The fast paths need 16-byte aligned operands and leading dimensions, K % 64 == 0 and
+ * N % 8 == 0 (M % 8 == 0 for layout TN); M is otherwise free (ragged tile edges are handled inside the kernels).
  */
 int mi355_hgemm(const void* A, const void* B, void* C, int M, int N, int K, int64_t lda, int64_t ldb,
                 int64_t ldc, int layout, void* stream);
@@ -64,7 +65,7 @@ int mi355_hgemm(const void* A, const void* B, void* C, int M, int N, int K, int6
  * gate and up projections of a Llama MLP computed by one GEMM on an interleaved weight matrix, with the activation
  * applied to the accumulators before the single rounding to fp16. Replaces `self.act_fn(self.gate_proj(x)) * self.up_proj(x)`
  * (benchmarks/flashattn-cuda/modeling_llama.py:227): two GEMMs, a SiLU kernel and a multiply kernel in the reference.
- * Layouts NN and NT. Only shapes the tiled kernels cover have the fused form (M and 2N multiples of 128, K a multiple of 64,
+ * Layouts NN and NT. Only shapes the tiled kernels cover have the fused form (M > 64, N a multiple of 32, K a multiple of 64,
  * 16-byte aligned operands and leading dimensions); others return MI355_ERR_UNSUPPORTED and nothing is launched: run
  * mi355_hgemm on the same operands followed by mi355_silu_mul with interleave = 32.
  */

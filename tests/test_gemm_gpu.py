@@ -88,6 +88,29 @@ def test_layouts_and_shapes(lib, gpu, layout, M, N, K):
     assert c.shape == (M, N)
 
 
+@pytest.mark.parametrize("variant", [0, 1, 2])
+@pytest.mark.parametrize("layout", ["NN", "TN", "NT"])
+@pytest.mark.parametrize("M,N,K", [(1000, 1000, 1024), (300, 4096, 512), (2056, 1032, 128), (130, 8, 64), (4104, 4096, 256),
+                                   (257, 264, 64)])
+def test_ragged_m_and_n_on_the_tiled_kernels(lib, gpu, variant, layout, M, N, K):
+    # token counts and widths that are not multiples of the tile (multiples of 8 where 16-byte chunks must not straddle the
+    # end): same kernels with the out-of-range rows folded back inside; the surrounding memory of C stays untouched
+    a, b = operands(M, N, K, layout, seed=M + N)
+    ref = so.gemm_ref(a, b, layout)
+    c = torch.full((M + 2, N + 8), 9.0, dtype=torch.float16, device=gpu)
+    ag, bg = a.to(gpu), b.to(gpu)
+    lib.set_variants(gemm=variant)
+    try:
+        lib.hgemm_raw(ag.data_ptr(), bg.data_ptr(), c.data_ptr(), M, N, K, ag.stride(0), bg.stride(0), c.stride(0),
+                      lib.LAYOUTS[layout], torch.cuda.current_stream().cuda_stream)
+        torch.cuda.synchronize()
+    finally:
+        lib.set_variants()
+    ok, st = so.gemm_tolerance_ok(c[:M, :N].cpu(), ref, K)
+    assert ok, st
+    assert bool((c[M:] == 9.0).all()) and bool((c[:, N:] == 9.0).all())
+
+
 @pytest.mark.parametrize("variant", [1, 2])
 @pytest.mark.parametrize("layout", ["NN", "TN", "NT"])
 def test_every_tile_variant(lib, gpu, variant, layout):

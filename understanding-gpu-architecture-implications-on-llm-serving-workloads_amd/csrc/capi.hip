@@ -81,7 +81,7 @@ int mi355_hgemm_silu_mul(const void* A, const void* B, void* C, int M, int N, in
     hipError_t e = mi355::hgemm_silu_mul_dispatch(A, B, C, M, 2 * N, K, lda, ldb, ldc, layout, static_cast<hipStream_t>(stream));
     if (e == hipErrorNotSupported)
         return fail(MI355_ERR_UNSUPPORTED,
-                    "mi355_hgemm_silu_mul: needs M and 2N multiples of 128, K a multiple of 64 and 16-byte aligned operands; "
+                    "mi355_hgemm_silu_mul: needs M > 64, N a multiple of 32, K a multiple of 64 and 16-byte aligned operands; "
                     "run mi355_hgemm and mi355_silu_mul(interleave = 32) instead");
     if (e != hipSuccess) return hip_fail(e, "mi355_hgemm_silu_mul launch");
     return 0;

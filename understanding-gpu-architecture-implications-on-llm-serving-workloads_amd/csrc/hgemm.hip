@@ -156,7 +156,10 @@ __device__ __forceinline__ void tile_of_block(int bid, int tiles_m, int tiles_n,
 // columns and their 32 up columns (`act_fn(gate_proj(x)) * up_proj(x)`, benchmarks/flashattn-cuda/modeling_llama.py:227,
 // with the two projections interleaved in one weight matrix): a wave then holds g and u of the same outputs in its two
 // column blocks, at the same accumulator positions, and C has N / 2 columns.
-template <bool A_KC, bool B_KC, int BM, int BN, int WM, int WN, int EPI = 0>
+// RAGGED: M (and N) need not be multiples of the tile. Copies of rows past the end are redirected to the last row (or, for
+// an operand whose M/N index is contiguous, to the last 8 columns; that dimension must be a multiple of 8), so every
+// load stays inside the matrices, and the epilogue stores only what exists.
+template <bool A_KC, bool B_KC, int BM, int BN, int WM, int WN, int EPI = 0, bool RAGGED = false>
 __global__ __launch_bounds__(WM * WN * 64) void hgemm_main_kernel(const half_t* __restrict__ A, const half_t* __restrict__ B,
                                                          half_t* __restrict__ C, int M, int N, int K, long lda,
                                                          long ldb, long ldc) {
@@ -177,7 +180,7 @@ __global__ __launch_bounds__(WM * WN * 64) void hgemm_main_kernel(const half_t* 
     const int wn = wave % Cfg::WN;
 
     int tile_m, tile_n;
-    tile_of_block(blockIdx.x, M / Cfg::BM, N / Cfg::BN, tile_m, tile_n);
+    tile_of_block(blockIdx.x, (M + Cfg::BM - 1) / Cfg::BM, (N + Cfg::BN - 1) / Cfg::BN, tile_m, tile_n);
     const long m0 = (long)tile_m * Cfg::BM;
     const long n0 = (long)tile_n * Cfg::BN;
 
@@ -205,9 +208,54 @@ __global__ __launch_bounds__(WM * WN * 64) void hgemm_main_kernel(const half_t* 
         b_k_stride = BTN::ktile_stride(ldb);
     }
 
+    // RAGGED: one pointer per copy, rows / column chunks past the end folded back inside
+    const half_t* a_ptr[RAGGED ? Cfg::A_INSTS : 1];
+    const half_t* b_ptr[RAGGED ? Cfg::B_INSTS : 1];
+    if constexpr (RAGGED) {
+        auto clamped = [&](const half_t* base, long ld, bool k_contig, int rows_per_inst, int chunks_per_row, int rows_per_pass,
+                           int i, long origin, long extent, int swz) {
+            const int row = wave * rows_per_inst + lane / chunks_per_row + i * rows_per_pass;
+            const int chunk = (lane % chunks_per_row) ^ swz;
+            if (k_contig) return base + min(origin + row, extent - 1) * ld + chunk * 8;   // row = M/N index
+            return base + (long)row * ld + min(origin + chunk * 8, extent - 8);           // row = K index
+        };
+#pragma unroll
+        for (int i = 0; i < Cfg::A_INSTS; ++i) {
+            if constexpr (A_KC) {
+                const int row = wave * ATK::kRowsPerInst + lane / ATK::kChunksPerRow;
+                a_ptr[i] = clamped(A, lda, true, ATK::kRowsPerInst, ATK::kChunksPerRow, ATK::kRowsPerPass, i, m0, M, ATK::swz(row));
+            } else {
+                const int row = wave * ATM::kRowsPerInst + lane / ATM::kChunksPerRow + i * ATM::kRowsPerPass;
+                a_ptr[i] = clamped(A, lda, false, ATM::kRowsPerInst, ATM::kChunksPerRow, ATM::kRowsPerPass, i, m0, M, ATM::swz(row));
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < Cfg::B_INSTS; ++i) {
+            if constexpr (B_KC) {
+                const int row = wave * BTK::kRowsPerInst + lane / BTK::kChunksPerRow;
+                b_ptr[i] = clamped(B, ldb, true, BTK::kRowsPerInst, BTK::kChunksPerRow, BTK::kRowsPerPass, i, n0, N, BTK::swz(row));
+            } else {
+                const int row = wave * BTN::kRowsPerInst + lane / BTN::kChunksPerRow + i * BTN::kRowsPerPass;
+                b_ptr[i] = clamped(B, ldb, false, BTN::kRowsPerInst, BTN::kChunksPerRow, BTN::kRowsPerPass, i, n0, N, BTN::swz(row));
+            }
+        }
+    }
     auto issue_copies = [&](int stage) {
         MI355_LDS char* sa = smem + stage * Cfg::STAGE_BYTES;
         MI355_LDS char* sb = sa + Cfg::A_BYTES;
+        if constexpr (RAGGED) {
+#pragma unroll
+            for (int i = 0; i < Cfg::A_INSTS; ++i) {
+                copy16_global_to_lds(a_ptr[i], sa + (i * Cfg::NWAVES + wave) * 1024);
+                a_ptr[i] += a_k_stride;
+            }
+#pragma unroll
+            for (int i = 0; i < Cfg::B_INSTS; ++i) {
+                copy16_global_to_lds(b_ptr[i], sb + (i * Cfg::NWAVES + wave) * 1024);
+                b_ptr[i] += b_k_stride;
+            }
+            return;
+        }
 #pragma unroll
         for (int i = 0; i < Cfg::A_INSTS; ++i)
             copy16_global_to_lds(a_src + i * a_copy_stride, sa + (i * Cfg::NWAVES + wave) * 1024);
@@ -373,11 +421,13 @@ __global__ __launch_bounds__(WM * WN * 64) void hgemm_main_kernel(const half_t* 
         const int rr = lane / kChunksC;
         const int cc = lane % kChunksC;
         half_t* cbase = C + (m0 + wm * TM * 32) * ldc + (EPI == 1 ? n0 / 2 : n0) + wn * TNO * 32 + cc * 8;
+        const long rows_left = M - (m0 + wm * TM * 32);   // RAGGED: rows and 8-column chunks that exist
+        const bool col_ok = (EPI == 1 ? n0 / 2 : n0) + wn * TNO * 32 + cc * 8 < (EPI == 1 ? N / 2 : N);
 #pragma unroll
         for (int it = 0; it < TM * 32 / kRowsPerStore; ++it) {
             const int row = it * kRowsPerStore + rr;
             half8 v = *(MI355_LDS const half8*)(cst + row * kRowBytesC + ((cc ^ (row & (kChunksC < 8 ? kChunksC - 1 : 7))) << 4));
-            *(half8*)(cbase + (long)row * ldc) = v;
+            if (!RAGGED || (row < rows_left && col_ok)) *(half8*)(cbase + (long)row * ldc) = v;
         }
     }
 }
@@ -680,14 +730,16 @@ static hipError_t launch_smallm_nt(const half_t* A, const half_t* B, half_t* C, 
 
 int g_gemm_variant = 0;  // tuning hook: 0 = heuristic, 1 = force 256x256 tiles, 2 = force 128x128 tiles
 
-template <bool A_KC, bool B_KC, int BM, int BN, int WM, int WN, int EPI = 0>
+template <bool A_KC, bool B_KC, int BM, int BN, int WM, int WN, int EPI = 0, bool RAGGED = false>
 static hipError_t launch_main(const half_t* A, const half_t* B, half_t* C, int M, int N, int K, long lda, long ldb,
                               long ldc, hipStream_t stream) {
     using Cfg = MainCfg<A_KC, B_KC, BM, BN, WM, WN>;
-    auto kern = hgemm_main_kernel<A_KC, B_KC, BM, BN, WM, WN, EPI>;
+    auto kern = hgemm_main_kernel<A_KC, B_KC, BM, BN, WM, WN, EPI, RAGGED>;
     static DynamicLdsOnce lds_once;
     if (hipError_t e = lds_once.ensure(reinterpret_cast<const void*>(kern), Cfg::LDS_BYTES); e != hipSuccess) return e;
-    int blocks = (M / BM) * (N / BN);
+    const long nblocks = (long)((M + BM - 1) / BM) * ((N + BN - 1) / BN);
+    if (nblocks > 0x7fffffffL) return hipErrorInvalidValue;
+    int blocks = (int)nblocks;
     kern<<<dim3(blocks), dim3(Cfg::NTHREADS), Cfg::LDS_BYTES, stream>>>(A, B, C, M, N, K, lda, ldb, ldc);
     return hipGetLastError();
 }
@@ -720,6 +772,13 @@ static hipError_t launch_layout(const half_t* A, const half_t* B, half_t* C, int
         case 2: return launch_main<A_KC, B_KC, 128, 128, 2, 2>(A, B, C, M, N, K, lda, ldb, ldc, stream);
         default: break;
     }
+    // ragged M / N on the same tiles: N (and M for layout TN) a multiple of 8, so 16-byte chunks never straddle the end
+    if (k_ok && N % 8 == 0 && N >= 8 && (A_KC || (M % 8 == 0 && M >= 8))) {
+        const long t256 = (long)((M + 255) / 256) * ((N + 255) / 256);
+        if ((t256 >= 192 && g_gemm_variant != 2) || g_gemm_variant == 1)
+            return launch_main<A_KC, B_KC, 256, 256, 2, 4, 0, true>(A, B, C, M, N, K, lda, ldb, ldc, stream);
+        return launch_main<A_KC, B_KC, 128, 128, 2, 2, 0, true>(A, B, C, M, N, K, lda, ldb, ldc, stream);
+    }
     dim3 grid((N + 63) / 64, (M + 63) / 64);
     hgemm_edge_kernel<A_KC, B_KC><<<grid, dim3(256), 0, stream>>>(A, B, C, M, N, K, lda, ldb, ldc);
     return hipGetLastError();
@@ -732,11 +791,17 @@ static hipError_t launch_silu_mul(const half_t* A, const half_t* B, half_t* C, i
                                   long ldc, hipStream_t stream) {
     const bool aligned = (reinterpret_cast<uintptr_t>(A) % 16 == 0) && (reinterpret_cast<uintptr_t>(B) % 16 == 0) &&
                          (reinterpret_cast<uintptr_t>(C) % 16 == 0) && (lda % 8 == 0) && (ldb % 8 == 0) && (ldc % 8 == 0);
-    if (!aligned || K % 64 != 0 || K < 64 || M % 128 != 0 || N % 128 != 0) return hipErrorNotSupported;
+    // N = columns of op(B); gate/up pairs are 64 columns wide. Few rows are better served by the small-M product.
+    if (!aligned || K % 64 != 0 || K < 64 || N % 64 != 0 || M <= 64) return hipErrorNotSupported;
+    const bool fits128 = M % 128 == 0 && N % 128 == 0;
     const bool fits256 = M % 256 == 0 && N % 256 == 0;
-    if (fits256 && (long)(M / 256) * (N / 256) >= 192)
-        return launch_main<A_KC, B_KC, 256, 256, 2, 4, 1>(A, B, C, M, N, K, lda, ldb, ldc, stream);
-    return launch_main<A_KC, B_KC, 128, 128, 2, 2, 1>(A, B, C, M, N, K, lda, ldb, ldc, stream);
+    const long t256 = (long)((M + 255) / 256) * ((N + 255) / 256);
+    if (t256 >= 192) {
+        if (fits256) return launch_main<A_KC, B_KC, 256, 256, 2, 4, 1>(A, B, C, M, N, K, lda, ldb, ldc, stream);
+        return launch_main<A_KC, B_KC, 256, 256, 2, 4, 1, true>(A, B, C, M, N, K, lda, ldb, ldc, stream);
+    }
+    if (fits128) return launch_main<A_KC, B_KC, 128, 128, 2, 2, 1>(A, B, C, M, N, K, lda, ldb, ldc, stream);
+    return launch_main<A_KC, B_KC, 128, 128, 2, 2, 1, true>(A, B, C, M, N, K, lda, ldb, ldc, stream);
 }
 
 hipError_t hgemm_silu_mul_dispatch(const void* A, const void* B, void* C, int M, int N2, int K, long lda, long ldb, long ldc,
