@@ -273,8 +273,8 @@ def main():
         ms_l = time_launches(lambda: layer(xl), 5, 2)
         other["L5_decoder_layer_prefill_s8192"] = {
             "ms": ms_l, "tflops": tot_fl / ms_l / 1e9,
-            "note": "whole FineLlamaDecoderLayer.forward (12 launches: norms, fused QKV GEMM, RoPE, attention on strided operands, "
-                    "O projection, gate/up GEMM, SiLU*up, down GEMM, residual adds), flops of the GEMMs and attention only"}
+            "note": "whole FineLlamaDecoderLayer.forward (11 launches: norms, fused QKV GEMM, RoPE, attention on strided operands, "
+                    "O projection, gate/up GEMM with SiLU*up epilogue, down GEMM, residual adds), flops of the GEMMs and attention only"}
         Bd = 8
         cache = FineKVCache(Bd, S5 + 64, 8, device=dev)
         cache.k.normal_(0, 1)
@@ -288,6 +288,20 @@ def main():
         other["L5_decoder_layer_generation_step_b8_past8192"] = {"ms": ms_s, "gbs": by_s / ms_s / 1e6,
                                                                  "pct_of_hbm_peak": 100 * by_s / ms_s / 1e6 / PEAK_HBM_GBS,
                                                                  "note": "bytes = layer weights + KV cache read once"}
+        # the same step captured once into a HIP graph and replayed (warm-up on the capture stream first)
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            step()
+        torch.cuda.current_stream().wait_stream(side)
+        graph = torch.cuda.CUDAGraph()
+        cache.length = S5
+        with torch.cuda.graph(graph, stream=side):
+            layer(xd1, kv_cache=cache)
+        ms_g = time_launches(graph.replay, 20, 3)
+        other["L5_decoder_layer_generation_step_b8_past8192_hip_graph"] = {"ms": ms_g, "gbs": by_s / ms_g / 1e6,
+                                                                           "pct_of_hbm_peak": 100 * by_s / ms_g / 1e6 / PEAK_HBM_GBS}
+        del graph
         del layer, cache
 
     # ---- CPU baseline: the same step with torch fp32 on the host cores -------------------------------------------------

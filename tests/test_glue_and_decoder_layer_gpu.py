@@ -206,3 +206,43 @@ def test_decoder_layer_from_transformers_weights(lib, gpu):
     out = layer(x.to(gpu))
     rel = float((out.float().cpu() - y).norm() / y.norm())
     assert rel <= 3e-3, rel
+
+
+def test_generation_step_replays_from_a_hip_graph(lib, gpu):
+    # A serving loop captures the launch-bound generation step once and replays it. Every kernel on the path is a plain
+    # launch on the current stream (no memsets, no synchronisation); the split-KV workspace is obtained by a warm-up call on
+    # the capture stream. Replays are interleaved with eager work and each is compared with the eager result.
+    from llama_layer import FineKVCache, FineLlamaDecoderLayer
+    B, S0, H, n_q, n_kv, F = 4, 640, 512, 8, 2, 1024
+    w = layer_weights(H, n_q, n_kv, F, seed=30)
+    layer = FineLlamaDecoderLayer({k: v.to(gpu) for k, v in w.items()}, n_q, n_kv, max_positions=1024)
+    cache = FineKVCache(B, S0 + 1, n_kv, device=gpu)
+    layer(so.randn_fp16((B, S0, H), 1).to(gpu), kv_cache=cache)
+    x_static = so.randn_fp16((B, 1, H), 2).to(gpu)
+    cache.length = S0
+    eager = layer(x_static, kv_cache=cache).clone()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        cache.length = S0
+        layer(x_static, kv_cache=cache)            # warm-up on the capture stream: workspace and allocator pools
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    cache.length = S0
+    with torch.cuda.graph(graph, stream=side):
+        out_static = layer(x_static, kv_cache=cache)
+    for it in range(3):
+        scratch = torch.randn(1 << 20, device=gpu).sum()      # unrelated eager work between replays
+        x_new = so.randn_fp16((B, 1, H), 50 + it).to(gpu)
+        x_static.copy_(x_new)
+        graph.replay()
+        torch.cuda.synchronize()
+        cache.length = S0
+        want = layer(x_new, kv_cache=cache)
+        torch.cuda.synchronize()
+        assert torch.equal(out_static, want), it
+        assert torch.isfinite(scratch)
+    x_static.copy_(so.randn_fp16((B, 1, H), 2).to(gpu))
+    graph.replay()
+    torch.cuda.synchronize()
+    assert torch.equal(out_static, eager)
