@@ -32,6 +32,7 @@ PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (KiB per dispatch), each scaled by what the same
 # counter reads for a 1 GiB device-to-device copy (FETCH_SIZE x2.0, WRITE_SIZE x1.0); see profiles/.
 MEASURED_TRAFFIC_BYTES = (786882 * 2.0 + 131072 * 1.0) * 1024        # hgemm_main_kernel, 8192^3 NN
+MEASURED_TRAFFIC_BYTES_G2C = (57881 * 2.0 + 448 * 1.0) * 1024          # hgemm_smallm_nn_kernel, 16 x 14336 x 4096
 MEASURED_TRAFFIC_BYTES_FMHA = (26371 * 2.0 + 33280 * 1.0) * 1024     # fmha_fwd_pingpong_kernel, F4
 
 
@@ -184,6 +185,7 @@ def main():
 
     # ---- the other benchmark configurations (quick timings) ----------------------------------------------------------
     other = {}
+    roofline_g2c = None
     if not args.no_other_configs:
         def t_gemm(m, n, kk, iters=20):
             x = so.randn_fp16((m, kk), 1).to(dev)
@@ -197,6 +199,9 @@ def main():
         other["G1_gemm_1024"] = t_gemm(1024, 1024, 1024)
         other["G2a_gemm_4096"] = t_gemm(4096, 4096, 4096)
         other["G2c_gemm_decode_16x14336x4096"] = t_gemm(16, 14336, 4096)
+        g2c = other["G2c_gemm_decode_16x14336x4096"]
+        roofline_g2c = {"kernel": "hgemm_smallm_nn_kernel (G2c: 16 x 14336 x 4096, NN)", "bound": "hbm", "achieved": g2c["gbs"],
+                        "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": g2c["gbs"] / PEAK_HBM_GBS, "traffic": MEASURED_TRAFFIC_BYTES_G2C}
         q3, k3, v3 = (t.to(dev) for t in so.fmha_inputs(4, 32, 32, 1024, 1024, seed=42))
         o3 = torch.empty_like(q3)
         ms3 = time_launches(lambda: lib.fmha_fwd_raw(q3.data_ptr(), k3.data_ptr(), v3.data_ptr(), o3.data_ptr(), None, 4, 32,
@@ -330,7 +335,8 @@ def main():
         "dtype": "fp16 (fp32 accumulate)", "data": "synthetic",
         "config": {"workload": "one step = hgemm 8192x8192x8192 NN (G2b) + fmha fwd causal GQA b1 h32/8 s4096 d128 with LSE (F4)",
                    "flops_per_step": gemm_flops + fmha_flops, "pct_of_fp16_mfma_peak": 100 * value / PEAK_FP16_TFLOPS},
-        "kernels": kernels, "roofline": roofline, "roofline_fmha": roofline_fmha, "cpu_baseline": cpu_baseline,
+        "kernels": kernels, "roofline": roofline, "roofline_fmha": roofline_fmha, "roofline_decode_gemm": roofline_g2c,
+        "cpu_baseline": cpu_baseline,
         "other_configs": other, "parity": checks,
     }
     print(json.dumps(out))
