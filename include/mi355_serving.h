@@ -33,7 +33,7 @@ extern "C" {
 #define MI355_ERR_BAD_ARGUMENT 10001
 #define MI355_ERR_UNSUPPORTED 10002
 
-/* element types (internal tags of the attention dispatcher; the entry points fix the type by name) */
+/* element types (internal tags of the dispatchers; the entry points fix the type by name) */
 #define MI355_DTYPE_FP16 0
 #define MI355_DTYPE_BF16 1
 
@@ -156,6 +156,23 @@ int mi355_rope(const void* x, void* out, int B, int S, int heads, int copy_heads
  */
 int mi355_silu_mul(const void* gate_up, void* out, int64_t rows, int inter, int interleave, int64_t ld_in, int64_t ld_out,
                    void* stream);
+
+/*
+ * bfloat16 twins of the fp16 entry points above: identical arguments and semantics, bfloat16 operands and results, fp32
+ * accumulation and arithmetic (MFMA bf16 instructions with the fp16 kernels' tiling). For models whose checkpoints are
+ * bfloat16; the reference's own bf16 use is its attention operator `finefmha_5` (see mi355_fmha_fwd_bf16).
+ */
+int mi355_gemm_bf16(const void* A, const void* B, void* C, int M, int N, int K, int64_t lda, int64_t ldb, int64_t ldc,
+                    int layout, void* stream);
+int mi355_gemm_silu_mul_bf16(const void* A, const void* B, void* C, int M, int N, int K, int64_t lda, int64_t ldb,
+                             int64_t ldc, int layout, void* stream);
+int mi355_rmsnorm_bf16(const void* x, const void* residual, void* residual_out, const void* weight, void* out, int64_t rows,
+                       int hidden, int64_t ldx, int64_t ldr, int64_t ldro, int64_t ldo, float eps, void* stream);
+int mi355_rope_bf16(const void* x, void* out, int B, int S, int heads, int copy_heads, int D, int64_t x_batch, int64_t x_row,
+                    int64_t out_batch, int64_t out_row, const float* cos_table, const float* sin_table,
+                    const int32_t* positions, int64_t pos_batch, int n_positions, void* stream);
+int mi355_silu_mul_bf16(const void* gate_up, void* out, int64_t rows, int inter, int interleave, int64_t ld_in, int64_t ld_out,
+                        void* stream);
 
 /* Thread-local text for the last non-zero return of this thread ("" if none). */
 const char* mi355_last_error(void);

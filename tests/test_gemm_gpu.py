@@ -201,3 +201,39 @@ def test_torch_operator_noncontiguous_inputs_and_stream(gpu):
     s.synchronize()
     ok, st = so.gemm_tolerance_ok(c, so.gemm_ref(a, b), 300)
     assert ok, st
+
+
+# ---- bfloat16 ---------------------------------------------------------------------------------------------------------
+# Tolerance for bfloat16 results (8 significand bits): |err| <= 2e-2 * sqrt(K / 1024) + 2^-8 |ref| against the fp32 product of
+# the bf16-rounded operands (the accumulation slack of the fp16 bound plus one bf16 rounding).
+def bf16_close(c, ref, K):
+    err = (c.float().cpu() - ref).abs()
+    return bool((err <= 2e-2 * (K / 1024) ** 0.5 + 2.0 ** -8 * ref.abs()).all()), float(err.max())
+
+
+@pytest.mark.parametrize("layout", ["NN", "NT", "TN"])
+@pytest.mark.parametrize("M,N,K", [(1024, 1024, 1024), (512, 768, 320), (1000, 264, 128), (16, 4096, 1024), (7, 72, 96),
+                                   (100, 70, 50)])
+def test_bfloat16_gemm(lib, gpu, layout, M, N, K):
+    a, b = operands(M, N, K, layout, seed=K, b_std=0.05)
+    a, b = a.float().bfloat16(), b.float().bfloat16()
+    c = lib.hgemm(a.to(gpu), b.to(gpu), layout)
+    assert c.dtype == torch.bfloat16
+    ok, worst = bf16_close(c, so.gemm_ref(a, b, layout), K)
+    assert ok, worst
+
+
+def test_bfloat16_gemm_exact_cases_and_torch_operator(lib, gpu):
+    import gemm_unified
+    n = 256
+    b = so.randn_fp16((n, n), 3).float().bfloat16()
+    eye = torch.eye(n, dtype=torch.bfloat16)
+    assert torch.equal(lib.hgemm(eye.to(gpu), b.to(gpu)).cpu(), b)            # identity: exact
+    ones = torch.ones((n, 1024), dtype=torch.bfloat16)
+    c = lib.hgemm(ones.to(gpu), torch.ones((1024, n), dtype=torch.bfloat16).to(gpu)).cpu()
+    assert bool((c == 1024).all())                                            # 1024 is representable in bf16
+    a = so.randn_fp16((n, n), 4).float().bfloat16()
+    out = gemm_unified.ops.fine_gemm(a.to(gpu), b.to(gpu), 13)                # NT index, bf16 tensors
+    assert out.dtype == torch.bfloat16 and bf16_close(out, so.gemm_ref(a, b, "NT"), n)[0]
+    with pytest.raises(RuntimeError, match="dtype"):
+        gemm_unified.ops.fine_gemm(a.to(gpu), b.half().to(gpu), 0)

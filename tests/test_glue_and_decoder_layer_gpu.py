@@ -246,3 +246,50 @@ def test_generation_step_replays_from_a_hip_graph(lib, gpu):
     graph.replay()
     torch.cuda.synchronize()
     assert torch.equal(out_static, eager)
+
+
+# ---- bfloat16 ---------------------------------------------------------------------------------------------------------
+def close_one_bf16_rounding(out, ref):
+    err = (out.float().cpu() - ref).abs()
+    return bool((err <= 2.0 ** -8 * ref.abs() + 1e-6).all()), float(err.max())
+
+
+def test_bfloat16_glue_kernels(lib, gpu):
+    bf = lambda t: t.float().bfloat16()
+    x, r, w = bf(so.randn_fp16((33, 1024), 1, 2.0)), bf(so.randn_fp16((33, 1024), 2)), bf(so.randn_fp16((1024,), 3))
+    ref, h_ref = so.rmsnorm_ref(x, w, 1e-5, residual=r, round_residual=False)
+    h_ref = h_ref.bfloat16().float()                      # the kernel stores and normalises the bf16-rounded sum
+    ref, _ = so.rmsnorm_ref(h_ref, w, 1e-5)
+    out, h = lib.rmsnorm(x.to(gpu), w.to(gpu), 1e-5, residual=r.to(gpu))
+    assert out.dtype == torch.bfloat16 and torch.equal(h.float().cpu(), h_ref) and close_one_bf16_rounding(out, ref)[0]
+    cos, sin = so.rope_tables(64, 128, 10000.0)
+    pos = torch.arange(5, 5 + 9, dtype=torch.int32)
+    q = bf(so.randn_fp16((2, 9, 6, 128), 4))
+    qg = q.to(gpu)
+    lib.rope(qg, cos.to(gpu), sin.to(gpu), pos.to(gpu), copy_heads=2)
+    ref_q = so.rope_ref(q[:, :, :4].transpose(1, 2), cos, sin, pos[None].expand(2, 9)).transpose(1, 2)
+    assert close_one_bf16_rounding(qg[:, :, :4], ref_q)[0] and torch.equal(qg[:, :, 4:].cpu(), q[:, :, 4:])
+    gu = bf(so.randn_fp16((17, 512), 5, 3.0))
+    assert close_one_bf16_rounding(lib.silu_mul(gu.to(gpu)), so.silu_mul_ref(gu))[0]
+
+
+def test_bfloat16_decoder_layer_prefill_and_step(lib, gpu):
+    # same layer in bfloat16 (weights, activations, cache); compared with the fp32 oracle on the bf16-rounded weights.
+    # bf16 intermediates carry 8 significand bits: relative Frobenius error <= 1.5e-2.
+    from llama_layer import FineKVCache, FineLlamaDecoderLayer
+    B, S0, H, n_q, n_kv, F = 2, 600, 512, 8, 2, 1024
+    w = {k: v.float().bfloat16() for k, v in layer_weights(H, n_q, n_kv, F, seed=40).items()}
+    layer = FineLlamaDecoderLayer({k: v.to(gpu) for k, v in w.items()}, n_q, n_kv, max_positions=1024, dtype=torch.bfloat16)
+    cache = FineKVCache(B, S0 + 2, n_kv, device=gpu, dtype=torch.bfloat16)
+    x = so.randn_fp16((B, S0, H), 1).float().bfloat16()
+    out = layer(x.to(gpu), kv_cache=cache)
+    ref, k_ref, v_ref = so.llama_decoder_layer_ref(x, w, torch.arange(S0)[None].expand(B, S0), n_q, n_kv, round_stages=False)
+    assert out.dtype == torch.bfloat16
+    rel = float((out.float().cpu() - ref).norm() / ref.norm())
+    assert rel <= 1.5e-2, rel
+    xt = so.randn_fp16((B, 1, H), 2).float().bfloat16()
+    out = layer(xt.to(gpu), kv_cache=cache)
+    ref, _, _ = so.llama_decoder_layer_ref(xt, w, torch.full((B, 1), S0), n_q, n_kv, past_k=k_ref, past_v=v_ref,
+                                           round_stages=False)
+    rel = float((out.float().cpu() - ref).norm() / ref.norm())
+    assert rel <= 1.5e-2, rel

@@ -23,21 +23,32 @@ int hip_fail(hipError_t e, const char* what) {
 
 extern "C" {
 
-int mi355_hgemm(const void* A, const void* B, void* C, int M, int N, int K, int64_t lda, int64_t ldb, int64_t ldc,
+static int hgemm_impl(const char* fn, int dtype, const void* A, const void* B, void* C, int M, int N, int K, int64_t lda, int64_t ldb, int64_t ldc,
                 int layout, void* stream) {
-    if (!A || !B || !C) return fail(MI355_ERR_BAD_ARGUMENT, "mi355_hgemm: null pointer");
-    if (M < 1 || N < 1 || K < 1) return fail(MI355_ERR_BAD_ARGUMENT, "mi355_hgemm: M, N, K must be >= 1 (got %d, %d, %d)", M, N, K);
+    if (!A || !B || !C) return fail(MI355_ERR_BAD_ARGUMENT, "%s: null pointer", fn);
+    if (M < 1 || N < 1 || K < 1) return fail(MI355_ERR_BAD_ARGUMENT, "%s: M, N, K must be >= 1 (got %d, %d, %d)", fn, M, N, K);
     if (layout != MI355_GEMM_NN && layout != MI355_GEMM_NT && layout != MI355_GEMM_TN)
-        return fail(MI355_ERR_BAD_ARGUMENT, "mi355_hgemm: unknown layout %d", layout);
+        return fail(MI355_ERR_BAD_ARGUMENT, "%s: unknown layout %d", fn, layout);
     const int64_t a_min = (layout == MI355_GEMM_TN) ? M : K;
     const int64_t b_min = (layout == MI355_GEMM_NT) ? K : N;
     if (lda < a_min || ldb < b_min || ldc < N)
-        return fail(MI355_ERR_BAD_ARGUMENT, "mi355_hgemm: leading dimension too small (lda %lld >= %lld, ldb %lld >= %lld, ldc %lld >= %d required)",
+        return fail(MI355_ERR_BAD_ARGUMENT, "%s: leading dimension too small (lda %lld >= %lld, ldb %lld >= %lld, ldc %lld >= %d required)", fn,
                     (long long)lda, (long long)a_min, (long long)ldb, (long long)b_min, (long long)ldc, N);
-    hipError_t e = mi355::hgemm_dispatch(A, B, C, M, N, K, lda, ldb, ldc, layout, static_cast<hipStream_t>(stream));
-    if (e != hipSuccess) return hip_fail(e, "mi355_hgemm launch");
+    hipError_t e = mi355::hgemm_dispatch(A, B, C, M, N, K, lda, ldb, ldc, layout, dtype, static_cast<hipStream_t>(stream));
+    if (e != hipSuccess) return hip_fail(e, fn);
     return 0;
 }
+
+int mi355_hgemm(const void* A, const void* B, void* C, int M, int N, int K, int64_t lda, int64_t ldb, int64_t ldc,
+                int layout, void* stream) {
+    return hgemm_impl("mi355_hgemm", MI355_DTYPE_FP16, A, B, C, M, N, K, lda, ldb, ldc, layout, stream);
+}
+
+int mi355_gemm_bf16(const void* A, const void* B, void* C, int M, int N, int K, int64_t lda, int64_t ldb, int64_t ldc,
+                int layout, void* stream) {
+    return hgemm_impl("mi355_gemm_bf16", MI355_DTYPE_BF16, A, B, C, M, N, K, lda, ldb, ldc, layout, stream);
+}
+
 
 static int fmha_checked(const char* fn, const void* Q, const void* K, const void* V, void* O, float* LSE, int B, int Hq, int Hkv,
                         int Sq, int Sk, int D, float scale, int causal, int kv_valid_len, const mi355::FmhaStrides& sd,
@@ -68,24 +79,35 @@ static int fmha_checked(const char* fn, const void* Q, const void* K, const void
     return 0;
 }
 
-int mi355_hgemm_silu_mul(const void* A, const void* B, void* C, int M, int N, int K, int64_t lda, int64_t ldb, int64_t ldc,
+static int hgemm_silu_mul_impl(const char* fn, int dtype, const void* A, const void* B, void* C, int M, int N, int K, int64_t lda, int64_t ldb, int64_t ldc,
                          int layout, void* stream) {
-    if (!A || !B || !C) return fail(MI355_ERR_BAD_ARGUMENT, "mi355_hgemm_silu_mul: null pointer");
-    if (M < 1 || N < 1 || K < 1) return fail(MI355_ERR_BAD_ARGUMENT, "mi355_hgemm_silu_mul: M, N, K must be >= 1");
+    if (!A || !B || !C) return fail(MI355_ERR_BAD_ARGUMENT, "%s: null pointer", fn);
+    if (M < 1 || N < 1 || K < 1) return fail(MI355_ERR_BAD_ARGUMENT, "%s: M, N, K must be >= 1", fn);
     if (layout != MI355_GEMM_NN && layout != MI355_GEMM_NT)
-        return fail(MI355_ERR_UNSUPPORTED, "mi355_hgemm_silu_mul: layout %d has no fused epilogue (NN and NT do)", layout);
+        return fail(MI355_ERR_UNSUPPORTED, "%s: layout %d has no fused epilogue (NN and NT do)", fn, layout);
     const int64_t b_min = (layout == MI355_GEMM_NT) ? K : 2 * (int64_t)N;
     if (lda < K || ldb < b_min || ldc < N)
-        return fail(MI355_ERR_BAD_ARGUMENT, "mi355_hgemm_silu_mul: leading dimension too small");
-    if (N > 0x3fffffff) return fail(MI355_ERR_BAD_ARGUMENT, "mi355_hgemm_silu_mul: N too large");
-    hipError_t e = mi355::hgemm_silu_mul_dispatch(A, B, C, M, 2 * N, K, lda, ldb, ldc, layout, static_cast<hipStream_t>(stream));
+        return fail(MI355_ERR_BAD_ARGUMENT, "%s: leading dimension too small", fn);
+    if (N > 0x3fffffff) return fail(MI355_ERR_BAD_ARGUMENT, "%s: N too large", fn);
+    hipError_t e = mi355::hgemm_silu_mul_dispatch(A, B, C, M, 2 * N, K, lda, ldb, ldc, layout, dtype, static_cast<hipStream_t>(stream));
     if (e == hipErrorNotSupported)
         return fail(MI355_ERR_UNSUPPORTED,
-                    "mi355_hgemm_silu_mul: needs M > 64, N a multiple of 32, K a multiple of 64 and 16-byte aligned operands; "
-                    "run mi355_hgemm and mi355_silu_mul(interleave = 32) instead");
-    if (e != hipSuccess) return hip_fail(e, "mi355_hgemm_silu_mul launch");
+                    "%s: needs M > 64, N a multiple of 32, K a multiple of 64 and 16-byte aligned operands; "
+                    "run mi355_hgemm and mi355_silu_mul(interleave = 32) instead", fn);
+    if (e != hipSuccess) return hip_fail(e, fn);
     return 0;
 }
+
+int mi355_hgemm_silu_mul(const void* A, const void* B, void* C, int M, int N, int K, int64_t lda, int64_t ldb, int64_t ldc,
+                         int layout, void* stream) {
+    return hgemm_silu_mul_impl("mi355_hgemm_silu_mul", MI355_DTYPE_FP16, A, B, C, M, N, K, lda, ldb, ldc, layout, stream);
+}
+
+int mi355_gemm_silu_mul_bf16(const void* A, const void* B, void* C, int M, int N, int K, int64_t lda, int64_t ldb, int64_t ldc,
+                         int layout, void* stream) {
+    return hgemm_silu_mul_impl("mi355_gemm_silu_mul_bf16", MI355_DTYPE_BF16, A, B, C, M, N, K, lda, ldb, ldc, layout, stream);
+}
+
 
 int mi355_fmha_fwd(const void* Q, const void* K, const void* V, void* O, float* LSE, int B, int Hq, int Hkv, int Sq,
                    int Sk, int D, float scale, int causal, int kv_valid_len, void* stream) {
@@ -119,59 +141,94 @@ int mi355_fmha_fwd_bf16(const void* Q, const void* K, const void* V, void* O, fl
 
 static bool aligned16(const void* p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; }
 
-int mi355_rmsnorm(const void* x, const void* residual, void* residual_out, const void* weight, void* out, int64_t rows,
+static int rmsnorm_impl(const char* fn, int dtype, const void* x, const void* residual, void* residual_out, const void* weight, void* out, int64_t rows,
                   int hidden, int64_t ldx, int64_t ldr, int64_t ldro, int64_t ldo, float eps, void* stream) {
-    if (!x || !weight || !out) return fail(MI355_ERR_BAD_ARGUMENT, "mi355_rmsnorm: null pointer");
+    if (!x || !weight || !out) return fail(MI355_ERR_BAD_ARGUMENT, "%s: null pointer", fn);
     if ((residual == nullptr) != (residual_out == nullptr))
-        return fail(MI355_ERR_BAD_ARGUMENT, "mi355_rmsnorm: residual and residual_out must both be given or both be NULL");
+        return fail(MI355_ERR_BAD_ARGUMENT, "%s: residual and residual_out must both be given or both be NULL", fn);
     if (rows < 1 || hidden < 8 || hidden % 8 != 0)
-        return fail(MI355_ERR_BAD_ARGUMENT, "mi355_rmsnorm: rows >= 1 and hidden a positive multiple of 8 required (got %lld, %d)",
+        return fail(MI355_ERR_BAD_ARGUMENT, "%s: rows >= 1 and hidden a positive multiple of 8 required (got %lld, %d)", fn,
                     (long long)rows, hidden);
     if (ldx < hidden || ldo < hidden || ldx % 8 || ldo % 8 ||
         (residual && (ldr < hidden || ldro < hidden || ldr % 8 || ldro % 8)))
-        return fail(MI355_ERR_BAD_ARGUMENT, "mi355_rmsnorm: row strides must be multiples of 8 and >= hidden");
+        return fail(MI355_ERR_BAD_ARGUMENT, "%s: row strides must be multiples of 8 and >= hidden", fn);
     if (!aligned16(x) || !aligned16(weight) || !aligned16(out) || !aligned16(residual) || !aligned16(residual_out))
-        return fail(MI355_ERR_BAD_ARGUMENT, "mi355_rmsnorm: pointers must be 16-byte aligned");
-    if (!(eps >= 0.f) || eps > 1.f) return fail(MI355_ERR_BAD_ARGUMENT, "mi355_rmsnorm: eps outside [0, 1] (got %g)", (double)eps);
-    hipError_t e = mi355::rmsnorm_dispatch(x, residual, residual_out, weight, out, rows, hidden, ldx, ldr, ldro, ldo, eps,
+        return fail(MI355_ERR_BAD_ARGUMENT, "%s: pointers must be 16-byte aligned", fn);
+    if (!(eps >= 0.f) || eps > 1.f) return fail(MI355_ERR_BAD_ARGUMENT, "%s: eps outside [0, 1] (got %g)", fn, (double)eps);
+    hipError_t e = mi355::rmsnorm_dispatch(x, residual, residual_out, weight, out, rows, hidden, ldx, ldr, ldro, ldo, eps, dtype,
                                            static_cast<hipStream_t>(stream));
-    if (e != hipSuccess) return hip_fail(e, "mi355_rmsnorm launch");
+    if (e != hipSuccess) return hip_fail(e, fn);
+    return 0;
+}
+
+int mi355_rmsnorm(const void* x, const void* residual, void* residual_out, const void* weight, void* out, int64_t rows,
+                  int hidden, int64_t ldx, int64_t ldr, int64_t ldro, int64_t ldo, float eps, void* stream) {
+    return rmsnorm_impl("mi355_rmsnorm", MI355_DTYPE_FP16, x, residual, residual_out, weight, out, rows, hidden, ldx, ldr, ldro, ldo, eps, stream);
+}
+
+int mi355_rmsnorm_bf16(const void* x, const void* residual, void* residual_out, const void* weight, void* out, int64_t rows,
+                  int hidden, int64_t ldx, int64_t ldr, int64_t ldro, int64_t ldo, float eps, void* stream) {
+    return rmsnorm_impl("mi355_rmsnorm_bf16", MI355_DTYPE_BF16, x, residual, residual_out, weight, out, rows, hidden, ldx, ldr, ldro, ldo, eps, stream);
+}
+
+
+static int rope_impl(const char* fn, int dtype, const void* x, void* out, int B, int S, int heads, int copy_heads, int D, int64_t x_batch, int64_t x_row,
+               int64_t out_batch, int64_t out_row, const float* cos_table, const float* sin_table, const int32_t* positions,
+               int64_t pos_batch, int n_positions, void* stream) {
+    if (!x || !out || !cos_table || !sin_table || !positions) return fail(MI355_ERR_BAD_ARGUMENT, "%s: null pointer", fn);
+    if (D != 128) return fail(MI355_ERR_UNSUPPORTED, "%s: head_dim must be 128 (got %d)", fn, D);
+    if (B < 1 || S < 1 || heads < 0 || copy_heads < 0 || heads + copy_heads < 1 || n_positions < 1 || pos_batch < 0)
+        return fail(MI355_ERR_BAD_ARGUMENT, "%s: B, S, heads + copy_heads, n_positions must be >= 1, pos_batch >= 0", fn);
+    const int64_t width = (int64_t)(heads + copy_heads) * D;
+    if (x_row < width || out_row < width || x_row % 8 || out_row % 8 || x_batch % 8 || out_batch % 8 || x_batch < 0 || out_batch < 0)
+        return fail(MI355_ERR_BAD_ARGUMENT, "%s: strides must be multiples of 8, row strides >= (heads + copy_heads) * 128", fn);
+    if (!aligned16(x) || !aligned16(out) || !aligned16(cos_table) || !aligned16(sin_table))
+        return fail(MI355_ERR_BAD_ARGUMENT, "%s: pointers must be 16-byte aligned", fn);
+    hipError_t e = mi355::rope_dispatch(x, out, B, S, heads, copy_heads, x_batch, x_row, out_batch, out_row, cos_table, sin_table,
+                                        positions, pos_batch, n_positions, dtype, static_cast<hipStream_t>(stream));
+    if (e != hipSuccess) return hip_fail(e, fn);
     return 0;
 }
 
 int mi355_rope(const void* x, void* out, int B, int S, int heads, int copy_heads, int D, int64_t x_batch, int64_t x_row,
                int64_t out_batch, int64_t out_row, const float* cos_table, const float* sin_table, const int32_t* positions,
                int64_t pos_batch, int n_positions, void* stream) {
-    if (!x || !out || !cos_table || !sin_table || !positions) return fail(MI355_ERR_BAD_ARGUMENT, "mi355_rope: null pointer");
-    if (D != 128) return fail(MI355_ERR_UNSUPPORTED, "mi355_rope: head_dim must be 128 (got %d)", D);
-    if (B < 1 || S < 1 || heads < 0 || copy_heads < 0 || heads + copy_heads < 1 || n_positions < 1 || pos_batch < 0)
-        return fail(MI355_ERR_BAD_ARGUMENT, "mi355_rope: B, S, heads + copy_heads, n_positions must be >= 1, pos_batch >= 0");
-    const int64_t width = (int64_t)(heads + copy_heads) * D;
-    if (x_row < width || out_row < width || x_row % 8 || out_row % 8 || x_batch % 8 || out_batch % 8 || x_batch < 0 || out_batch < 0)
-        return fail(MI355_ERR_BAD_ARGUMENT, "mi355_rope: strides must be multiples of 8, row strides >= (heads + copy_heads) * 128");
-    if (!aligned16(x) || !aligned16(out) || !aligned16(cos_table) || !aligned16(sin_table))
-        return fail(MI355_ERR_BAD_ARGUMENT, "mi355_rope: pointers must be 16-byte aligned");
-    hipError_t e = mi355::rope_dispatch(x, out, B, S, heads, copy_heads, x_batch, x_row, out_batch, out_row, cos_table, sin_table,
-                                        positions, pos_batch, n_positions, static_cast<hipStream_t>(stream));
-    if (e != hipSuccess) return hip_fail(e, "mi355_rope launch");
+    return rope_impl("mi355_rope", MI355_DTYPE_FP16, x, out, B, S, heads, copy_heads, D, x_batch, x_row, out_batch, out_row, cos_table, sin_table, positions, pos_batch, n_positions, stream);
+}
+
+int mi355_rope_bf16(const void* x, void* out, int B, int S, int heads, int copy_heads, int D, int64_t x_batch, int64_t x_row,
+               int64_t out_batch, int64_t out_row, const float* cos_table, const float* sin_table, const int32_t* positions,
+               int64_t pos_batch, int n_positions, void* stream) {
+    return rope_impl("mi355_rope_bf16", MI355_DTYPE_BF16, x, out, B, S, heads, copy_heads, D, x_batch, x_row, out_batch, out_row, cos_table, sin_table, positions, pos_batch, n_positions, stream);
+}
+
+
+static int silu_mul_impl(const char* fn, int dtype, const void* gate_up, void* out, int64_t rows, int inter, int interleave, int64_t ld_in, int64_t ld_out,
+                   void* stream) {
+    if (!gate_up || !out) return fail(MI355_ERR_BAD_ARGUMENT, "%s: null pointer", fn);
+    if (rows < 1 || inter < 8 || inter % 8 != 0)
+        return fail(MI355_ERR_BAD_ARGUMENT, "%s: rows >= 1 and inter a positive multiple of 8 required", fn);
+    if (interleave < 0 || interleave % 8 != 0 || (interleave > 0 && inter % interleave != 0))
+        return fail(MI355_ERR_BAD_ARGUMENT, "%s: interleave must be 0 or a multiple of 8 that divides inter (got %d)", fn,
+                    interleave);
+    if (ld_in < 2 * (int64_t)inter || ld_out < inter || ld_in % 8 || ld_out % 8)
+        return fail(MI355_ERR_BAD_ARGUMENT, "%s: ld_in >= 2 * inter, ld_out >= inter, both multiples of 8 required", fn);
+    if (!aligned16(gate_up) || !aligned16(out)) return fail(MI355_ERR_BAD_ARGUMENT, "%s: pointers must be 16-byte aligned", fn);
+    hipError_t e = mi355::silu_mul_dispatch(gate_up, out, rows, inter, interleave, ld_in, ld_out, dtype, static_cast<hipStream_t>(stream));
+    if (e != hipSuccess) return hip_fail(e, fn);
     return 0;
 }
 
 int mi355_silu_mul(const void* gate_up, void* out, int64_t rows, int inter, int interleave, int64_t ld_in, int64_t ld_out,
                    void* stream) {
-    if (!gate_up || !out) return fail(MI355_ERR_BAD_ARGUMENT, "mi355_silu_mul: null pointer");
-    if (rows < 1 || inter < 8 || inter % 8 != 0)
-        return fail(MI355_ERR_BAD_ARGUMENT, "mi355_silu_mul: rows >= 1 and inter a positive multiple of 8 required");
-    if (interleave < 0 || interleave % 8 != 0 || (interleave > 0 && inter % interleave != 0))
-        return fail(MI355_ERR_BAD_ARGUMENT, "mi355_silu_mul: interleave must be 0 or a multiple of 8 that divides inter (got %d)",
-                    interleave);
-    if (ld_in < 2 * (int64_t)inter || ld_out < inter || ld_in % 8 || ld_out % 8)
-        return fail(MI355_ERR_BAD_ARGUMENT, "mi355_silu_mul: ld_in >= 2 * inter, ld_out >= inter, both multiples of 8 required");
-    if (!aligned16(gate_up) || !aligned16(out)) return fail(MI355_ERR_BAD_ARGUMENT, "mi355_silu_mul: pointers must be 16-byte aligned");
-    hipError_t e = mi355::silu_mul_dispatch(gate_up, out, rows, inter, interleave, ld_in, ld_out, static_cast<hipStream_t>(stream));
-    if (e != hipSuccess) return hip_fail(e, "mi355_silu_mul launch");
-    return 0;
+    return silu_mul_impl("mi355_silu_mul", MI355_DTYPE_FP16, gate_up, out, rows, inter, interleave, ld_in, ld_out, stream);
 }
+
+int mi355_silu_mul_bf16(const void* gate_up, void* out, int64_t rows, int inter, int interleave, int64_t ld_in, int64_t ld_out,
+                   void* stream) {
+    return silu_mul_impl("mi355_silu_mul_bf16", MI355_DTYPE_BF16, gate_up, out, rows, inter, interleave, ld_in, ld_out, stream);
+}
+
 
 const char* mi355_last_error(void) { return g_err; }
 

@@ -159,10 +159,13 @@ __device__ __forceinline__ void tile_of_block(int bid, int tiles_m, int tiles_n,
 // RAGGED: M (and N) need not be multiples of the tile. Copies of rows past the end are redirected to the last row (or, for
 // an operand whose M/N index is contiguous, to the last 8 columns; that dimension must be a multiple of 8), so every
 // load stays inside the matrices, and the epilogue stores only what exists.
-template <bool A_KC, bool B_KC, int BM, int BN, int WM, int WN, int EPI = 0, bool RAGGED = false>
-__global__ __launch_bounds__(WM * WN * 64) void hgemm_main_kernel(const half_t* __restrict__ A, const half_t* __restrict__ B,
-                                                         half_t* __restrict__ C, int M, int N, int K, long lda,
+template <typename T, bool A_KC, bool B_KC, int BM, int BN, int WM, int WN, int EPI = 0, bool RAGGED = false>
+__global__ __launch_bounds__(WM * WN * 64) void hgemm_main_kernel(const T* __restrict__ A, const T* __restrict__ B,
+                                                         T* __restrict__ C, int M, int N, int K, long lda,
                                                          long ldb, long ldc) {
+    using V8 = typename Elem<T>::v8;
+    using V4 = typename Elem<T>::v4;
+    using V2 = typename Elem<T>::v2;
     using Cfg = MainCfg<A_KC, B_KC, BM, BN, WM, WN>;
     using ATK = typename Cfg::ATileK;
     using ATM = typename Cfg::ATileM;
@@ -185,7 +188,7 @@ __global__ __launch_bounds__(WM * WN * 64) void hgemm_main_kernel(const half_t* 
     const long n0 = (long)tile_n * Cfg::BN;
 
     // ---- global -> LDS copy descriptors --------------------------------------------------------------
-    const half_t* a_src;
+    const T* a_src;
     long a_copy_stride, a_k_stride;
     if constexpr (A_KC) {  // A stored [M,K]
         a_src = A + m0 * lda + ATK::first_copy_offset(wave, lane, lda);
@@ -196,7 +199,7 @@ __global__ __launch_bounds__(WM * WN * 64) void hgemm_main_kernel(const half_t* 
         a_copy_stride = ATM::copy_stride(lda);
         a_k_stride = ATM::ktile_stride(lda);
     }
-    const half_t* b_src;
+    const T* b_src;
     long b_copy_stride, b_k_stride;
     if constexpr (B_KC) {  // B stored [N,K]
         b_src = B + n0 * ldb + BTK::first_copy_offset(wave, lane, ldb);
@@ -209,10 +212,10 @@ __global__ __launch_bounds__(WM * WN * 64) void hgemm_main_kernel(const half_t* 
     }
 
     // RAGGED: one pointer per copy, rows / column chunks past the end folded back inside
-    const half_t* a_ptr[RAGGED ? Cfg::A_INSTS : 1];
-    const half_t* b_ptr[RAGGED ? Cfg::B_INSTS : 1];
+    const T* a_ptr[RAGGED ? Cfg::A_INSTS : 1];
+    const T* b_ptr[RAGGED ? Cfg::B_INSTS : 1];
     if constexpr (RAGGED) {
-        auto clamped = [&](const half_t* base, long ld, bool k_contig, int rows_per_inst, int chunks_per_row, int rows_per_pass,
+        auto clamped = [&](const T* base, long ld, bool k_contig, int rows_per_inst, int chunks_per_row, int rows_per_pass,
                            int i, long origin, long extent, int swz) {
             const int row = wave * rows_per_inst + lane / chunks_per_row + i * rows_per_pass;
             const int chunk = (lane % chunks_per_row) ^ swz;
@@ -294,34 +297,34 @@ __global__ __launch_bounds__(WM * WN * 64) void hgemm_main_kernel(const half_t* 
             for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 
     // fragment loads of one k-substep (16 deep) from stage `st`
-    auto load_frags = [&](MI355_LDS char* st, int kk, half8(&af)[TM], half8(&bf)[TN]) {
+    auto load_frags = [&](MI355_LDS char* st, int kk, V8(&af)[TM], V8(&bf)[TN]) {
 #pragma unroll
         for (int i = 0; i < TM; ++i) {
             if constexpr (A_KC) {
-                af[i] = lds_read_b128(st + a_off[kk] + i * 32 * ATK::kRowBytes);
+                af[i] = Elem<T>::frag(lds_read_b128(st + a_off[kk] + i * 32 * ATK::kRowBytes));
             } else {
                 half4 lo = lds_read_tr16_b64(st + a_off[i] + (kk * 16) * ATM::kRowBytes);
                 half4 hi = lds_read_tr16_b64(st + a_off[i] + (kk * 16 + 4) * ATM::kRowBytes);
-                af[i] = concat(lo, hi);
+                af[i] = Elem<T>::frag(concat(lo, hi));
             }
         }
 #pragma unroll
         for (int j = 0; j < TN; ++j) {
             if constexpr (B_KC) {
-                bf[j] = lds_read_b128(st + b_off[kk] + j * 32 * BTK::kRowBytes);
+                bf[j] = Elem<T>::frag(lds_read_b128(st + b_off[kk] + j * 32 * BTK::kRowBytes));
             } else {
                 half4 lo = lds_read_tr16_b64(st + b_off[j] + (kk * 16) * BTN::kRowBytes);
                 half4 hi = lds_read_tr16_b64(st + b_off[j] + (kk * 16 + 4) * BTN::kRowBytes);
-                bf[j] = concat(lo, hi);
+                bf[j] = Elem<T>::frag(concat(lo, hi));
             }
         }
     };
-    auto mma = [&](const half8(&af)[TM], const half8(&bf)[TN]) {
+    auto mma = [&](const V8(&af)[TM], const V8(&bf)[TN]) {
 #pragma unroll
         for (int i = 0; i < TM; ++i)
 #pragma unroll
             for (int j = 0; j < TN; ++j)
-                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bf[j], af[i], acc[i][j], 0, 0, 0);
+                acc[i][j] = Elem<T>::mfma32(bf[j], af[i], acc[i][j]);
     };
     // ask the scheduler to alternate the TM*TN MFMAs of one substep with the LDS reads of the next one
     constexpr int kDsReads = (A_KC ? TM : 2 * TM) + (B_KC ? TN : 2 * TN);
@@ -334,7 +337,7 @@ __global__ __launch_bounds__(WM * WN * 64) void hgemm_main_kernel(const half_t* 
     // the first fragments of the next tile are read under that substep's MFMAs and no wave starts a tile
     // with an exposed LDS round trip.
     const int ktiles = K / BK;
-    half8 af[2][TM], bf[2][TN];
+    V8 af[2][TM], bf[2][TN];
     issue_copies(0);
     wait_vmcnt<0>();
     __syncthreads();
@@ -399,19 +402,19 @@ __global__ __launch_bounds__(WM * WN * 64) void hgemm_main_kernel(const half_t* 
             for (int j = 0; j < TNO; ++j) {
 #pragma unroll
                 for (int p = 0; p < 4; ++p) {
-                    half4 v;
+                    V4 v;
 #pragma unroll
                     for (int q = 0; q < 4; ++q) {
                         if constexpr (EPI == 1) {
                             const float g = acc[i][2 * j][4 * p + q];
                             const float sig = __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(-g * 1.4426950408889634f));
-                            v[q] = (half_t)(g * sig * acc[i][2 * j + 1][4 * p + q]);
+                            v[q] = (T)(g * sig * acc[i][2 * j + 1][4 * p + q]);
                         } else {
-                            v[q] = (half_t)acc[i][j][4 * p + q];
+                            v[q] = (T)acc[i][j][4 * p + q];
                         }
                     }
                     const int chunk = (j * 4 + p) ^ (row & (kChunksC < 8 ? kChunksC - 1 : 7));
-                    *(MI355_LDS half4*)(cst + row * kRowBytesC + chunk * 16 + hh * 8) = v;
+                    *(MI355_LDS V4*)(cst + row * kRowBytesC + chunk * 16 + hh * 8) = v;
                 }
             }
         }
@@ -420,14 +423,14 @@ __global__ __launch_bounds__(WM * WN * 64) void hgemm_main_kernel(const half_t* 
     {
         const int rr = lane / kChunksC;
         const int cc = lane % kChunksC;
-        half_t* cbase = C + (m0 + wm * TM * 32) * ldc + (EPI == 1 ? n0 / 2 : n0) + wn * TNO * 32 + cc * 8;
+        T* cbase = C + (m0 + wm * TM * 32) * ldc + (EPI == 1 ? n0 / 2 : n0) + wn * TNO * 32 + cc * 8;
         const long rows_left = M - (m0 + wm * TM * 32);   // RAGGED: rows and 8-column chunks that exist
         const bool col_ok = (EPI == 1 ? n0 / 2 : n0) + wn * TNO * 32 + cc * 8 < (EPI == 1 ? N / 2 : N);
 #pragma unroll
         for (int it = 0; it < TM * 32 / kRowsPerStore; ++it) {
             const int row = it * kRowsPerStore + rr;
-            half8 v = *(MI355_LDS const half8*)(cst + row * kRowBytesC + ((cc ^ (row & (kChunksC < 8 ? kChunksC - 1 : 7))) << 4));
-            if (!RAGGED || (row < rows_left && col_ok)) *(half8*)(cbase + (long)row * ldc) = v;
+            V8 v = *(MI355_LDS const V8*)(cst + row * kRowBytesC + ((cc ^ (row & (kChunksC < 8 ? kChunksC - 1 : 7))) << 4));
+            if (!RAGGED || (row < rows_left && col_ok)) *(V8*)(cbase + (long)row * ldc) = v;
         }
     }
 }
@@ -436,10 +439,13 @@ __global__ __launch_bounds__(WM * WN * 64) void hgemm_main_kernel(const half_t* 
 // Bounds-checked kernel for any shape: 64x64 tile per wave-quad, operands gathered with guarded scalar loads
 // into the MFMA layout. Used for shapes the tiled kernels do not cover; correctness first.
 // ---------------------------------------------------------------------------------------------------------
-template <bool A_KC, bool B_KC>
-__global__ __launch_bounds__(256) void hgemm_edge_kernel(const half_t* __restrict__ A, const half_t* __restrict__ B,
-                                                         half_t* __restrict__ C, int M, int N, int K, long lda,
+template <typename T, bool A_KC, bool B_KC>
+__global__ __launch_bounds__(256) void hgemm_edge_kernel(const T* __restrict__ A, const T* __restrict__ B,
+                                                         T* __restrict__ C, int M, int N, int K, long lda,
                                                          long ldb, long ldc) {
+    using V8 = typename Elem<T>::v8;
+    using V4 = typename Elem<T>::v4;
+    using V2 = typename Elem<T>::v2;
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
     const long m = (long)blockIdx.y * 64 + (wave >> 1) * 32 + (lane & 31);
@@ -449,18 +455,18 @@ __global__ __launch_bounds__(256) void hgemm_edge_kernel(const half_t* __restric
 #pragma unroll
     for (int e = 0; e < 16; ++e) acc[e] = 0.f;
     for (int k0 = 0; k0 < K; k0 += 16) {
-        half8 a, b;
+        V8 a, b;
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
             int k = k0 + kh + j;
             bool kin = k < K;
-            half_t av = (half_t)0.f, bv = (half_t)0.f;
+            T av = (T)0.f, bv = (T)0.f;
             if (kin && m < M) av = A_KC ? A[m * lda + k] : A[(long)k * lda + m];
             if (kin && n < N) bv = B_KC ? B[n * ldb + k] : B[(long)k * ldb + n];
             a[j] = av;
             b[j] = bv;
         }
-        acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, acc, 0, 0, 0);
+        acc = Elem<T>::mfma32(a, b, acc);
     }
     // acc element 4p+q is C[row 8p + 4*(lane/32) + q][col lane%32] of this wave's 32x32 block
     const long rb = (long)blockIdx.y * 64 + (wave >> 1) * 32 + 4 * (lane >> 5);
@@ -469,7 +475,7 @@ __global__ __launch_bounds__(256) void hgemm_edge_kernel(const half_t* __restric
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
             long r = rb + 8 * p + q;
-            if (r < M && n < N) C[r * ldc + n] = (half_t)acc[4 * p + q];
+            if (r < M && n < N) C[r * ldc + n] = (T)acc[4 * p + q];
         }
 }
 
@@ -487,9 +493,13 @@ constexpr int kSmallMStageBytes = 5 * 1024;  // 4 KiB of B + 1 KiB of A
 constexpr int kSmallMWaveBytes = kSmallMStages * kSmallMStageBytes;
 constexpr int kSmallMLdsBytes = 8 * kSmallMWaveBytes;
 
-__global__ __launch_bounds__(512) void hgemm_smallm_nn_kernel(const half_t* __restrict__ A, const half_t* __restrict__ B,
-                                                              half_t* __restrict__ C, int M, int N, int K, long lda,
+template <typename T>
+__global__ __launch_bounds__(512) void hgemm_smallm_nn_kernel(const T* __restrict__ A, const T* __restrict__ B,
+                                                              T* __restrict__ C, int M, int N, int K, long lda,
                                                               long ldb, long ldc, int n_tiles) {
+    using V8 = typename Elem<T>::v8;
+    using V4 = typename Elem<T>::v4;
+    using V2 = typename Elem<T>::v2;
     extern __shared__ __attribute__((aligned(1024))) char smem_raw[];
     MI355_LDS char* smem = (MI355_LDS char*)smem_raw;
     const int tid = threadIdx.x;
@@ -515,11 +525,11 @@ __global__ __launch_bounds__(512) void hgemm_smallm_nn_kernel(const half_t* __re
     const int b_chunk = (lane & 7) ^ (2 * (b_row & 3));           // (8i + b_row) % 4 == b_row % 4
     const int n_chunk_max = N / 8 - 1;
     const int b_col = min(n0 / 8 + b_chunk, n_chunk_max) * 8;     // clamp: columns past N are never stored
-    const half_t* b_src = B + (long)(s_begin * 32 + b_row) * ldb + b_col;
+    const T* b_src = B + (long)(s_begin * 32 + b_row) * ldb + b_col;
     // A slab: 16 rows (m) x 64 bytes; row lane/4, chunk position lane%4, chunk c of row r at c ^ ((r>>1)&3)
     const int a_row = lane >> 2;
     const int a_chunk = (lane & 3) ^ ((a_row >> 1) & 3);
-    const half_t* a_src = A + (long)min(m0 + a_row, M - 1) * lda + (long)s_begin * 32 + a_chunk * 8;
+    const T* a_src = A + (long)min(m0 + a_row, M - 1) * lda + (long)s_begin * 32 + a_chunk * 8;
 
     auto issue_stage = [&](int slot) {
         MI355_LDS char* st = wbase + slot * kSmallMStageBytes;
@@ -567,12 +577,12 @@ __global__ __launch_bounds__(512) void hgemm_smallm_nn_kernel(const half_t* __re
         }
         MI355_LDS char* st = wbase + slot * kSmallMStageBytes;
         slot = (slot + 1 == kSmallMStages) ? 0 : slot + 1;
-        half8 af = lds_read_b128(st + a_off);
+        V8 af = Elem<T>::frag(lds_read_b128(st + a_off));
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             half4 lo = lds_read_tr16_b64(st + b_off[j]);
             half4 hi = lds_read_tr16_b64(st + b_off[j] + 4 * 128);
-            acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(af, concat(lo, hi), acc[j], 0, 0, 0);
+            acc[j] = Elem<T>::mfma16(af, Elem<T>::frag(concat(lo, hi)), acc[j]);
         }
         // the reads of this slot must be complete before a later copy refills it
         wait_lgkmcnt<0>();
@@ -597,20 +607,21 @@ __global__ __launch_bounds__(512) void hgemm_smallm_nn_kernel(const half_t* __re
     const int m = m0 + (o >> 6);
     const int n = n0 + (o & 63);
     if (m < M && n < N) {
-        half2v v;
-        v[0] = (half_t)s0;
-        v[1] = (half_t)s1;
-        *(half2v*)(C + (long)m * ldc + n) = v;
+        V2 v;
+        v[0] = (T)s0;
+        v[1] = (T)s1;
+        *(V2*)(C + (long)m * ldc + n) = v;
     }
 }
 
-static hipError_t launch_smallm_nn(const half_t* A, const half_t* B, half_t* C, int M, int N, int K, long lda, long ldb,
+template <typename T>
+static hipError_t launch_smallm_nn(const T* A, const T* B, T* C, int M, int N, int K, long lda, long ldb,
                                    long ldc, hipStream_t stream) {
     static DynamicLdsOnce lds_once;
-    if (hipError_t e = lds_once.ensure(reinterpret_cast<const void*>(hgemm_smallm_nn_kernel), kSmallMLdsBytes); e != hipSuccess) return e;
+    if (hipError_t e = lds_once.ensure(reinterpret_cast<const void*>(hgemm_smallm_nn_kernel<T>), kSmallMLdsBytes); e != hipSuccess) return e;
     const int n_tiles = (N + 63) / 64;
     dim3 grid(n_tiles, (M + 15) / 16);
-    hgemm_smallm_nn_kernel<<<grid, dim3(512), kSmallMLdsBytes, stream>>>(A, B, C, M, N, K, lda, ldb, ldc, n_tiles);
+    hgemm_smallm_nn_kernel<T><<<grid, dim3(512), kSmallMLdsBytes, stream>>>(A, B, C, M, N, K, lda, ldb, ldc, n_tiles);
     return hipGetLastError();
 }
 
@@ -626,9 +637,13 @@ constexpr int kSmallMNtStageBytes = 4 * 1024;  // 2 KiB of B + 2 KiB of A
 constexpr int kSmallMNtWaveBytes = kSmallMNtStages * kSmallMNtStageBytes;
 constexpr int kSmallMNtLdsBytes = 8 * kSmallMNtWaveBytes;
 
-__global__ __launch_bounds__(512) void hgemm_smallm_nt_kernel(const half_t* __restrict__ A, const half_t* __restrict__ B,
-                                                              half_t* __restrict__ C, int M, int N, int K, long lda,
+template <typename T>
+__global__ __launch_bounds__(512) void hgemm_smallm_nt_kernel(const T* __restrict__ A, const T* __restrict__ B,
+                                                              T* __restrict__ C, int M, int N, int K, long lda,
                                                               long ldb, long ldc, int n_tiles) {
+    using V8 = typename Elem<T>::v8;
+    using V4 = typename Elem<T>::v4;
+    using V2 = typename Elem<T>::v2;
     extern __shared__ __attribute__((aligned(1024))) char smem_raw[];
     MI355_LDS char* smem = (MI355_LDS char*)smem_raw;
     const int tid = threadIdx.x;
@@ -649,10 +664,10 @@ __global__ __launch_bounds__(512) void hgemm_smallm_nt_kernel(const half_t* __re
     // chunk c of row r is stored at position c ^ (r & 7)
     const int c_row = lane >> 3;  // + 8*i
     const int c_chunk = (lane & 7) ^ (c_row & 7);
-    const half_t* b_src0 = B + (long)min(n0 + c_row, N - 1) * ldb + (long)s_begin * 64 + c_chunk * 8;
-    const half_t* b_src1 = B + (long)min(n0 + c_row + 8, N - 1) * ldb + (long)s_begin * 64 + c_chunk * 8;
-    const half_t* a_src0 = A + (long)min(m0 + c_row, M - 1) * lda + (long)s_begin * 64 + c_chunk * 8;
-    const half_t* a_src1 = A + (long)min(m0 + c_row + 8, M - 1) * lda + (long)s_begin * 64 + c_chunk * 8;
+    const T* b_src0 = B + (long)min(n0 + c_row, N - 1) * ldb + (long)s_begin * 64 + c_chunk * 8;
+    const T* b_src1 = B + (long)min(n0 + c_row + 8, N - 1) * ldb + (long)s_begin * 64 + c_chunk * 8;
+    const T* a_src0 = A + (long)min(m0 + c_row, M - 1) * lda + (long)s_begin * 64 + c_chunk * 8;
+    const T* a_src1 = A + (long)min(m0 + c_row + 8, M - 1) * lda + (long)s_begin * 64 + c_chunk * 8;
 
     auto issue_stage = [&](int slot) {
         MI355_LDS char* st = wbase + slot * kSmallMNtStageBytes;
@@ -695,9 +710,9 @@ __global__ __launch_bounds__(512) void hgemm_smallm_nt_kernel(const half_t* __re
         slot = (slot + 1 == kSmallMNtStages) ? 0 : slot + 1;
 #pragma unroll
         for (int sub = 0; sub < 2; ++sub) {
-            half8 bf = lds_read_b128(st + f_off[sub]);
-            half8 af = lds_read_b128(st + 2048 + f_off[sub]);
-            acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(af, bf, acc, 0, 0, 0);
+            V8 bf = Elem<T>::frag(lds_read_b128(st + f_off[sub]));
+            V8 af = Elem<T>::frag(lds_read_b128(st + 2048 + f_off[sub]));
+            acc = Elem<T>::mfma16(af, bf, acc);
         }
         wait_lgkmcnt<0>();  // the reads of this slot are complete before a later copy refills it
     }
@@ -714,27 +729,28 @@ __global__ __launch_bounds__(512) void hgemm_smallm_nt_kernel(const half_t* __re
         for (int w = 0; w < 8; ++w) sum += red[w * 256 + tid];
         const int m = m0 + (tid >> 4);
         const int n = n0 + (tid & 15);
-        if (m < M && n < N) C[(long)m * ldc + n] = (half_t)sum;
+        if (m < M && n < N) C[(long)m * ldc + n] = (T)sum;
     }
 }
 
-static hipError_t launch_smallm_nt(const half_t* A, const half_t* B, half_t* C, int M, int N, int K, long lda, long ldb,
+template <typename T>
+static hipError_t launch_smallm_nt(const T* A, const T* B, T* C, int M, int N, int K, long lda, long ldb,
                                    long ldc, hipStream_t stream) {
     static DynamicLdsOnce lds_once;
-    if (hipError_t e = lds_once.ensure(reinterpret_cast<const void*>(hgemm_smallm_nt_kernel), kSmallMNtLdsBytes); e != hipSuccess) return e;
+    if (hipError_t e = lds_once.ensure(reinterpret_cast<const void*>(hgemm_smallm_nt_kernel<T>), kSmallMNtLdsBytes); e != hipSuccess) return e;
     const int n_tiles = (N + 15) / 16;
     dim3 grid(n_tiles, (M + 15) / 16);
-    hgemm_smallm_nt_kernel<<<grid, dim3(512), kSmallMNtLdsBytes, stream>>>(A, B, C, M, N, K, lda, ldb, ldc, n_tiles);
+    hgemm_smallm_nt_kernel<T><<<grid, dim3(512), kSmallMNtLdsBytes, stream>>>(A, B, C, M, N, K, lda, ldb, ldc, n_tiles);
     return hipGetLastError();
 }
 
 int g_gemm_variant = 0;  // tuning hook: 0 = heuristic, 1 = force 256x256 tiles, 2 = force 128x128 tiles
 
-template <bool A_KC, bool B_KC, int BM, int BN, int WM, int WN, int EPI = 0, bool RAGGED = false>
-static hipError_t launch_main(const half_t* A, const half_t* B, half_t* C, int M, int N, int K, long lda, long ldb,
+template <typename T, bool A_KC, bool B_KC, int BM, int BN, int WM, int WN, int EPI = 0, bool RAGGED = false>
+static hipError_t launch_main(const T* A, const T* B, T* C, int M, int N, int K, long lda, long ldb,
                               long ldc, hipStream_t stream) {
     using Cfg = MainCfg<A_KC, B_KC, BM, BN, WM, WN>;
-    auto kern = hgemm_main_kernel<A_KC, B_KC, BM, BN, WM, WN, EPI, RAGGED>;
+    auto kern = hgemm_main_kernel<T, A_KC, B_KC, BM, BN, WM, WN, EPI, RAGGED>;
     static DynamicLdsOnce lds_once;
     if (hipError_t e = lds_once.ensure(reinterpret_cast<const void*>(kern), Cfg::LDS_BYTES); e != hipSuccess) return e;
     const long nblocks = (long)((M + BM - 1) / BM) * ((N + BN - 1) / BN);
@@ -744,8 +760,8 @@ static hipError_t launch_main(const half_t* A, const half_t* B, half_t* C, int M
     return hipGetLastError();
 }
 
-template <bool A_KC, bool B_KC>
-static hipError_t launch_layout(const half_t* A, const half_t* B, half_t* C, int M, int N, int K, long lda, long ldb,
+template <typename T, bool A_KC, bool B_KC>
+static hipError_t launch_layout(const T* A, const T* B, T* C, int M, int N, int K, long lda, long ldb,
                                 long ldc, hipStream_t stream) {
     const bool aligned = (reinterpret_cast<uintptr_t>(A) % 16 == 0) && (reinterpret_cast<uintptr_t>(B) % 16 == 0) &&
                          (reinterpret_cast<uintptr_t>(C) % 16 == 0) && (lda % 8 == 0) && (ldb % 8 == 0) &&
@@ -755,10 +771,10 @@ static hipError_t launch_layout(const half_t* A, const half_t* B, half_t* C, int
     const bool fits128 = k_ok && M % 128 == 0 && N % 128 == 0;
     if constexpr (A_KC && !B_KC) {
         if (aligned && M <= 64 && K % 32 == 0 && K >= 32 && N % 8 == 0 && ldc % 2 == 0)
-            return launch_smallm_nn(A, B, C, M, N, K, lda, ldb, ldc, stream);
+            return launch_smallm_nn<T>(A, B, C, M, N, K, lda, ldb, ldc, stream);
     }
     if constexpr (A_KC && B_KC) {
-        if (aligned && M <= 64 && K % 64 == 0 && K >= 64) return launch_smallm_nt(A, B, C, M, N, K, lda, ldb, ldc, stream);
+        if (aligned && M <= 64 && K % 64 == 0 && K >= 64) return launch_smallm_nt<T>(A, B, C, M, N, K, lda, ldb, ldc, stream);
     }
     // 256x256 tiles when they fill the machine (>= ~3/4 of the 256 CUs), 128x128 tiles for smaller problems
     const long tiles256 = fits256 ? (long)(M / 256) * (N / 256) : 0;
@@ -768,26 +784,26 @@ static hipError_t launch_layout(const half_t* A, const half_t* B, half_t* C, int
     if (g_gemm_variant == 1 && fits256) choice = 1;
     if (g_gemm_variant == 2 && fits128) choice = 2;
     switch (choice) {
-        case 1: return launch_main<A_KC, B_KC, 256, 256, 2, 4>(A, B, C, M, N, K, lda, ldb, ldc, stream);
-        case 2: return launch_main<A_KC, B_KC, 128, 128, 2, 2>(A, B, C, M, N, K, lda, ldb, ldc, stream);
+        case 1: return launch_main<T, A_KC, B_KC, 256, 256, 2, 4>(A, B, C, M, N, K, lda, ldb, ldc, stream);
+        case 2: return launch_main<T, A_KC, B_KC, 128, 128, 2, 2>(A, B, C, M, N, K, lda, ldb, ldc, stream);
         default: break;
     }
     // ragged M / N on the same tiles: N (and M for layout TN) a multiple of 8, so 16-byte chunks never straddle the end
     if (k_ok && N % 8 == 0 && N >= 8 && (A_KC || (M % 8 == 0 && M >= 8))) {
         const long t256 = (long)((M + 255) / 256) * ((N + 255) / 256);
         if ((t256 >= 192 && g_gemm_variant != 2) || g_gemm_variant == 1)
-            return launch_main<A_KC, B_KC, 256, 256, 2, 4, 0, true>(A, B, C, M, N, K, lda, ldb, ldc, stream);
-        return launch_main<A_KC, B_KC, 128, 128, 2, 2, 0, true>(A, B, C, M, N, K, lda, ldb, ldc, stream);
+            return launch_main<T, A_KC, B_KC, 256, 256, 2, 4, 0, true>(A, B, C, M, N, K, lda, ldb, ldc, stream);
+        return launch_main<T, A_KC, B_KC, 128, 128, 2, 2, 0, true>(A, B, C, M, N, K, lda, ldb, ldc, stream);
     }
     dim3 grid((N + 63) / 64, (M + 63) / 64);
-    hgemm_edge_kernel<A_KC, B_KC><<<grid, dim3(256), 0, stream>>>(A, B, C, M, N, K, lda, ldb, ldc);
+    hgemm_edge_kernel<T, A_KC, B_KC><<<grid, dim3(256), 0, stream>>>(A, B, C, M, N, K, lda, ldb, ldc);
     return hipGetLastError();
 }
 
 // Product with the gate/up epilogue (EPI = 1): N counts the columns of op(B) (twice those of C). Only the tiled kernels
 // have it; other shapes report hipErrorNotSupported and the caller runs the product and mi355_silu_mul separately.
-template <bool A_KC, bool B_KC>
-static hipError_t launch_silu_mul(const half_t* A, const half_t* B, half_t* C, int M, int N, int K, long lda, long ldb,
+template <typename T, bool A_KC, bool B_KC>
+static hipError_t launch_silu_mul(const T* A, const T* B, T* C, int M, int N, int K, long lda, long ldb,
                                   long ldc, hipStream_t stream) {
     const bool aligned = (reinterpret_cast<uintptr_t>(A) % 16 == 0) && (reinterpret_cast<uintptr_t>(B) % 16 == 0) &&
                          (reinterpret_cast<uintptr_t>(C) % 16 == 0) && (lda % 8 == 0) && (ldb % 8 == 0) && (ldc % 8 == 0);
@@ -797,36 +813,50 @@ static hipError_t launch_silu_mul(const half_t* A, const half_t* B, half_t* C, i
     const bool fits256 = M % 256 == 0 && N % 256 == 0;
     const long t256 = (long)((M + 255) / 256) * ((N + 255) / 256);
     if (t256 >= 192) {
-        if (fits256) return launch_main<A_KC, B_KC, 256, 256, 2, 4, 1>(A, B, C, M, N, K, lda, ldb, ldc, stream);
-        return launch_main<A_KC, B_KC, 256, 256, 2, 4, 1, true>(A, B, C, M, N, K, lda, ldb, ldc, stream);
+        if (fits256) return launch_main<T, A_KC, B_KC, 256, 256, 2, 4, 1>(A, B, C, M, N, K, lda, ldb, ldc, stream);
+        return launch_main<T, A_KC, B_KC, 256, 256, 2, 4, 1, true>(A, B, C, M, N, K, lda, ldb, ldc, stream);
     }
-    if (fits128) return launch_main<A_KC, B_KC, 128, 128, 2, 2, 1>(A, B, C, M, N, K, lda, ldb, ldc, stream);
-    return launch_main<A_KC, B_KC, 128, 128, 2, 2, 1, true>(A, B, C, M, N, K, lda, ldb, ldc, stream);
+    if (fits128) return launch_main<T, A_KC, B_KC, 128, 128, 2, 2, 1>(A, B, C, M, N, K, lda, ldb, ldc, stream);
+    return launch_main<T, A_KC, B_KC, 128, 128, 2, 2, 1, true>(A, B, C, M, N, K, lda, ldb, ldc, stream);
 }
 
-hipError_t hgemm_silu_mul_dispatch(const void* A, const void* B, void* C, int M, int N2, int K, long lda, long ldb, long ldc,
-                                   int layout, hipStream_t stream) {
-    const half_t* a = static_cast<const half_t*>(A);
-    const half_t* b = static_cast<const half_t*>(B);
-    half_t* c = static_cast<half_t*>(C);
+template <typename T>
+static hipError_t silu_mul_dispatch_t(const void* A, const void* B, void* C, int M, int N2, int K, long lda, long ldb, long ldc,
+                                      int layout, hipStream_t stream) {
+    const T* a = static_cast<const T*>(A);
+    const T* b = static_cast<const T*>(B);
+    T* c = static_cast<T*>(C);
     switch (layout) {
-        case MI355_GEMM_NN: return launch_silu_mul<true, false>(a, b, c, M, N2, K, lda, ldb, ldc, stream);
-        case MI355_GEMM_NT: return launch_silu_mul<true, true>(a, b, c, M, N2, K, lda, ldb, ldc, stream);
+        case MI355_GEMM_NN: return launch_silu_mul<T, true, false>(a, b, c, M, N2, K, lda, ldb, ldc, stream);
+        case MI355_GEMM_NT: return launch_silu_mul<T, true, true>(a, b, c, M, N2, K, lda, ldb, ldc, stream);
         default: return hipErrorNotSupported;
     }
 }
 
-hipError_t hgemm_dispatch(const void* A, const void* B, void* C, int M, int N, int K, long lda, long ldb, long ldc,
-                          int layout, hipStream_t stream) {
-    const half_t* a = static_cast<const half_t*>(A);
-    const half_t* b = static_cast<const half_t*>(B);
-    half_t* c = static_cast<half_t*>(C);
+hipError_t hgemm_silu_mul_dispatch(const void* A, const void* B, void* C, int M, int N2, int K, long lda, long ldb, long ldc,
+                                   int layout, int dtype, hipStream_t stream) {
+    if (dtype == MI355_DTYPE_BF16) return silu_mul_dispatch_t<bf16_t>(A, B, C, M, N2, K, lda, ldb, ldc, layout, stream);
+    return silu_mul_dispatch_t<half_t>(A, B, C, M, N2, K, lda, ldb, ldc, layout, stream);
+}
+
+template <typename T>
+static hipError_t gemm_dispatch_t(const void* A, const void* B, void* C, int M, int N, int K, long lda, long ldb, long ldc,
+                                  int layout, hipStream_t stream) {
+    const T* a = static_cast<const T*>(A);
+    const T* b = static_cast<const T*>(B);
+    T* c = static_cast<T*>(C);
     switch (layout) {
-        case MI355_GEMM_NN: return launch_layout<true, false>(a, b, c, M, N, K, lda, ldb, ldc, stream);
-        case MI355_GEMM_NT: return launch_layout<true, true>(a, b, c, M, N, K, lda, ldb, ldc, stream);
-        case MI355_GEMM_TN: return launch_layout<false, false>(a, b, c, M, N, K, lda, ldb, ldc, stream);
+        case MI355_GEMM_NN: return launch_layout<T, true, false>(a, b, c, M, N, K, lda, ldb, ldc, stream);
+        case MI355_GEMM_NT: return launch_layout<T, true, true>(a, b, c, M, N, K, lda, ldb, ldc, stream);
+        case MI355_GEMM_TN: return launch_layout<T, false, false>(a, b, c, M, N, K, lda, ldb, ldc, stream);
         default: return hipErrorInvalidValue;
     }
+}
+
+hipError_t hgemm_dispatch(const void* A, const void* B, void* C, int M, int N, int K, long lda, long ldb, long ldc,
+                          int layout, int dtype, hipStream_t stream) {
+    if (dtype == MI355_DTYPE_BF16) return gemm_dispatch_t<bf16_t>(A, B, C, M, N, K, lda, ldb, ldc, layout, stream);
+    return gemm_dispatch_t<half_t>(A, B, C, M, N, K, lda, ldb, ldc, layout, stream);
 }
 
 }  // namespace mi355

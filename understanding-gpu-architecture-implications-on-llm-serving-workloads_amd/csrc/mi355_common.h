@@ -85,11 +85,12 @@ __device__ __forceinline__ half8 concat(half4 lo, half4 hi) {
     return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
 }
 
-// Element types of the attention kernels. LDS traffic is type-blind (16-bit lanes); only the MFMA opcode and the
+// Element types of the kernels. LDS traffic is type-blind (16-bit lanes); only the MFMA opcode and the
 // float conversions differ. The register layouts of the bf16 MFMAs are those of their fp16 twins.
 typedef __bf16 bf16_t;
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 
 template <typename T>
 struct Elem;
@@ -97,18 +98,26 @@ template <>
 struct Elem<half_t> {
     using v8 = half8;
     using v4 = half4;
+    using v2 = half2v;
     static __device__ __forceinline__ v8 frag(half8 raw) { return raw; }
     static __device__ __forceinline__ float16v mfma32(v8 a, v8 b, float16v c) {
         return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ float4v mfma16(v8 a, v8 b, float4v c) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
     }
 };
 template <>
 struct Elem<bf16_t> {
     using v8 = bf16x8;
     using v4 = bf16x4;
+    using v2 = bf16x2;
     static __device__ __forceinline__ v8 frag(half8 raw) { return __builtin_bit_cast(bf16x8, raw); }
     static __device__ __forceinline__ float16v mfma32(v8 a, v8 b, float16v c) {
         return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ float4v mfma16(v8 a, v8 b, float4v c) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
     }
 };
 

@@ -23,7 +23,7 @@ struct DynamicLdsOnce {
 
 // Launches the GEMM kernels; arguments as mi355_hgemm after validation.
 hipError_t hgemm_dispatch(const void* A, const void* B, void* C, int M, int N, int K, long lda, long ldb, long ldc,
-                          int layout, hipStream_t stream);
+                          int layout, int dtype, hipStream_t stream);
 
 // Element strides of the attention operands: tensor[b][h][s][d] lives at b*batch + h*head + s*row + d (d contiguous).
 struct FmhaStrides {
@@ -35,7 +35,7 @@ struct FmhaStrides {
 
 // The product fused with silu(gate) * up (see hgemm_main_kernel's EPI); hipErrorNotSupported for shapes without it.
 hipError_t hgemm_silu_mul_dispatch(const void* A, const void* B, void* C, int M, int N2, int K, long lda, long ldb, long ldc,
-                                   int layout, hipStream_t stream);
+                                   int layout, int dtype, hipStream_t stream);
 
 // Launches the attention forward kernels; arguments as mi355_fmha_fwd_strided after validation.
 hipError_t fmha_fwd_dispatch(const void* Q, const void* K, const void* V, void* O, float* LSE, int B, int Hq, int Hkv,
@@ -50,11 +50,11 @@ hipError_t fmha_decode_dispatch(const T* Q, const T* K, const T* V, T* O, float*
 
 // Layer glue (glue.hip); arguments as the mi355_rmsnorm / mi355_rope / mi355_silu_mul entry points after validation.
 hipError_t rmsnorm_dispatch(const void* x, const void* residual, void* res_out, const void* weight, void* out, long rows,
-                            int hidden, long ldx, long ldr, long ldro, long ldo, float eps, hipStream_t stream);
+                            int hidden, long ldx, long ldr, long ldro, long ldo, float eps, int dtype, hipStream_t stream);
 hipError_t rope_dispatch(const void* x, void* out, int B, int S, int heads, int copy_heads, long x_batch, long x_row,
                          long o_batch, long o_row, const float* cos_t, const float* sin_t, const int* positions, long pos_batch,
-                         int n_pos, hipStream_t stream);
-hipError_t silu_mul_dispatch(const void* in, void* out, long rows, int inter, int block, long ld_in, long ld_out,
+                         int n_pos, int dtype, hipStream_t stream);
+hipError_t silu_mul_dispatch(const void* in, void* out, long rows, int inter, int block, long ld_in, long ld_out, int dtype,
                              hipStream_t stream);
 
 }  // namespace mi355

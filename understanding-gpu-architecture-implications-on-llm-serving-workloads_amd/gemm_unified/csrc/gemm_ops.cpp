@@ -27,8 +27,9 @@ namespace {
 
 at::Tensor run_gemm(const at::Tensor& a, const at::Tensor& b, int layout, const char* name) {
     TORCH_CHECK(a.dim() == 2 && b.dim() == 2, name, ": a and b must be 2-D, got ", a.dim(), "-D and ", b.dim(), "-D");
-    TORCH_CHECK(a.scalar_type() == at::kHalf, name, ": a must be float16, got ", a.scalar_type());
-    TORCH_CHECK(b.scalar_type() == at::kHalf, name, ": b must be float16, got ", b.scalar_type());
+    const bool bf16 = a.scalar_type() == at::kBFloat16;
+    TORCH_CHECK(a.scalar_type() == at::kHalf || bf16, name, ": a must be float16 or bfloat16, got ", a.scalar_type());
+    TORCH_CHECK(b.scalar_type() == a.scalar_type(), name, ": b must have a's dtype ", a.scalar_type(), ", got ", b.scalar_type());
     int64_t M, N, K, Kb;
     if (layout == MI355_GEMM_TN) {
         K = a.size(0); M = a.size(1);
@@ -52,7 +53,8 @@ at::Tensor run_gemm(const at::Tensor& a, const at::Tensor& b, int layout, const 
     at::Tensor bc = b.contiguous();
     at::Tensor c = at::empty({M, N}, a.options());
     hipStream_t stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream();
-    int rc = mi355_hgemm(ac.data_ptr(), bc.data_ptr(), c.data_ptr(), (int)M, (int)N, (int)K, ac.stride(0), bc.stride(0), N,
+    auto entry = bf16 ? &mi355_gemm_bf16 : &mi355_hgemm;
+    int rc = entry(ac.data_ptr(), bc.data_ptr(), c.data_ptr(), (int)M, (int)N, (int)K, ac.stride(0), bc.stride(0), N,
                          layout, stream);
     TORCH_CHECK(rc == 0, name, ": ", mi355_last_error(), " (code ", rc, ")");
     return c;

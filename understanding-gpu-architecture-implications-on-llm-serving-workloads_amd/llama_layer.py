@@ -33,8 +33,8 @@ class FineKVCache:
     row) with the key heads of a token followed by its value heads, so one kernel launch files both. `k` and `v` are the
     [B, max_len, n_kv, 128] views the attention kernel reads in place."""
 
-    def __init__(self, batch, max_len, n_kv, head_dim=128, device="cuda"):
-        self.kv = torch.empty((batch, max_len, 2 * n_kv, head_dim), dtype=torch.float16, device=device)
+    def __init__(self, batch, max_len, n_kv, head_dim=128, device="cuda", dtype=torch.float16):
+        self.kv = torch.empty((batch, max_len, 2 * n_kv, head_dim), dtype=dtype, device=device)
         self.k = self.kv[:, :, :n_kv]
         self.v = self.kv[:, :, n_kv:]
         self.length = 0
@@ -45,12 +45,16 @@ class FineKVCache:
 
 
 class FineLlamaDecoderLayer:
-    """forward(hidden_states [B, S, H] fp16, position_ids [B, S]) -> [B, S, H]; causal attention over the cache (if
-    any) plus the new tokens. `weights`: dict of fp16 GPU tensors in nn.Linear layout: q, k, v, o, gate, up, down,
-    and the norm weights ln1, ln2."""
+    """forward(hidden_states [B, S, H], position_ids [B, S]) -> [B, S, H]; causal attention over the cache (if any)
+    plus the new tokens. `weights`: dict of GPU tensors in nn.Linear layout: q, k, v, o, gate, up, down, and the norm
+    weights ln1, ln2. `dtype` (float16 or bfloat16) is the type of the weights, activations and KV cache."""
 
-    def __init__(self, weights, n_q_heads, n_kv_heads, rms_eps=1e-5, rope_base=10000.0, max_positions=8192):
-        w = {k: v.detach().to(torch.float16).contiguous() for k, v in weights.items()}
+    def __init__(self, weights, n_q_heads, n_kv_heads, rms_eps=1e-5, rope_base=10000.0, max_positions=8192,
+                 dtype=torch.float16):
+        if dtype not in (torch.float16, torch.bfloat16):
+            raise ValueError("dtype must be float16 or bfloat16")
+        self.dtype = dtype
+        w = {k: v.detach().to(dtype).contiguous() for k, v in weights.items()}
         self.n_q, self.n_kv = int(n_q_heads), int(n_kv_heads)
         self.hidden = w["q"].shape[1]
         self.head_dim = w["q"].shape[0] // self.n_q
@@ -71,7 +75,7 @@ class FineLlamaDecoderLayer:
         self.attn_ms = {"prefill": [], "decode": []}  # filled when time_attention=True (modeling_llama.py:762-775)
 
     @classmethod
-    def from_hf(cls, hf_layer, config, max_positions=8192, device="cuda"):
+    def from_hf(cls, hf_layer, config, max_positions=8192, device="cuda", dtype=torch.float16):
         """Wrap the weights of a transformers LlamaDecoderLayer."""
         a, m = hf_layer.self_attn, hf_layer.mlp
         w = dict(q=a.q_proj.weight, k=a.k_proj.weight, v=a.v_proj.weight, o=a.o_proj.weight, gate=m.gate_proj.weight,
@@ -79,7 +83,7 @@ class FineLlamaDecoderLayer:
                  ln2=hf_layer.post_attention_layernorm.weight)
         w = {k: v.detach().to(device) for k, v in w.items()}
         base = getattr(config, "rope_theta", None) or (getattr(config, "rope_parameters", None) or {}).get("rope_theta", 10000.0)
-        return cls(w, config.num_attention_heads, config.num_key_value_heads, config.rms_norm_eps, base, max_positions)
+        return cls(w, config.num_attention_heads, config.num_key_value_heads, config.rms_norm_eps, base, max_positions, dtype)
 
     def forward(self, hidden_states, position_ids=None, kv_cache=None, time_attention=False):
         B, S, H = hidden_states.shape
@@ -109,7 +113,7 @@ class FineLlamaDecoderLayer:
             lib.rope(qkv[:, :, Hq:], self.cos, self.sin, pos, out=kv_cache.kv[:, past:past + S], copy_heads=Hkv)
             kv_cache.length = past + S
             k, v = kv_cache.k[:, :past + S], kv_cache.v[:, :past + S]
-        attn = torch.empty((B, S, Hq, D), dtype=torch.float16, device=x.device)
+        attn = torch.empty((B, S, Hq, D), dtype=self.dtype, device=x.device)
         # [B, S, heads, D] viewed as [B, heads, S, D]: the kernel reads and writes these layouts in place
         lib.fmha_fwd(q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2), causal=True, return_lse=False,
                      out=attn.transpose(1, 2))

@@ -15,6 +15,7 @@ LAYOUTS = {"NN": GEMM_NN, "NT": GEMM_NT, "TN": GEMM_TN}
 ERR_BAD_ARGUMENT, ERR_UNSUPPORTED = 10001, 10002
 
 EXPORTED_SYMBOLS = ("mi355_hgemm", "mi355_fmha_fwd", "mi355_fmha_fwd_strided", "mi355_fmha_fwd_bf16", "mi355_hgemm_silu_mul", "mi355_rmsnorm", "mi355_rope", "mi355_silu_mul",
+                    "mi355_gemm_bf16", "mi355_gemm_silu_mul_bf16", "mi355_rmsnorm_bf16", "mi355_rope_bf16", "mi355_silu_mul_bf16",
                     "mi355_last_error", "mi355_serving_version",
                     "mi355_debug_set_gemm_variant", "mi355_debug_set_fmha_variant")
 
@@ -55,6 +56,11 @@ def load():
     lib.mi355_hgemm_silu_mul.argtypes = lib.mi355_hgemm.argtypes
     lib.mi355_hgemm_silu_mul.restype = i32
     lib.mi355_silu_mul.restype = i32
+    for fp16_name, bf16_name in (("mi355_hgemm", "mi355_gemm_bf16"), ("mi355_hgemm_silu_mul", "mi355_gemm_silu_mul_bf16"),
+                                 ("mi355_rmsnorm", "mi355_rmsnorm_bf16"), ("mi355_rope", "mi355_rope_bf16"),
+                                 ("mi355_silu_mul", "mi355_silu_mul_bf16")):
+        getattr(lib, bf16_name).argtypes = getattr(lib, fp16_name).argtypes
+        getattr(lib, bf16_name).restype = i32
     lib.mi355_last_error.argtypes = []
     lib.mi355_last_error.restype = ctypes.c_char_p
     lib.mi355_serving_version.argtypes = []
@@ -100,7 +106,7 @@ def hgemm(a, b, layout="NN", out=None):
     """C = op(a) op(b) through the C ABI on torch's current stream. a, b: contiguous fp16 GPU tensors."""
     import torch
     lay = LAYOUTS[layout] if isinstance(layout, str) else int(layout)
-    assert a.dtype == torch.float16 and b.dtype == torch.float16 and a.is_cuda and b.is_cuda
+    assert a.dtype in (torch.float16, torch.bfloat16) and b.dtype == a.dtype and a.is_cuda and b.is_cuda
     assert a.is_contiguous() and b.is_contiguous()
     if lay == GEMM_TN:
         K, M = a.shape
@@ -113,9 +119,10 @@ def hgemm(a, b, layout="NN", out=None):
     if K != Kb:
         raise ValueError("inner dimensions differ: %d vs %d" % (K, Kb))
     if out is None:
-        out = torch.empty((M, N), dtype=torch.float16, device=a.device)
+        out = torch.empty((M, N), dtype=a.dtype, device=a.device)
     stream = torch.cuda.current_stream(a.device).cuda_stream
-    hgemm_raw(_ptr(a), _ptr(b), _ptr(out), M, N, K, a.stride(0), b.stride(0), out.stride(0), lay, stream)
+    entry = load().mi355_gemm_bf16 if a.dtype == torch.bfloat16 else load().mi355_hgemm
+    _check(entry(_ptr(a), _ptr(b), _ptr(out), M, N, K, a.stride(0), b.stride(0), out.stride(0), lay, stream))
     return out
 
 
@@ -174,13 +181,15 @@ def rmsnorm(x, weight, eps, residual=None, residual_out=None, out=None):
     """RMSNorm over the last dimension of a [rows, hidden] fp16 tensor (row stride free). With `residual`, normalises
     h = fp16(residual + x) and writes h to `residual_out` (default: a new tensor). Returns out or (out, h)."""
     import torch
-    assert x.dim() == 2 and x.stride(1) == 1 and x.dtype == torch.float16 and weight.is_contiguous()
+    assert x.dim() == 2 and x.stride(1) == 1 and x.dtype in (torch.float16, torch.bfloat16) and weight.is_contiguous()
+    assert weight.dtype == x.dtype
     rows, hidden = x.shape
     if out is None:
-        out = torch.empty((rows, hidden), dtype=torch.float16, device=x.device)
+        out = torch.empty((rows, hidden), dtype=x.dtype, device=x.device)
     if residual is not None and residual_out is None:
-        residual_out = torch.empty((rows, hidden), dtype=torch.float16, device=x.device)
-    _check(load().mi355_rmsnorm(_ptr(x), _ptr(residual), _ptr(residual_out), _ptr(weight), _ptr(out), rows, hidden,
+        residual_out = torch.empty((rows, hidden), dtype=x.dtype, device=x.device)
+    entry = load().mi355_rmsnorm_bf16 if x.dtype == torch.bfloat16 else load().mi355_rmsnorm
+    _check(entry(_ptr(x), _ptr(residual), _ptr(residual_out), _ptr(weight), _ptr(out), rows, hidden,
                                 x.stride(0), residual.stride(0) if residual is not None else 0,
                                 residual_out.stride(0) if residual_out is not None else 0, out.stride(0), float(eps),
                                 _stream_of(x)))
@@ -194,11 +203,13 @@ def rope(x, cos, sin, positions, out=None, copy_heads=0):
     import torch
     B, S, heads, D = x.shape
     out = x if out is None else out
-    assert x.dtype == torch.float16 and x.stride(3) == 1 and x.stride(2) == D and out.stride(3) == 1 and out.stride(2) == D
+    assert x.dtype in (torch.float16, torch.bfloat16) and out.dtype == x.dtype
+    assert x.stride(3) == 1 and x.stride(2) == D and out.stride(3) == 1 and out.stride(2) == D
     assert cos.dtype == torch.float32 and cos.is_contiguous() and sin.is_contiguous() and cos.shape == sin.shape
     assert positions.dtype == torch.int32 and positions.is_contiguous() and positions.numel() in (S, B * S)
     pos_batch = S if (positions.numel() == B * S and B > 1) else 0
-    _check(load().mi355_rope(_ptr(x), _ptr(out), B, S, heads - copy_heads, copy_heads, D, x.stride(0), x.stride(1),
+    entry = load().mi355_rope_bf16 if x.dtype == torch.bfloat16 else load().mi355_rope
+    _check(entry(_ptr(x), _ptr(out), B, S, heads - copy_heads, copy_heads, D, x.stride(0), x.stride(1),
                              out.stride(0), out.stride(1), _ptr(cos), _ptr(sin), _ptr(positions), pos_batch, cos.shape[0],
                              _stream_of(x)))
     return out
@@ -208,12 +219,13 @@ def silu_mul(gate_up, out=None, interleave=0):
     """silu(gate) * up for a [rows, 2F] fp16 tensor holding gate in its first F columns and up in the rest
     (interleave=0), or gate and up alternating in groups of `interleave` columns."""
     import torch
-    assert gate_up.dim() == 2 and gate_up.stride(1) == 1 and gate_up.dtype == torch.float16
+    assert gate_up.dim() == 2 and gate_up.stride(1) == 1 and gate_up.dtype in (torch.float16, torch.bfloat16)
     rows, two_f = gate_up.shape
     inter = two_f // 2
     if out is None:
-        out = torch.empty((rows, inter), dtype=torch.float16, device=gate_up.device)
-    _check(load().mi355_silu_mul(_ptr(gate_up), _ptr(out), rows, inter, int(interleave), gate_up.stride(0), out.stride(0),
+        out = torch.empty((rows, inter), dtype=gate_up.dtype, device=gate_up.device)
+    entry = load().mi355_silu_mul_bf16 if gate_up.dtype == torch.bfloat16 else load().mi355_silu_mul
+    _check(entry(_ptr(gate_up), _ptr(out), rows, inter, int(interleave), gate_up.stride(0), out.stride(0),
                                  _stream_of(gate_up)))
     return out
 
@@ -241,13 +253,15 @@ def hgemm_silu_mul(a, w, layout="NT", out=None):
     shape (mi355_hgemm_silu_mul), otherwise the product followed by silu_mul on the interleaved columns."""
     import torch
     lay = LAYOUTS[layout] if isinstance(layout, str) else int(layout)
-    assert lay in (GEMM_NN, GEMM_NT) and a.is_contiguous() and w.is_contiguous() and a.dtype == torch.float16
+    assert lay in (GEMM_NN, GEMM_NT) and a.is_contiguous() and w.is_contiguous()
+    assert a.dtype in (torch.float16, torch.bfloat16) and w.dtype == a.dtype
     M, K = a.shape
     N2 = w.shape[0] if lay == GEMM_NT else w.shape[1]
     N = N2 // 2
     if out is None:
-        out = torch.empty((M, N), dtype=torch.float16, device=a.device)
-    rc = load().mi355_hgemm_silu_mul(_ptr(a), _ptr(w), _ptr(out), M, N, K, a.stride(0), w.stride(0), out.stride(0), lay,
+        out = torch.empty((M, N), dtype=a.dtype, device=a.device)
+    entry = load().mi355_gemm_silu_mul_bf16 if a.dtype == torch.bfloat16 else load().mi355_hgemm_silu_mul
+    rc = entry(_ptr(a), _ptr(w), _ptr(out), M, N, K, a.stride(0), w.stride(0), out.stride(0), lay,
                                      _stream_of(a))
     if rc == ERR_UNSUPPORTED:
         return silu_mul(hgemm(a, w, layout), out=out, interleave=GATE_UP_BLOCK)
