@@ -308,6 +308,33 @@ def main():
                                                                            "pct_of_hbm_peak": 100 * by_s / ms_g / 1e6 / PEAK_HBM_GBS}
         del graph
         del layer, cache
+        torch.cuda.empty_cache()
+        # 32 such layers with their own weights and caches (a Llama-3-8B-sized decoder stack without embedding and LM head):
+        # cold weights for every GEMM, as in serving
+        n_layers = 32
+        layers = [llama3_8b_layer(torch, so, dev)[0] for _ in range(n_layers)]
+        caches = [FineKVCache(Bd, S5 + 64, 8, device=dev) for _ in range(n_layers)]
+        for cch in caches:
+            cch.kv.normal_(0, 1)
+        def stack_prefill():
+            hcur = xl
+            for lyr in layers:
+                hcur = lyr(hcur)
+            return hcur
+        def stack_step():
+            hcur = xd1
+            for lyr, cch in zip(layers, caches):
+                cch.length = S5
+                hcur = lyr(hcur, kv_cache=cch)
+            return hcur
+        ms_sp = time_launches(stack_prefill, 3, 1)
+        ms_ss = time_launches(stack_step, 10, 2)
+        other["L5_stack_of_32_layers"] = {
+            "prefill_s8192_ms": ms_sp, "prefill_tokens_per_s": S5 / ms_sp * 1e3, "prefill_tflops": n_layers * tot_fl / ms_sp / 1e9,
+            "generation_step_b8_past8192_ms": ms_ss, "generation_tokens_per_s": Bd / ms_ss * 1e3,
+            "generation_gbs": n_layers * by_s / ms_ss / 1e6,
+            "note": "32 decoder layers with distinct random weights and KV caches, no embedding / LM head / sampling"}
+        del layers, caches
 
     # ---- CPU baseline: the same step with torch fp32 on the host cores -------------------------------------------------
     cpu_baseline = None
