@@ -220,7 +220,13 @@ def main():
             "torch_matmul_hipblaslt_8192_nn": {"ms": ms_v, "tflops": gemm_flops / ms_v / 1e9},
             "torch_matmul_hipblaslt_8192_nt": {"ms": ms_vt, "tflops": gemm_flops / ms_vt / 1e9},
             "torch_sdpa_f4_causal_gqa": {"ms": ms_sd, "tflops": fmha_flops / ms_sd / 1e9}}
-        del cv, bt
+        for tag, (mv, nv, kv) in (("g1_1024", (1024, 1024, 1024)), ("g2a_4096", (4096, 4096, 4096)), ("g2c_16x14336x4096", (16, 14336, 4096))):
+            xv = so.randn_fp16((mv, kv), 1).to(dev)
+            wv = so.randn_fp16((kv, nv), 2, 0.02).to(dev)
+            ov = torch.empty((mv, nv), dtype=torch.float16, device=dev)
+            msv = time_launches(lambda: torch.matmul(xv, wv, out=ov), 20, 3)
+            other["vendor_libraries_same_box"]["torch_matmul_hipblaslt_" + tag] = {"ms": msv, "tflops": 2.0 * mv * nv * kv / msv / 1e9}
+        del cv, bt, xv, wv, ov
         # generation-step shapes (HBM bound): nn.Linear-layout weight GEMM and attention over a long KV cache
         xd = so.randn_fp16((16, 4096), 1).to(dev)
         wd_nt = so.randn_fp16((14336, 4096), 2, 0.02).to(dev)
