@@ -284,8 +284,8 @@ def main():
         ms_l = time_launches(lambda: layer(xl), 5, 2)
         other["L5_decoder_layer_prefill_s8192"] = {
             "ms": ms_l, "tflops": tot_fl / ms_l / 1e9,
-            "note": "whole FineLlamaDecoderLayer.forward (11 launches: norms, fused QKV GEMM, RoPE, attention on strided operands, "
-                    "O projection, gate/up GEMM with SiLU*up epilogue, down GEMM, residual adds), flops of the GEMMs and attention only"}
+            "note": "whole FineLlamaDecoderLayer.forward (8 launches: norms, fused QKV GEMM, RoPE, attention on strided operands, "
+                    "O projection + residual, gate/up GEMM with SiLU*up epilogue, down GEMM + residual), flops of the GEMMs and attention only"}
         Bd = 8
         cache = FineKVCache(Bd, S5 + 64, 8, device=dev)
         cache.k.normal_(0, 1)

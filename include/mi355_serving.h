@@ -73,6 +73,17 @@ int mi355_hgemm_silu_mul(const void* A, const void* B, void* C, int M, int N, in
                          int layout, void* stream);
 
 /*
+ * C[M,N] = R[M,N] + op(A) * op(B): the product of mi355_hgemm with a residual added in its epilogue, for the two
+ * projections of a decoder layer whose result is added to the residual stream (`hidden_states = residual + hidden_states`
+ * after o_proj and after down_proj, benchmarks/flashattn-cuda/modeling_llama.py:776,781; an elementwise kernel of its own
+ * in the reference). The product is rounded to fp16 first and the sum once more, so the result equals that of the two
+ * separate operations bit for bit. R may be C (in place; then ldr must equal ldc), otherwise R and C must not overlap;
+ * ldr >= N. Layouts, shapes and fast-path conditions as mi355_hgemm (R and ldr aligned like C and ldc).
+ */
+int mi355_hgemm_add(const void* A, const void* B, const void* R, void* C, int M, int N, int K, int64_t lda, int64_t ldb,
+                    int64_t ldr, int64_t ldc, int layout, void* stream);
+
+/*
  * Fused attention forward, O = softmax(scale * Q K^T + mask) V, online softmax with fp32 statistics.
  *
  * Replaces the device side of `torch::Tensor finefmha_N(Q, K, V, causal, is_decode, decode_length)`
@@ -164,6 +175,8 @@ int mi355_silu_mul(const void* gate_up, void* out, int64_t rows, int inter, int 
  */
 int mi355_gemm_bf16(const void* A, const void* B, void* C, int M, int N, int K, int64_t lda, int64_t ldb, int64_t ldc,
                     int layout, void* stream);
+int mi355_gemm_add_bf16(const void* A, const void* B, const void* R, void* C, int M, int N, int K, int64_t lda, int64_t ldb,
+                        int64_t ldr, int64_t ldc, int layout, void* stream);
 int mi355_gemm_silu_mul_bf16(const void* A, const void* B, void* C, int M, int N, int K, int64_t lda, int64_t ldb,
                              int64_t ldc, int layout, void* stream);
 int mi355_rmsnorm_bf16(const void* x, const void* residual, void* residual_out, const void* weight, void* out, int64_t rows,

@@ -32,6 +32,7 @@ def test_capi_rejects_bad_arguments_without_a_gpu(lib):
     assert cdll.mi355_hgemm(None, None, None, 4, 4, 4, 4, 4, 4, 0, None) == 10001
     assert b"null pointer" in cdll.mi355_last_error()
     p = ctypes.c_void_p(0x1000)
+    p2 = ctypes.c_void_p(0x100000)
     assert cdll.mi355_hgemm(p, p, p, 0, 4, 4, 4, 4, 4, 0, None) == 10001
     assert cdll.mi355_hgemm(p, p, p, 4, 4, 4, 4, 4, 4, 7, None) == 10001
     assert b"layout" in cdll.mi355_last_error()
@@ -65,6 +66,11 @@ def test_capi_rejects_bad_arguments_without_a_gpu(lib):
     assert cdll.mi355_hgemm_silu_mul(p, p, p, 256, 128, 64, 64, 64, 64, 1, None) == 10001           # ldc < N
     assert cdll.mi355_hgemm_silu_mul(p, p, p, 32, 128, 64, 64, 64, 128, 1, None) == 10002           # few rows: small-M product + silu_mul
     assert b"mi355_silu_mul" in cdll.mi355_last_error()
+    assert cdll.mi355_hgemm_add(p, p, None, p, 64, 64, 64, 64, 64, 64, 64, 0, None) == 10001            # residual missing
+    assert cdll.mi355_hgemm_add(p, p, p2, p, 64, 64, 64, 64, 64, 32, 64, 0, None) == 10001              # ldr < N
+    assert b"ldr" in cdll.mi355_last_error()
+    assert cdll.mi355_hgemm_add(p, p, p, p, 64, 64, 64, 64, 64, 128, 64, 0, None) == 10001              # in place with ldr != ldc
+    assert cdll.mi355_gemm_add_bf16(p, p, p2, p, 64, 64, 0, 64, 64, 64, 64, 0, None) == 10001           # K < 1
     with pytest.raises(lib.Mi355Error):
         lib.hgemm_raw(0, 0, 0, 4, 4, 4, 4, 4, 4, 0)
 

@@ -237,3 +237,44 @@ def test_bfloat16_gemm_exact_cases_and_torch_operator(lib, gpu):
     assert out.dtype == torch.bfloat16 and bf16_close(out, so.gemm_ref(a, b, "NT"), n)[0]
     with pytest.raises(RuntimeError, match="dtype"):
         gemm_unified.ops.fine_gemm(a.to(gpu), b.half().to(gpu), 0)
+
+
+# ---- residual added in the epilogue (mi355_hgemm_add) -----------------------------------------------------------
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("layout", ["NN", "NT", "TN"])
+@pytest.mark.parametrize("M,N,K", [(512, 512, 256),      # 128x128 tiles
+                                   (4096, 4096, 128),    # 256x256 tiles
+                                   (1000, 264, 128),     # ragged tiles
+                                   (16, 4096, 1024),     # small-M kernels (NN, NT)
+                                   (8, 72, 192),
+                                   (100, 70, 50)])       # bounds-checked kernel
+def test_residual_epilogue_equals_product_then_add(lib, gpu, dtype, layout, M, N, K):
+    """residual + proj(x) (modeling_llama.py:776,781): the fused form must give, bit for bit, what the product followed by
+    an elementwise add in the same type gives, for a separate output, for a residual with a row stride, and in place."""
+    a, b = operands(M, N, K, layout, seed=5)
+    a, b = a.to(gpu, dtype), b.to(gpu, dtype)
+    g = torch.Generator().manual_seed(6)
+    wide = (torch.randn(M, N + 8, generator=g) * 3).to(dtype).to(gpu)
+    r = wide[:, :N]                                      # row stride N + 8
+    want = lib.hgemm(a, b, layout) + r
+    got = lib.hgemm(a, b, layout, residual=r)
+    assert torch.equal(got, want)
+    rc = r.contiguous()
+    got2 = lib.hgemm(a, b, layout, out=rc, residual=rc)  # in place
+    assert got2.data_ptr() == rc.data_ptr() and torch.equal(rc, want)
+    if dtype == torch.float16:                           # and against the oracle, rounding as the unfused sequence
+        ref = so.gemm_ref(a.cpu(), b.cpu(), layout).to(dtype).float() + r.cpu().float()
+        ok, st = so.gemm_tolerance_ok(got.cpu(), ref, K)
+        assert ok, st
+
+
+def test_residual_epilogue_full_size_projection(lib, gpu):
+    """Llama-3-8B down projection at s = 8192 with the residual stream updated in place."""
+    M, N, K = 8192, 4096, 14336
+    g = torch.Generator(device=gpu).manual_seed(1)
+    a = torch.randn(M, K, generator=g, device=gpu, dtype=torch.float16)
+    w = (torch.randn(N, K, generator=g, device=gpu) * 0.02).half()
+    res = torch.randn(M, N, generator=g, device=gpu, dtype=torch.float16)
+    want = lib.hgemm(a, w, "NT") + res
+    lib.hgemm(a, w, "NT", out=res, residual=res)
+    assert torch.equal(res, want)

@@ -23,8 +23,9 @@ int hip_fail(hipError_t e, const char* what) {
 
 extern "C" {
 
-static int hgemm_impl(const char* fn, int dtype, const void* A, const void* B, void* C, int M, int N, int K, int64_t lda, int64_t ldb, int64_t ldc,
-                int layout, void* stream) {
+// R == nullptr: the plain product; otherwise the residual operand of the *_add entry points (checked by the caller)
+static int hgemm_impl(const char* fn, int dtype, const void* A, const void* B, void* C, const void* R, int M, int N, int K, int64_t lda,
+                      int64_t ldb, int64_t ldc, int64_t ldr, int layout, void* stream) {
     if (!A || !B || !C) return fail(MI355_ERR_BAD_ARGUMENT, "%s: null pointer", fn);
     if (M < 1 || N < 1 || K < 1) return fail(MI355_ERR_BAD_ARGUMENT, "%s: M, N, K must be >= 1 (got %d, %d, %d)", fn, M, N, K);
     if (layout != MI355_GEMM_NN && layout != MI355_GEMM_NT && layout != MI355_GEMM_TN)
@@ -34,19 +35,35 @@ static int hgemm_impl(const char* fn, int dtype, const void* A, const void* B, v
     if (lda < a_min || ldb < b_min || ldc < N)
         return fail(MI355_ERR_BAD_ARGUMENT, "%s: leading dimension too small (lda %lld >= %lld, ldb %lld >= %lld, ldc %lld >= %d required)", fn,
                     (long long)lda, (long long)a_min, (long long)ldb, (long long)b_min, (long long)ldc, N);
-    hipError_t e = mi355::hgemm_dispatch(A, B, C, M, N, K, lda, ldb, ldc, layout, dtype, static_cast<hipStream_t>(stream));
+    if (R != nullptr && ldr < N)
+        return fail(MI355_ERR_BAD_ARGUMENT, "%s: leading dimension too small (ldr %lld >= %d required)", fn, (long long)ldr, N);
+    if (R != nullptr && R == C && ldr != ldc)
+        return fail(MI355_ERR_BAD_ARGUMENT, "%s: R aliases C but ldr (%lld) differs from ldc (%lld)", fn, (long long)ldr, (long long)ldc);
+    hipError_t e = mi355::hgemm_dispatch(A, B, C, R, M, N, K, lda, ldb, ldc, R ? ldr : 0, layout, dtype, static_cast<hipStream_t>(stream));
     if (e != hipSuccess) return hip_fail(e, fn);
     return 0;
 }
 
 int mi355_hgemm(const void* A, const void* B, void* C, int M, int N, int K, int64_t lda, int64_t ldb, int64_t ldc,
                 int layout, void* stream) {
-    return hgemm_impl("mi355_hgemm", MI355_DTYPE_FP16, A, B, C, M, N, K, lda, ldb, ldc, layout, stream);
+    return hgemm_impl("mi355_hgemm", MI355_DTYPE_FP16, A, B, C, nullptr, M, N, K, lda, ldb, ldc, 0, layout, stream);
 }
 
 int mi355_gemm_bf16(const void* A, const void* B, void* C, int M, int N, int K, int64_t lda, int64_t ldb, int64_t ldc,
                 int layout, void* stream) {
-    return hgemm_impl("mi355_gemm_bf16", MI355_DTYPE_BF16, A, B, C, M, N, K, lda, ldb, ldc, layout, stream);
+    return hgemm_impl("mi355_gemm_bf16", MI355_DTYPE_BF16, A, B, C, nullptr, M, N, K, lda, ldb, ldc, 0, layout, stream);
+}
+
+int mi355_hgemm_add(const void* A, const void* B, const void* R, void* C, int M, int N, int K, int64_t lda, int64_t ldb, int64_t ldr,
+                    int64_t ldc, int layout, void* stream) {
+    if (!R) return fail(MI355_ERR_BAD_ARGUMENT, "mi355_hgemm_add: null pointer");
+    return hgemm_impl("mi355_hgemm_add", MI355_DTYPE_FP16, A, B, C, R, M, N, K, lda, ldb, ldc, ldr, layout, stream);
+}
+
+int mi355_gemm_add_bf16(const void* A, const void* B, const void* R, void* C, int M, int N, int K, int64_t lda, int64_t ldb, int64_t ldr,
+                        int64_t ldc, int layout, void* stream) {
+    if (!R) return fail(MI355_ERR_BAD_ARGUMENT, "mi355_gemm_add_bf16: null pointer");
+    return hgemm_impl("mi355_gemm_add_bf16", MI355_DTYPE_BF16, A, B, C, R, M, N, K, lda, ldb, ldc, ldr, layout, stream);
 }
 
 

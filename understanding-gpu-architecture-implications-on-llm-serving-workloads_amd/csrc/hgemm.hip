@@ -156,13 +156,15 @@ __device__ __forceinline__ void tile_of_block(int bid, int tiles_m, int tiles_n,
 // columns and their 32 up columns (`act_fn(gate_proj(x)) * up_proj(x)`, benchmarks/flashattn-cuda/modeling_llama.py:227,
 // with the two projections interleaved in one weight matrix): a wave then holds g and u of the same outputs in its two
 // column blocks, at the same accumulator positions, and C has N / 2 columns.
+// R (may be null, may be C itself): a residual of C's shape added to the rounded product, `residual + proj(x)` of
+// modeling_llama.py:776,781 with the rounding of the unfused sequence (product to T, then the sum to T).
 // RAGGED: M (and N) need not be multiples of the tile. Copies of rows past the end are redirected to the last row (or, for
 // an operand whose M/N index is contiguous, to the last 8 columns; that dimension must be a multiple of 8), so every
 // load stays inside the matrices, and the epilogue stores only what exists.
 template <typename T, bool A_KC, bool B_KC, int BM, int BN, int WM, int WN, int EPI = 0, bool RAGGED = false>
 __global__ __launch_bounds__(WM * WN * 64) void hgemm_main_kernel(const T* __restrict__ A, const T* __restrict__ B,
-                                                         T* __restrict__ C, int M, int N, int K, long lda,
-                                                         long ldb, long ldc) {
+                                                         T* C, const T* R, int M, int N, int K, long lda,
+                                                         long ldb, long ldc, long ldr) {
     using V8 = typename Elem<T>::v8;
     using V4 = typename Elem<T>::v4;
     using V2 = typename Elem<T>::v2;
@@ -426,11 +428,19 @@ __global__ __launch_bounds__(WM * WN * 64) void hgemm_main_kernel(const T* __res
         T* cbase = C + (m0 + wm * TM * 32) * ldc + (EPI == 1 ? n0 / 2 : n0) + wn * TNO * 32 + cc * 8;
         const long rows_left = M - (m0 + wm * TM * 32);   // RAGGED: rows and 8-column chunks that exist
         const bool col_ok = (EPI == 1 ? n0 / 2 : n0) + wn * TNO * 32 + cc * 8 < (EPI == 1 ? N / 2 : N);
+        const T* rbase = R + (m0 + wm * TM * 32) * ldr + (EPI == 1 ? n0 / 2 : n0) + wn * TNO * 32 + cc * 8;
 #pragma unroll
         for (int it = 0; it < TM * 32 / kRowsPerStore; ++it) {
             const int row = it * kRowsPerStore + rr;
             V8 v = *(MI355_LDS const V8*)(cst + row * kRowBytesC + ((cc ^ (row & (kChunksC < 8 ? kChunksC - 1 : 7))) << 4));
-            if (!RAGGED || (row < rows_left && col_ok)) *(V8*)(cbase + (long)row * ldc) = v;
+            if (!RAGGED || (row < rows_left && col_ok)) {
+                if (R != nullptr) {
+                    const V8 r = *(const V8*)(rbase + (long)row * ldr);
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) v[j] = (T)((float)v[j] + (float)r[j]);
+                }
+                *(V8*)(cbase + (long)row * ldc) = v;
+            }
         }
     }
 }
@@ -441,8 +451,8 @@ __global__ __launch_bounds__(WM * WN * 64) void hgemm_main_kernel(const T* __res
 // ---------------------------------------------------------------------------------------------------------
 template <typename T, bool A_KC, bool B_KC>
 __global__ __launch_bounds__(256) void hgemm_edge_kernel(const T* __restrict__ A, const T* __restrict__ B,
-                                                         T* __restrict__ C, int M, int N, int K, long lda,
-                                                         long ldb, long ldc) {
+                                                         T* C, const T* R, int M, int N, int K, long lda,
+                                                         long ldb, long ldc, long ldr) {
     using V8 = typename Elem<T>::v8;
     using V4 = typename Elem<T>::v4;
     using V2 = typename Elem<T>::v2;
@@ -475,7 +485,11 @@ __global__ __launch_bounds__(256) void hgemm_edge_kernel(const T* __restrict__ A
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
             long r = rb + 8 * p + q;
-            if (r < M && n < N) C[r * ldc + n] = (T)acc[4 * p + q];
+            if (r < M && n < N) {
+                T v = (T)acc[4 * p + q];
+                if (R != nullptr) v = (T)((float)v + (float)R[r * ldr + n]);
+                C[r * ldc + n] = v;
+            }
         }
 }
 
@@ -495,8 +509,8 @@ constexpr int kSmallMLdsBytes = 8 * kSmallMWaveBytes;
 
 template <typename T>
 __global__ __launch_bounds__(512) void hgemm_smallm_nn_kernel(const T* __restrict__ A, const T* __restrict__ B,
-                                                              T* __restrict__ C, int M, int N, int K, long lda,
-                                                              long ldb, long ldc, int n_tiles) {
+                                                              T* C, const T* R, int M, int N, int K, long lda,
+                                                              long ldb, long ldc, long ldr, int n_tiles) {
     using V8 = typename Elem<T>::v8;
     using V4 = typename Elem<T>::v4;
     using V2 = typename Elem<T>::v2;
@@ -610,18 +624,23 @@ __global__ __launch_bounds__(512) void hgemm_smallm_nn_kernel(const T* __restric
         V2 v;
         v[0] = (T)s0;
         v[1] = (T)s1;
+        if (R != nullptr) {
+            const V2 r = *(const V2*)(R + (long)m * ldr + n);
+            v[0] = (T)((float)v[0] + (float)r[0]);
+            v[1] = (T)((float)v[1] + (float)r[1]);
+        }
         *(V2*)(C + (long)m * ldc + n) = v;
     }
 }
 
 template <typename T>
-static hipError_t launch_smallm_nn(const T* A, const T* B, T* C, int M, int N, int K, long lda, long ldb,
-                                   long ldc, hipStream_t stream) {
+static hipError_t launch_smallm_nn(const T* A, const T* B, T* C, const T* R, int M, int N, int K, long lda, long ldb,
+                                   long ldc, long ldr, hipStream_t stream) {
     static DynamicLdsOnce lds_once;
     if (hipError_t e = lds_once.ensure(reinterpret_cast<const void*>(hgemm_smallm_nn_kernel<T>), kSmallMLdsBytes); e != hipSuccess) return e;
     const int n_tiles = (N + 63) / 64;
     dim3 grid(n_tiles, (M + 15) / 16);
-    hgemm_smallm_nn_kernel<T><<<grid, dim3(512), kSmallMLdsBytes, stream>>>(A, B, C, M, N, K, lda, ldb, ldc, n_tiles);
+    hgemm_smallm_nn_kernel<T><<<grid, dim3(512), kSmallMLdsBytes, stream>>>(A, B, C, R, M, N, K, lda, ldb, ldc, ldr, n_tiles);
     return hipGetLastError();
 }
 
@@ -639,8 +658,8 @@ constexpr int kSmallMNtLdsBytes = 8 * kSmallMNtWaveBytes;
 
 template <typename T>
 __global__ __launch_bounds__(512) void hgemm_smallm_nt_kernel(const T* __restrict__ A, const T* __restrict__ B,
-                                                              T* __restrict__ C, int M, int N, int K, long lda,
-                                                              long ldb, long ldc, int n_tiles) {
+                                                              T* C, const T* R, int M, int N, int K, long lda,
+                                                              long ldb, long ldc, long ldr, int n_tiles) {
     using V8 = typename Elem<T>::v8;
     using V4 = typename Elem<T>::v4;
     using V2 = typename Elem<T>::v2;
@@ -729,26 +748,30 @@ __global__ __launch_bounds__(512) void hgemm_smallm_nt_kernel(const T* __restric
         for (int w = 0; w < 8; ++w) sum += red[w * 256 + tid];
         const int m = m0 + (tid >> 4);
         const int n = n0 + (tid & 15);
-        if (m < M && n < N) C[(long)m * ldc + n] = (T)sum;
+        if (m < M && n < N) {
+            T v = (T)sum;
+            if (R != nullptr) v = (T)((float)v + (float)R[(long)m * ldr + n]);
+            C[(long)m * ldc + n] = v;
+        }
     }
 }
 
 template <typename T>
-static hipError_t launch_smallm_nt(const T* A, const T* B, T* C, int M, int N, int K, long lda, long ldb,
-                                   long ldc, hipStream_t stream) {
+static hipError_t launch_smallm_nt(const T* A, const T* B, T* C, const T* R, int M, int N, int K, long lda, long ldb,
+                                   long ldc, long ldr, hipStream_t stream) {
     static DynamicLdsOnce lds_once;
     if (hipError_t e = lds_once.ensure(reinterpret_cast<const void*>(hgemm_smallm_nt_kernel<T>), kSmallMNtLdsBytes); e != hipSuccess) return e;
     const int n_tiles = (N + 15) / 16;
     dim3 grid(n_tiles, (M + 15) / 16);
-    hgemm_smallm_nt_kernel<T><<<grid, dim3(512), kSmallMNtLdsBytes, stream>>>(A, B, C, M, N, K, lda, ldb, ldc, n_tiles);
+    hgemm_smallm_nt_kernel<T><<<grid, dim3(512), kSmallMNtLdsBytes, stream>>>(A, B, C, R, M, N, K, lda, ldb, ldc, ldr, n_tiles);
     return hipGetLastError();
 }
 
 int g_gemm_variant = 0;  // tuning hook: 0 = heuristic, 1 = force 256x256 tiles, 2 = force 128x128 tiles
 
 template <typename T, bool A_KC, bool B_KC, int BM, int BN, int WM, int WN, int EPI = 0, bool RAGGED = false>
-static hipError_t launch_main(const T* A, const T* B, T* C, int M, int N, int K, long lda, long ldb,
-                              long ldc, hipStream_t stream) {
+static hipError_t launch_main(const T* A, const T* B, T* C, const T* R, int M, int N, int K, long lda, long ldb,
+                              long ldc, long ldr, hipStream_t stream) {
     using Cfg = MainCfg<A_KC, B_KC, BM, BN, WM, WN>;
     auto kern = hgemm_main_kernel<T, A_KC, B_KC, BM, BN, WM, WN, EPI, RAGGED>;
     static DynamicLdsOnce lds_once;
@@ -756,25 +779,25 @@ static hipError_t launch_main(const T* A, const T* B, T* C, int M, int N, int K,
     const long nblocks = (long)((M + BM - 1) / BM) * ((N + BN - 1) / BN);
     if (nblocks > 0x7fffffffL) return hipErrorInvalidValue;
     int blocks = (int)nblocks;
-    kern<<<dim3(blocks), dim3(Cfg::NTHREADS), Cfg::LDS_BYTES, stream>>>(A, B, C, M, N, K, lda, ldb, ldc);
+    kern<<<dim3(blocks), dim3(Cfg::NTHREADS), Cfg::LDS_BYTES, stream>>>(A, B, C, R, M, N, K, lda, ldb, ldc, ldr);
     return hipGetLastError();
 }
 
 template <typename T, bool A_KC, bool B_KC>
-static hipError_t launch_layout(const T* A, const T* B, T* C, int M, int N, int K, long lda, long ldb,
-                                long ldc, hipStream_t stream) {
+static hipError_t launch_layout(const T* A, const T* B, T* C, const T* R, int M, int N, int K, long lda, long ldb,
+                                long ldc, long ldr, hipStream_t stream) {
     const bool aligned = (reinterpret_cast<uintptr_t>(A) % 16 == 0) && (reinterpret_cast<uintptr_t>(B) % 16 == 0) &&
                          (reinterpret_cast<uintptr_t>(C) % 16 == 0) && (lda % 8 == 0) && (ldb % 8 == 0) &&
-                         (ldc % 8 == 0);
+                         (ldc % 8 == 0) && (reinterpret_cast<uintptr_t>(R) % 16 == 0) && (ldr % 8 == 0);
     const bool k_ok = aligned && K % 64 == 0 && K >= 64;
     const bool fits256 = k_ok && M % 256 == 0 && N % 256 == 0;
     const bool fits128 = k_ok && M % 128 == 0 && N % 128 == 0;
     if constexpr (A_KC && !B_KC) {
         if (aligned && M <= 64 && K % 32 == 0 && K >= 32 && N % 8 == 0 && ldc % 2 == 0)
-            return launch_smallm_nn<T>(A, B, C, M, N, K, lda, ldb, ldc, stream);
+            return launch_smallm_nn<T>(A, B, C, R, M, N, K, lda, ldb, ldc, ldr, stream);
     }
     if constexpr (A_KC && B_KC) {
-        if (aligned && M <= 64 && K % 64 == 0 && K >= 64) return launch_smallm_nt<T>(A, B, C, M, N, K, lda, ldb, ldc, stream);
+        if (aligned && M <= 64 && K % 64 == 0 && K >= 64) return launch_smallm_nt<T>(A, B, C, R, M, N, K, lda, ldb, ldc, ldr, stream);
     }
     // 256x256 tiles when they fill the machine (>= ~3/4 of the 256 CUs), 128x128 tiles for smaller problems
     const long tiles256 = fits256 ? (long)(M / 256) * (N / 256) : 0;
@@ -784,19 +807,19 @@ static hipError_t launch_layout(const T* A, const T* B, T* C, int M, int N, int 
     if (g_gemm_variant == 1 && fits256) choice = 1;
     if (g_gemm_variant == 2 && fits128) choice = 2;
     switch (choice) {
-        case 1: return launch_main<T, A_KC, B_KC, 256, 256, 2, 4>(A, B, C, M, N, K, lda, ldb, ldc, stream);
-        case 2: return launch_main<T, A_KC, B_KC, 128, 128, 2, 2>(A, B, C, M, N, K, lda, ldb, ldc, stream);
+        case 1: return launch_main<T, A_KC, B_KC, 256, 256, 2, 4>(A, B, C, R, M, N, K, lda, ldb, ldc, ldr, stream);
+        case 2: return launch_main<T, A_KC, B_KC, 128, 128, 2, 2>(A, B, C, R, M, N, K, lda, ldb, ldc, ldr, stream);
         default: break;
     }
     // ragged M / N on the same tiles: N (and M for layout TN) a multiple of 8, so 16-byte chunks never straddle the end
     if (k_ok && N % 8 == 0 && N >= 8 && (A_KC || (M % 8 == 0 && M >= 8))) {
         const long t256 = (long)((M + 255) / 256) * ((N + 255) / 256);
         if ((t256 >= 192 && g_gemm_variant != 2) || g_gemm_variant == 1)
-            return launch_main<T, A_KC, B_KC, 256, 256, 2, 4, 0, true>(A, B, C, M, N, K, lda, ldb, ldc, stream);
-        return launch_main<T, A_KC, B_KC, 128, 128, 2, 2, 0, true>(A, B, C, M, N, K, lda, ldb, ldc, stream);
+            return launch_main<T, A_KC, B_KC, 256, 256, 2, 4, 0, true>(A, B, C, R, M, N, K, lda, ldb, ldc, ldr, stream);
+        return launch_main<T, A_KC, B_KC, 128, 128, 2, 2, 0, true>(A, B, C, R, M, N, K, lda, ldb, ldc, ldr, stream);
     }
     dim3 grid((N + 63) / 64, (M + 63) / 64);
-    hgemm_edge_kernel<T, A_KC, B_KC><<<grid, dim3(256), 0, stream>>>(A, B, C, M, N, K, lda, ldb, ldc);
+    hgemm_edge_kernel<T, A_KC, B_KC><<<grid, dim3(256), 0, stream>>>(A, B, C, R, M, N, K, lda, ldb, ldc, ldr);
     return hipGetLastError();
 }
 
@@ -813,11 +836,11 @@ static hipError_t launch_silu_mul(const T* A, const T* B, T* C, int M, int N, in
     const bool fits256 = M % 256 == 0 && N % 256 == 0;
     const long t256 = (long)((M + 255) / 256) * ((N + 255) / 256);
     if (t256 >= 192) {
-        if (fits256) return launch_main<T, A_KC, B_KC, 256, 256, 2, 4, 1>(A, B, C, M, N, K, lda, ldb, ldc, stream);
-        return launch_main<T, A_KC, B_KC, 256, 256, 2, 4, 1, true>(A, B, C, M, N, K, lda, ldb, ldc, stream);
+        if (fits256) return launch_main<T, A_KC, B_KC, 256, 256, 2, 4, 1>(A, B, C, nullptr, M, N, K, lda, ldb, ldc, 0, stream);
+        return launch_main<T, A_KC, B_KC, 256, 256, 2, 4, 1, true>(A, B, C, nullptr, M, N, K, lda, ldb, ldc, 0, stream);
     }
-    if (fits128) return launch_main<T, A_KC, B_KC, 128, 128, 2, 2, 1>(A, B, C, M, N, K, lda, ldb, ldc, stream);
-    return launch_main<T, A_KC, B_KC, 128, 128, 2, 2, 1, true>(A, B, C, M, N, K, lda, ldb, ldc, stream);
+    if (fits128) return launch_main<T, A_KC, B_KC, 128, 128, 2, 2, 1>(A, B, C, nullptr, M, N, K, lda, ldb, ldc, 0, stream);
+    return launch_main<T, A_KC, B_KC, 128, 128, 2, 2, 1, true>(A, B, C, nullptr, M, N, K, lda, ldb, ldc, 0, stream);
 }
 
 template <typename T>
@@ -840,23 +863,24 @@ hipError_t hgemm_silu_mul_dispatch(const void* A, const void* B, void* C, int M,
 }
 
 template <typename T>
-static hipError_t gemm_dispatch_t(const void* A, const void* B, void* C, int M, int N, int K, long lda, long ldb, long ldc,
-                                  int layout, hipStream_t stream) {
+static hipError_t gemm_dispatch_t(const void* A, const void* B, void* C, const void* R, int M, int N, int K, long lda,
+                                  long ldb, long ldc, long ldr, int layout, hipStream_t stream) {
     const T* a = static_cast<const T*>(A);
     const T* b = static_cast<const T*>(B);
     T* c = static_cast<T*>(C);
+    const T* r = static_cast<const T*>(R);
     switch (layout) {
-        case MI355_GEMM_NN: return launch_layout<T, true, false>(a, b, c, M, N, K, lda, ldb, ldc, stream);
-        case MI355_GEMM_NT: return launch_layout<T, true, true>(a, b, c, M, N, K, lda, ldb, ldc, stream);
-        case MI355_GEMM_TN: return launch_layout<T, false, false>(a, b, c, M, N, K, lda, ldb, ldc, stream);
+        case MI355_GEMM_NN: return launch_layout<T, true, false>(a, b, c, r, M, N, K, lda, ldb, ldc, ldr, stream);
+        case MI355_GEMM_NT: return launch_layout<T, true, true>(a, b, c, r, M, N, K, lda, ldb, ldc, ldr, stream);
+        case MI355_GEMM_TN: return launch_layout<T, false, false>(a, b, c, r, M, N, K, lda, ldb, ldc, ldr, stream);
         default: return hipErrorInvalidValue;
     }
 }
 
-hipError_t hgemm_dispatch(const void* A, const void* B, void* C, int M, int N, int K, long lda, long ldb, long ldc,
-                          int layout, int dtype, hipStream_t stream) {
-    if (dtype == MI355_DTYPE_BF16) return gemm_dispatch_t<bf16_t>(A, B, C, M, N, K, lda, ldb, ldc, layout, stream);
-    return gemm_dispatch_t<half_t>(A, B, C, M, N, K, lda, ldb, ldc, layout, stream);
+hipError_t hgemm_dispatch(const void* A, const void* B, void* C, const void* R, int M, int N, int K, long lda, long ldb,
+                          long ldc, long ldr, int layout, int dtype, hipStream_t stream) {
+    if (dtype == MI355_DTYPE_BF16) return gemm_dispatch_t<bf16_t>(A, B, C, R, M, N, K, lda, ldb, ldc, ldr, layout, stream);
+    return gemm_dispatch_t<half_t>(A, B, C, R, M, N, K, lda, ldb, ldc, ldr, layout, stream);
 }
 
 }  // namespace mi355

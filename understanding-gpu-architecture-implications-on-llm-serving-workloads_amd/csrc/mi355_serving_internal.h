@@ -21,9 +21,9 @@ struct DynamicLdsOnce {
     }
 };
 
-// Launches the GEMM kernels; arguments as mi355_hgemm after validation.
-hipError_t hgemm_dispatch(const void* A, const void* B, void* C, int M, int N, int K, long lda, long ldb, long ldc,
-                          int layout, int dtype, hipStream_t stream);
+// Launches the GEMM kernels; arguments as mi355_hgemm_add after validation (R == nullptr: no residual).
+hipError_t hgemm_dispatch(const void* A, const void* B, void* C, const void* R, int M, int N, int K, long lda, long ldb,
+                          long ldc, long ldr, int layout, int dtype, hipStream_t stream);
 
 // Element strides of the attention operands: tensor[b][h][s][d] lives at b*batch + h*head + s*row + d (d contiguous).
 struct FmhaStrides {

@@ -6,11 +6,13 @@ calls, transposes to [B, H, S, D], applies RoPE, expands K/V with repeat_kv (:67
 ``fmha_unified.ops.fine_fmha`` (:687-690), transposes back with a copy (:700) and projects; LlamaDecoderLayer.forward
 (:755-781) wraps it in RMSNorm, residual adds and the gate/up/down MLP (:227), all as separate PyTorch kernels.
 
-Here one layer is eleven launches (twelve for shapes off the tiled GEMM's grid) with no layout copies:
+Here one layer is nine launches with a KV cache (ten on a generation step, whose split attention ends in a merge
+kernel; one more where the gate/up epilogue does not apply and SiLU*up runs on its own) with no layout copies:
     rmsnorm -> QKV GEMM (one fused NT GEMM on the nn.Linear weights) -> RoPE in place on the q and k heads of the
     projection (k goes straight into the KV cache when there is one) -> attention reading q, k, v where they lie
-    (strided operands, GQA inside the kernel, output written as [B, S, Hq*D]) -> O projection -> residual add fused
-    into the second rmsnorm -> gate/up GEMM with SiLU(gate)*up applied in its epilogue -> down GEMM -> residual add.
+    (strided operands, GQA inside the kernel, output written as [B, S, Hq*D]) -> O projection with the residual
+    added in its epilogue -> rmsnorm -> gate/up GEMM with SiLU(gate)*up applied in its epilogue -> down GEMM with the
+    residual added in its epilogue.
 Weights keep the nn.Linear layout ([out_features, in_features]); nothing is transposed or repacked beyond
 concatenating q/k/v and interleaving gate/up along the output dimension once at construction.
 """
@@ -117,14 +119,13 @@ class FineLlamaDecoderLayer:
         # [B, S, heads, D] viewed as [B, heads, S, D]: the kernel reads and writes these layouts in place
         lib.fmha_fwd(q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2), causal=True, return_lse=False,
                      out=attn.transpose(1, 2))
-        proj = lib.hgemm(attn.view(B * S, Hq * D), self.w_o, "NT")
+        res = lib.hgemm(attn.view(B * S, Hq * D), self.w_o, "NT", residual=x)   # x + o_proj(attn)
         if time_attention:
             t1.record()
             torch.cuda.synchronize()
             self.attn_ms["decode" if (S == 1 and past > 0) else "prefill"].append(t0.elapsed_time(t1))
-        h2, res = lib.rmsnorm(proj, self.ln2, self.eps, residual=x)
+        h2 = lib.rmsnorm(res, self.ln2, self.eps)
         act = lib.hgemm_silu_mul(h2, self.w_gu, "NT") if self.gu_block else lib.silu_mul(lib.hgemm(h2, self.w_gu, "NT"))
-        down = lib.hgemm(act, self.w_d, "NT")
-        return res.add_(down).view(B, S, H)
+        return lib.hgemm(act, self.w_d, "NT", out=res, residual=res).view(B, S, H)   # res + down_proj(act), in place
 
     __call__ = forward

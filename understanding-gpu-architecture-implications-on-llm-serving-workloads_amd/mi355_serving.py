@@ -14,8 +14,8 @@ GEMM_NN, GEMM_NT, GEMM_TN = 0, 1, 2
 LAYOUTS = {"NN": GEMM_NN, "NT": GEMM_NT, "TN": GEMM_TN}
 ERR_BAD_ARGUMENT, ERR_UNSUPPORTED = 10001, 10002
 
-EXPORTED_SYMBOLS = ("mi355_hgemm", "mi355_fmha_fwd", "mi355_fmha_fwd_strided", "mi355_fmha_fwd_bf16", "mi355_hgemm_silu_mul", "mi355_rmsnorm", "mi355_rope", "mi355_silu_mul",
-                    "mi355_gemm_bf16", "mi355_gemm_silu_mul_bf16", "mi355_rmsnorm_bf16", "mi355_rope_bf16", "mi355_silu_mul_bf16",
+EXPORTED_SYMBOLS = ("mi355_hgemm", "mi355_fmha_fwd", "mi355_fmha_fwd_strided", "mi355_fmha_fwd_bf16", "mi355_hgemm_silu_mul", "mi355_hgemm_add", "mi355_rmsnorm", "mi355_rope", "mi355_silu_mul",
+                    "mi355_gemm_bf16", "mi355_gemm_silu_mul_bf16", "mi355_gemm_add_bf16", "mi355_rmsnorm_bf16", "mi355_rope_bf16", "mi355_silu_mul_bf16",
                     "mi355_last_error", "mi355_serving_version",
                     "mi355_debug_set_gemm_variant", "mi355_debug_set_fmha_variant")
 
@@ -55,8 +55,11 @@ def load():
     lib.mi355_silu_mul.argtypes = [vp, vp, i64, i32, i32, i64, i64, vp]
     lib.mi355_hgemm_silu_mul.argtypes = lib.mi355_hgemm.argtypes
     lib.mi355_hgemm_silu_mul.restype = i32
+    lib.mi355_hgemm_add.argtypes = [vp, vp, vp, vp, i32, i32, i32, i64, i64, i64, i64, i32, vp]
+    lib.mi355_hgemm_add.restype = i32
     lib.mi355_silu_mul.restype = i32
     for fp16_name, bf16_name in (("mi355_hgemm", "mi355_gemm_bf16"), ("mi355_hgemm_silu_mul", "mi355_gemm_silu_mul_bf16"),
+                                 ("mi355_hgemm_add", "mi355_gemm_add_bf16"),
                                  ("mi355_rmsnorm", "mi355_rmsnorm_bf16"), ("mi355_rope", "mi355_rope_bf16"),
                                  ("mi355_silu_mul", "mi355_silu_mul_bf16")):
         getattr(lib, bf16_name).argtypes = getattr(lib, fp16_name).argtypes
@@ -102,8 +105,10 @@ def fmha_fwd_raw(q_ptr, k_ptr, v_ptr, o_ptr, lse_ptr, B, Hq, Hkv, Sq, Sk, D, sca
                                  kv_valid_len, stream))
 
 
-def hgemm(a, b, layout="NN", out=None):
-    """C = op(a) op(b) through the C ABI on torch's current stream. a, b: contiguous fp16 GPU tensors."""
+def hgemm(a, b, layout="NN", out=None, residual=None):
+    """C = op(a) op(b) (+ residual) through the C ABI on torch's current stream. a, b: contiguous fp16 or bf16 GPU
+    tensors; `residual`: [M, N] rows with a contiguous last dimension, added in the GEMM's epilogue (mi355_hgemm_add);
+    it may be `out` itself."""
     import torch
     lay = LAYOUTS[layout] if isinstance(layout, str) else int(layout)
     assert a.dtype in (torch.float16, torch.bfloat16) and b.dtype == a.dtype and a.is_cuda and b.is_cuda
@@ -121,6 +126,13 @@ def hgemm(a, b, layout="NN", out=None):
     if out is None:
         out = torch.empty((M, N), dtype=a.dtype, device=a.device)
     stream = torch.cuda.current_stream(a.device).cuda_stream
+    if residual is not None:
+        if tuple(residual.shape) != (M, N) or residual.dtype != a.dtype or residual.stride(1) != 1:
+            raise ValueError("residual must be [%d, %d] %s with a contiguous last dimension" % (M, N, a.dtype))
+        entry = load().mi355_gemm_add_bf16 if a.dtype == torch.bfloat16 else load().mi355_hgemm_add
+        _check(entry(_ptr(a), _ptr(b), _ptr(residual), _ptr(out), M, N, K, a.stride(0), b.stride(0), residual.stride(0),
+                     out.stride(0), lay, stream))
+        return out
     entry = load().mi355_gemm_bf16 if a.dtype == torch.bfloat16 else load().mi355_hgemm
     _check(entry(_ptr(a), _ptr(b), _ptr(out), M, N, K, a.stride(0), b.stride(0), out.stride(0), lay, stream))
     return out
