@@ -9,6 +9,8 @@
 // Main kernel: one workgroup of 8 waves computes a 256x256 tile of C, K is walked in steps of 64.
 //   * global -> LDS staging uses 16-byte direct-to-LDS copies (no VGPR bounce), double buffered; every
 //     wave-instruction writes 1 KiB of contiguous LDS, the XOR swizzle is applied on the global-address side.
+//     The copies are buffer loads (scalar tile base + one 32-bit lane offset): a global load with 64-bit lane
+//     addresses takes about twice as much issue time away from the MFMAs it runs beside.
 //   * an operand whose K index is contiguous in memory is read from LDS with ds_read_b128; an operand whose
 //     M/N index is contiguous (B in the NN case) is read with the transposing ds_read_b64_tr_b16, so no
 //     transpose pass over B is ever made.
@@ -16,6 +18,7 @@
 //     The MFMA is issued with the B fragment as first operand, i.e. it produces the transposed block, so a
 //     lane ends up with 4 consecutive N of one row of C; the epilogue parks the sub-tile in LDS and stores whole
 //     128-byte lines.
+#include <type_traits>
 #include "mi355_common.h"
 #include "mi355_serving_internal.h"
 
@@ -117,19 +120,14 @@ struct MainCfg {
     static constexpr int FRAG_SLOTS = (TM > TN ? TM : TN) > 4 ? (TM > TN ? TM : TN) : 4;
 };
 
-// Scheduling hint: alternate NMFMA matrix instructions with NDS LDS reads, spreading the reads evenly
-// (sched_group_barrier wants literal counts, hence the recursion over the MFMA index).
-template <int M, int NMFMA, int NDS>
-struct InterleaveMfmaWithLdsReads {
-    __device__ static __forceinline__ void emit() {
-        if constexpr (M < NMFMA) {
-            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // one MFMA
-            constexpr int nds = NDS * (M + 1) / NMFMA - NDS * M / NMFMA;
-            if constexpr (nds > 0) __builtin_amdgcn_sched_group_barrier(0x100, nds, 0);  // LDS reads
-            InterleaveMfmaWithLdsReads<M + 1, NMFMA, NDS>::emit();
-        }
+// f(std::integral_constant<int, I>) for I = BEGIN .. END-1, unrolled at compile time
+template <int BEGIN, int END, class F>
+__device__ __forceinline__ void static_for(F&& f) {
+    if constexpr (BEGIN < END) {
+        f(std::integral_constant<int, BEGIN>{});
+        static_for<BEGIN + 1, END>(f);
     }
-};
+}
 
 // Map the linear workgroup id to a C tile so that the workgroups resident on one XCD (ids congruent mod 8)
 // cover a compact rectangle of tiles: they then share A row-panels and B column-panels in that XCD's L2.
@@ -190,86 +188,72 @@ __global__ __launch_bounds__(WM * WN * 64) void hgemm_main_kernel(const T* __res
     const long n0 = (long)tile_n * Cfg::BN;
 
     // ---- global -> LDS copy descriptors --------------------------------------------------------------
-    const T* a_src;
-    long a_copy_stride, a_k_stride;
+    // A copy reads (tile base, kept in scalar registers and advanced per K tile) + (this lane's byte offset inside the
+    // tile, a loop-invariant 32-bit VGPR) + (copy index * uniform step). Offsets inside a tile fit 32 bits because the
+    // launcher only takes leading dimensions below 2^22 elements.
+    const char* a_base;
+    const char* b_base;
+    uint32_t a_lane_off, b_lane_off, a_copy_step, b_copy_step;
+    long a_k_step, b_k_step;
     if constexpr (A_KC) {  // A stored [M,K]
-        a_src = A + m0 * lda + ATK::first_copy_offset(wave, lane, lda);
-        a_copy_stride = ATK::copy_stride(lda);
-        a_k_stride = ATK::ktile_stride(lda);
+        a_base = (const char*)(A + m0 * lda);
+        a_lane_off = (uint32_t)(ATK::first_copy_offset(wave, lane, lda) * 2);
+        a_copy_step = (uint32_t)(ATK::copy_stride(lda) * 2);
+        a_k_step = ATK::ktile_stride(lda) * 2;
     } else {  // A stored [K,M]
-        a_src = A + m0 + ATM::first_copy_offset(wave, lane, lda);
-        a_copy_stride = ATM::copy_stride(lda);
-        a_k_stride = ATM::ktile_stride(lda);
+        a_base = (const char*)(A + m0);
+        a_lane_off = (uint32_t)(ATM::first_copy_offset(wave, lane, lda) * 2);
+        a_copy_step = (uint32_t)(ATM::copy_stride(lda) * 2);
+        a_k_step = ATM::ktile_stride(lda) * 2;
     }
-    const T* b_src;
-    long b_copy_stride, b_k_stride;
     if constexpr (B_KC) {  // B stored [N,K]
-        b_src = B + n0 * ldb + BTK::first_copy_offset(wave, lane, ldb);
-        b_copy_stride = BTK::copy_stride(ldb);
-        b_k_stride = BTK::ktile_stride(ldb);
+        b_base = (const char*)(B + n0 * ldb);
+        b_lane_off = (uint32_t)(BTK::first_copy_offset(wave, lane, ldb) * 2);
+        b_copy_step = (uint32_t)(BTK::copy_stride(ldb) * 2);
+        b_k_step = BTK::ktile_stride(ldb) * 2;
     } else {  // B stored [K,N]
-        b_src = B + n0 + BTN::first_copy_offset(wave, lane, ldb);
-        b_copy_stride = BTN::copy_stride(ldb);
-        b_k_stride = BTN::ktile_stride(ldb);
+        b_base = (const char*)(B + n0);
+        b_lane_off = (uint32_t)(BTN::first_copy_offset(wave, lane, ldb) * 2);
+        b_copy_step = (uint32_t)(BTN::copy_stride(ldb) * 2);
+        b_k_step = BTN::ktile_stride(ldb) * 2;
     }
 
-    // RAGGED: one pointer per copy, rows / column chunks past the end folded back inside
-    const T* a_ptr[RAGGED ? Cfg::A_INSTS : 1];
-    const T* b_ptr[RAGGED ? Cfg::B_INSTS : 1];
+    // RAGGED: one lane offset per copy, rows / column chunks past the end folded back inside the matrix (never in
+    // front of the tile origin: the tile exists, so its first row and its first 8 columns do)
+    uint32_t a_voff[RAGGED ? Cfg::A_INSTS : 1];
+    uint32_t b_voff[RAGGED ? Cfg::B_INSTS : 1];
     if constexpr (RAGGED) {
-        auto clamped = [&](const T* base, long ld, bool k_contig, int rows_per_inst, int chunks_per_row, int rows_per_pass,
-                           int i, long origin, long extent, int swz) {
+        // byte offset from the tile base of copy i of this lane; origin / extent along the tile's M (or N) axis
+        auto clamped = [&](long ld, bool k_contig, int rows_per_inst, int chunks_per_row, int rows_per_pass, int i,
+                           long origin, long extent, int swz) {
             const int row = wave * rows_per_inst + lane / chunks_per_row + i * rows_per_pass;
             const int chunk = (lane % chunks_per_row) ^ swz;
-            if (k_contig) return base + min(origin + row, extent - 1) * ld + chunk * 8;   // row = M/N index
-            return base + (long)row * ld + min(origin + chunk * 8, extent - 8);           // row = K index
+            if (k_contig) return (uint32_t)(((min(origin + row, extent - 1) - origin) * ld + chunk * 8) * 2);   // row = M/N index
+            return (uint32_t)(((long)row * ld + min(origin + chunk * 8, extent - 8) - origin) * 2);              // row = K index
         };
 #pragma unroll
         for (int i = 0; i < Cfg::A_INSTS; ++i) {
             if constexpr (A_KC) {
                 const int row = wave * ATK::kRowsPerInst + lane / ATK::kChunksPerRow;
-                a_ptr[i] = clamped(A, lda, true, ATK::kRowsPerInst, ATK::kChunksPerRow, ATK::kRowsPerPass, i, m0, M, ATK::swz(row));
+                a_voff[i] = clamped(lda, true, ATK::kRowsPerInst, ATK::kChunksPerRow, ATK::kRowsPerPass, i, m0, M, ATK::swz(row));
             } else {
                 const int row = wave * ATM::kRowsPerInst + lane / ATM::kChunksPerRow + i * ATM::kRowsPerPass;
-                a_ptr[i] = clamped(A, lda, false, ATM::kRowsPerInst, ATM::kChunksPerRow, ATM::kRowsPerPass, i, m0, M, ATM::swz(row));
+                a_voff[i] = clamped(lda, false, ATM::kRowsPerInst, ATM::kChunksPerRow, ATM::kRowsPerPass, i, m0, M, ATM::swz(row));
             }
         }
 #pragma unroll
         for (int i = 0; i < Cfg::B_INSTS; ++i) {
             if constexpr (B_KC) {
                 const int row = wave * BTK::kRowsPerInst + lane / BTK::kChunksPerRow;
-                b_ptr[i] = clamped(B, ldb, true, BTK::kRowsPerInst, BTK::kChunksPerRow, BTK::kRowsPerPass, i, n0, N, BTK::swz(row));
+                b_voff[i] = clamped(ldb, true, BTK::kRowsPerInst, BTK::kChunksPerRow, BTK::kRowsPerPass, i, n0, N, BTK::swz(row));
             } else {
                 const int row = wave * BTN::kRowsPerInst + lane / BTN::kChunksPerRow + i * BTN::kRowsPerPass;
-                b_ptr[i] = clamped(B, ldb, false, BTN::kRowsPerInst, BTN::kChunksPerRow, BTN::kRowsPerPass, i, n0, N, BTN::swz(row));
+                b_voff[i] = clamped(ldb, false, BTN::kRowsPerInst, BTN::kChunksPerRow, BTN::kRowsPerPass, i, n0, N, BTN::swz(row));
             }
         }
     }
-    auto issue_copies = [&](int stage) {
-        MI355_LDS char* sa = smem + stage * Cfg::STAGE_BYTES;
-        MI355_LDS char* sb = sa + Cfg::A_BYTES;
-        if constexpr (RAGGED) {
-#pragma unroll
-            for (int i = 0; i < Cfg::A_INSTS; ++i) {
-                copy16_global_to_lds(a_ptr[i], sa + (i * Cfg::NWAVES + wave) * 1024);
-                a_ptr[i] += a_k_stride;
-            }
-#pragma unroll
-            for (int i = 0; i < Cfg::B_INSTS; ++i) {
-                copy16_global_to_lds(b_ptr[i], sb + (i * Cfg::NWAVES + wave) * 1024);
-                b_ptr[i] += b_k_stride;
-            }
-            return;
-        }
-#pragma unroll
-        for (int i = 0; i < Cfg::A_INSTS; ++i)
-            copy16_global_to_lds(a_src + i * a_copy_stride, sa + (i * Cfg::NWAVES + wave) * 1024);
-#pragma unroll
-        for (int i = 0; i < Cfg::B_INSTS; ++i)
-            copy16_global_to_lds(b_src + i * b_copy_stride, sb + (i * Cfg::NWAVES + wave) * 1024);
-        a_src += a_k_stride;
-        b_src += b_k_stride;
-    };
+    int4v a_res = make_buffer_resource(a_base);
+    int4v b_res = make_buffer_resource(b_base);
 
     // ---- LDS fragment read offsets (bytes inside one stage) -------------------------------------------
     // A fragments: TM blocks of 32 rows; B fragments: TN blocks of 32 columns.
@@ -328,55 +312,149 @@ __global__ __launch_bounds__(WM * WN * 64) void hgemm_main_kernel(const T* __res
             for (int j = 0; j < TN; ++j)
                 acc[i][j] = Elem<T>::mfma32(bf[j], af[i], acc[i][j]);
     };
-    // ask the scheduler to alternate the TM*TN MFMAs of one substep with the LDS reads of the next one
-    constexpr int kDsReads = (A_KC ? TM : 2 * TM) + (B_KC ? TN : 2 * TN);
-    auto interleave = [&]() {
-        InterleaveMfmaWithLdsReads<0, TM * TN, kDsReads>::emit();
+    // Software pipeline, pinned slot by slot (a slot = one MFMA and what is issued in its shadow; sched_barrier keeps the
+    // compiler from moving anything between slots):
+    //   * the fragments of substep kk+1 are read during the FIRST slots of substep kk, in the order the MFMAs will need
+    //     them, so they have landed long before that substep ends and no MFMA waits on a read it has just issued;
+    //   * the barrier that hands over the next K tile sits in front of the last substep: the reads of that substep
+    //     were issued a substep earlier, so the wave reaches the barrier with nothing in flight, and goes on with
+    //     MFMAs whose operands are already in registers;
+    //   * the copies of the tile after next go out one per slot during that last substep, behind the reads of the next
+    //     tile's first fragments.
+    constexpr int NSLOT = TM * TN;
+    constexpr int NFRAG = TM + TN;
+    constexpr int NCOPY = Cfg::A_INSTS + Cfg::B_INSTS;
+    // fragment f of substep kk, f in the order of first use: A0, B0 .. B(TN-1), A1 .. A(TM-1)
+    auto load_frag = [&](MI355_LDS char* st, int kk, auto fc, V8(&afn)[TM], V8(&bfn)[TN]) {
+        constexpr int f = decltype(fc)::value;
+#ifdef EXP_NOREAD
+        return;
+#endif
+        if constexpr (f == 0 || f > TN) {
+            constexpr int i = f == 0 ? 0 : f - TN;
+            if constexpr (A_KC) {
+                afn[i] = Elem<T>::frag(lds_read_b128(st + a_off[kk] + i * 32 * ATK::kRowBytes));
+            } else {
+                half4 lo = lds_read_tr16_b64(st + a_off[i] + (kk * 16) * ATM::kRowBytes);
+                half4 hi = lds_read_tr16_b64(st + a_off[i] + (kk * 16 + 4) * ATM::kRowBytes);
+                afn[i] = Elem<T>::frag(concat(lo, hi));
+            }
+        } else {
+            constexpr int j = f - 1;
+            if constexpr (B_KC) {
+                bfn[j] = Elem<T>::frag(lds_read_b128(st + b_off[kk] + j * 32 * BTK::kRowBytes));
+            } else {
+                half4 lo = lds_read_tr16_b64(st + b_off[j] + (kk * 16) * BTN::kRowBytes);
+                half4 hi = lds_read_tr16_b64(st + b_off[j] + (kk * 16 + 4) * BTN::kRowBytes);
+                bfn[j] = Elem<T>::frag(concat(lo, hi));
+            }
+        }
+    };
+    auto issue_copy = [&](int stage, auto dc) {
+        constexpr int d = decltype(dc)::value;
+#ifdef EXP_NOCOPY
+        return;
+#endif
+        MI355_LDS char* sa = smem + stage * Cfg::STAGE_BYTES;
+        if constexpr (d < Cfg::A_INSTS) {
+            MI355_LDS char* dst = sa + (d * Cfg::NWAVES + wave) * 1024;
+            if constexpr (RAGGED) copy16_buffer_to_lds(a_res, a_voff[d], 0u, dst);
+            else copy16_buffer_to_lds(a_res, a_lane_off, d * a_copy_step, dst);
+        } else {
+            constexpr int e = d - Cfg::A_INSTS;
+            MI355_LDS char* dst = sa + Cfg::A_BYTES + (e * Cfg::NWAVES + wave) * 1024;
+            if constexpr (RAGGED) copy16_buffer_to_lds(b_res, b_voff[e], 0u, dst);
+            else copy16_buffer_to_lds(b_res, b_lane_off, e * b_copy_step, dst);
+        }
+    };
+    auto advance_copies = [&]() {   // next K tile: scalar arithmetic on the two bases
+        a_base += a_k_step;
+        b_base += b_k_step;
+        a_res = make_buffer_resource(a_base);
+        b_res = make_buffer_resource(b_base);
+    };
+    auto issue_copies = [&](int stage) {
+        static_for<0, NCOPY>([&](auto dc) { issue_copy(stage, dc); });
+        advance_copies();
+    };
+    // one substep: the MFMAs on (afc, bfc); in slot m, `hook(m)` issues what rides along
+    auto substep = [&](const V8(&afc)[TM], const V8(&bfc)[TN], auto&& hook) {
+        static_for<0, NSLOT>([&](auto mc) {
+            constexpr int m = decltype(mc)::value;
+            constexpr int i = m / TN, j = m % TN;
+            acc[i][j] = Elem<T>::mfma32(bfc[j], afc[i], acc[i][j]);
+            hook(mc);
+            __builtin_amdgcn_sched_barrier(0);
+        });
+    };
+    auto reads_of = [&](MI355_LDS char* st, int kk, V8(&afn)[TM], V8(&bfn)[TN]) {
+        return [&, st, kk](auto mc) {
+            if constexpr (decltype(mc)::value < NFRAG) load_frag(st, kk, mc, afn, bfn);
+        };
     };
 
-    // Software pipeline: the fragments of substep kk+1 are read from LDS while the MFMAs of substep kk run;
-    // the barrier that hands over the next K tile sits in front of the LAST substep of the current tile, so
-    // the first fragments of the next tile are read under that substep's MFMAs and no wave starts a tile
-    // with an exposed LDS round trip.
+#ifndef EXP_SP
+#define EXP_SP 1
+#endif
+    // copy d of a tile goes out in slot d * kCopySpacing, counted from the first slot after the barrier that frees its
+    // stage: the slots of the substep behind the barrier (the "head") and, beyond those, of the next tile's first
+    // substeps (the "tail")
+    constexpr int kCopySpacingNum = EXP_SP * NSLOT, kCopySpacingDen = NCOPY;
+    static_assert((NCOPY - 1) * kCopySpacingNum / kCopySpacingDen < 3 * NSLOT, "copies must be out two substeps before the barrier");
+    auto copies_of_slot = [&](int stage, auto gc) {   // issue the copies whose slot is g
+        constexpr int g = decltype(gc)::value;
+        static_for<0, NCOPY>([&](auto dc) {
+            if constexpr (decltype(dc)::value * kCopySpacingNum / kCopySpacingDen == g) issue_copy(stage, dc);
+        });
+    };
     const int ktiles = K / BK;
     V8 af[2][TM], bf[2][TN];
     issue_copies(0);
     wait_vmcnt<0>();
     __syncthreads();
-    if (ktiles > 1) issue_copies(1);
+    if (ktiles > 1) static_for<0, NSLOT>([&](auto gc) { copies_of_slot(1, gc); });   // head of tile 1
     load_frags(smem, 0, af[0], bf[0]);
+#ifdef EXP_NOREAD
+    load_frags(smem, 1, af[1], bf[1]);
+#endif
 
-    for (int kt = 0; kt + 1 < ktiles; ++kt) {
+    auto tile = [&](int kt, auto with_copies) {
         MI355_LDS char* st = smem + (kt & 1) * Cfg::STAGE_BYTES;
         MI355_LDS char* stn = smem + ((kt + 1) & 1) * Cfg::STAGE_BYTES;
-        load_frags(st, 1, af[1], bf[1]);
-        mma(af[0], bf[0]);
-        interleave();
-        load_frags(st, 2, af[0], bf[0]);
-        mma(af[1], bf[1]);
-        interleave();
-        load_frags(st, 3, af[1], bf[1]);
-        mma(af[0], bf[0]);
-        interleave();
-        // my copies of tile kt+1 have landed and my reads of this stage are complete; after the barrier that
-        // holds for every wave, so this stage may be refilled and the next one may be read
+        // (tail of the copies of tile kt+1 rides along)
+        substep(af[0], bf[0], [&](auto mc) {
+            constexpr int m = decltype(mc)::value;
+            if constexpr (m < NFRAG) load_frag(st, 1, mc, af[1], bf[1]);
+            copies_of_slot((kt + 1) & 1, std::integral_constant<int, NSLOT + m>{});
+        });
+        substep(af[1], bf[1], [&](auto mc) {
+            constexpr int m = decltype(mc)::value;
+            if constexpr (m < NFRAG) load_frag(st, 2, mc, af[0], bf[0]);
+            copies_of_slot((kt + 1) & 1, std::integral_constant<int, 2 * NSLOT + m>{});
+        });
+        advance_copies();
+        substep(af[0], bf[0], reads_of(st, 3, af[1], bf[1]));
+        // my copies of tile kt+1 have landed and my reads of this stage are complete; after the barrier that holds for
+        // every wave, so this stage may be refilled and the next one may be read
+#ifndef EXP_NOVMWAIT
         wait_vmcnt<0>();
+#endif
+#ifndef EXP_NOBAR
         __syncthreads();
-        if (kt + 2 < ktiles) issue_copies(kt & 1);
-        load_frags(stn, 0, af[0], bf[0]);
-        mma(af[1], bf[1]);
-        interleave();
-    }
+#endif
+        substep(af[1], bf[1], [&](auto mc) {
+            constexpr int m = decltype(mc)::value;
+            if constexpr (m < NFRAG) load_frag(stn, 0, mc, af[0], bf[0]);
+            if constexpr (decltype(with_copies)::value) copies_of_slot(kt & 1, mc);   // head of tile kt+2
+        });
+    };
+    for (int kt = 0; kt + 2 < ktiles; ++kt) tile(kt, std::true_type{});
+    if (ktiles >= 2) tile(ktiles - 2, std::false_type{});
     {  // last tile: nothing left to fetch
         MI355_LDS char* st = smem + ((ktiles - 1) & 1) * Cfg::STAGE_BYTES;
-        load_frags(st, 1, af[1], bf[1]);
-        mma(af[0], bf[0]);
-        interleave();
-        load_frags(st, 2, af[0], bf[0]);
-        mma(af[1], bf[1]);
-        interleave();
-        load_frags(st, 3, af[1], bf[1]);
-        mma(af[0], bf[0]);
+        substep(af[0], bf[0], reads_of(st, 1, af[1], bf[1]));
+        substep(af[1], bf[1], reads_of(st, 2, af[0], bf[0]));
+        substep(af[0], bf[0], reads_of(st, 3, af[1], bf[1]));
         mma(af[1], bf[1]);
     }
 
@@ -789,7 +867,8 @@ static hipError_t launch_layout(const T* A, const T* B, T* C, const T* R, int M,
     const bool aligned = (reinterpret_cast<uintptr_t>(A) % 16 == 0) && (reinterpret_cast<uintptr_t>(B) % 16 == 0) &&
                          (reinterpret_cast<uintptr_t>(C) % 16 == 0) && (lda % 8 == 0) && (ldb % 8 == 0) &&
                          (ldc % 8 == 0) && (reinterpret_cast<uintptr_t>(R) % 16 == 0) && (ldr % 8 == 0);
-    const bool k_ok = aligned && K % 64 == 0 && K >= 64;
+    // the tiled kernels address a tile with 32-bit byte offsets: up to 256 rows of lda (ldb) elements
+    const bool k_ok = aligned && K % 64 == 0 && K >= 64 && lda < (1L << 22) && ldb < (1L << 22);
     const bool fits256 = k_ok && M % 256 == 0 && N % 256 == 0;
     const bool fits128 = k_ok && M % 128 == 0 && N % 128 == 0;
     if constexpr (A_KC && !B_KC) {
@@ -807,7 +886,11 @@ static hipError_t launch_layout(const T* A, const T* B, T* C, const T* R, int M,
     if (g_gemm_variant == 1 && fits256) choice = 1;
     if (g_gemm_variant == 2 && fits128) choice = 2;
     switch (choice) {
+#ifdef EXP_W4
+        case 1: return launch_main<T, A_KC, B_KC, 256, 256, 2, 2>(A, B, C, R, M, N, K, lda, ldb, ldc, ldr, stream);
+#else
         case 1: return launch_main<T, A_KC, B_KC, 256, 256, 2, 4>(A, B, C, R, M, N, K, lda, ldb, ldc, ldr, stream);
+#endif
         case 2: return launch_main<T, A_KC, B_KC, 128, 128, 2, 2>(A, B, C, R, M, N, K, lda, ldb, ldc, ldr, stream);
         default: break;
     }
@@ -831,7 +914,8 @@ static hipError_t launch_silu_mul(const T* A, const T* B, T* C, int M, int N, in
     const bool aligned = (reinterpret_cast<uintptr_t>(A) % 16 == 0) && (reinterpret_cast<uintptr_t>(B) % 16 == 0) &&
                          (reinterpret_cast<uintptr_t>(C) % 16 == 0) && (lda % 8 == 0) && (ldb % 8 == 0) && (ldc % 8 == 0);
     // N = columns of op(B); gate/up pairs are 64 columns wide. Few rows are better served by the small-M product.
-    if (!aligned || K % 64 != 0 || K < 64 || N % 64 != 0 || M <= 64) return hipErrorNotSupported;
+    if (!aligned || K % 64 != 0 || K < 64 || N % 64 != 0 || M <= 64 || lda >= (1L << 22) || ldb >= (1L << 22))
+        return hipErrorNotSupported;
     const bool fits128 = M % 128 == 0 && N % 128 == 0;
     const bool fits256 = M % 256 == 0 && N % 256 == 0;
     const long t256 = (long)((M + 255) / 256) * ((N + 255) / 256);

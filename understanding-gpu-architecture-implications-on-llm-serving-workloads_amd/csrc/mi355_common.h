@@ -2,7 +2,7 @@
 //
 // Everything here is written for wave64 and for the gfx950 instruction set only:
 //   * v_mfma_f32_32x32x16_f16 / v_mfma_f32_16x16x32_f16 (fp16 in, fp32 accumulate)
-//   * global_load_lds_dwordx4 (16-byte global -> LDS copies that bypass the VGPRs)
+//   * global_load_lds_dwordx4 / buffer_load_dwordx4 ... lds (16-byte global -> LDS copies that bypass the VGPRs)
 //   * ds_read_b64_tr_b16 (LDS read that transposes a 4x16 block of 16-bit values)
 //
 // Register layouts (checked on hardware):
@@ -69,6 +69,33 @@ __device__ __forceinline__ void copy16_global_to_lds(const void* uniform_base, u
         "global_load_lds_dwordx4 %0, %1"
         :
         : "v"(lane_byte_offset), "s"(uniform_base), "s"((uint32_t)(uintptr_t)lds_wave_base)
+        : "memory", "m0");
+}
+
+// Buffer resource (V#) over a whole address range: 48-bit base, no stride, no swizzle, the largest record count, raw
+// 32-bit data format. The four words must sit in scalar registers, so every word is made wave-uniform explicitly.
+__device__ __forceinline__ int4v make_buffer_resource(const void* base) {
+    const uint64_t b = (uint64_t)(uintptr_t)base;
+    int4v r;
+    r[0] = __builtin_amdgcn_readfirstlane((int)(uint32_t)b);
+    r[1] = __builtin_amdgcn_readfirstlane((int)(uint32_t)(b >> 32) & 0xffff);
+    r[2] = __builtin_amdgcn_readfirstlane((int)0xffffffffu);
+    r[3] = __builtin_amdgcn_readfirstlane(0x00020000);
+    return r;
+}
+
+// The same 16-byte global -> LDS copy through a buffer resource: lane address = resource base + lane_byte_offset (one
+// 32-bit VGPR) + uniform_byte_offset (a scalar register). A wave instruction that reads one address VGPR instead of a
+// 64-bit pair takes about half as much issue time away from the MFMAs it runs beside, and all per-tile address
+// arithmetic (advancing the base) runs on the scalar unit.
+__device__ __forceinline__ void copy16_buffer_to_lds(int4v resource, uint32_t lane_byte_offset, uint32_t uniform_byte_offset,
+                                                     MI355_LDS void* lds_wave_base) {
+    asm volatile(
+        "s_mov_b32 m0, %3\n\t"
+        "s_nop 0\n\t"
+        "buffer_load_dwordx4 %0, %1, %2 offen lds"
+        :
+        : "v"(lane_byte_offset), "s"(resource), "s"(uniform_byte_offset), "s"((uint32_t)(uintptr_t)lds_wave_base)
         : "memory", "m0");
 }
 
