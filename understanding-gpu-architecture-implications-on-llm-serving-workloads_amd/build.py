@@ -27,6 +27,9 @@ DEVICE_FLAGS = [
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
 ]
 KERNEL_SOURCES = ["csrc/hgemm.hip", "csrc/fmha_fwd.hip", "csrc/fmha_decode.hip", "csrc/glue.hip", "csrc/capi.hip"]
+# Per-source additions. The GEMM keeps its MFMA accumulators in ordinary VGPRs: left to itself the compiler moves part of
+# them to AGPRs in the 4-wave kernels and then shuffles them back and forth inside the K loop.
+SOURCE_FLAGS = {"csrc/hgemm.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"]}
 
 
 def _run(cmd, quiet_patterns=("is not a recognized feature for this target",)):
@@ -39,11 +42,24 @@ def _run(cmd, quiet_patterns=("is not a recognized feature for this target",)):
 
 
 def build_library(verbose=True):
-    """Compile the HIP kernels and the C ABI into libmi355_serving.so."""
-    cmd = [HIPCC] + DEVICE_FLAGS + ["-shared", "-I", INCLUDE] + KERNEL_SOURCES + ["-o", LIB_PATH]
-    if verbose:
-        print("[build] " + " ".join(cmd))
-    _run(cmd)
+    """Compile the HIP kernels and the C ABI into libmi355_serving.so (one object per source, compiled side by side)."""
+    import tempfile
+    from concurrent.futures import ThreadPoolExecutor
+
+    with tempfile.TemporaryDirectory(prefix="mi355_build_") as tmp:
+        jobs = []
+        for src in KERNEL_SOURCES:
+            obj = os.path.join(tmp, os.path.basename(src) + ".o")
+            cmd = [HIPCC] + DEVICE_FLAGS + SOURCE_FLAGS.get(src, []) + ["-I", INCLUDE, "-c", src, "-o", obj]
+            if verbose:
+                print("[build] " + " ".join(cmd))
+            jobs.append((cmd, obj))
+        with ThreadPoolExecutor(max_workers=min(len(jobs), os.cpu_count() or 1, 8)) as pool:
+            list(pool.map(lambda job: _run(job[0]), jobs))
+        link = [HIPCC, "--offload-arch=gfx950", "-fPIC", "-shared"] + [obj for _, obj in jobs] + ["-o", LIB_PATH]
+        if verbose:
+            print("[build] " + " ".join(link))
+        _run(link)
     return LIB_PATH
 
 

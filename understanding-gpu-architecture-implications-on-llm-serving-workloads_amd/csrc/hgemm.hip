@@ -14,7 +14,8 @@
 //   * an operand whose K index is contiguous in memory is read from LDS with ds_read_b128; an operand whose
 //     M/N index is contiguous (B in the NN case) is read with the transposing ds_read_b64_tr_b16, so no
 //     transpose pass over B is ever made.
-//   * each wave owns a 128x64 sub-tile = 4x2 MFMA 32x32x16 blocks (128 fp32 accumulators per lane).
+//   * each wave owns a 128x64 sub-tile = 8x4 MFMA 16x16x32 blocks (128 fp32 accumulators per lane); with random
+//     operands the 16x16x32 instruction sustains a ~14 % higher rate than 32x32x16 under the board's power limit.
 //     The MFMA is issued with the B fragment as first operand, i.e. it produces the transposed block, so a
 //     lane ends up with 4 consecutive N of one row of C; the epilogue parks the sub-tile in LDS and stores whole
 //     128-byte lines.
@@ -53,10 +54,11 @@ struct KContigTile {
     __device__ static __forceinline__ long ktile_stride(long /*ld*/) { return BK; }
     __device__ static __forceinline__ int lds_inst_offset(int inst, int wave) { return (inst * NWAVES + wave) * 1024; }
 
-    // byte offset inside the tile of the fragment (32 rows x 16 k) for k-substep kk, first row row0
+    // byte offset inside the tile of this lane's 16 bytes of the fragment (16 rows x 32 k) for k-substep kk, first
+    // row row0 (a multiple of 16): lane l holds k = 32 kk + 8 (l / 16) .. +7 of row l % 16
     __device__ static __forceinline__ int frag_offset(int row0, int kk, int lane) {
-        int row = row0 + (lane & 31);
-        int chunk = (kk * 2 + (lane >> 5)) ^ swz(row);
+        int row = row0 + (lane & 15);
+        int chunk = (kk * 4 + (lane >> 4)) ^ swz(row);
         return row * kRowBytes + chunk * 16;
     }
 };
@@ -73,11 +75,10 @@ struct MNContigTile {
     static_assert(COLS == 256 || COLS == 128, "swizzle below needs at least 16 chunks per row");
     static_assert(BK % kRowsPerPass == 0, "tile depth must be a multiple of one pass of the workgroup");
 
-    // depends on (row % 4) only; keeps the 16 lanes of one transposing read on distinct banks
-    __device__ static __forceinline__ int swz(int row) {
-        int r = row & 3;
-        return (r << 1) | ((r & 1) << 3);  // 0, 10, 4, 14
-    }
+    // A transposing read touches, per 16 lanes, 4 k-rows x 32 bytes (two neighbouring chunks); lanes 0..31 of a
+    // fragment read cover rows {0..3} and {8..11} (+ a multiple of 4 that does not change what follows). XOR-ing the
+    // chunk index with an even number that differs for those 8 rows keeps their 8 chunk pairs on distinct banks.
+    __device__ static __forceinline__ int swz(int row) { return ((row & 3) | (((row >> 3) & 1) << 2)) << 1; }
     __device__ static __forceinline__ long first_copy_offset(int wave, int lane, long ld) {
         int row = wave * kRowsPerInst + lane / kChunksPerRow;
         int chunk = (lane % kChunksPerRow) ^ swz(row);
@@ -87,12 +88,14 @@ struct MNContigTile {
     __device__ static __forceinline__ long ktile_stride(long ld) { return (long)BK * ld; }
     __device__ static __forceinline__ int lds_inst_offset(int inst, int wave) { return (inst * NWAVES + wave) * 1024; }
 
-    // byte offset of this lane's transposing read for the fragment (16 k x 32 cols) whose first column is
-    // col0, at k rows [8*(lane/32) .. +3]; add (kk*16 + 4*t) * kRowBytes for substep kk and half t.
+    // byte offset of this lane's transposing read for the fragment (32 k x 16 cols) whose first column is col0 (a
+    // multiple of 16): group g = lane / 16 reads k rows 8g .. 8g+3, input lane j of the group supplies the 4 columns
+    // 4 (j % 4) .. +3 of row j / 4. Add (kk*32 + 4*t) * kRowBytes for substep kk and half t (neither changes swz).
     __device__ static __forceinline__ int frag_offset(int col0, int lane) {
-        int row = 8 * (lane >> 5) + ((lane & 15) >> 2);
-        int chunk = (col0 >> 3) + 2 * ((lane >> 4) & 1) + ((lane & 3) >> 1);
-        return row * kRowBytes + ((chunk ^ swz(row)) << 4) + (lane & 1) * 8;
+        int j = lane & 15;
+        int row = 8 * (lane >> 4) + (j >> 2);
+        int chunk = (col0 >> 3) + ((j & 3) >> 1);
+        return row * kRowBytes + ((chunk ^ swz(row)) << 4) + (j & 1) * 8;
     }
 };
 
@@ -104,8 +107,8 @@ template <bool A_KC, bool B_KC, int BM_, int BN_, int WM_, int WN_>
 struct MainCfg {
     static constexpr int BM = BM_, BN = BN_, BK = 64;
     static constexpr int WM = WM_, WN = WN_, NWAVES = WM_ * WN_, NTHREADS = NWAVES * 64;
-    static constexpr int TM = BM / WM / 32;  // MFMA blocks along M per wave
-    static constexpr int TN = BN / WN / 32;  // along N
+    static constexpr int TM = BM / WM / 16;  // MFMA 16x16 blocks along M per wave
+    static constexpr int TN = BN / WN / 16;  // along N
     using ATileK = KContigTile<BM, BK, NWAVES>;
     using ATileM = MNContigTile<BM, BK, NWAVES>;
     using BTileK = KContigTile<BN, BK, NWAVES>;
@@ -113,11 +116,13 @@ struct MainCfg {
     static constexpr int A_BYTES = BM * BK * 2;
     static constexpr int B_BYTES = BN * BK * 2;
     static constexpr int STAGE_BYTES = A_BYTES + B_BYTES;
-    static constexpr int NSTAGE = 2;
+    // 64 KiB stages: two of them fit; the 32 KiB stages of the 128x128 tile get a third, which gives every copy one more
+    // K tile of time to land (small problems run few tiles per workgroup and are bound by that latency)
+    static constexpr int NSTAGE = STAGE_BYTES > 48 * 1024 ? 2 : 3;
     static constexpr int LDS_BYTES = STAGE_BYTES * NSTAGE;
     static constexpr int A_INSTS = A_BYTES / (NWAVES * 1024);  // 16-byte copies per lane per K tile
     static constexpr int B_INSTS = B_BYTES / (NWAVES * 1024);
-    static constexpr int FRAG_SLOTS = (TM > TN ? TM : TN) > 4 ? (TM > TN ? TM : TN) : 4;
+    static constexpr int FRAG_SLOTS = TM > TN ? TM : TN;
 };
 
 // f(std::integral_constant<int, I>) for I = BEGIN .. END-1, unrolled at compile time
@@ -160,7 +165,8 @@ __device__ __forceinline__ void tile_of_block(int bid, int tiles_m, int tiles_n,
 // an operand whose M/N index is contiguous, to the last 8 columns; that dimension must be a multiple of 8), so every
 // load stays inside the matrices, and the epilogue stores only what exists.
 template <typename T, bool A_KC, bool B_KC, int BM, int BN, int WM, int WN, int EPI = 0, bool RAGGED = false>
-__global__ __launch_bounds__(WM * WN * 64) void hgemm_main_kernel(const T* __restrict__ A, const T* __restrict__ B,
+__global__ __launch_bounds__(WM * WN * 64) __attribute__((amdgpu_waves_per_eu(WM * WN / 4, WM * WN / 4)))
+void hgemm_main_kernel(const T* __restrict__ A, const T* __restrict__ B,
                                                          T* C, const T* R, int M, int N, int K, long lda,
                                                          long ldb, long ldc, long ldr) {
     using V8 = typename Elem<T>::v8;
@@ -256,71 +262,42 @@ __global__ __launch_bounds__(WM * WN * 64) void hgemm_main_kernel(const T* __res
     int4v b_res = make_buffer_resource(b_base);
 
     // ---- LDS fragment read offsets (bytes inside one stage) -------------------------------------------
-    // A fragments: TM blocks of 32 rows; B fragments: TN blocks of 32 columns.
-    int a_off[Cfg::FRAG_SLOTS];  // K-contiguous operand: one per k-substep; M/N-contiguous: one per 32-wide block
+    // A fragments: TM blocks of 16 rows; B fragments: TN blocks of 16 columns; a K tile is two 32-deep substeps.
+    constexpr int NSUB = BK / 32;
+    static_assert(NSUB == 2, "the pipeline below is written for two substeps per K tile");
+    int a_off[Cfg::FRAG_SLOTS];  // K-contiguous operand: one per k-substep; M/N-contiguous: one per 16-wide block
     int b_off[Cfg::FRAG_SLOTS];
     if constexpr (A_KC) {
 #pragma unroll
-        for (int kk = 0; kk < 4; ++kk) a_off[kk] = ATK::frag_offset(wm * TM * 32, kk, lane);
+        for (int kk = 0; kk < NSUB; ++kk) a_off[kk] = ATK::frag_offset(wm * TM * 16, kk, lane);
     } else {
 #pragma unroll
-        for (int i = 0; i < TM; ++i) a_off[i] = ATM::frag_offset(wm * TM * 32 + i * 32, lane);
+        for (int i = 0; i < TM; ++i) a_off[i] = ATM::frag_offset(wm * TM * 16 + i * 16, lane);
     }
     if constexpr (B_KC) {
 #pragma unroll
-        for (int kk = 0; kk < 4; ++kk) b_off[kk] = Cfg::A_BYTES + BTK::frag_offset(wn * TN * 32, kk, lane);
+        for (int kk = 0; kk < NSUB; ++kk) b_off[kk] = Cfg::A_BYTES + BTK::frag_offset(wn * TN * 16, kk, lane);
     } else {
 #pragma unroll
-        for (int j = 0; j < TN; ++j) b_off[j] = Cfg::A_BYTES + BTN::frag_offset(wn * TN * 32 + j * 32, lane);
+        for (int j = 0; j < TN; ++j) b_off[j] = Cfg::A_BYTES + BTN::frag_offset(wn * TN * 16 + j * 16, lane);
     }
 
-    float16v acc[TM][TN];
+    float4v acc[TM][TN];
 #pragma unroll
     for (int i = 0; i < TM; ++i)
 #pragma unroll
-        for (int j = 0; j < TN; ++j)
-#pragma unroll
-            for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+        for (int j = 0; j < TN; ++j) acc[i][j] = float4v{0.f, 0.f, 0.f, 0.f};
 
-    // fragment loads of one k-substep (16 deep) from stage `st`
-    auto load_frags = [&](MI355_LDS char* st, int kk, V8(&af)[TM], V8(&bf)[TN]) {
-#pragma unroll
-        for (int i = 0; i < TM; ++i) {
-            if constexpr (A_KC) {
-                af[i] = Elem<T>::frag(lds_read_b128(st + a_off[kk] + i * 32 * ATK::kRowBytes));
-            } else {
-                half4 lo = lds_read_tr16_b64(st + a_off[i] + (kk * 16) * ATM::kRowBytes);
-                half4 hi = lds_read_tr16_b64(st + a_off[i] + (kk * 16 + 4) * ATM::kRowBytes);
-                af[i] = Elem<T>::frag(concat(lo, hi));
-            }
-        }
-#pragma unroll
-        for (int j = 0; j < TN; ++j) {
-            if constexpr (B_KC) {
-                bf[j] = Elem<T>::frag(lds_read_b128(st + b_off[kk] + j * 32 * BTK::kRowBytes));
-            } else {
-                half4 lo = lds_read_tr16_b64(st + b_off[j] + (kk * 16) * BTN::kRowBytes);
-                half4 hi = lds_read_tr16_b64(st + b_off[j] + (kk * 16 + 4) * BTN::kRowBytes);
-                bf[j] = Elem<T>::frag(concat(lo, hi));
-            }
-        }
-    };
-    auto mma = [&](const V8(&af)[TM], const V8(&bf)[TN]) {
-#pragma unroll
-        for (int i = 0; i < TM; ++i)
-#pragma unroll
-            for (int j = 0; j < TN; ++j)
-                acc[i][j] = Elem<T>::mfma32(bf[j], af[i], acc[i][j]);
-    };
-    // Software pipeline, pinned slot by slot (a slot = one MFMA and what is issued in its shadow; sched_barrier keeps the
-    // compiler from moving anything between slots):
-    //   * the fragments of substep kk+1 are read during the FIRST slots of substep kk, in the order the MFMAs will need
-    //     them, so they have landed long before that substep ends and no MFMA waits on a read it has just issued;
+    // Software pipeline, pinned slot by slot (a slot = one MFMA 16x16x32 and what is issued in its shadow;
+    // sched_barrier keeps the compiler from moving anything between slots):
+    //   * the fragments of the next substep are read during the FIRST slots of the current one, in the order the MFMAs
+    //     will need them, so they have landed long before that substep ends and no MFMA waits on a read it has just
+    //     issued;
     //   * the barrier that hands over the next K tile sits in front of the last substep: the reads of that substep
     //     were issued a substep earlier, so the wave reaches the barrier with nothing in flight, and goes on with
     //     MFMAs whose operands are already in registers;
-    //   * the copies of the tile after next go out one per slot during that last substep, behind the reads of the next
-    //     tile's first fragments.
+    //   * the copies of the tile after next go out during that last substep, spread over its slots, behind the reads of
+    //     the next tile's first fragments.
     constexpr int NSLOT = TM * TN;
     constexpr int NFRAG = TM + TN;
     constexpr int NCOPY = Cfg::A_INSTS + Cfg::B_INSTS;
@@ -333,22 +310,25 @@ __global__ __launch_bounds__(WM * WN * 64) void hgemm_main_kernel(const T* __res
         if constexpr (f == 0 || f > TN) {
             constexpr int i = f == 0 ? 0 : f - TN;
             if constexpr (A_KC) {
-                afn[i] = Elem<T>::frag(lds_read_b128(st + a_off[kk] + i * 32 * ATK::kRowBytes));
+                afn[i] = Elem<T>::frag(lds_read_b128(st + a_off[kk] + i * 16 * ATK::kRowBytes));
             } else {
-                half4 lo = lds_read_tr16_b64(st + a_off[i] + (kk * 16) * ATM::kRowBytes);
-                half4 hi = lds_read_tr16_b64(st + a_off[i] + (kk * 16 + 4) * ATM::kRowBytes);
+                half4 lo = lds_read_tr16_b64(st + a_off[i] + (kk * 32) * ATM::kRowBytes);
+                half4 hi = lds_read_tr16_b64(st + a_off[i] + (kk * 32 + 4) * ATM::kRowBytes);
                 afn[i] = Elem<T>::frag(concat(lo, hi));
             }
         } else {
             constexpr int j = f - 1;
             if constexpr (B_KC) {
-                bfn[j] = Elem<T>::frag(lds_read_b128(st + b_off[kk] + j * 32 * BTK::kRowBytes));
+                bfn[j] = Elem<T>::frag(lds_read_b128(st + b_off[kk] + j * 16 * BTK::kRowBytes));
             } else {
-                half4 lo = lds_read_tr16_b64(st + b_off[j] + (kk * 16) * BTN::kRowBytes);
-                half4 hi = lds_read_tr16_b64(st + b_off[j] + (kk * 16 + 4) * BTN::kRowBytes);
+                half4 lo = lds_read_tr16_b64(st + b_off[j] + (kk * 32) * BTN::kRowBytes);
+                half4 hi = lds_read_tr16_b64(st + b_off[j] + (kk * 32 + 4) * BTN::kRowBytes);
                 bfn[j] = Elem<T>::frag(concat(lo, hi));
             }
         }
+    };
+    auto load_frags = [&](MI355_LDS char* st, int kk, V8(&afn)[TM], V8(&bfn)[TN]) {
+        static_for<0, NFRAG>([&](auto fc) { load_frag(st, kk, fc, afn, bfn); });
     };
     auto issue_copy = [&](int stage, auto dc) {
         constexpr int d = decltype(dc)::value;
@@ -377,12 +357,14 @@ __global__ __launch_bounds__(WM * WN * 64) void hgemm_main_kernel(const T* __res
         static_for<0, NCOPY>([&](auto dc) { issue_copy(stage, dc); });
         advance_copies();
     };
+    // The MFMA is issued with the B fragment as first operand, i.e. it produces the transposed block: lane l ends up
+    // with C[m = l % 16][n = 4 (l / 16) .. +3] of the block, 4 consecutive columns of one row.
     // one substep: the MFMAs on (afc, bfc); in slot m, `hook(m)` issues what rides along
     auto substep = [&](const V8(&afc)[TM], const V8(&bfc)[TN], auto&& hook) {
         static_for<0, NSLOT>([&](auto mc) {
             constexpr int m = decltype(mc)::value;
             constexpr int i = m / TN, j = m % TN;
-            acc[i][j] = Elem<T>::mfma32(bfc[j], afc[i], acc[i][j]);
+            acc[i][j] = Elem<T>::mfma16(bfc[j], afc[i], acc[i][j]);
             hook(mc);
             __builtin_amdgcn_sched_barrier(0);
         });
@@ -392,52 +374,44 @@ __global__ __launch_bounds__(WM * WN * 64) void hgemm_main_kernel(const T* __res
             if constexpr (decltype(mc)::value < NFRAG) load_frag(st, kk, mc, afn, bfn);
         };
     };
-
-#ifndef EXP_SP
-#define EXP_SP 1
+#ifndef EXP_SPQ
+#define EXP_SPQ (NSLOT >= 2 * NCOPY ? 8 : 4 * NSLOT / NCOPY)
 #endif
-    // copy d of a tile goes out in slot d * kCopySpacing, counted from the first slot after the barrier that frees its
-    // stage: the slots of the substep behind the barrier (the "head") and, beyond those, of the next tile's first
-    // substeps (the "tail")
-    constexpr int kCopySpacingNum = EXP_SP * NSLOT, kCopySpacingDen = NCOPY;
-    static_assert((NCOPY - 1) * kCopySpacingNum / kCopySpacingDen < 3 * NSLOT, "copies must be out two substeps before the barrier");
+    // copy d of a tile goes out in slot d * kCopySpacing of the substep behind the barrier that frees its stage
+    constexpr int kCopySpacingNum = EXP_SPQ, kCopySpacingDen = 4;
+    static_assert((NCOPY - 1) * kCopySpacingNum / kCopySpacingDen < NSLOT, "copies go out within one substep");
     auto copies_of_slot = [&](int stage, auto gc) {   // issue the copies whose slot is g
         constexpr int g = decltype(gc)::value;
         static_for<0, NCOPY>([&](auto dc) {
             if constexpr (decltype(dc)::value * kCopySpacingNum / kCopySpacingDen == g) issue_copy(stage, dc);
         });
     };
+    // Ring of NSTAGE stages, tile t in stage t % NSTAGE. The prologue fills every stage; in tile kt, behind the barrier,
+    // the copies of tile kt + NSTAGE go into the stage tile kt has just left. At that barrier tile kt+1 must have
+    // landed: all but the copies of the NSTAGE-2 tiles issued after it.
+    constexpr int NSTAGE = Cfg::NSTAGE;
     const int ktiles = K / BK;
     V8 af[2][TM], bf[2][TN];
-    issue_copies(0);
-    wait_vmcnt<0>();
+    for (int t = 0; t < NSTAGE && t < ktiles; ++t) issue_copies(t);
+    if (ktiles >= NSTAGE) wait_vmcnt<NCOPY * (NSTAGE - 1)>();
+    else wait_vmcnt<0>();
     __syncthreads();
-    if (ktiles > 1) static_for<0, NSLOT>([&](auto gc) { copies_of_slot(1, gc); });   // head of tile 1
     load_frags(smem, 0, af[0], bf[0]);
 #ifdef EXP_NOREAD
     load_frags(smem, 1, af[1], bf[1]);
 #endif
 
-    auto tile = [&](int kt, auto with_copies) {
-        MI355_LDS char* st = smem + (kt & 1) * Cfg::STAGE_BYTES;
-        MI355_LDS char* stn = smem + ((kt + 1) & 1) * Cfg::STAGE_BYTES;
-        // (tail of the copies of tile kt+1 rides along)
-        substep(af[0], bf[0], [&](auto mc) {
-            constexpr int m = decltype(mc)::value;
-            if constexpr (m < NFRAG) load_frag(st, 1, mc, af[1], bf[1]);
-            copies_of_slot((kt + 1) & 1, std::integral_constant<int, NSLOT + m>{});
-        });
-        substep(af[1], bf[1], [&](auto mc) {
-            constexpr int m = decltype(mc)::value;
-            if constexpr (m < NFRAG) load_frag(st, 2, mc, af[0], bf[0]);
-            copies_of_slot((kt + 1) & 1, std::integral_constant<int, 2 * NSLOT + m>{});
-        });
-        advance_copies();
-        substep(af[0], bf[0], reads_of(st, 3, af[1], bf[1]));
-        // my copies of tile kt+1 have landed and my reads of this stage are complete; after the barrier that holds for
-        // every wave, so this stage may be refilled and the next one may be read
+    int stage = 0;   // kt % NSTAGE
+    auto tile = [&](auto with_copies) {
+        const int next = stage + 1 == NSTAGE ? 0 : stage + 1;
+        MI355_LDS char* st = smem + stage * Cfg::STAGE_BYTES;
+        MI355_LDS char* stn = smem + next * Cfg::STAGE_BYTES;
+        substep(af[0], bf[0], reads_of(st, 1, af[1], bf[1]));
+        // my copies of the next tile have landed and my reads of this stage are complete; after the barrier that holds
+        // for every wave, so this stage may be refilled and the next one may be read
 #ifndef EXP_NOVMWAIT
-        wait_vmcnt<0>();
+        if constexpr (decltype(with_copies)::value) wait_vmcnt<NCOPY * (NSTAGE - 2)>();
+        else wait_vmcnt<0>();
 #endif
 #ifndef EXP_NOBAR
         __syncthreads();
@@ -445,57 +419,59 @@ __global__ __launch_bounds__(WM * WN * 64) void hgemm_main_kernel(const T* __res
         substep(af[1], bf[1], [&](auto mc) {
             constexpr int m = decltype(mc)::value;
             if constexpr (m < NFRAG) load_frag(stn, 0, mc, af[0], bf[0]);
-            if constexpr (decltype(with_copies)::value) copies_of_slot(kt & 1, mc);   // head of tile kt+2
+            if constexpr (decltype(with_copies)::value) copies_of_slot(stage, mc);   // tile kt + NSTAGE
         });
+        if constexpr (decltype(with_copies)::value) advance_copies();
+        stage = next;
     };
-    for (int kt = 0; kt + 2 < ktiles; ++kt) tile(kt, std::true_type{});
-    if (ktiles >= 2) tile(ktiles - 2, std::false_type{});
+    int kt = 0;
+    for (; kt + NSTAGE < ktiles; ++kt) tile(std::true_type{});
+    for (; kt + 1 < ktiles; ++kt) tile(std::false_type{});
     {  // last tile: nothing left to fetch
-        MI355_LDS char* st = smem + ((ktiles - 1) & 1) * Cfg::STAGE_BYTES;
+        MI355_LDS char* st = smem + stage * Cfg::STAGE_BYTES;
         substep(af[0], bf[0], reads_of(st, 1, af[1], bf[1]));
-        substep(af[1], bf[1], reads_of(st, 2, af[0], bf[0]));
-        substep(af[0], bf[0], reads_of(st, 3, af[1], bf[1]));
-        mma(af[1], bf[1]);
+        substep(af[1], bf[1], [](auto) {});
     }
 
     // ---- epilogue ------------------------------------------------------------------------------------------------
-    // A lane holds C[m][n .. n+3] for m = l%32, n = 8p + 4*(l/32) of every 32x32 block. Storing that directly would
-    // write 8-byte pieces of 32 different rows per instruction (partial cache lines, read-modify-write in the
-    // memory system), so each wave first parks its sub-tile in its own slice of LDS (fp16, 16-byte chunks XOR-
-    // swizzled by row) and then stores whole rows: every store instruction writes complete 128-byte lines.
-    static_assert(EPI == 0 || TN == 2, "the gate/up epilogue pairs the two column blocks of a wave");
+    // A lane holds C[m][n .. n+3] for m = l%16, n = 4*(l/16) of every 16x16 block. Storing that directly would write
+    // 8-byte pieces of 16 different rows per instruction (partial cache lines, read-modify-write in the memory
+    // system), so each wave first parks its sub-tile in its own slice of LDS (fp16, 16-byte chunks XOR-swizzled by
+    // row) and then stores whole rows: every store instruction writes complete 128-byte lines.
+    // EPI == 1: the wave's columns come in groups of [32 gate | 32 up]; output block jo takes its gate from block
+    // 4 (jo / 2) + jo % 2 and its up from two blocks further.
+    static_assert(EPI == 0 || TN % 4 == 0, "the gate/up epilogue pairs column blocks 32 columns apart");
     constexpr int TNO = EPI == 1 ? TN / 2 : TN;   // column blocks a wave stores
-    constexpr int kRowHalfs = TNO * 32;           // width of the stored wave sub-tile
+    constexpr int kRowHalfs = TNO * 16;           // width of the stored wave sub-tile
     constexpr int kRowBytesC = kRowHalfs * 2;
-    constexpr int kChunksC = kRowBytesC / 16;     // 16-byte chunks per row (8 or 16)
+    constexpr int kChunksC = kRowBytesC / 16;     // 16-byte chunks per row (4, 8 or 16)
     constexpr int kRowsPerStore = 64 / kChunksC;  // rows covered by one store instruction
-    static_assert(Cfg::NWAVES * TM * 32 * kRowBytesC <= Cfg::LDS_BYTES, "epilogue staging does not fit in LDS");
+    constexpr int kSwzC = kChunksC < 8 ? kChunksC - 1 : 7;
+    static_assert(Cfg::NWAVES * TM * 16 * kRowBytesC <= Cfg::LDS_BYTES, "epilogue staging does not fit in LDS");
     __syncthreads();  // every wave has finished reading the operand stages
-    MI355_LDS char* cst = smem + wave * (TM * 32 * kRowBytesC);
+    MI355_LDS char* cst = smem + wave * (TM * 16 * kRowBytesC);
     {
-        const int r = lane & 31;
-        const int hh = lane >> 5;
+        const int r = lane & 15;
+        const int g = lane >> 4;
 #pragma unroll
         for (int i = 0; i < TM; ++i) {
-            const int row = i * 32 + r;
+            const int row = i * 16 + r;
 #pragma unroll
-            for (int j = 0; j < TNO; ++j) {
+            for (int jo = 0; jo < TNO; ++jo) {
+                V4 v;
 #pragma unroll
-                for (int p = 0; p < 4; ++p) {
-                    V4 v;
-#pragma unroll
-                    for (int q = 0; q < 4; ++q) {
-                        if constexpr (EPI == 1) {
-                            const float g = acc[i][2 * j][4 * p + q];
-                            const float sig = __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(-g * 1.4426950408889634f));
-                            v[q] = (T)(g * sig * acc[i][2 * j + 1][4 * p + q]);
-                        } else {
-                            v[q] = (T)acc[i][j][4 * p + q];
-                        }
+                for (int q = 0; q < 4; ++q) {
+                    if constexpr (EPI == 1) {
+                        const int gj = (jo / 2) * 4 + (jo % 2);
+                        const float gt = acc[i][gj][q];
+                        const float sig = __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(-gt * 1.4426950408889634f));
+                        v[q] = (T)(gt * sig * acc[i][gj + 2][q]);
+                    } else {
+                        v[q] = (T)acc[i][jo][q];
                     }
-                    const int chunk = (j * 4 + p) ^ (row & (kChunksC < 8 ? kChunksC - 1 : 7));
-                    *(MI355_LDS V4*)(cst + row * kRowBytesC + chunk * 16 + hh * 8) = v;
                 }
+                const int chunk = (2 * jo + (g >> 1)) ^ (row & kSwzC);
+                *(MI355_LDS V4*)(cst + row * kRowBytesC + chunk * 16 + (g & 1) * 8) = v;
             }
         }
     }
@@ -503,14 +479,14 @@ __global__ __launch_bounds__(WM * WN * 64) void hgemm_main_kernel(const T* __res
     {
         const int rr = lane / kChunksC;
         const int cc = lane % kChunksC;
-        T* cbase = C + (m0 + wm * TM * 32) * ldc + (EPI == 1 ? n0 / 2 : n0) + wn * TNO * 32 + cc * 8;
-        const long rows_left = M - (m0 + wm * TM * 32);   // RAGGED: rows and 8-column chunks that exist
-        const bool col_ok = (EPI == 1 ? n0 / 2 : n0) + wn * TNO * 32 + cc * 8 < (EPI == 1 ? N / 2 : N);
-        const T* rbase = R + (m0 + wm * TM * 32) * ldr + (EPI == 1 ? n0 / 2 : n0) + wn * TNO * 32 + cc * 8;
+        T* cbase = C + (m0 + wm * TM * 16) * ldc + (EPI == 1 ? n0 / 2 : n0) + wn * TNO * 16 + cc * 8;
+        const long rows_left = M - (m0 + wm * TM * 16);   // RAGGED: rows and 8-column chunks that exist
+        const bool col_ok = (EPI == 1 ? n0 / 2 : n0) + wn * TNO * 16 + cc * 8 < (EPI == 1 ? N / 2 : N);
+        const T* rbase = R + (m0 + wm * TM * 16) * ldr + (EPI == 1 ? n0 / 2 : n0) + wn * TNO * 16 + cc * 8;
 #pragma unroll
-        for (int it = 0; it < TM * 32 / kRowsPerStore; ++it) {
+        for (int it = 0; it < TM * 16 / kRowsPerStore; ++it) {
             const int row = it * kRowsPerStore + rr;
-            V8 v = *(MI355_LDS const V8*)(cst + row * kRowBytesC + ((cc ^ (row & (kChunksC < 8 ? kChunksC - 1 : 7))) << 4));
+            V8 v = *(MI355_LDS const V8*)(cst + row * kRowBytesC + ((cc ^ (row & kSwzC)) << 4));
             if (!RAGGED || (row < rows_left && col_ok)) {
                 if (R != nullptr) {
                     const V8 r = *(const V8*)(rbase + (long)row * ldr);
