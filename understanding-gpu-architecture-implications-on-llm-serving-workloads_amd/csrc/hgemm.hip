@@ -7,10 +7,12 @@
 // [N,K]) for 13..15.
 //
 // Main kernel: one workgroup of 8 waves computes a 256x256 tile of C, K is walked in steps of 64.
-//   * global -> LDS staging uses 16-byte direct-to-LDS copies (no VGPR bounce), double buffered; every
-//     wave-instruction writes 1 KiB of contiguous LDS, the XOR swizzle is applied on the global-address side.
+//   * global -> LDS staging uses 16-byte direct-to-LDS copies (no VGPR bounce) into a ring of stages (two 64 KiB
+//     stages for the 256x256 tile, three 32 KiB stages for the 128x128 tile); every wave-instruction writes 1 KiB
+//     of contiguous LDS, the XOR swizzle is applied on the global-address side.
 //     The copies are buffer loads (scalar tile base + one 32-bit lane offset): a global load with 64-bit lane
-//     addresses takes about twice as much issue time away from the MFMAs it runs beside.
+//     addresses takes about twice as much issue time away from the MFMAs it runs beside, and several times as
+//     much when such loads are issued back to back.
 //   * an operand whose K index is contiguous in memory is read from LDS with ds_read_b128; an operand whose
 //     M/N index is contiguous (B in the NN case) is read with the transposing ds_read_b64_tr_b16, so no
 //     transpose pass over B is ever made.
@@ -73,6 +75,7 @@ struct MNContigTile {
     static constexpr int kInsts = BK / kRowsPerPass;
     static constexpr int kBytes = BK * kRowBytes;
     static_assert(COLS == 256 || COLS == 128, "swizzle below needs at least 16 chunks per row");
+    static_assert(kRowsPerPass % 16 == 0, "copy i of a lane is 16 rows or a multiple further down: same swizzle for all i");
     static_assert(BK % kRowsPerPass == 0, "tile depth must be a multiple of one pass of the workgroup");
 
     // A transposing read touches, per 16 lanes, 4 k-rows x 32 bytes (two neighbouring chunks); lanes 0..31 of a
@@ -304,9 +307,6 @@ void hgemm_main_kernel(const T* __restrict__ A, const T* __restrict__ B,
     // fragment f of substep kk, f in the order of first use: A0, B0 .. B(TN-1), A1 .. A(TM-1)
     auto load_frag = [&](MI355_LDS char* st, int kk, auto fc, V8(&afn)[TM], V8(&bfn)[TN]) {
         constexpr int f = decltype(fc)::value;
-#ifdef EXP_NOREAD
-        return;
-#endif
         if constexpr (f == 0 || f > TN) {
             constexpr int i = f == 0 ? 0 : f - TN;
             if constexpr (A_KC) {
@@ -332,9 +332,6 @@ void hgemm_main_kernel(const T* __restrict__ A, const T* __restrict__ B,
     };
     auto issue_copy = [&](int stage, auto dc) {
         constexpr int d = decltype(dc)::value;
-#ifdef EXP_NOCOPY
-        return;
-#endif
         MI355_LDS char* sa = smem + stage * Cfg::STAGE_BYTES;
         if constexpr (d < Cfg::A_INSTS) {
             MI355_LDS char* dst = sa + (d * Cfg::NWAVES + wave) * 1024;
@@ -374,11 +371,10 @@ void hgemm_main_kernel(const T* __restrict__ A, const T* __restrict__ B,
             if constexpr (decltype(mc)::value < NFRAG) load_frag(st, kk, mc, afn, bfn);
         };
     };
-#ifndef EXP_SPQ
-#define EXP_SPQ (NSLOT >= 2 * NCOPY ? 8 : 4 * NSLOT / NCOPY)
-#endif
-    // copy d of a tile goes out in slot d * kCopySpacing of the substep behind the barrier that frees its stage
-    constexpr int kCopySpacingNum = EXP_SPQ, kCopySpacingDen = 4;
+    // copy d of a tile goes out in slot d * kCopySpacing of the substep behind the barrier that frees its stage: every
+    // second slot where there are that many (buffer loads are cheap to issue in a row, and the earlier a copy leaves the
+    // more time it has to land), evenly over the substep otherwise
+    constexpr int kCopySpacingNum = NSLOT >= 2 * NCOPY ? 8 : 4 * NSLOT / NCOPY, kCopySpacingDen = 4;
     static_assert((NCOPY - 1) * kCopySpacingNum / kCopySpacingDen < NSLOT, "copies go out within one substep");
     auto copies_of_slot = [&](int stage, auto gc) {   // issue the copies whose slot is g
         constexpr int g = decltype(gc)::value;
@@ -397,9 +393,6 @@ void hgemm_main_kernel(const T* __restrict__ A, const T* __restrict__ B,
     else wait_vmcnt<0>();
     __syncthreads();
     load_frags(smem, 0, af[0], bf[0]);
-#ifdef EXP_NOREAD
-    load_frags(smem, 1, af[1], bf[1]);
-#endif
 
     int stage = 0;   // kt % NSTAGE
     auto tile = [&](auto with_copies) {
@@ -409,13 +402,9 @@ void hgemm_main_kernel(const T* __restrict__ A, const T* __restrict__ B,
         substep(af[0], bf[0], reads_of(st, 1, af[1], bf[1]));
         // my copies of the next tile have landed and my reads of this stage are complete; after the barrier that holds
         // for every wave, so this stage may be refilled and the next one may be read
-#ifndef EXP_NOVMWAIT
         if constexpr (decltype(with_copies)::value) wait_vmcnt<NCOPY * (NSTAGE - 2)>();
         else wait_vmcnt<0>();
-#endif
-#ifndef EXP_NOBAR
         __syncthreads();
-#endif
         substep(af[1], bf[1], [&](auto mc) {
             constexpr int m = decltype(mc)::value;
             if constexpr (m < NFRAG) load_frag(stn, 0, mc, af[0], bf[0]);
@@ -862,11 +851,7 @@ static hipError_t launch_layout(const T* A, const T* B, T* C, const T* R, int M,
     if (g_gemm_variant == 1 && fits256) choice = 1;
     if (g_gemm_variant == 2 && fits128) choice = 2;
     switch (choice) {
-#ifdef EXP_W4
-        case 1: return launch_main<T, A_KC, B_KC, 256, 256, 2, 2>(A, B, C, R, M, N, K, lda, ldb, ldc, ldr, stream);
-#else
         case 1: return launch_main<T, A_KC, B_KC, 256, 256, 2, 4>(A, B, C, R, M, N, K, lda, ldb, ldc, ldr, stream);
-#endif
         case 2: return launch_main<T, A_KC, B_KC, 128, 128, 2, 2>(A, B, C, R, M, N, K, lda, ldb, ldc, ldr, stream);
         default: break;
     }
