@@ -44,7 +44,13 @@ struct KContigTile {
     static_assert(ROWS % kRowsPerPass == 0, "tile rows must be a multiple of one pass of the workgroup");
     static_assert(BK == 64, "swizzle below is written for 128-byte rows");
 
-    __device__ static __forceinline__ int swz(int row) { return (row & 7) ^ ((row >> 3) & 1); }
+    // A fragment read (ds_read_b128) has lane l at row l % 16, chunk c0 + l / 16. Rows of equal parity share the same
+    // half of the 256-byte bank window, so their chunk positions must differ: over 16 consecutive lanes (16 rows, one
+    // chunk), and over the lanes l and l + 32 that the hardware serves together (8 rows, chunks c and c + 2, i.e. c ^ 2).
+    // Bits 0 and 2 of the XOR value tell the 4 rows of one parity inside an 8-row group apart, bit 1 the two groups.
+    __device__ static __forceinline__ int swz(int row) {
+        return ((row >> 1) & 1) | (((row >> 2) & 1) << 2) | (((row >> 3) & 1) << 1);
+    }
 
     // element offset (in halfs, relative to the tile origin in global memory) of this lane's first copy
     __device__ static __forceinline__ long first_copy_offset(int wave, int lane, long ld) {
