@@ -151,6 +151,24 @@ def test_strided_leading_dimensions(lib, gpu):
     assert bool((cbig[:, N:] == 0).all())  # nothing written outside the N columns
 
 
+@pytest.mark.parametrize("layout", ["NN", "NT"])
+def test_leading_dimension_beyond_the_tiled_kernels_reach(lib, gpu, layout):
+    """The tiled kernels address a tile with 32-bit byte offsets and take leading dimensions below 2^22 elements; a wider
+    operand must take the bounds-checked kernel and still be right (A is a 128 x 64 corner of a 128 x 2^22 buffer)."""
+    M, N, K, lda = 128, 64, 64, 1 << 22
+    abig = torch.zeros((M, lda), dtype=torch.float16, device=gpu)
+    a = so.randn_fp16((M, K), 3)
+    abig[:, :K] = a.to(gpu)
+    b = so.randn_fp16((N, K) if layout == "NT" else (K, N), 4)
+    bg = b.to(gpu)
+    c = torch.zeros((M, N), dtype=torch.float16, device=gpu)
+    lib.hgemm_raw(abig.data_ptr(), bg.data_ptr(), c.data_ptr(), M, N, K, lda, bg.stride(0), N, lib.LAYOUTS[layout],
+                  torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    ok, st = so.gemm_tolerance_ok(c.cpu(), so.gemm_ref(a, b, layout), K)
+    assert ok, st
+
+
 # ---- size-independent properties at the full benchmark size -------------------------------------------------------
 def test_full_size_linearity_and_column_selection(lib, gpu):
     n = 8192
