@@ -129,6 +129,15 @@ def test_decode_shaped_small_m(lib, gpu, layout, M, N, K):
     check(lib, gpu, a, b, layout, K)
 
 
+@pytest.mark.parametrize("layout", ["NN", "NT", "TN"])
+@pytest.mark.parametrize("M,N,K", [(24, 14336, 512), (64, 14336, 256), (32, 28672, 128), (40, 4096, 1024), (17, 12800, 192)])
+def test_17_to_64_rows_small_m_or_tiles(lib, gpu, layout, M, N, K):
+    """Between 17 and 64 rows the dispatcher weighs the small-M kernels (B streamed once per 16 rows) against the 128x128
+    tiles (wide products); both sides of that choice, all layouts (TN with M a multiple of 8 has a small-M kernel too)."""
+    a, b = operands(M, N, K, layout, seed=9, b_std=0.05)
+    check(lib, gpu, a, b, layout, K)
+
+
 def test_reference_seeded_case_from_golden_fixture(lib, gpu):
     z = np.load(os.path.join(GOLDEN, "gemm_seed0_256.npz"))
     a, b, rows = torch.from_numpy(z["a"]), torch.from_numpy(z["b"]), z["rows"]

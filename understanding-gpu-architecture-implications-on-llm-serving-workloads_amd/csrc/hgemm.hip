@@ -543,20 +543,22 @@ __global__ __launch_bounds__(256) void hgemm_edge_kernel(const T* __restrict__ A
 }
 
 // ---------------------------------------------------------------------------------------------------------
-// Small-M kernel (decode-shaped GEMM, M <= 16 rows per workgroup row), layout NN. HBM-bound: B is streamed once.
+// Small-M kernel (decode-shaped GEMM, M <= 16 rows per workgroup row), layouts NN and TN. HBM-bound: B is streamed once.
 //   * a workgroup owns 64 columns of C; its 8 waves split K between them (in-workgroup split-K, reduced
 //     through LDS at the end, so no global workspace and no atomics);
 //   * every wave runs its own copy pipeline, without workgroup barriers: per 32-deep k-step it copies a
 //     32x64 slab of B (4 KiB) and a 16x32 slab of A (1 KiB) global -> LDS with 16-byte direct-to-LDS copies,
 //     keeps kSmallMStages-1 steps in flight, and waits for the oldest with s_waitcnt vmcnt;
-//   * B fragments are read with the transposing LDS read, the product is MFMA 16x16x32.
+//   * B fragments are read with the transposing LDS read, the product is MFMA 16x16x32;
+//   * layout TN (A stored [K,M], A_KC = false): the A slab of a k-step is 32 rows (k) x 16 m, copied as it lies and read
+//     with the transposing read like B; M must be a multiple of 8.
 // ---------------------------------------------------------------------------------------------------------
 constexpr int kSmallMStages = 3;
 constexpr int kSmallMStageBytes = 5 * 1024;  // 4 KiB of B + 1 KiB of A
 constexpr int kSmallMWaveBytes = kSmallMStages * kSmallMStageBytes;
 constexpr int kSmallMLdsBytes = 8 * kSmallMWaveBytes;
 
-template <typename T>
+template <typename T, bool A_KC>
 __global__ __launch_bounds__(512) void hgemm_smallm_nn_kernel(const T* __restrict__ A, const T* __restrict__ B,
                                                               T* C, const T* R, int M, int N, int K, long lda,
                                                               long ldb, long ldc, long ldr, int n_tiles) {
@@ -590,9 +592,15 @@ __global__ __launch_bounds__(512) void hgemm_smallm_nn_kernel(const T* __restric
     const int b_col = min(n0 / 8 + b_chunk, n_chunk_max) * 8;     // clamp: columns past N are never stored
     const T* b_src = B + (long)(s_begin * 32 + b_row) * ldb + b_col;
     // A slab: 16 rows (m) x 64 bytes; row lane/4, chunk position lane%4, chunk c of row r at c ^ ((r>>1)&3)
+    // A stored [K,M]: slab of 32 rows (k) x 32 bytes; LDS row slot lane/2 holds k row = slot with bits 2 and 3 swapped,
+    // which puts the 8 rows that lanes 0..31 of a transposing read touch (k 0..3 and 8..11, + 4 for the second read)
+    // into 8 consecutive slots = 256 bytes = distinct banks. Chunks past M fold back onto the last 8 rows of A.
     const int a_row = lane >> 2;
     const int a_chunk = (lane & 3) ^ ((a_row >> 1) & 3);
-    const T* a_src = A + (long)min(m0 + a_row, M - 1) * lda + (long)s_begin * 32 + a_chunk * 8;
+    const int at_slot = lane >> 1;
+    const int at_k = (at_slot & ~12) | ((at_slot & 4) << 1) | ((at_slot & 8) >> 1);
+    const T* a_src = A_KC ? A + (long)min(m0 + a_row, M - 1) * lda + (long)s_begin * 32 + a_chunk * 8
+                          : A + (long)(s_begin * 32 + at_k) * lda + min(m0 + 8 * (lane & 1), M - 8);
 
     auto issue_stage = [&](int slot) {
         MI355_LDS char* st = wbase + slot * kSmallMStageBytes;
@@ -600,12 +608,17 @@ __global__ __launch_bounds__(512) void hgemm_smallm_nn_kernel(const T* __restric
         for (int i = 0; i < 4; ++i) copy16_global_to_lds(b_src + (long)(8 * i) * ldb, st + i * 1024);
         copy16_global_to_lds(a_src, st + 4096);
         b_src += 32 * ldb;
-        a_src += 32;
+        a_src += A_KC ? 32 : 32 * lda;
     };
 
     // ---- fragment read offsets inside a stage ---------------------------------------------------------------
     // A fragment: lane holds A[m = lane%16][k = 8*(lane/16) .. +7]
-    const int a_off = 4096 + (lane & 15) * 64 + (((lane >> 4) ^ (((lane & 15) >> 1) & 3)) << 4);
+    // (A stored [K,M]: transposing read of k rows 8*(lane/16) + 4t + (lane%16)/4, m = 4*(lane%4) .. +3; the second read
+    //  (t = 1, k + 4) lies 8 slots = 256 bytes further)
+    const int at_read_k = 8 * (lane >> 4) + ((lane & 15) >> 2);
+    const int at_read_slot = (at_read_k & ~12) | ((at_read_k & 4) << 1) | ((at_read_k & 8) >> 1);
+    const int a_off = A_KC ? 4096 + (lane & 15) * 64 + (((lane >> 4) ^ (((lane & 15) >> 1) & 3)) << 4)
+                           : 4096 + at_read_slot * 32 + (lane & 3) * 8;
     // B fragment of column block j: rows 8*(lane/16) + 4t + (lane%16)/4, columns 16j + 4*(lane%4) .. +3
     const int bt_row = 8 * (lane >> 4) + ((lane & 15) >> 2);
     const int bt_swz = 2 * (bt_row & 3);
@@ -640,7 +653,9 @@ __global__ __launch_bounds__(512) void hgemm_smallm_nn_kernel(const T* __restric
         }
         MI355_LDS char* st = wbase + slot * kSmallMStageBytes;
         slot = (slot + 1 == kSmallMStages) ? 0 : slot + 1;
-        V8 af = Elem<T>::frag(lds_read_b128(st + a_off));
+        V8 af;
+        if constexpr (A_KC) af = Elem<T>::frag(lds_read_b128(st + a_off));
+        else af = Elem<T>::frag(concat(lds_read_tr16_b64(st + a_off), lds_read_tr16_b64(st + a_off + 256)));
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             half4 lo = lds_read_tr16_b64(st + b_off[j]);
@@ -682,14 +697,14 @@ __global__ __launch_bounds__(512) void hgemm_smallm_nn_kernel(const T* __restric
     }
 }
 
-template <typename T>
+template <typename T, bool A_KC>
 static hipError_t launch_smallm_nn(const T* A, const T* B, T* C, const T* R, int M, int N, int K, long lda, long ldb,
                                    long ldc, long ldr, hipStream_t stream) {
     static DynamicLdsOnce lds_once;
-    if (hipError_t e = lds_once.ensure(reinterpret_cast<const void*>(hgemm_smallm_nn_kernel<T>), kSmallMLdsBytes); e != hipSuccess) return e;
+    if (hipError_t e = lds_once.ensure(reinterpret_cast<const void*>(hgemm_smallm_nn_kernel<T, A_KC>), kSmallMLdsBytes); e != hipSuccess) return e;
     const int n_tiles = (N + 63) / 64;
     dim3 grid(n_tiles, (M + 15) / 16);
-    hgemm_smallm_nn_kernel<T><<<grid, dim3(512), kSmallMLdsBytes, stream>>>(A, B, C, R, M, N, K, lda, ldb, ldc, ldr, n_tiles);
+    hgemm_smallm_nn_kernel<T, A_KC><<<grid, dim3(512), kSmallMLdsBytes, stream>>>(A, B, C, R, M, N, K, lda, ldb, ldc, ldr, n_tiles);
     return hipGetLastError();
 }
 
@@ -832,6 +847,17 @@ static hipError_t launch_main(const T* A, const T* B, T* C, const T* R, int M, i
     return hipGetLastError();
 }
 
+// 17..64 rows: the small-M kernels stream B once per 16 rows (the L2 catches part of the repeats), the 128x128 tiles
+// stream it once but run K / 64 dependent tile steps of ~0.4 us on at most one workgroup per 128 columns. Cost models
+// from measurements of both at Llama projection shapes; true = the tiles are expected to be faster.
+static bool few_rows_prefer_tiles(int M, int N, int K) {
+    if (M <= 16) return false;
+    const double small_us = (double)((M + 15) / 16) * (double)N * (double)K * 2.0 / 6.5e6;
+    const long tiles = (long)((M + 127) / 128) * ((N + 127) / 128);
+    const double tiles_us = (double)(K / 64) * 0.42 * (double)((tiles + 255) / 256);
+    return tiles_us < small_us;
+}
+
 template <typename T, bool A_KC, bool B_KC>
 static hipError_t launch_layout(const T* A, const T* B, T* C, const T* R, int M, int N, int K, long lda, long ldb,
                                 long ldc, long ldr, hipStream_t stream) {
@@ -842,12 +868,14 @@ static hipError_t launch_layout(const T* A, const T* B, T* C, const T* R, int M,
     const bool k_ok = aligned && K % 64 == 0 && K >= 64 && lda < (1L << 22) && ldb < (1L << 22);
     const bool fits256 = k_ok && M % 256 == 0 && N % 256 == 0;
     const bool fits128 = k_ok && M % 128 == 0 && N % 128 == 0;
-    if constexpr (A_KC && !B_KC) {
-        if (aligned && M <= 64 && K % 32 == 0 && K >= 32 && N % 8 == 0 && ldc % 2 == 0)
-            return launch_smallm_nn<T>(A, B, C, R, M, N, K, lda, ldb, ldc, ldr, stream);
+    const bool ragged_ok = k_ok && N % 8 == 0 && N >= 8 && (A_KC || (M % 8 == 0 && M >= 8));
+    const bool small_m = M <= 64 && !(ragged_ok && few_rows_prefer_tiles(M, N, K));
+    if constexpr (!B_KC) {   // NN, and TN with M a multiple of 8 (its A slab is copied in 8-row chunks)
+        if (aligned && small_m && K % 32 == 0 && K >= 32 && N % 8 == 0 && ldc % 2 == 0 && (A_KC || M % 8 == 0))
+            return launch_smallm_nn<T, A_KC>(A, B, C, R, M, N, K, lda, ldb, ldc, ldr, stream);
     }
     if constexpr (A_KC && B_KC) {
-        if (aligned && M <= 64 && K % 64 == 0 && K >= 64) return launch_smallm_nt<T>(A, B, C, R, M, N, K, lda, ldb, ldc, ldr, stream);
+        if (aligned && small_m && K % 64 == 0 && K >= 64) return launch_smallm_nt<T>(A, B, C, R, M, N, K, lda, ldb, ldc, ldr, stream);
     }
     // 256x256 tiles when they fill the machine (>= ~3/4 of the 256 CUs), 128x128 tiles for smaller problems
     const long tiles256 = fits256 ? (long)(M / 256) * (N / 256) : 0;
@@ -862,7 +890,7 @@ static hipError_t launch_layout(const T* A, const T* B, T* C, const T* R, int M,
         default: break;
     }
     // ragged M / N on the same tiles: N (and M for layout TN) a multiple of 8, so 16-byte chunks never straddle the end
-    if (k_ok && N % 8 == 0 && N >= 8 && (A_KC || (M % 8 == 0 && M >= 8))) {
+    if (ragged_ok) {
         const long t256 = (long)((M + 255) / 256) * ((N + 255) / 256);
         if ((t256 >= 192 && g_gemm_variant != 2) || g_gemm_variant == 1)
             return launch_main<T, A_KC, B_KC, 256, 256, 2, 4, 0, true>(A, B, C, R, M, N, K, lda, ldb, ldc, ldr, stream);
@@ -881,8 +909,8 @@ static hipError_t launch_silu_mul(const T* A, const T* B, T* C, int M, int N, in
     const bool aligned = (reinterpret_cast<uintptr_t>(A) % 16 == 0) && (reinterpret_cast<uintptr_t>(B) % 16 == 0) &&
                          (reinterpret_cast<uintptr_t>(C) % 16 == 0) && (lda % 8 == 0) && (ldb % 8 == 0) && (ldc % 8 == 0);
     // N = columns of op(B); gate/up pairs are 64 columns wide. Few rows are better served by the small-M product.
-    if (!aligned || K % 64 != 0 || K < 64 || N % 64 != 0 || M <= 64 || lda >= (1L << 22) || ldb >= (1L << 22))
-        return hipErrorNotSupported;
+    if (!aligned || K % 64 != 0 || K < 64 || N % 64 != 0 || lda >= (1L << 22) || ldb >= (1L << 22)) return hipErrorNotSupported;
+    if (M <= 64 && !few_rows_prefer_tiles(M, N, K)) return hipErrorNotSupported;   // the small-M product + silu_mul is faster
     const bool fits128 = M % 128 == 0 && N % 128 == 0;
     const bool fits256 = M % 256 == 0 && N % 256 == 0;
     const long t256 = (long)((M + 255) / 256) * ((N + 255) / 256);
