@@ -8,7 +8,7 @@
 //
 // Main kernel: one workgroup of 8 waves computes a 256x256 tile of C, K is walked in steps of 64.
 //   * global -> LDS staging uses 16-byte direct-to-LDS copies (no VGPR bounce) into a ring of stages (two 64 KiB
-//     stages for the 256x256 tile, three 32 KiB stages for the 128x128 tile); every wave-instruction writes 1 KiB
+//     stages for the 256x256 tile, three stages for the 128x128 and 128x64 tiles); every wave-instruction writes 1 KiB
 //     of contiguous LDS, the XOR swizzle is applied on the global-address side.
 //     The copies are buffer loads (scalar tile base + one 32-bit lane offset): a global load with 64-bit lane
 //     addresses takes about twice as much issue time away from the MFMAs it runs beside, and several times as
@@ -850,12 +850,16 @@ static hipError_t launch_main(const T* A, const T* B, T* C, const T* R, int M, i
 // 17..64 rows: the small-M kernels stream B once per 16 rows (the L2 catches part of the repeats), the 128x128 tiles
 // stream it once but run K / 64 dependent tile steps of ~0.4 us on at most one workgroup per 128 columns. Cost models
 // from measurements of both at Llama projection shapes; true = the tiles are expected to be faster.
-static bool few_rows_prefer_tiles(int M, int N, int K) {
+static bool few_rows_prefer_tiles(int M, int N, int K, bool nt) {
     if (M <= 16) return false;
     const double small_us = (double)((M + 15) / 16) * (double)N * (double)K * 2.0 / 6.5e6;
-    const long tiles = (long)((M + 127) / 128) * ((N + 127) / 128);
-    const double tiles_us = (double)(K / 64) * 0.42 * (double)((tiles + 255) / 256);
-    return tiles_us < small_us;
+    long tiles = (long)((M + 127) / 128) * ((N + 127) / 128);
+    double step_us = 0.42;
+    if (nt && tiles < 192) {   // layout NT runs 128x64 tiles then
+        tiles = (long)((M + 127) / 128) * ((N + 63) / 64);
+        step_us = 0.34;
+    }
+    return (double)(K / 64) * step_us * (double)((tiles + 255) / 256) < small_us;
 }
 
 template <typename T, bool A_KC, bool B_KC>
@@ -869,13 +873,33 @@ static hipError_t launch_layout(const T* A, const T* B, T* C, const T* R, int M,
     const bool fits256 = k_ok && M % 256 == 0 && N % 256 == 0;
     const bool fits128 = k_ok && M % 128 == 0 && N % 128 == 0;
     const bool ragged_ok = k_ok && N % 8 == 0 && N >= 8 && (A_KC || (M % 8 == 0 && M >= 8));
-    const bool small_m = M <= 64 && !(ragged_ok && few_rows_prefer_tiles(M, N, K));
+    const bool small_m = M <= 64 && !(ragged_ok && few_rows_prefer_tiles(M, N, K, A_KC && B_KC));
     if constexpr (!B_KC) {   // NN, and TN with M a multiple of 8 (its A slab is copied in 8-row chunks)
         if (aligned && small_m && K % 32 == 0 && K >= 32 && N % 8 == 0 && ldc % 2 == 0 && (A_KC || M % 8 == 0))
             return launch_smallm_nn<T, A_KC>(A, B, C, R, M, N, K, lda, ldb, ldc, ldr, stream);
     }
     if constexpr (A_KC && B_KC) {
         if (aligned && small_m && K % 64 == 0 && K >= 64) return launch_smallm_nt<T>(A, B, C, R, M, N, K, lda, ldb, ldc, ldr, stream);
+    }
+    // Fewer than ~3/4 x 256 tiles of 128x128 cannot occupy the CUs: halve the tile so that twice as many workgroups pull
+    // on the memory system (64 x 14336 x 4096 NT: 22 us instead of 27.5; 1024^3: 7 us instead of 9.5). Layout NT halves
+    // the tile along N (128x64).
+    const bool few_tiles = ragged_ok && (long)((M + 127) / 128) * ((N + 127) / 128) < 192 && g_gemm_variant == 0;
+    if constexpr (A_KC && B_KC) {
+        if (few_tiles) {
+            if (M % 128 == 0 && N % 64 == 0)
+                return launch_main<T, A_KC, B_KC, 128, 64, 2, 2>(A, B, C, R, M, N, K, lda, ldb, ldc, ldr, stream);
+            return launch_main<T, A_KC, B_KC, 128, 64, 2, 2, 0, true>(A, B, C, R, M, N, K, lda, ldb, ldc, ldr, stream);
+        }
+    }
+    // layout NN: the N-contiguous B tile cannot be narrower than 128 columns, so the tile is halved along M (64x128);
+    // that helps products with several row tiles (1024^3), not the few-row ones
+    if constexpr (A_KC && !B_KC) {
+        if (few_tiles && M > 64) {
+            if (M % 64 == 0 && N % 128 == 0)
+                return launch_main<T, A_KC, B_KC, 64, 128, 1, 4>(A, B, C, R, M, N, K, lda, ldb, ldc, ldr, stream);
+            return launch_main<T, A_KC, B_KC, 64, 128, 1, 4, 0, true>(A, B, C, R, M, N, K, lda, ldb, ldc, ldr, stream);
+        }
     }
     // 256x256 tiles when they fill the machine (>= ~3/4 of the 256 CUs), 128x128 tiles for smaller problems
     const long tiles256 = fits256 ? (long)(M / 256) * (N / 256) : 0;
@@ -910,7 +934,7 @@ static hipError_t launch_silu_mul(const T* A, const T* B, T* C, int M, int N, in
                          (reinterpret_cast<uintptr_t>(C) % 16 == 0) && (lda % 8 == 0) && (ldb % 8 == 0) && (ldc % 8 == 0);
     // N = columns of op(B); gate/up pairs are 64 columns wide. Few rows are better served by the small-M product.
     if (!aligned || K % 64 != 0 || K < 64 || N % 64 != 0 || lda >= (1L << 22) || ldb >= (1L << 22)) return hipErrorNotSupported;
-    if (M <= 64 && !few_rows_prefer_tiles(M, N, K)) return hipErrorNotSupported;   // the small-M product + silu_mul is faster
+    if (M <= 64 && !few_rows_prefer_tiles(M, N, K, false)) return hipErrorNotSupported;   // the small-M product + silu_mul is faster
     const bool fits128 = M % 128 == 0 && N % 128 == 0;
     const bool fits256 = M % 256 == 0 && N % 256 == 0;
     const long t256 = (long)((M + 255) / 256) * ((N + 255) / 256);
