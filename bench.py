@@ -235,6 +235,23 @@ def main():
                                                   14336, lib.GEMM_NT, stream), 20, 3)
         byd = 2.0 * (16 * 4096 + 4096 * 14336 + 16 * 14336)
         other["gemm_decode_nt_16x14336x4096"] = {"ms": msd, "gbs": byd / msd / 1e6, "pct_of_hbm_peak": 100 * byd / msd / 1e6 / PEAK_HBM_GBS}
+        # the same projection at batch 64 (128x64 tiles instead of the small-M kernel), and bf16 twins of the two headline kernels
+        x64 = so.randn_fp16((64, 4096), 3).to(dev)
+        o64 = torch.empty((64, 14336), dtype=torch.float16, device=dev)
+        ms64 = time_launches(lambda: lib.hgemm_raw(x64.data_ptr(), wd_nt.data_ptr(), o64.data_ptr(), 64, 14336, 4096, 4096, 4096,
+                                                   14336, lib.GEMM_NT, stream), 20, 3)
+        by64 = 2.0 * (64 * 4096 + 4096 * 14336 + 64 * 14336)
+        other["gemm_decode_nt_64x14336x4096"] = {"ms": ms64, "gbs": by64 / ms64 / 1e6, "pct_of_hbm_peak": 100 * by64 / ms64 / 1e6 / PEAK_HBM_GBS}
+        del x64, o64
+        ab, bb = a.to(torch.bfloat16), b.to(torch.bfloat16)
+        cb = torch.empty((M, N), dtype=torch.bfloat16, device=dev)
+        msb = time_launches(lambda: lib.hgemm(ab, bb, "NN", out=cb), 10, 2)
+        qb_, kb_, vb_ = q.to(torch.bfloat16), k.to(torch.bfloat16), v.to(torch.bfloat16)
+        ob_ = torch.empty_like(qb_)
+        msfb = time_launches(lambda: lib.fmha_fwd(qb_, kb_, vb_, causal=True, return_lse=False, out=ob_), 10, 2)
+        other["bf16"] = {"gemm_8192_nn": {"ms": msb, "tflops": gemm_flops / msb / 1e9},
+                         "fmha_f4_causal_gqa": {"ms": msfb, "tflops": fmha_flops / msfb / 1e9}}
+        del ab, bb, cb, qb_, kb_, vb_, ob_
         for bd, skd in ((1, 8192), (8, 8192), (1, 32768)):
             qd, kd, vd = (t.to(dev) for t in so.fmha_inputs(bd, 32, 8, 1, skd, seed=7))
             o_d = torch.empty_like(qd)
