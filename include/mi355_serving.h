@@ -9,25 +9,31 @@
  *   - every pointer is a DEVICE pointer owned by the caller; none is retained. The only memory the library ever
  *     allocates is a workspace for the partial results of the split-KV attention path (taken when
  *     Hq/Hkv * Sq <= 32 and kv_valid_len >= 512, i.e. generation steps): one buffer per (device, stream), obtained
- *     with hipMallocAsync on that stream at first use (>= 4 MiB, regrown when a call needs more, kept until the
- *     process ends), so steady-state calls allocate nothing and calls on different streams never share it;
+ *     with hipMalloc at first use (>= 4 MiB; when a later call needs more, a larger buffer is allocated and the old
+ *     one is kept, because a HIP graph captured earlier may still hold its address; nothing is freed before the
+ *     process ends), so steady-state calls allocate nothing and calls on different streams never share a buffer.
+ *     A call that would have to allocate while its stream is being captured fails (hipErrorStreamCaptureUnsupported)
+ *     and launches nothing: run the step once on that stream before capturing it, and replay the graph on the stream it
+ *     was captured on (or use mi355_fmha_fwd_ws with memory of your own);
  *   - `stream` is a hipStream_t passed as void* (NULL = the null stream); calls are asynchronous;
  *   - fp16 data is IEEE binary16 (`_Float16` / `__half` / torch.float16);
  *   - return value 0 = launched; non-zero = a hipError_t value or MI355_ERR_* below, nothing was launched.
  *     mi355_last_error() returns a thread-local description of the last failure.
  *   - calls are re-entrant and thread-safe; the only mutable global state is one-time kernel attribute
- *     initialisation and the mutex-protected table of those workspaces.
+ *     initialisation (atomic flags) and the mutex-protected table of those workspaces. Which kernel runs depends on
+ *     the arguments alone.
  */
 #ifndef MI355_SERVING_H
 #define MI355_SERVING_H
 
+#include <stddef.h>
 #include <stdint.h>
 
 #ifdef __cplusplus
 extern "C" {
 #endif
 
-#define MI355_SERVING_VERSION 100
+#define MI355_SERVING_VERSION 200
 
 /* argument errors (distinct from hipError_t values, which are < 10000) */
 #define MI355_ERR_BAD_ARGUMENT 10001
@@ -188,22 +194,26 @@ int mi355_rope_bf16(const void* x, void* out, int B, int S, int heads, int copy_
 int mi355_silu_mul_bf16(const void* gate_up, void* out, int64_t rows, int inter, int interleave, int64_t ld_in, int64_t ld_out,
                         void* stream);
 
+/*
+ * The attention forward with a workspace owned by the caller, for callers that manage all device memory themselves
+ * (HIP graph capture, arena allocators). mi355_fmha_fwd_workspace_bytes returns how many bytes a call with these sizes
+ * needs: 0 for every shape outside the split-KV path (then `workspace` may be NULL), otherwise the size of its partial
+ * results (at most a few MiB for B * Hkv <= 768). mi355_fmha_fwd_ws is mi355_fmha_fwd_strided (strides == NULL:
+ * contiguous [B, H, S, D] operands) for dtype MI355_DTYPE_FP16 or MI355_DTYPE_BF16 that keeps those partial results in
+ * `workspace` (16-byte aligned, at least that many bytes, contents irrelevant before and after the call) and never
+ * allocates. Calls that share a workspace must be ordered on one stream. No counterpart in the reference, whose
+ * generation step runs the prefill kernel (kernels/fmha/pkg/fmha_unified/ops.py:19-25).
+ */
+size_t mi355_fmha_fwd_workspace_bytes(int B, int Hq, int Hkv, int Sq, int Sk, int kv_valid_len);
+int mi355_fmha_fwd_ws(const void* Q, const void* K, const void* V, void* O, float* LSE, int B, int Hq, int Hkv, int Sq,
+                      int Sk, int D, float scale, int causal, int kv_valid_len, const int64_t* strides, int dtype,
+                      void* workspace, size_t workspace_bytes, void* stream);
+
 /* Thread-local text for the last non-zero return of this thread ("" if none). */
 const char* mi355_last_error(void);
 
 /* MI355_SERVING_VERSION of the loaded library. */
 int mi355_serving_version(void);
-
-/*
- * Diagnostics (no counterpart in the reference): pin the kernel variant instead of letting the dispatcher choose
- * by shape, so tests and tuning runs can exercise every variant on every shape. Process-wide; 0 restores the
- * heuristic. A variant that does not fit the shape (e.g. tile sizes that do not divide it) is ignored.
- *   gemm: 1 = 256x256 tiles, 2 = 128x128 tiles
- *   fmha: 1 = 4 waves x 32 queries, 2 = 8 waves x 32 queries, 3 = 8 waves x 32 queries ping-pong (1..3 also
- *         keep generation-step shapes off the split-KV path)
- */
-void mi355_debug_set_gemm_variant(int variant);
-void mi355_debug_set_fmha_variant(int variant);
 
 #ifdef __cplusplus
 }

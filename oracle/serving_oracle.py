@@ -123,10 +123,13 @@ def visible_mask(Sq: int, Sk: int, causal: bool, kv_valid_len=None) -> torch.Ten
     return vis
 
 
-def attention_ref(q, k, v, causal: bool = False, kv_valid_len=None, scale=None):
+def attention_ref(q, k, v, causal: bool = False, kv_valid_len=None, scale=None, q_rows=None):
     """fp32 softmax attention. q [B,Hq,Sq,D], k, v [B,Hkv,Sk,D]. Returns (O [B,Hq,Sq,D], LSE [B,Hq,Sq]) fp32.
 
     Rows with no visible key give O = 0 and LSE = -inf.
+    q_rows (1-D index tensor): evaluate only these query rows of the Sq-row problem (same mask rows, same keys) and
+    return O [B,Hq,len(q_rows),D], LSE [B,Hq,len(q_rows)]: the rows of the full result, for checks at sizes where the
+    full score matrix is too much host work.
     """
     q32 = q.detach().to("cpu", torch.float32)
     k32 = k.detach().to("cpu", torch.float32)
@@ -141,8 +144,12 @@ def attention_ref(q, k, v, causal: bool = False, kv_valid_len=None, scale=None):
     if scale is None:
         scale = 1.0 / math.sqrt(D)
     vis = visible_mask(Sq, Sk, causal, kv_valid_len)
+    if q_rows is not None:
+        q_rows = torch.as_tensor(q_rows, dtype=torch.long)
+        q32 = q32[:, :, q_rows]
+        vis = vis[q_rows]
     out = torch.empty_like(q32)
-    lse = torch.empty((B, Hq, Sq), dtype=torch.float32)
+    lse = torch.empty((B, Hq, q32.shape[2]), dtype=torch.float32)
     for b in range(B):  # head by head keeps the score matrix small
         for h in range(Hq):
             s = (q32[b, h] @ k32[b, h].t()) * scale
@@ -233,34 +240,39 @@ def fmha_tolerance_ok(o, lse, o_ref, lse_ref):
 # ---------------------------------------------------------------------------------------------------------------
 # Llama-3-8B-shaped prefill layer (benchmark configuration 5): hidden 4096, 32 q / 8 kv heads, d 128, FFN 14336
 # ---------------------------------------------------------------------------------------------------------------
-def llama_layer_ref(x, w_qkv, w_o, w_gu, w_d, n_q=32, n_kv=8, d=128, stage_inputs=None):
+def llama_layer_ref(x, w_qkv, w_o, w_gu, w_d, n_q=32, n_kv=8, d=128, stage_inputs=None, rows=None):
     """fp32 chain. x [S, H]; weights stored [K, N]. Returns dict of every stage's fp32 output.
 
     stage_inputs, when given, maps a stage name to the tensor to feed INTO that stage instead of the oracle's own
-    previous output (used to check each GPU stage against an oracle fed the GPU's previous-stage result)."""
+    previous output (used to check each GPU stage against an oracle fed the GPU's previous-stage result).
+    rows (1-D index tensor): every returned stage holds only these token rows of the full result (the QKV product is
+    still formed for all rows, because every key and value feeds the attention of the sampled rows; stage_inputs stay
+    full-size tensors). For S = 8192, where the full chain is minutes of host work."""
     si = stage_inputs or {}
     f = lambda t: t.detach().to("cpu", torch.float32)
     S = x.shape[0]
+    sel = (lambda t: t) if rows is None else (lambda t: t[torch.as_tensor(rows, dtype=torch.long)])
     out = {}
     qkv = f(si.get("qkv_in", x)) @ f(w_qkv)
-    out["qkv"] = qkv
+    out["qkv"] = sel(qkv)
     qkv_used = f(si.get("attn_in", qkv.half()))
     q = qkv_used[:, : n_q * d].reshape(S, n_q, d).permute(1, 0, 2)[None]
     k = qkv_used[:, n_q * d: (n_q + n_kv) * d].reshape(S, n_kv, d).permute(1, 0, 2)[None]
     v = qkv_used[:, (n_q + n_kv) * d:].reshape(S, n_kv, d).permute(1, 0, 2)[None]
-    o, lse = attention_ref(q, k, v, causal=True)
+    o, lse = attention_ref(q, k, v, causal=True, q_rows=rows)
     out["attn"] = o
     out["attn_lse"] = lse
-    attn_used = f(si.get("oproj_in", o.half()))
-    a2 = attn_used[0].permute(1, 0, 2).reshape(S, n_q * d)
+    attn_used = f(si["oproj_in"])[:, :, torch.as_tensor(rows, dtype=torch.long)] if ("oproj_in" in si and rows is not None) \
+        else f(si.get("oproj_in", o.half()))
+    a2 = attn_used[0].permute(1, 0, 2).reshape(-1, n_q * d)
     out["oproj"] = a2 @ f(w_o)
-    gu = f(si.get("gu_in", out["oproj"].half())) @ f(w_gu)
+    gu = sel(f(si["gu_in"])) @ f(w_gu) if "gu_in" in si else f(out["oproj"].half()) @ f(w_gu)
     out["gate_up"] = gu
-    gu_used = f(si.get("act_in", gu.half()))
+    gu_used = sel(f(si["act_in"])) if "act_in" in si else f(gu.half())
     ffn = w_gu.shape[1] // 2
     act = torch.nn.functional.silu(gu_used[:, :ffn]) * gu_used[:, ffn:]
     out["act"] = act
-    out["down"] = f(si.get("down_in", act.half())) @ f(w_d)
+    out["down"] = (sel(f(si["down_in"])) if "down_in" in si else f(act.half())) @ f(w_d)
     return out
 
 
@@ -312,34 +324,45 @@ def silu_mul_ref(gate_up):
 
 
 def llama_decoder_layer_ref(x, w, positions, n_q, n_kv, eps=1e-5, rope_base=10000.0, past_k=None, past_v=None,
-                            round_stages=True):
+                            round_stages=True, rows=None):
     """One Llama decoder layer in fp32 on the CPU. x [B, S, H]; w: dict with nn.Linear-layout ([out, in]) weights
     'q', 'k', 'v', 'o', 'gate', 'up', 'down' and norm weights 'ln1', 'ln2'; positions [B, S]; past_k / past_v
     [B, n_kv, P, D] (already rotated keys). Follows LlamaDecoderLayer.forward (:755-781) and
     LlamaSdpaAttention.forward (:652-704); attention is causal with the mask aligned bottom-right (prefill: P = 0;
     generation step: S = 1). round_stages rounds every intermediate to fp16 where an fp16 pipeline stores it, so a
     kernel chain is compared against the same sequence of roundings. Returns (out fp32 [B,S,H], k, v) with k, v the
-    updated caches [B, n_kv, P+S, D] fp32."""
+    updated caches [B, n_kv, P+S, D] fp32. rows (1-D index tensor): `out` holds only these token rows [B,len(rows),H]
+    (keys and values are still formed for every token; queries, attention and everything after it only for `rows`)."""
     r = (lambda t: t.to(torch.float16).float()) if round_stages else (lambda t: t)
     x = _f32(x)
     B, S, H = x.shape
     D = w["q"].shape[0] // n_q
     h1, _ = rmsnorm_ref(x, w["ln1"], eps)
     h1 = r(h1)
-    q = r(h1 @ _f32(w["q"]).T).view(B, S, n_q, D).transpose(1, 2)
+    if rows is not None:
+        rows = torch.as_tensor(rows, dtype=torch.long)
+    Sr = S if rows is None else len(rows)
+    h1q = h1 if rows is None else h1[:, rows]
+    pos_q = positions if rows is None else positions[:, rows]
+    q = r(h1q @ _f32(w["q"]).T).view(B, Sr, n_q, D).transpose(1, 2)
     k = r(h1 @ _f32(w["k"]).T).view(B, S, n_kv, D).transpose(1, 2)
     v = r(h1 @ _f32(w["v"]).T).view(B, S, n_kv, D).transpose(1, 2)
     n_pos = int(positions.max()) + 1
     cos, sin = rope_tables(n_pos, D, rope_base)
-    q = r(rope_ref(q, cos, sin, positions))
+    q = r(rope_ref(q, cos, sin, pos_q))
     k = r(rope_ref(k, cos, sin, positions))
     if past_k is not None:
         k = torch.cat((_f32(past_k), k), 2)
         v = torch.cat((_f32(past_v), v), 2)
-    o, _ = attention_ref(q, k, v, causal=True)
-    o = r(o).transpose(1, 2).reshape(B, S, n_q * D)
+    if rows is None:
+        o, _ = attention_ref(q, k, v, causal=True)
+    else:   # the sampled queries keep their place in the S-row causal problem
+        qfull = torch.zeros((B, n_q, S, D), dtype=torch.float32)
+        qfull[:, :, rows] = q
+        o, _ = attention_ref(qfull, k, v, causal=True, q_rows=rows)
+    o = r(o).transpose(1, 2).reshape(B, Sr, n_q * D)
     attn = r(o @ _f32(w["o"]).T)
-    h2, res = rmsnorm_ref(attn, w["ln2"], eps, residual=x, round_residual=round_stages)
+    h2, res = rmsnorm_ref(attn, w["ln2"], eps, residual=x if rows is None else x[:, rows], round_residual=round_stages)
     h2 = r(h2)
     gu = r(torch.cat((h2 @ _f32(w["gate"]).T, h2 @ _f32(w["up"]).T), -1))
     act = r(silu_mul_ref(gu))

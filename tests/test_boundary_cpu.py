@@ -24,7 +24,12 @@ def test_library_exports_every_declared_symbol(lib):
     cdll = lib.load()
     for n in names:
         assert getattr(cdll, n) is not None
-    assert cdll.mi355_serving_version() == 100
+    assert cdll.mi355_serving_version() == 200
+    # the test / tuning hooks are exported but stay out of the public header, and no process-wide switch exists any more
+    for n in lib.INTERNAL_SYMBOLS:
+        assert n not in names and getattr(cdll, n) is not None
+    assert not any("debug" in n for n in names)
+    assert not hasattr(cdll, "mi355_debug_set_gemm_variant") and not hasattr(cdll, "mi355_debug_set_fmha_variant")
 
 
 def test_capi_rejects_bad_arguments_without_a_gpu(lib):
@@ -52,6 +57,18 @@ def test_capi_rejects_bad_arguments_without_a_gpu(lib):
     assert strided(good[:11] + [64]) == 10001              # rows of O overlap
     assert b"overlap" in cdll.mi355_last_error()
     assert cdll.mi355_fmha_fwd_strided(p, p, p, p, None, 2, 4, 2, 8, 8, 128, 0.1, 0, 8, None, None) == 10001
+    # caller-owned workspace: size query and the checks that run before any launch
+    wsb = cdll.mi355_fmha_fwd_workspace_bytes
+    assert wsb(1, 32, 8, 4096, 4096, 4096) == 0 and wsb(1, 32, 8, 1, 400, 400) == 0     # prefill, short cache: no split-KV
+    need = wsb(1, 32, 8, 1, 8192, 8192)
+    assert 0 < need <= 16 << 20 and need % 16 == 0
+    assert wsb(8, 32, 8, 1, 8192, 8192) > 0 and wsb(1, 32, 8, 1, 8192, 9000) == 0         # invalid sizes report 0
+    ws_call = lambda ptr, nbytes, dtype=0: cdll.mi355_fmha_fwd_ws(p, p, p, p, None, 1, 32, 8, 1, 8192, 128, 0.1, 0, 8192, None,
+                                                                  dtype, ptr, nbytes, None)
+    assert ws_call(None, 0) == 10001 and b"workspace" in cdll.mi355_last_error()
+    assert ws_call(p2, need - 16) == 10001
+    assert ws_call(ctypes.c_void_p(0x100008), need) == 10001                                 # misaligned
+    assert ws_call(p2, need, dtype=5) == 10001 and b"dtype" in cdll.mi355_last_error()
     # layer glue
     assert cdll.mi355_rmsnorm(p, None, None, p, p, 4, 100, 104, 0, 0, 104, 1e-5, None) == 10001   # hidden % 8
     assert cdll.mi355_rmsnorm(p, p, None, p, p, 4, 128, 128, 128, 128, 128, 1e-5, None) == 10001   # residual without residual_out

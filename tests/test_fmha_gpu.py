@@ -14,14 +14,14 @@ pytestmark = pytest.mark.gpu
 GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
 
 
-def run(lib, gpu, q, k, v, causal=False, kv_valid_len=None):
-    o, lse = lib.fmha_fwd(q.to(gpu), k.to(gpu), v.to(gpu), causal=causal, kv_valid_len=kv_valid_len)
+def run(lib, gpu, q, k, v, causal=False, kv_valid_len=None, variant=0):
+    o, lse = lib.fmha_fwd(q.to(gpu), k.to(gpu), v.to(gpu), causal=causal, kv_valid_len=kv_valid_len, variant=variant)
     torch.cuda.synchronize()
     return o.cpu(), lse.cpu()
 
 
-def check(lib, gpu, q, k, v, causal=False, kv_valid_len=None):
-    o, lse = run(lib, gpu, q, k, v, causal, kv_valid_len)
+def check(lib, gpu, q, k, v, causal=False, kv_valid_len=None, variant=0):
+    o, lse = run(lib, gpu, q, k, v, causal, kv_valid_len, variant)
     o_ref, lse_ref = so.attention_ref(q, k, v, causal=causal, kv_valid_len=kv_valid_len)
     ok, st = so.fmha_tolerance_ok(o, lse, o_ref, lse_ref)
     assert ok, (tuple(q.shape), tuple(k.shape), causal, kv_valid_len, st)
@@ -121,11 +121,7 @@ def test_ragged_shapes_and_masks(lib, gpu, B, Hq, Hkv, Sq, Sk, causal, kvv):
 ])
 def test_every_kernel_variant_on_ragged_shapes(lib, gpu, variant, B, Hq, Hkv, Sq, Sk, causal, kvv):
     q, k, v = so.fmha_inputs(B, Hq, Hkv, Sq, Sk, seed=Sq + 3 * Sk + variant)
-    lib.set_variants(fmha=variant)
-    try:
-        check(lib, gpu, q, k, v, causal, kvv)
-    finally:
-        lib.set_variants()
+    check(lib, gpu, q, k, v, causal, kvv, variant=variant)   # pinned through the library's internal test hook
 
 
 @pytest.mark.parametrize("B,Hq,Hkv,Sq,Sk,causal,kvv", [
@@ -138,11 +134,7 @@ def test_generation_step_split_kv_path(lib, gpu, B, Hq, Hkv, Sq, Sk, causal, kvv
     # prefill kernel on the same inputs
     q, k, v = so.fmha_inputs(B, Hq, Hkv, Sq, Sk, seed=Sk + Hq)
     o, lse = check(lib, gpu, q, k, v, causal, kvv)
-    lib.set_variants(fmha=1)
-    try:
-        o1, lse1 = run(lib, gpu, q, k, v, causal, kvv)
-    finally:
-        lib.set_variants()
+    o1, lse1 = run(lib, gpu, q, k, v, causal, kvv, variant=1)
     assert (o.float() - o1.float()).abs().max() <= 2e-3 and (lse - lse1).abs().max() <= 1e-3
 
 
@@ -162,6 +154,87 @@ def test_generation_step_on_two_streams(lib, gpu):
             outs_b.append(lib.fmha_fwd(qb, kb, vb)[0])
     torch.cuda.synchronize()
     assert all(torch.equal(o, ref_a) for o in outs_a) and all(torch.equal(o, ref_b) for o in outs_b)
+
+
+def test_split_kv_workspace_outlives_growth_under_a_captured_graph(lib, gpu):
+    # A generation step is captured into a HIP graph; afterwards an eager call on the same stream needs a larger
+    # workspace than the one the graph's kernels hold the address of. The library must keep the old buffer alive (it
+    # only ever adds buffers), so replays of the graph still write valid memory and still give the eager result.
+    qs, ks, vs = (t.to(gpu) for t in so.fmha_inputs(1, 32, 8, 1, 4096, seed=31))
+    qb, kb, vb = (t.to(gpu) for t in so.fmha_inputs(8, 32, 1, 1, 16384, seed=32))     # 768 units x 32 columns: ~13 MB
+    assert lib.fmha_workspace_bytes(8, 32, 1, 1, 16384) > (4 << 20) > lib.fmha_workspace_bytes(1, 32, 8, 1, 4096) > 0
+    ref_s = lib.fmha_fwd(qs, ks, vs)[0].clone()
+    ref_b = lib.fmha_fwd(qb, kb, vb)[0].clone()
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    out_g = torch.zeros_like(qs)
+    with torch.cuda.stream(side):
+        lib.fmha_fwd(qs, ks, vs, return_lse=False, out=out_g)        # first use on this stream: allocates its 4 MiB buffer
+    side.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        lib.fmha_fwd(qs, ks, vs, return_lse=False, out=out_g)
+    for rep in range(3):
+        out_g.zero_()
+        with torch.cuda.stream(side):
+            big = lib.fmha_fwd(qb, kb, vb)[0]                        # eager, same stream, larger workspace
+        side.synchronize()
+        assert torch.equal(big, ref_b), rep
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out_g, ref_s), rep
+    del graph
+
+
+def test_split_kv_call_that_would_allocate_during_capture_is_refused(lib, gpu):
+    # The capture stream has no workspace large enough (this shape needs more than any other test's: torch hands out
+    # pooled streams, so "never used" cannot be relied on): the library must not allocate under capture; it reports an
+    # error and launches nothing. The same capture then succeeds with a caller-owned workspace.
+    B, Hq, Hkv, Sk = 1536, 32, 1, 512
+    q, k, v = (t.to(gpu) for t in so.fmha_inputs(B, Hq, Hkv, 1, Sk, seed=33))
+    assert lib.fmha_workspace_bytes(B, Hq, Hkv, 1, Sk) > (24 << 20)
+    ref = lib.fmha_fwd(q, k, v)[0].clone()      # default stream (also sets the kernel attributes outside capture)
+    ws = torch.empty(lib.fmha_workspace_bytes(B, Hq, Hkv, 1, Sk), dtype=torch.uint8, device=gpu)
+    out_g = torch.zeros_like(q)
+    torch.cuda.synchronize()
+    fresh = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    refused = None
+    with torch.cuda.graph(graph, stream=fresh):
+        try:
+            lib.fmha_fwd(q, k, v, return_lse=False, out=out_g)
+        except lib.Mi355Error as e:
+            refused = e
+        lib.fmha_fwd(q, k, v, return_lse=False, out=out_g, workspace=ws)
+    assert refused is not None and "capturing" in str(refused)
+    for _ in range(2):
+        out_g.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out_g, ref)
+    del graph
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_caller_owned_workspace_entry_point(lib, gpu, dtype):
+    # mi355_fmha_fwd_ws: same kernels, partial results in the caller's memory; bit-identical to the library-owned path,
+    # also when the workspace is larger than needed, holds garbage, and is reused by a smaller call
+    for (B, Hq, Hkv, Sq, Sk, causal) in ((2, 32, 8, 1, 5000, False), (1, 8, 2, 3, 1200, True)):
+        q, k, v = (t.to(gpu).to(dtype) for t in so.fmha_inputs(B, Hq, Hkv, Sq, Sk, seed=Sk))
+        need = lib.fmha_workspace_bytes(B, Hq, Hkv, Sq, Sk)
+        assert need > 0
+        ws = torch.full((need + 4096,), 0xFF, dtype=torch.uint8, device=gpu)
+        o_ref, l_ref = lib.fmha_fwd(q, k, v, causal=causal)
+        o, l = lib.fmha_fwd(q, k, v, causal=causal, workspace=ws)
+        torch.cuda.synchronize()
+        assert torch.equal(o, o_ref) and torch.equal(l, l_ref)
+        with pytest.raises(lib.Mi355Error, match="workspace"):
+            lib.fmha_fwd(q, k, v, causal=causal, workspace=ws[:need - 16])
+    # prefill shapes need no workspace at all
+    q, k, v = (t.to(gpu).to(dtype) for t in so.fmha_inputs(1, 4, 2, 200, 200, seed=5))
+    assert lib.fmha_workspace_bytes(1, 4, 2, 200, 200) == 0
+    o = lib.fmha_fwd(q, k, v, causal=True, workspace=torch.empty(0, dtype=torch.uint8, device=gpu))[0]
+    assert torch.equal(o, lib.fmha_fwd(q, k, v, causal=True)[0])
 
 
 # ---- operands read in place from other layouts ------------------------------------------------------------------------
@@ -285,7 +358,8 @@ def test_torch_operator_accepts_reference_style_padded_call(gpu):
 
 def test_torch_operator_reads_transposed_views_in_place(gpu):
     # the in-model call of the reference: [B, S, H, D] projections viewed as [B, H, S, D]
-    # (benchmarks/flashattn-cuda/modeling_llama.py:658-660); the result has q's layout, so transposing it back is free
+    # (benchmarks/flashattn-cuda/modeling_llama.py:658-660), read where they lie; the result is a contiguous [B, H, S, D]
+    # tensor like the reference's (semi/fmha_2_amd.cpp:336), so a caller may .view() it
     import fmha_unified
     B, S, Hq, Hkv = 2, 384, 8, 2
     q, k, v = so.fmha_inputs(B, Hq, Hkv, S, S, seed=21)
@@ -294,7 +368,8 @@ def test_torch_operator_reads_transposed_views_in_place(gpu):
     vp = v.transpose(1, 2).contiguous().to(gpu)
     out = fmha_unified.ops.fine_fmha(qp.transpose(1, 2), kp.transpose(1, 2), vp.transpose(1, 2), causal=True,
                                      is_decode=False, kernel_index=5)
-    assert out.shape == (B, Hq, S, 128) and out.transpose(1, 2).is_contiguous()
+    assert out.shape == (B, Hq, S, 128) and out.is_contiguous()
+    assert out.view(B * Hq, S * 128).shape == (B * Hq, S * 128)
     o_ref, _ = so.attention_ref(q, k, v, causal=True)
     assert (out.cpu().float() - o_ref).abs().max() <= 2e-3
     # a view the kernel cannot read in place (last dimension strided) is copied, as the reference does

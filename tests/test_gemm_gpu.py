@@ -14,14 +14,14 @@ pytestmark = pytest.mark.gpu
 GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
 
 
-def run(lib, gpu, a, b, layout="NN"):
-    c = lib.hgemm(a.to(gpu), b.to(gpu), layout)
+def run(lib, gpu, a, b, layout="NN", variant=0):
+    c = lib.hgemm(a.to(gpu), b.to(gpu), layout, variant=variant)
     torch.cuda.synchronize()
     return c.cpu()
 
 
-def check(lib, gpu, a, b, layout, K):
-    c = run(lib, gpu, a, b, layout)
+def check(lib, gpu, a, b, layout, K, variant=0):
+    c = run(lib, gpu, a, b, layout, variant)
     ok, st = so.gemm_tolerance_ok(c, so.gemm_ref(a, b, layout), K)
     assert ok, (layout, tuple(a.shape), tuple(b.shape), st)
     return c
@@ -99,13 +99,8 @@ def test_ragged_m_and_n_on_the_tiled_kernels(lib, gpu, variant, layout, M, N, K)
     ref = so.gemm_ref(a, b, layout)
     c = torch.full((M + 2, N + 8), 9.0, dtype=torch.float16, device=gpu)
     ag, bg = a.to(gpu), b.to(gpu)
-    lib.set_variants(gemm=variant)
-    try:
-        lib.hgemm_raw(ag.data_ptr(), bg.data_ptr(), c.data_ptr(), M, N, K, ag.stride(0), bg.stride(0), c.stride(0),
-                      lib.LAYOUTS[layout], torch.cuda.current_stream().cuda_stream)
-        torch.cuda.synchronize()
-    finally:
-        lib.set_variants()
+    lib.hgemm(ag, bg, layout, out=c[:M, :N], variant=variant)   # variant 0: the public entry point
+    torch.cuda.synchronize()
     ok, st = so.gemm_tolerance_ok(c[:M, :N].cpu(), ref, K)
     assert ok, st
     assert bool((c[M:] == 9.0).all()) and bool((c[:, N:] == 9.0).all())
@@ -115,11 +110,7 @@ def test_ragged_m_and_n_on_the_tiled_kernels(lib, gpu, variant, layout, M, N, K)
 @pytest.mark.parametrize("layout", ["NN", "TN", "NT"])
 def test_every_tile_variant(lib, gpu, variant, layout):
     a, b = operands(512, 768, 448, layout, seed=variant)
-    lib.set_variants(gemm=variant)
-    try:
-        check(lib, gpu, a, b, layout, 448)
-    finally:
-        lib.set_variants()
+    check(lib, gpu, a, b, layout, 448, variant=variant)
 
 
 @pytest.mark.parametrize("layout", ["NN", "NT", "TN"])
@@ -227,6 +218,29 @@ def test_torch_operator_noncontiguous_inputs_and_stream(gpu):
         c = gemm_unified.ops.fine_gemm(at, b, 0)
     s.synchronize()
     ok, st = so.gemm_tolerance_ok(c, so.gemm_ref(a, b), 300)
+    assert ok, st
+
+
+def test_torch_operator_single_row_operand_with_arbitrary_row_stride(lib, gpu):
+    # torch calls a [1, K] tensor contiguous whatever its stride(0) (expand / as_strided / keepdim views produce such
+    # tensors); the operators and the ctypes wrapper must pass the logical leading dimension, not that stride
+    import gemm_unified
+    K, N = 512, 256
+    a, b = so.gemm_inputs(1, N, K, seed=5)
+    base = torch.zeros(4 * K, dtype=torch.float16, device=gpu)
+    base[:K] = a[0].to(gpu)
+    for stride0 in (7, 0, 3 * K):
+        a1 = base.as_strided((1, K), (stride0, 1))
+        assert a1.is_contiguous() and a1.stride(0) == stride0
+        for c in (gemm_unified.ops.fine_gemm(a1, b.to(gpu), 0), lib.hgemm(a1, b.to(gpu), "NN"),
+                  gemm_unified.ops.fine_gemm(a1, b.t().contiguous().to(gpu), 13)):
+            ok, st = so.gemm_tolerance_ok(c, so.gemm_ref(a, b), K)
+            assert ok, (stride0, st)
+    # the same for a [K, 1] second operand
+    a2, b2 = so.gemm_inputs(64, 1, K, seed=6)
+    bcol = b2.to(gpu).as_strided((K, 1), (1, 5))
+    assert bcol.is_contiguous()
+    ok, st = so.gemm_tolerance_ok(gemm_unified.ops.fine_gemm(a2.to(gpu), bcol, 0), so.gemm_ref(a2, b2), K)
     assert ok, st
 
 

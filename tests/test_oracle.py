@@ -284,3 +284,39 @@ def test_decoder_layer_against_transformers_llama():
     full, _, _ = so.llama_decoder_layer_ref(torch.cat((x, x1), 1), w, torch.arange(S + 1)[None].expand(B, S + 1), 4, 2,
                                             round_stages=False)
     assert torch.allclose(out1[:, 0], full[:, -1], atol=1e-4)
+
+
+def test_sampled_rows_are_the_rows_of_the_full_result():
+    # q_rows / rows restrict the (pinned) full-size functions to some token rows for the 8192-token checks; they must
+    # reproduce exactly those rows, masks included (up to fp32 summation order inside the BLAS call)
+    q, k, v = so.fmha_inputs(2, 4, 2, 70, 101, seed=3)
+    rows = torch.tensor([0, 3, 17, 69])
+    for causal, kvv in ((True, None), (False, 90), (True, 95), (True, 20)):
+        o, l = so.attention_ref(q, k, v, causal, kvv)
+        o2, l2 = so.attention_ref(q, k, v, causal, kvv, q_rows=rows)
+        assert (o[:, :, rows] - o2).abs().max() <= 1e-5
+        fin = torch.isfinite(l[:, :, rows])
+        assert torch.equal(fin, torch.isfinite(l2)) and (l[:, :, rows][fin] - l2[fin]).abs().max() <= 1e-5
+    S, H, F = 300, 256, 512
+    x = so.randn_fp16((S, H), 0)
+    wq, wo = so.randn_fp16((H, 512), 1, 0.05), so.randn_fp16((256, H), 2, 0.05)
+    wgu, wd = so.randn_fp16((H, 2 * F), 3, 0.05), so.randn_fp16((F, H), 4, 0.05)
+    rows = torch.tensor([0, 5, 128, 299])
+    full = so.llama_layer_ref(x, wq, wo, wgu, wd, n_q=2, n_kv=1)
+    part = so.llama_layer_ref(x, wq, wo, wgu, wd, n_q=2, n_kv=1, rows=rows)
+    si = {"attn_in": full["qkv"].half(), "oproj_in": full["attn"].half(), "gu_in": full["oproj"].half(),
+          "act_in": full["gate_up"].half(), "down_in": full["act"].half()}
+    a = so.llama_layer_ref(x, wq, wo, wgu, wd, n_q=2, n_kv=1, stage_inputs=si)
+    b = so.llama_layer_ref(x, wq, wo, wgu, wd, n_q=2, n_kv=1, stage_inputs=si, rows=rows)
+    for name in ("qkv", "oproj", "gate_up", "act", "down"):
+        assert (full[name][rows] - part[name]).abs().max() <= 1e-4 * full[name].abs().max(), name
+        assert (a[name][rows] - b[name]).abs().max() <= 1e-4 * a[name].abs().max(), name
+    assert (full["attn"][:, :, rows] - part["attn"]).abs().max() <= 1e-5
+    g = lambda shape, s_: so.randn_fp16(shape, s_, 0.05)
+    w = dict(q=g((256, H), 1), k=g((128, H), 2), v=g((128, H), 3), o=g((H, 256), 4), gate=g((F, H), 5), up=g((F, H), 6),
+             down=g((H, F), 7), ln1=torch.ones(H).half(), ln2=torch.ones(H).half())
+    xb = so.randn_fp16((2, S, H), 9)
+    pos = torch.arange(S)[None].expand(2, S)
+    f, kf, vf = so.llama_decoder_layer_ref(xb, w, pos, 2, 1, round_stages=False)
+    p, kp, vp = so.llama_decoder_layer_ref(xb, w, pos, 2, 1, round_stages=False, rows=rows)
+    assert (f[:, rows] - p).abs().max() <= 1e-4 * f.abs().max() and torch.equal(kf, kp) and torch.equal(vf, vp)

@@ -1,12 +1,17 @@
 """Build script for the MI355X serving kernels (gfx950 only).
 
-Produces, next to the sources:
-    libmi355_serving.so        HIP kernels + C ABI (include/mi355_serving.h); no torch dependency
-    gemm_unified/_C.so         torch operators gemm_unified::finegemm_N, linked against the library above
-    fmha_unified/_C.so         torch operators fmha_unified::finefmha_N
+Produces, inside the three packages:
+    mi355_serving/libmi355_serving.so   HIP kernels + C ABI (include/mi355_serving.h); no torch dependency
+    gemm_unified/_C.so                  torch operators gemm_unified::finegemm_N, linked against the library above
+    fmha_unified/_C.so                  torch operators fmha_unified::finefmha_N
+Each _C.so finds the library through RUNPATH $ORIGIN/../mi355_serving: the packages sit side by side both in the source
+tree and in site-packages.
 
 hipcc cross-compiles for gfx950 without a GPU. Usage: ``python build.py [--only lib|ops]`` or
 ``from build import build_all``.
+
+Environment (the knobs of the reference's kernels/*/pkg/setup.py): GPU_ARCHS (setup.py:222; only "gfx950" or "native" are
+accepted here), MAX_JOBS (setup.py:284-305; number of sources compiled side by side), HIPCC, CXX.
 """
 import os
 import subprocess
@@ -17,7 +22,8 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(HERE)
 INCLUDE = os.path.join(ROOT, "include")
 LIB_NAME = "libmi355_serving.so"
-LIB_PATH = os.path.join(HERE, LIB_NAME)
+LIB_DIR = os.path.join(HERE, "mi355_serving")
+LIB_PATH = os.path.join(LIB_DIR, LIB_NAME)
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 
@@ -30,6 +36,24 @@ KERNEL_SOURCES = ["csrc/hgemm.hip", "csrc/fmha_fwd.hip", "csrc/fmha_decode.hip",
 # Per-source additions. The GEMM keeps its MFMA accumulators in ordinary VGPRs: left to itself the compiler moves part of
 # them to AGPRs in the 4-wave kernels and then shuffles them back and forth inside the K loop.
 SOURCE_FLAGS = {"csrc/hgemm.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"]}
+
+
+def check_archs():
+    """GPU_ARCHS as the reference's setup.py reads it (';'-separated). This build has gfx950 code only."""
+    archs = [a for a in os.environ.get("GPU_ARCHS", "gfx950").split(";") if a]
+    bad = [a for a in archs if a not in ("gfx950", "native")]
+    if bad:
+        raise SystemExit("GPU_ARCHS=%s: these kernels are written for gfx950 (MI355X) only" % ";".join(archs))
+
+
+def max_jobs(n_sources):
+    try:
+        jobs = int(os.environ.get("MAX_JOBS", "0"))
+    except ValueError:
+        jobs = 0
+    if jobs < 1:
+        jobs = min(os.cpu_count() or 1, 8)
+    return max(1, min(jobs, n_sources))
 
 
 def _run(cmd, quiet_patterns=("is not a recognized feature for this target",)):
@@ -46,6 +70,7 @@ def build_library(verbose=True):
     import tempfile
     from concurrent.futures import ThreadPoolExecutor
 
+    check_archs()
     with tempfile.TemporaryDirectory(prefix="mi355_build_") as tmp:
         jobs = []
         for src in KERNEL_SOURCES:
@@ -54,7 +79,7 @@ def build_library(verbose=True):
             if verbose:
                 print("[build] " + " ".join(cmd))
             jobs.append((cmd, obj))
-        with ThreadPoolExecutor(max_workers=min(len(jobs), os.cpu_count() or 1, 8)) as pool:
+        with ThreadPoolExecutor(max_workers=max_jobs(len(jobs))) as pool:
             list(pool.map(lambda job: _run(job[0]), jobs))
         link = [HIPCC, "--offload-arch=gfx950", "-fPIC", "-shared"] + [obj for _, obj in jobs] + ["-o", LIB_PATH]
         if verbose:
@@ -86,7 +111,7 @@ def build_operator(pkg, source, verbose=True):
     out = os.path.join(HERE, pkg, "_C.so")
     cxx = os.environ.get("CXX", "g++")
     cmd = [cxx, "-O2", "-std=c++17", "-fPIC", "-shared", "-Wno-attributes"] + defs + ["-I", INCLUDE] + inc + \
-          [os.path.join(pkg, "csrc", source), "-o", out, "-L" + HERE, "-lmi355_serving", "-Wl,-rpath,$ORIGIN/.."] + libs
+          [os.path.join(pkg, "csrc", source), "-o", out, "-L" + LIB_DIR, "-lmi355_serving", "-Wl,-rpath,$ORIGIN/../mi355_serving"] + libs
     if verbose:
         print("[build] " + " ".join(cmd))
     _run(cmd)
@@ -102,6 +127,51 @@ def build_all(verbose=True):
 def is_built():
     return all(os.path.exists(p) for p in (LIB_PATH, os.path.join(HERE, "gemm_unified", "_C.so"),
                                            os.path.join(HERE, "fmha_unified", "_C.so")))
+
+
+def run_setup(dist_name, op_packages, rel, py_modules=()):
+    """setuptools.setup() for `op_packages` (gemm_unified and / or fmha_unified) plus the mi355_serving package that
+    holds the kernel library. `rel` is the path from the calling setup.py (the current directory) to this directory.
+    The shared objects are package data: they are compiled (if missing) by build_py, before the data files are
+    collected, so a clean checkout installs complete packages."""
+    from setuptools import Command, setup
+    from setuptools.command.build_py import build_py
+
+    class BuildExt(Command):
+        description = "compile libmi355_serving.so and the torch operator modules in-tree"
+        user_options = [("inplace", "i", "accepted for compatibility; the build is always in-tree")]
+
+        def initialize_options(self):
+            self.inplace = True
+
+        def finalize_options(self):
+            pass
+
+        def run(self):
+            build_all(verbose=True)
+
+    class BuildPy(build_py):
+        def run(self):
+            check_archs()
+            if not is_built():
+                build_all(verbose=True)
+            super().run()
+
+    packages = list(op_packages) + ["mi355_serving"]
+    data = {p: ["_C.so"] for p in op_packages}
+    data["mi355_serving"] = [LIB_NAME]
+    setup(
+        name=dist_name,
+        version="2.0.0",
+        description="MI355X (gfx950) fp16 GEMM and fused attention forward behind the gemm_unified / fmha_unified operators",
+        packages=packages,
+        package_dir={p: os.path.join(rel, p) for p in packages} if rel != "." else {"": "."},
+        package_data=data,
+        py_modules=list(py_modules),
+        cmdclass={"build_ext": BuildExt, "build_py": BuildPy},
+        python_requires=">=3.8",
+        zip_safe=False,
+    )
 
 
 if __name__ == "__main__":

@@ -1,5 +1,6 @@
 // C ABI of libmi355_serving.so (see include/mi355_serving.h): argument validation and error reporting around
-// the kernel dispatchers. Nothing here allocates device memory or synchronises.
+// the kernel dispatchers. Nothing here allocates device memory or synchronises (the one allocation the library ever
+// makes, the split-KV workspace of mi355_fmha_fwd*, lives in fmha_decode.hip).
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
@@ -19,13 +20,21 @@ int fail(int code, const char* fmt, ...) {
 int hip_fail(hipError_t e, const char* what) {
     return fail(static_cast<int>(e), "%s: %s", what, hipGetErrorString(e));
 }
+mi355::FmhaStrides contiguous_strides(int Hq, int Hkv, int Sq, int Sk, int D) {
+    const long q_head = (long)Sq * D, k_head = (long)Sk * D;
+    return {Hq * q_head, q_head, D, Hkv * k_head, k_head, D, Hkv * k_head, k_head, D, Hq * q_head, q_head, D};
+}
+mi355::FmhaStrides strides_from(const int64_t* s) {
+    return {(long)s[0], (long)s[1], (long)s[2], (long)s[3], (long)s[4], (long)s[5],
+            (long)s[6], (long)s[7], (long)s[8], (long)s[9], (long)s[10], (long)s[11]};
+}
 }  // namespace
 
 extern "C" {
 
 // R == nullptr: the plain product; otherwise the residual operand of the *_add entry points (checked by the caller)
 static int hgemm_impl(const char* fn, int dtype, const void* A, const void* B, void* C, const void* R, int M, int N, int K, int64_t lda,
-                      int64_t ldb, int64_t ldc, int64_t ldr, int layout, void* stream) {
+                      int64_t ldb, int64_t ldc, int64_t ldr, int layout, void* stream, int variant = 0) {
     if (!A || !B || !C) return fail(MI355_ERR_BAD_ARGUMENT, "%s: null pointer", fn);
     if (M < 1 || N < 1 || K < 1) return fail(MI355_ERR_BAD_ARGUMENT, "%s: M, N, K must be >= 1 (got %d, %d, %d)", fn, M, N, K);
     if (layout != MI355_GEMM_NN && layout != MI355_GEMM_NT && layout != MI355_GEMM_TN)
@@ -39,7 +48,7 @@ static int hgemm_impl(const char* fn, int dtype, const void* A, const void* B, v
         return fail(MI355_ERR_BAD_ARGUMENT, "%s: leading dimension too small (ldr %lld >= %d required)", fn, (long long)ldr, N);
     if (R != nullptr && R == C && ldr != ldc)
         return fail(MI355_ERR_BAD_ARGUMENT, "%s: R aliases C but ldr (%lld) differs from ldc (%lld)", fn, (long long)ldr, (long long)ldc);
-    hipError_t e = mi355::hgemm_dispatch(A, B, C, R, M, N, K, lda, ldb, ldc, R ? ldr : 0, layout, dtype, static_cast<hipStream_t>(stream));
+    hipError_t e = mi355::hgemm_dispatch(A, B, C, R, M, N, K, lda, ldb, ldc, R ? ldr : 0, layout, dtype, variant, static_cast<hipStream_t>(stream));
     if (e != hipSuccess) return hip_fail(e, fn);
     return 0;
 }
@@ -69,7 +78,7 @@ int mi355_gemm_add_bf16(const void* A, const void* B, const void* R, void* C, in
 
 static int fmha_checked(const char* fn, const void* Q, const void* K, const void* V, void* O, float* LSE, int B, int Hq, int Hkv,
                         int Sq, int Sk, int D, float scale, int causal, int kv_valid_len, const mi355::FmhaStrides& sd,
-                        int dtype, void* stream) {
+                        int dtype, void* stream, int variant = 0, const mi355::FmhaWorkspace& ws = mi355::FmhaWorkspace()) {
     if (!Q || !K || !V || !O) return fail(MI355_ERR_BAD_ARGUMENT, "%s: null pointer", fn);
     if (B < 1 || Hq < 1 || Hkv < 1 || Sq < 1 || Sk < 1)
         return fail(MI355_ERR_BAD_ARGUMENT, "%s: B, Hq, Hkv, Sq, Sk must be >= 1", fn);
@@ -90,8 +99,17 @@ static int fmha_checked(const char* fn, const void* Q, const void* K, const void
                         all[i]);
     if (sd.o_row < D || (Hq > 1 && sd.o_head < D) || (B > 1 && sd.o_batch < D))
         return fail(MI355_ERR_BAD_ARGUMENT, "%s: rows of O overlap (o strides %ld, %ld, %ld)", fn, sd.o_batch, sd.o_head, sd.o_row);
+    if (ws.kind == mi355::FmhaWorkspace::kCaller) {
+        const size_t need = mi355::fmha_decode_workspace_bytes(B, Hq, Hkv, Sq, Sk, kv_valid_len);
+        if (need > 0 && (ws.ptr == nullptr || ws.bytes < need || reinterpret_cast<uintptr_t>(ws.ptr) % 16 != 0))
+            return fail(MI355_ERR_BAD_ARGUMENT, "%s: workspace of %zu bytes at %p; this call needs %zu bytes, 16-byte aligned "
+                        "(mi355_fmha_fwd_workspace_bytes)", fn, ws.bytes, ws.ptr, need);
+    }
     hipError_t e = mi355::fmha_fwd_dispatch(Q, K, V, O, LSE, B, Hq, Hkv, Sq, Sk, scale, causal != 0, kv_valid_len, sd, dtype,
-                                            static_cast<hipStream_t>(stream));
+                                            variant, ws, static_cast<hipStream_t>(stream));
+    if (e == hipErrorStreamCaptureUnsupported)
+        return fail(static_cast<int>(e), "%s: the split-KV workspace of this stream would have to be allocated or enlarged while "
+                    "the stream is capturing; run the call once before capture, or use mi355_fmha_fwd_ws", fn);
     if (e != hipSuccess) return hip_fail(e, fn);
     return 0;
 }
@@ -128,32 +146,51 @@ int mi355_gemm_silu_mul_bf16(const void* A, const void* B, void* C, int M, int N
 
 int mi355_fmha_fwd(const void* Q, const void* K, const void* V, void* O, float* LSE, int B, int Hq, int Hkv, int Sq,
                    int Sk, int D, float scale, int causal, int kv_valid_len, void* stream) {
-    const long q_head = (long)Sq * D, k_head = (long)Sk * D;
-    const mi355::FmhaStrides sd = {Hq * q_head, q_head, D, Hkv * k_head, k_head, D, Hkv * k_head, k_head, D, Hq * q_head, q_head, D};
-    return fmha_checked("mi355_fmha_fwd", Q, K, V, O, LSE, B, Hq, Hkv, Sq, Sk, D, scale, causal, kv_valid_len, sd,
-                        MI355_DTYPE_FP16, stream);
+    return fmha_checked("mi355_fmha_fwd", Q, K, V, O, LSE, B, Hq, Hkv, Sq, Sk, D, scale, causal, kv_valid_len,
+                        contiguous_strides(Hq, Hkv, Sq, Sk, D), MI355_DTYPE_FP16, stream);
 }
 
 int mi355_fmha_fwd_strided(const void* Q, const void* K, const void* V, void* O, float* LSE, int B, int Hq, int Hkv, int Sq,
                            int Sk, int D, float scale, int causal, int kv_valid_len, const int64_t* strides, void* stream) {
     if (!strides) return fail(MI355_ERR_BAD_ARGUMENT, "mi355_fmha_fwd_strided: null strides");
-    const mi355::FmhaStrides sd = {(long)strides[0], (long)strides[1], (long)strides[2],  (long)strides[3],
-                                   (long)strides[4], (long)strides[5], (long)strides[6],  (long)strides[7],
-                                   (long)strides[8], (long)strides[9], (long)strides[10], (long)strides[11]};
-    return fmha_checked("mi355_fmha_fwd_strided", Q, K, V, O, LSE, B, Hq, Hkv, Sq, Sk, D, scale, causal, kv_valid_len, sd,
-                        MI355_DTYPE_FP16, stream);
+    return fmha_checked("mi355_fmha_fwd_strided", Q, K, V, O, LSE, B, Hq, Hkv, Sq, Sk, D, scale, causal, kv_valid_len,
+                        strides_from(strides), MI355_DTYPE_FP16, stream);
 }
 
 int mi355_fmha_fwd_bf16(const void* Q, const void* K, const void* V, void* O, float* LSE, int B, int Hq, int Hkv, int Sq,
                         int Sk, int D, float scale, int causal, int kv_valid_len, const int64_t* strides, void* stream) {
-    const long q_head = (long)Sq * D, k_head = (long)Sk * D;
-    mi355::FmhaStrides sd = {Hq * q_head, q_head, D, Hkv * k_head, k_head, D, Hkv * k_head, k_head, D, Hq * q_head, q_head, D};
-    if (strides)
-        sd = {(long)strides[0], (long)strides[1], (long)strides[2],  (long)strides[3],
-              (long)strides[4], (long)strides[5], (long)strides[6],  (long)strides[7],
-              (long)strides[8], (long)strides[9], (long)strides[10], (long)strides[11]};
-    return fmha_checked("mi355_fmha_fwd_bf16", Q, K, V, O, LSE, B, Hq, Hkv, Sq, Sk, D, scale, causal, kv_valid_len, sd,
-                        MI355_DTYPE_BF16, stream);
+    return fmha_checked("mi355_fmha_fwd_bf16", Q, K, V, O, LSE, B, Hq, Hkv, Sq, Sk, D, scale, causal, kv_valid_len,
+                        strides ? strides_from(strides) : contiguous_strides(Hq, Hkv, Sq, Sk, D), MI355_DTYPE_BF16, stream);
+}
+
+size_t mi355_fmha_fwd_workspace_bytes(int B, int Hq, int Hkv, int Sq, int Sk, int kv_valid_len) {
+    if (B < 1 || Hq < 1 || Hkv < 1 || Sq < 1 || Sk < 1 || Hq % Hkv != 0 || kv_valid_len < 1 || kv_valid_len > Sk) return 0;
+    return mi355::fmha_decode_workspace_bytes(B, Hq, Hkv, Sq, Sk, kv_valid_len);
+}
+
+int mi355_fmha_fwd_ws(const void* Q, const void* K, const void* V, void* O, float* LSE, int B, int Hq, int Hkv, int Sq,
+                      int Sk, int D, float scale, int causal, int kv_valid_len, const int64_t* strides, int dtype,
+                      void* workspace, size_t workspace_bytes, void* stream) {
+    if (dtype != MI355_DTYPE_FP16 && dtype != MI355_DTYPE_BF16)
+        return fail(MI355_ERR_BAD_ARGUMENT, "mi355_fmha_fwd_ws: unknown dtype %d", dtype);
+    mi355::FmhaWorkspace ws;
+    ws.kind = mi355::FmhaWorkspace::kCaller;
+    ws.ptr = workspace;
+    ws.bytes = workspace_bytes;
+    return fmha_checked("mi355_fmha_fwd_ws", Q, K, V, O, LSE, B, Hq, Hkv, Sq, Sk, D, scale, causal, kv_valid_len,
+                        strides ? strides_from(strides) : contiguous_strides(Hq, Hkv, Sq, Sk, D), dtype, stream, 0, ws);
+}
+
+int mi355_internal_fmha_fwd_variant(const void* Q, const void* K, const void* V, void* O, float* LSE, int B, int Hq, int Hkv,
+                                    int Sq, int Sk, int D, float scale, int causal, int kv_valid_len, const int64_t* strides,
+                                    int dtype, int variant, void* stream) {
+    return fmha_checked("mi355_internal_fmha_fwd_variant", Q, K, V, O, LSE, B, Hq, Hkv, Sq, Sk, D, scale, causal, kv_valid_len,
+                        strides ? strides_from(strides) : contiguous_strides(Hq, Hkv, Sq, Sk, D), dtype, stream, variant);
+}
+
+int mi355_internal_hgemm_variant(const void* A, const void* B, void* C, int M, int N, int K, int64_t lda, int64_t ldb,
+                                 int64_t ldc, int layout, int dtype, int variant, void* stream) {
+    return hgemm_impl("mi355_internal_hgemm_variant", dtype, A, B, C, nullptr, M, N, K, lda, ldb, ldc, 0, layout, stream, variant);
 }
 
 static bool aligned16(const void* p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; }

@@ -16,6 +16,7 @@
 //
 // Mask semantics are those of the prefill kernel (keys >= kv_valid_len masked; causal: key j visible to query i
 // iff j <= i + Sk - Sq).
+#include <atomic>
 #include <map>
 #include <mutex>
 #include <utility>
@@ -306,9 +307,42 @@ bool fmha_decode_applicable(int B, int Hq, int Hkv, int Sq, int Sk, int kv_valid
     return (long)group * Sq <= 32 && kv_valid_len >= 512 && Sk >= kv_valid_len && B >= 1;
 }
 
-// Workspace for the partial results: one buffer per (device, stream), allocated stream-ordered on first use and
-// regrown (never shrunk) when a call needs more. Calls on one stream are ordered, so they can share it; calls on
-// different streams get different buffers. Steady-state calls allocate nothing.
+// How a call is cut into work units, and what its partial results occupy.
+struct DecodePlan {
+    int splits, tiles_per_split;
+    long units;
+    size_t bytes;
+};
+static DecodePlan decode_plan(int B, int Hq, int Hkv, int Sq, int kv_valid) {
+    using namespace dec;
+    const int ncols = (Hq / Hkv) * Sq;
+    const int tiles = (kv_valid + TK - 1) / TK;
+    // about three waves (one workgroup) per CU in flight, at least 4 key tiles (128 keys) per wave
+    int splits = (256 * WAVES) / (B * Hkv);
+    splits = splits < 1 ? 1 : splits;
+    const int max_splits = (tiles + 3) / 4;
+    if (splits > max_splits) splits = max_splits;
+    if (splits > kMaxSplits) splits = kMaxSplits;
+    DecodePlan p;
+    p.tiles_per_split = (tiles + splits - 1) / splits;
+    p.splits = (tiles + p.tiles_per_split - 1) / p.tiles_per_split;
+    p.units = (long)B * Hkv * p.splits;
+    p.bytes = (size_t)p.units * ncols * PART_STRIDE * sizeof(float);
+    return p;
+}
+
+size_t fmha_decode_workspace_bytes(int B, int Hq, int Hkv, int Sq, int Sk, int kv_valid_len) {
+    if (!fmha_decode_applicable(B, Hq, Hkv, Sq, Sk, kv_valid_len)) return 0;
+    return decode_plan(B, Hq, Hkv, Sq, kv_valid_len).bytes;
+}
+
+// The library's own workspace: one buffer per (device, stream), allocated on first use and replaced by a larger one when
+// a call needs more. A buffer that has been handed to a kernel is NEVER freed: a HIP graph captured earlier may hold
+// its address, so replaced buffers stay allocated until the process ends (each replacement is at least 1.5x larger, so
+// together they hold less than three times the largest request). Calls on one stream are ordered, so they can share a
+// buffer; calls on different streams get different ones. Nothing can be allocated while the stream is capturing: such a
+// call fails with hipErrorStreamCaptureUnsupported unless an earlier call on the same stream already made the buffer
+// large enough (run the step once before capturing it, or hand in a workspace of your own).
 static hipError_t decode_workspace(size_t bytes, hipStream_t stream, float** out) {
     struct Buf {
         void* ptr = nullptr;
@@ -322,18 +356,15 @@ static hipError_t decode_workspace(size_t bytes, hipStream_t stream, float** out
     std::lock_guard<std::mutex> lock(mu);
     Buf& b = bufs[std::make_pair(dev, stream)];
     if (b.size < bytes) {
-        if (b.ptr != nullptr) {
-            e = hipFreeAsync(b.ptr, stream);  // ordered after the kernels already queued on this stream
-            b.ptr = nullptr;
-            b.size = 0;
-            if (e != hipSuccess) return e;
-        }
-        size_t want = bytes < (size_t(4) << 20) ? (size_t(4) << 20) : bytes + bytes / 2;
-        e = hipMallocAsync(&b.ptr, want, stream);
-        if (e != hipSuccess) {
-            b.ptr = nullptr;
-            return e;
-        }
+        hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+        e = hipStreamIsCapturing(stream, &cap);
+        if (e != hipSuccess) return e;
+        if (cap != hipStreamCaptureStatusNone) return hipErrorStreamCaptureUnsupported;
+        const size_t want = bytes < (size_t(4) << 20) ? (size_t(4) << 20) : bytes + bytes / 2;
+        void* fresh = nullptr;
+        e = hipMalloc(&fresh, want);
+        if (e != hipSuccess) return e;
+        b.ptr = fresh;   // the previous buffer, if any, stays allocated (see above)
         b.size = want;
     }
     *out = static_cast<float*>(b.ptr);
@@ -343,26 +374,25 @@ static hipError_t decode_workspace(size_t bytes, hipStream_t stream, float** out
 template <typename T>
 hipError_t fmha_decode_dispatch(const T* Q, const T* K, const T* V, T* O, float* LSE, int B, int Hq,
                                 int Hkv, int Sq, int Sk, float scale, int causal, int kv_valid, const FmhaStrides& sd,
-                                hipStream_t stream) {
+                                const FmhaWorkspace& ws, hipStream_t stream) {
     using namespace dec;
     static DynamicLdsOnce lds_once;
     if (hipError_t e = lds_once.ensure(reinterpret_cast<const void*>(fmha_decode_split_kernel<T>), LDS_BYTES); e != hipSuccess) return e;
-    const int group = Hq / Hkv;
-    const int ncols = group * Sq;
-    const int tiles = (kv_valid + TK - 1) / TK;
-    // about three waves (one workgroup) per CU in flight, at least 4 key tiles (128 keys) per wave
-    int splits = (256 * WAVES) / (B * Hkv);
-    splits = splits < 1 ? 1 : splits;
-    int max_splits = (tiles + 3) / 4;
-    if (splits > max_splits) splits = max_splits;
-    if (splits > kMaxSplits) splits = kMaxSplits;
-    const int tiles_per_split = (tiles + splits - 1) / splits;
-    splits = (tiles + tiles_per_split - 1) / tiles_per_split;
-    const long units = (long)B * Hkv * splits;
-    const size_t bytes = (size_t)units * ncols * PART_STRIDE * sizeof(float);
+    const DecodePlan plan = decode_plan(B, Hq, Hkv, Sq, kv_valid);
+    const int splits = plan.splits, tiles_per_split = plan.tiles_per_split;
+    const long units = plan.units;
 
     float* part = nullptr;
-    hipError_t e = decode_workspace(bytes, stream, &part);
+    hipError_t e = hipSuccess;
+    switch (ws.kind) {
+        case FmhaWorkspace::kCaller:
+            if (ws.ptr == nullptr || ws.bytes < plan.bytes || reinterpret_cast<uintptr_t>(ws.ptr) % 16 != 0) return hipErrorInvalidValue;
+            part = static_cast<float*>(ws.ptr);
+            break;
+        default:
+            e = decode_workspace(plan.bytes, stream, &part);
+            break;
+    }
     if (e != hipSuccess) return e;
     const float scale_log2 = scale * 1.4426950408889634f;
     const unsigned blocks = (unsigned)((units + WAVES - 1) / WAVES);
@@ -377,8 +407,8 @@ hipError_t fmha_decode_dispatch(const T* Q, const T* K, const T* V, T* O, float*
 }
 
 template hipError_t fmha_decode_dispatch<half_t>(const half_t*, const half_t*, const half_t*, half_t*, float*, int, int, int, int,
-                                                  int, float, int, int, const FmhaStrides&, hipStream_t);
+                                                  int, float, int, int, const FmhaStrides&, const FmhaWorkspace&, hipStream_t);
 template hipError_t fmha_decode_dispatch<bf16_t>(const bf16_t*, const bf16_t*, const bf16_t*, bf16_t*, float*, int, int, int, int,
-                                                 int, float, int, int, const FmhaStrides&, hipStream_t);
+                                                 int, float, int, int, const FmhaStrides&, const FmhaWorkspace&, hipStream_t);
 
 }  // namespace mi355

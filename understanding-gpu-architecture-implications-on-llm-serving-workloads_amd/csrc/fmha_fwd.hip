@@ -657,21 +657,18 @@ static hipError_t launch_fmha(const T* Q, const T* K, const T* V, T* O, float* L
     return hipGetLastError();
 }
 
-int g_fmha_variant = 0;  // tuning hook: 0 = heuristic, 1 = 4 waves x 32 queries, 2 = 8 waves x 32 queries, 3 = ping-pong
-
 template <typename T>
 static hipError_t fmha_fwd_dispatch_t(const void* Q, const void* K, const void* V, void* O, float* LSE, int B, int Hq, int Hkv,
                                       int Sq, int Sk, float scale, int causal, int kv_valid_len, const FmhaStrides& sd,
-                                      hipStream_t stream) {
+                                      int variant, const FmhaWorkspace& ws, hipStream_t stream) {
     const T* q = static_cast<const T*>(Q);
     const T* k = static_cast<const T*>(K);
     const T* v = static_cast<const T*>(V);
     T* o = static_cast<T*>(O);
-    int variant = g_fmha_variant;
     // the split-KV and ping-pong kernels address a K/V tile with 32-bit byte offsets from its first row
     const bool rows_fit_32bit = sd.k_row < (1L << 24) && sd.v_row < (1L << 24);
     if ((variant == 0 || variant == 4) && rows_fit_32bit && fmha_decode_applicable(B, Hq, Hkv, Sq, Sk, kv_valid_len))
-        return fmha_decode_dispatch<T>(q, k, v, o, LSE, B, Hq, Hkv, Sq, Sk, scale, causal, kv_valid_len, sd, stream);
+        return fmha_decode_dispatch<T>(q, k, v, o, LSE, B, Hq, Hkv, Sq, Sk, scale, causal, kv_valid_len, sd, ws, stream);
     if (variant == 0 || variant == 4) {
         // 256-query ping-pong workgroups once there are enough of them to fill the 256 CUs, otherwise 128-query ones
         const long wg256 = (long)((Sq + 255) / 256) * Hq * B;
@@ -687,12 +684,10 @@ static hipError_t fmha_fwd_dispatch_t(const void* Q, const void* K, const void* 
 
 hipError_t fmha_fwd_dispatch(const void* Q, const void* K, const void* V, void* O, float* LSE, int B, int Hq, int Hkv,
                              int Sq, int Sk, float scale, int causal, int kv_valid_len, const FmhaStrides& sd, int dtype,
-                             hipStream_t stream) {
+                             int variant, const FmhaWorkspace& ws, hipStream_t stream) {
     if (dtype == MI355_DTYPE_BF16)
-        return fmha_fwd_dispatch_t<bf16_t>(Q, K, V, O, LSE, B, Hq, Hkv, Sq, Sk, scale, causal, kv_valid_len, sd, stream);
-    return fmha_fwd_dispatch_t<half_t>(Q, K, V, O, LSE, B, Hq, Hkv, Sq, Sk, scale, causal, kv_valid_len, sd, stream);
+        return fmha_fwd_dispatch_t<bf16_t>(Q, K, V, O, LSE, B, Hq, Hkv, Sq, Sk, scale, causal, kv_valid_len, sd, variant, ws, stream);
+    return fmha_fwd_dispatch_t<half_t>(Q, K, V, O, LSE, B, Hq, Hkv, Sq, Sk, scale, causal, kv_valid_len, sd, variant, ws, stream);
 }
 
 }  // namespace mi355
-
-extern "C" void mi355_debug_set_fmha_variant(int v) { mi355::g_fmha_variant = v; }

@@ -831,8 +831,6 @@ static hipError_t launch_smallm_nt(const T* A, const T* B, T* C, const T* R, int
     return hipGetLastError();
 }
 
-int g_gemm_variant = 0;  // tuning hook: 0 = heuristic, 1 = force 256x256 tiles, 2 = force 128x128 tiles
-
 template <typename T, bool A_KC, bool B_KC, int BM, int BN, int WM, int WN, int EPI = 0, bool RAGGED = false>
 static hipError_t launch_main(const T* A, const T* B, T* C, const T* R, int M, int N, int K, long lda, long ldb,
                               long ldc, long ldr, hipStream_t stream) {
@@ -864,7 +862,7 @@ static bool few_rows_prefer_tiles(int M, int N, int K, bool nt) {
 
 template <typename T, bool A_KC, bool B_KC>
 static hipError_t launch_layout(const T* A, const T* B, T* C, const T* R, int M, int N, int K, long lda, long ldb,
-                                long ldc, long ldr, hipStream_t stream) {
+                                long ldc, long ldr, int variant, hipStream_t stream) {
     const bool aligned = (reinterpret_cast<uintptr_t>(A) % 16 == 0) && (reinterpret_cast<uintptr_t>(B) % 16 == 0) &&
                          (reinterpret_cast<uintptr_t>(C) % 16 == 0) && (lda % 8 == 0) && (ldb % 8 == 0) &&
                          (ldc % 8 == 0) && (reinterpret_cast<uintptr_t>(R) % 16 == 0) && (ldr % 8 == 0);
@@ -884,7 +882,7 @@ static hipError_t launch_layout(const T* A, const T* B, T* C, const T* R, int M,
     // Fewer than ~3/4 x 256 tiles of 128x128 cannot occupy the CUs: halve the tile so that twice as many workgroups pull
     // on the memory system (64 x 14336 x 4096 NT: 22 us instead of 27.5; 1024^3: 7 us instead of 9.5). Layout NT halves
     // the tile along N (128x64).
-    const bool few_tiles = ragged_ok && (long)((M + 127) / 128) * ((N + 127) / 128) < 192 && g_gemm_variant == 0;
+    const bool few_tiles = ragged_ok && (long)((M + 127) / 128) * ((N + 127) / 128) < 192 && variant == 0;
     if constexpr (A_KC && B_KC) {
         if (few_tiles) {
             if (M % 128 == 0 && N % 64 == 0)
@@ -906,8 +904,8 @@ static hipError_t launch_layout(const T* A, const T* B, T* C, const T* R, int M,
     int choice = 0;
     if (fits256 && (tiles256 >= 192 || !fits128)) choice = 1;
     else if (fits128) choice = 2;
-    if (g_gemm_variant == 1 && fits256) choice = 1;
-    if (g_gemm_variant == 2 && fits128) choice = 2;
+    if (variant == 1 && fits256) choice = 1;
+    if (variant == 2 && fits128) choice = 2;
     switch (choice) {
         case 1: return launch_main<T, A_KC, B_KC, 256, 256, 2, 4>(A, B, C, R, M, N, K, lda, ldb, ldc, ldr, stream);
         case 2: return launch_main<T, A_KC, B_KC, 128, 128, 2, 2>(A, B, C, R, M, N, K, lda, ldb, ldc, ldr, stream);
@@ -916,7 +914,7 @@ static hipError_t launch_layout(const T* A, const T* B, T* C, const T* R, int M,
     // ragged M / N on the same tiles: N (and M for layout TN) a multiple of 8, so 16-byte chunks never straddle the end
     if (ragged_ok) {
         const long t256 = (long)((M + 255) / 256) * ((N + 255) / 256);
-        if ((t256 >= 192 && g_gemm_variant != 2) || g_gemm_variant == 1)
+        if ((t256 >= 192 && variant != 2) || variant == 1)
             return launch_main<T, A_KC, B_KC, 256, 256, 2, 4, 0, true>(A, B, C, R, M, N, K, lda, ldb, ldc, ldr, stream);
         return launch_main<T, A_KC, B_KC, 128, 128, 2, 2, 0, true>(A, B, C, R, M, N, K, lda, ldb, ldc, ldr, stream);
     }
@@ -967,25 +965,23 @@ hipError_t hgemm_silu_mul_dispatch(const void* A, const void* B, void* C, int M,
 
 template <typename T>
 static hipError_t gemm_dispatch_t(const void* A, const void* B, void* C, const void* R, int M, int N, int K, long lda,
-                                  long ldb, long ldc, long ldr, int layout, hipStream_t stream) {
+                                  long ldb, long ldc, long ldr, int layout, int variant, hipStream_t stream) {
     const T* a = static_cast<const T*>(A);
     const T* b = static_cast<const T*>(B);
     T* c = static_cast<T*>(C);
     const T* r = static_cast<const T*>(R);
     switch (layout) {
-        case MI355_GEMM_NN: return launch_layout<T, true, false>(a, b, c, r, M, N, K, lda, ldb, ldc, ldr, stream);
-        case MI355_GEMM_NT: return launch_layout<T, true, true>(a, b, c, r, M, N, K, lda, ldb, ldc, ldr, stream);
-        case MI355_GEMM_TN: return launch_layout<T, false, false>(a, b, c, r, M, N, K, lda, ldb, ldc, ldr, stream);
+        case MI355_GEMM_NN: return launch_layout<T, true, false>(a, b, c, r, M, N, K, lda, ldb, ldc, ldr, variant, stream);
+        case MI355_GEMM_NT: return launch_layout<T, true, true>(a, b, c, r, M, N, K, lda, ldb, ldc, ldr, variant, stream);
+        case MI355_GEMM_TN: return launch_layout<T, false, false>(a, b, c, r, M, N, K, lda, ldb, ldc, ldr, variant, stream);
         default: return hipErrorInvalidValue;
     }
 }
 
 hipError_t hgemm_dispatch(const void* A, const void* B, void* C, const void* R, int M, int N, int K, long lda, long ldb,
-                          long ldc, long ldr, int layout, int dtype, hipStream_t stream) {
-    if (dtype == MI355_DTYPE_BF16) return gemm_dispatch_t<bf16_t>(A, B, C, R, M, N, K, lda, ldb, ldc, ldr, layout, stream);
-    return gemm_dispatch_t<half_t>(A, B, C, R, M, N, K, lda, ldb, ldc, ldr, layout, stream);
+                          long ldc, long ldr, int layout, int dtype, int variant, hipStream_t stream) {
+    if (dtype == MI355_DTYPE_BF16) return gemm_dispatch_t<bf16_t>(A, B, C, R, M, N, K, lda, ldb, ldc, ldr, layout, variant, stream);
+    return gemm_dispatch_t<half_t>(A, B, C, R, M, N, K, lda, ldb, ldc, ldr, layout, variant, stream);
 }
 
 }  // namespace mi355
-
-extern "C" void mi355_debug_set_gemm_variant(int v) { mi355::g_gemm_variant = v; }

@@ -68,9 +68,10 @@ std::tuple<at::Tensor, at::Tensor> run_fmha(const at::Tensor& q, const at::Tenso
     at::Tensor qc = readable_in_place(q) ? q : q.contiguous();
     at::Tensor kc = readable_in_place(k) ? k : k.contiguous();
     at::Tensor vc = readable_in_place(v) ? v : v.contiguous();
-    // The output takes q's memory layout when q is a dense permuted view (so `out.transpose(1, 2).contiguous()` in the
-    // caller costs nothing for a [B, S, H, D] projection); otherwise it is a contiguous [B, H, S, D] tensor.
-    at::Tensor o = qc.is_non_overlapping_and_dense() ? at::empty_like(qc) : at::empty(qc.sizes(), qc.options());
+    // The result is a freshly allocated contiguous [B, H, S, D] tensor whatever the strides of q, as in the reference
+    // (`zeros_like` of a `.contiguous()` input, semi/fmha_2_amd.cpp:336; kernels/fmha/pkg/fmha_unified/ops.py:23-29), so
+    // callers may `.view()` it. empty() instead of zeros(): the kernel writes every element.
+    at::Tensor o = at::empty(qc.sizes(), qc.options());
     at::Tensor lse;
     float* lse_ptr = nullptr;
     if (want_lse) {

@@ -54,8 +54,10 @@ at::Tensor run_gemm(const at::Tensor& a, const at::Tensor& b, int layout, const 
     at::Tensor c = at::empty({M, N}, a.options());
     hipStream_t stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream();
     auto entry = bf16 ? &mi355_gemm_bf16 : &mi355_hgemm;
-    int rc = entry(ac.data_ptr(), bc.data_ptr(), c.data_ptr(), (int)M, (int)N, (int)K, ac.stride(0), bc.stride(0), N,
-                         layout, stream);
+    // Leading dimensions are the logical row lengths of the contiguous operands, not stride(0): torch ignores the stride of
+    // a size-1 dimension when it decides contiguity, so a [1, K] operand may carry any stride(0).
+    const int64_t lda = ac.size(1), ldb = bc.size(1);
+    int rc = entry(ac.data_ptr(), bc.data_ptr(), c.data_ptr(), (int)M, (int)N, (int)K, lda, ldb, N, layout, stream);
     TORCH_CHECK(rc == 0, name, ": ", mi355_last_error(), " (code ", rc, ")");
     return c;
 }

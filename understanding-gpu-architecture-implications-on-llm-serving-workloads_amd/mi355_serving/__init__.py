@@ -1,4 +1,5 @@
-"""ctypes binding of libmi355_serving.so (the C ABI declared in include/mi355_serving.h).
+"""ctypes binding of libmi355_serving.so (the C ABI declared in include/mi355_serving.h); the shared library is this
+package's data file, so it is found the same way in the source tree and after `python setup.py install`.
 
 This is the torch-free boundary: plain device pointers and sizes. Tensors are used here only as a convenient way
 to own device memory and a stream; ``hgemm`` / ``fmha_fwd`` take anything with ``data_ptr()``.
@@ -16,8 +17,10 @@ ERR_BAD_ARGUMENT, ERR_UNSUPPORTED = 10001, 10002
 
 EXPORTED_SYMBOLS = ("mi355_hgemm", "mi355_fmha_fwd", "mi355_fmha_fwd_strided", "mi355_fmha_fwd_bf16", "mi355_hgemm_silu_mul", "mi355_hgemm_add", "mi355_rmsnorm", "mi355_rope", "mi355_silu_mul",
                     "mi355_gemm_bf16", "mi355_gemm_silu_mul_bf16", "mi355_gemm_add_bf16", "mi355_rmsnorm_bf16", "mi355_rope_bf16", "mi355_silu_mul_bf16",
-                    "mi355_last_error", "mi355_serving_version",
-                    "mi355_debug_set_gemm_variant", "mi355_debug_set_fmha_variant")
+                    "mi355_fmha_fwd_workspace_bytes", "mi355_fmha_fwd_ws",
+                    "mi355_last_error", "mi355_serving_version")
+# exported for tests and tuning runs, declared in csrc/mi355_serving_internal.h and not in the public header
+INTERNAL_SYMBOLS = ("mi355_internal_hgemm_variant", "mi355_internal_fmha_fwd_variant")
 
 _lib = None
 
@@ -35,7 +38,8 @@ def load():
         return _lib
     if not os.path.exists(LIB_PATH):
         raise FileNotFoundError(
-            "%s is missing: build it with `python build.py` in %s (there is no CPU fallback)" % (LIB_PATH, _HERE))
+            "%s is missing: build it with `python build.py` in %s (there is no CPU fallback)"
+            % (LIB_PATH, os.path.dirname(_HERE)))
     import torch  # noqa: F401  loads the HIP runtime the library binds to
     lib = ctypes.CDLL(LIB_PATH, mode=ctypes.RTLD_GLOBAL)
     vp, i32, i64, f32 = ctypes.c_void_p, ctypes.c_int, ctypes.c_int64, ctypes.c_float
@@ -68,19 +72,21 @@ def load():
     lib.mi355_last_error.restype = ctypes.c_char_p
     lib.mi355_serving_version.argtypes = []
     lib.mi355_serving_version.restype = i32
-    lib.mi355_debug_set_gemm_variant.argtypes = [i32]
-    lib.mi355_debug_set_gemm_variant.restype = None
-    lib.mi355_debug_set_fmha_variant.argtypes = [i32]
-    lib.mi355_debug_set_fmha_variant.restype = None
+    lib.mi355_fmha_fwd_workspace_bytes.argtypes = [i32] * 6
+    lib.mi355_fmha_fwd_workspace_bytes.restype = ctypes.c_size_t
+    lib.mi355_fmha_fwd_ws.argtypes = [vp, vp, vp, vp, vp, i32, i32, i32, i32, i32, i32, f32, i32, i32, ctypes.POINTER(i64), i32,
+                                      vp, ctypes.c_size_t, vp]
+    lib.mi355_fmha_fwd_ws.restype = i32
+    lib.mi355_internal_hgemm_variant.argtypes = [vp, vp, vp, i32, i32, i32, i64, i64, i64, i32, i32, i32, vp]
+    lib.mi355_internal_hgemm_variant.restype = i32
+    lib.mi355_internal_fmha_fwd_variant.argtypes = [vp, vp, vp, vp, vp, i32, i32, i32, i32, i32, i32, f32, i32, i32,
+                                                    ctypes.POINTER(i64), i32, i32, vp]
+    lib.mi355_internal_fmha_fwd_variant.restype = i32
     _lib = lib
     return lib
 
 
-def set_variants(gemm=0, fmha=0):
-    """Pin kernel variants (diagnostics; 0 = let the dispatcher choose by shape)."""
-    lib = load()
-    lib.mi355_debug_set_gemm_variant(int(gemm))
-    lib.mi355_debug_set_fmha_variant(int(fmha))
+DTYPE_FP16, DTYPE_BF16 = 0, 1
 
 
 def _ptr(x):
@@ -105,10 +111,11 @@ def fmha_fwd_raw(q_ptr, k_ptr, v_ptr, o_ptr, lse_ptr, B, Hq, Hkv, Sq, Sk, D, sca
                                  kv_valid_len, stream))
 
 
-def hgemm(a, b, layout="NN", out=None, residual=None):
+def hgemm(a, b, layout="NN", out=None, residual=None, variant=0):
     """C = op(a) op(b) (+ residual) through the C ABI on torch's current stream. a, b: contiguous fp16 or bf16 GPU
     tensors; `residual`: [M, N] rows with a contiguous last dimension, added in the GEMM's epilogue (mi355_hgemm_add);
-    it may be `out` itself."""
+    it may be `out` itself. `variant` != 0 pins a tile shape through the library's internal test hook (1 = 256x256,
+    2 = 128x128) instead of the choice by shape."""
     import torch
     lay = LAYOUTS[layout] if isinstance(layout, str) else int(layout)
     assert a.dtype in (torch.float16, torch.bfloat16) and b.dtype == a.dtype and a.is_cuda and b.is_cuda
@@ -126,15 +133,21 @@ def hgemm(a, b, layout="NN", out=None, residual=None):
     if out is None:
         out = torch.empty((M, N), dtype=a.dtype, device=a.device)
     stream = torch.cuda.current_stream(a.device).cuda_stream
+    # leading dimensions of the contiguous operands (stride(0) of a size-1 dimension is arbitrary in torch)
+    lda, ldb = a.shape[1], b.shape[1]
     if residual is not None:
         if tuple(residual.shape) != (M, N) or residual.dtype != a.dtype or residual.stride(1) != 1:
             raise ValueError("residual must be [%d, %d] %s with a contiguous last dimension" % (M, N, a.dtype))
         entry = load().mi355_gemm_add_bf16 if a.dtype == torch.bfloat16 else load().mi355_hgemm_add
-        _check(entry(_ptr(a), _ptr(b), _ptr(residual), _ptr(out), M, N, K, a.stride(0), b.stride(0), residual.stride(0),
-                     out.stride(0), lay, stream))
+        _check(entry(_ptr(a), _ptr(b), _ptr(residual), _ptr(out), M, N, K, lda, ldb, max(residual.stride(0), N),
+                     max(out.stride(0), N), lay, stream))
+        return out
+    if variant:
+        _check(load().mi355_internal_hgemm_variant(_ptr(a), _ptr(b), _ptr(out), M, N, K, lda, ldb, max(out.stride(0), N), lay,
+                                                   DTYPE_BF16 if a.dtype == torch.bfloat16 else DTYPE_FP16, int(variant), stream))
         return out
     entry = load().mi355_gemm_bf16 if a.dtype == torch.bfloat16 else load().mi355_hgemm
-    _check(entry(_ptr(a), _ptr(b), _ptr(out), M, N, K, a.stride(0), b.stride(0), out.stride(0), lay, stream))
+    _check(entry(_ptr(a), _ptr(b), _ptr(out), M, N, K, lda, ldb, max(out.stride(0), N), lay, stream))
     return out
 
 
@@ -150,12 +163,19 @@ def _bhs_strides(t):
     return [t.stride(0), t.stride(1), t.stride(2)]
 
 
-def fmha_fwd(q, k, v, causal=False, kv_valid_len=None, scale=None, return_lse=True, out=None):
+def fmha_workspace_bytes(B, Hq, Hkv, Sq, Sk, kv_valid_len=None):
+    """Bytes of caller workspace mi355_fmha_fwd_ws needs for these sizes (0 outside the split-KV path)."""
+    return int(load().mi355_fmha_fwd_workspace_bytes(B, Hq, Hkv, Sq, Sk, Sk if kv_valid_len is None else kv_valid_len))
+
+
+def fmha_fwd(q, k, v, causal=False, kv_valid_len=None, scale=None, return_lse=True, out=None, variant=0, workspace=None):
     """Attention forward through the C ABI on torch's current stream. Returns (O, LSE) or O.
 
     q, k, v (and `out`, if given) are [B, H, S, D] fp16 GPU tensors or views with a contiguous last dimension, e.g.
     `x.view(B, S, H, D).transpose(1, 2)`; contiguous tensors take mi355_fmha_fwd, views mi355_fmha_fwd_strided.
-    bfloat16 tensors take mi355_fmha_fwd_bf16.
+    bfloat16 tensors take mi355_fmha_fwd_bf16. `workspace` (a uint8 GPU tensor): mi355_fmha_fwd_ws, which keeps the
+    split-KV partial results there and never allocates. `variant` != 0 pins a kernel through the library's internal test
+    hook (1 = 4 waves, 2 = 8 waves, 3 = 8 waves ping-pong; all keep generation steps off the split-KV path).
     """
     import torch
     assert q.dtype in (torch.float16, torch.bfloat16) and q.dtype == k.dtype == v.dtype and q.is_cuda
@@ -168,7 +188,19 @@ def fmha_fwd(q, k, v, causal=False, kv_valid_len=None, scale=None, return_lse=Tr
     o = torch.empty_like(q) if out is None else out
     lse = torch.empty((B, Hq, Sq), dtype=torch.float32, device=q.device) if return_lse else None
     stream = torch.cuda.current_stream(q.device).cuda_stream
-    if q.dtype == torch.bfloat16:
+    if variant or workspace is not None:
+        assert all(t.stride(3) == 1 for t in (q, k, v, o)), "the last dimension must be contiguous"
+        arr = (ctypes.c_int64 * 12)(*(_bhs_strides(q) + _bhs_strides(k) + _bhs_strides(v) + _bhs_strides(o)))
+        dt = DTYPE_BF16 if q.dtype == torch.bfloat16 else DTYPE_FP16
+        if variant:
+            _check(load().mi355_internal_fmha_fwd_variant(_ptr(q), _ptr(k), _ptr(v), _ptr(o), _ptr(lse), B, Hq, Hkv, Sq, Sk, D,
+                                                          float(scale), int(bool(causal)), int(kv_valid_len), arr, dt, int(variant),
+                                                          stream))
+        else:
+            _check(load().mi355_fmha_fwd_ws(_ptr(q), _ptr(k), _ptr(v), _ptr(o), _ptr(lse), B, Hq, Hkv, Sq, Sk, D, float(scale),
+                                            int(bool(causal)), int(kv_valid_len), arr, dt, _ptr(workspace),
+                                            workspace.numel() * workspace.element_size(), stream))
+    elif q.dtype == torch.bfloat16:
         assert all(t.stride(3) == 1 for t in (q, k, v, o)), "the last dimension must be contiguous"
         arr = (ctypes.c_int64 * 12)(*(_bhs_strides(q) + _bhs_strides(k) + _bhs_strides(v) + _bhs_strides(o)))
         _check(load().mi355_fmha_fwd_bf16(_ptr(q), _ptr(k), _ptr(v), _ptr(o), _ptr(lse), B, Hq, Hkv, Sq, Sk, D, float(scale),
