@@ -34,25 +34,39 @@ PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 MEASURED_TRAFFIC_BYTES = (786975 * 2.0 + 131072 * 1.0) * 1024        # hgemm_main_kernel, 8192^3 NN
 MEASURED_TRAFFIC_BYTES_G2C = (57881 * 2.0 + 448 * 1.0) * 1024          # hgemm_smallm_nn_kernel, 16 x 14336 x 4096
 MEASURED_TRAFFIC_BYTES_FMHA = (26705 * 2.0 + 33280 * 1.0) * 1024     # fmha_fwd_pingpong_kernel, F4
+# the figures above are constants copied from these counter summaries (they are not read at run time)
+TRAFFIC_SOURCE = {"gemm": "constant from profiles/hgemm_main_kernel_8192_nn.md (rocprofv3 --pmc FETCH_SIZE, WRITE_SIZE)",
+                  "g2c": "constant from profiles/hgemm_smallm_nn_kernel_g2c_decode.md",
+                  "fmha": "constant from profiles/fmha_fwd_pingpong_kernel_f4_causal_gqa.md"}
 
 
 def log(*a):
     print(*a, file=sys.stderr, flush=True)
 
 
-def time_launches(fn, iters, warmup):
-    """Average duration (ms) of `iters` back-to-back launches, HIP events on the current stream."""
+def time_launches(fn, iters, warmup, stats=False):
+    """Durations (ms) of `iters` back-to-back launches after `warmup` untimed ones, HIP events on the current stream.
+    The mean is (last event - first event) / iters; with stats=True also the median and minimum of the per-launch
+    intervals between consecutive events (each interval includes the event's own overhead of a few microseconds, which
+    matters only for the microsecond-scale kernels)."""
     import torch
     for _ in range(warmup):
         fn()
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(iters + 1 if stats else 2)]
     torch.cuda.synchronize()
-    e0.record()
-    for _ in range(iters):
+    ev[0].record()
+    for i in range(iters):
         fn()
-    e1.record()
-    e1.synchronize()
-    return e0.elapsed_time(e1) / iters
+        if stats:
+            ev[i + 1].record()
+    if not stats:
+        ev[1].record()
+    ev[-1].synchronize()
+    mean = ev[0].elapsed_time(ev[-1]) / iters
+    if not stats:
+        return mean
+    per = sorted(ev[i].elapsed_time(ev[i + 1]) for i in range(iters))
+    return {"ms": mean, "ms_median": per[len(per) // 2], "ms_min": per[0], "launches": iters, "warmup": warmup}
 
 
 def causal_pairs(Sq, Sk):
@@ -168,48 +182,66 @@ def main():
     value = (gemm_flops + fmha_flops) / (ms_per_step * 1e-3) / 1e12
 
     # ---- per-kernel launch durations (HIP events on the launch stream) --------------------------------------------
-    gemm_ms = time_launches(gemm, args.steps, 2)
-    fmha_ms = time_launches(fmha, args.steps, 2)
+    n_timed, n_warm = max(args.steps, 50), max(args.warmup, 10)
+    gemm_t = time_launches(gemm, n_timed, n_warm, stats=True)
+    fmha_t = time_launches(fmha, n_timed, n_warm, stats=True)
+    gemm_ms, fmha_ms = gemm_t["ms"], fmha_t["ms"]
     gemm_tf = gemm_flops / (gemm_ms * 1e-3) / 1e12
     fmha_tf = fmha_flops / (fmha_ms * 1e-3) / 1e12
     kernels = {
-        "hgemm_8192x8192x8192_nn": {"ms": gemm_ms, "tflops": gemm_tf, "pct_of_fp16_mfma_peak": 100 * gemm_tf / PEAK_FP16_TFLOPS},
-        "fmha_fwd_causal_gqa_b1_h32_8_s4096_d128": {
-            "ms": fmha_ms, "tflops": fmha_tf, "pct_of_fp16_mfma_peak": 100 * fmha_tf / PEAK_FP16_TFLOPS,
-            "tflops_reference_convention_4s2dh": fmha_flops_ref_convention / (fmha_ms * 1e-3) / 1e12},
+        "hgemm_8192x8192x8192_nn": dict(gemm_t, tflops=gemm_tf, pct_of_fp16_mfma_peak=100 * gemm_tf / PEAK_FP16_TFLOPS,
+                                        tflops_at_median=gemm_flops / gemm_t["ms_median"] / 1e9,
+                                        tflops_at_min=gemm_flops / gemm_t["ms_min"] / 1e9),
+        "fmha_fwd_causal_gqa_b1_h32_8_s4096_d128": dict(
+            fmha_t, tflops=fmha_tf, pct_of_fp16_mfma_peak=100 * fmha_tf / PEAK_FP16_TFLOPS,
+            tflops_at_median=fmha_flops / fmha_t["ms_median"] / 1e9, tflops_at_min=fmha_flops / fmha_t["ms_min"] / 1e9,
+            tflops_reference_convention_4s2dh=fmha_flops_ref_convention / (fmha_ms * 1e-3) / 1e12),
     }
     roofline = {"kernel": "hgemm_main_kernel (8192^3, NN)", "bound": "mfma", "achieved": gemm_tf, "peak": PEAK_FP16_TFLOPS,
-                "unit": "TFLOP/s", "frac": gemm_tf / PEAK_FP16_TFLOPS, "traffic": MEASURED_TRAFFIC_BYTES}
+                "unit": "TFLOP/s", "frac": gemm_tf / PEAK_FP16_TFLOPS, "traffic": MEASURED_TRAFFIC_BYTES,
+                "traffic_source": TRAFFIC_SOURCE["gemm"]}
     roofline_fmha = {"kernel": "fmha_fwd_pingpong_kernel (F4)", "bound": "mfma", "achieved": fmha_tf, "peak": PEAK_FP16_TFLOPS,
-                     "unit": "TFLOP/s", "frac": fmha_tf / PEAK_FP16_TFLOPS, "traffic": MEASURED_TRAFFIC_BYTES_FMHA}
+                     "unit": "TFLOP/s", "frac": fmha_tf / PEAK_FP16_TFLOPS, "traffic": MEASURED_TRAFFIC_BYTES_FMHA,
+                     "traffic_source": TRAFFIC_SOURCE["fmha"]}
 
     # ---- the other benchmark configurations (quick timings) ----------------------------------------------------------
     other = {}
     roofline_g2c = None
     if not args.no_other_configs:
-        def t_gemm(m, n, kk, iters=20):
-            x = so.randn_fp16((m, kk), 1).to(dev)
-            w = so.randn_fp16((kk, n), 2, 0.02).to(dev)
+        def t_gemm(m, n, kk, iters=50):
+            x_h, w_h = so.randn_fp16((m, kk), 1), so.randn_fp16((kk, n), 2, 0.02)
+            x, w = x_h.to(dev), w_h.to(dev)
             out = torch.empty((m, n), dtype=torch.float16, device=dev)
-            ms = time_launches(lambda: lib.hgemm_raw(x.data_ptr(), w.data_ptr(), out.data_ptr(), m, n, kk, kk, n, n,
-                                                     lib.GEMM_NN, stream), iters, 3)
+            t = time_launches(lambda: lib.hgemm_raw(x.data_ptr(), w.data_ptr(), out.data_ptr(), m, n, kk, kk, n, n,
+                                                    lib.GEMM_NN, stream), iters, 10, stats=True)
+            ms = t["ms"]
             fl, by = 2.0 * m * n * kk, 2.0 * (m * kk + kk * n + m * n)
-            return {"ms": ms, "tflops": fl / ms / 1e9, "pct_of_fp16_mfma_peak": 100 * fl / ms / 1e9 / PEAK_FP16_TFLOPS,
-                    "gbs": by / ms / 1e6, "pct_of_hbm_peak": 100 * by / ms / 1e6 / PEAK_HBM_GBS}
+            rows_ = torch.arange(0, m, max(1, m // 64))
+            ok_, _ = so.gemm_tolerance_ok(out[rows_.to(dev)], so.gemm_ref(x_h[rows_], w_h), kk)
+            return dict(t, tflops=fl / ms / 1e9, pct_of_fp16_mfma_peak=100 * fl / ms / 1e9 / PEAK_FP16_TFLOPS,
+                        gbs=by / ms / 1e6, pct_of_hbm_peak=100 * by / ms / 1e6 / PEAK_HBM_GBS, within_tolerance=bool(ok_))
         other["G1_gemm_1024"] = t_gemm(1024, 1024, 1024)
         other["G2a_gemm_4096"] = t_gemm(4096, 4096, 4096)
         other["G2c_gemm_decode_16x14336x4096"] = t_gemm(16, 14336, 4096)
         g2c = other["G2c_gemm_decode_16x14336x4096"]
         roofline_g2c = {"kernel": "hgemm_smallm_nn_kernel (G2c: 16 x 14336 x 4096, NN)", "bound": "hbm", "achieved": g2c["gbs"],
-                        "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": g2c["gbs"] / PEAK_HBM_GBS, "traffic": MEASURED_TRAFFIC_BYTES_G2C}
-        q3, k3, v3 = (t.to(dev) for t in so.fmha_inputs(4, 32, 32, 1024, 1024, seed=42))
+                        "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": g2c["gbs"] / PEAK_HBM_GBS, "traffic": MEASURED_TRAFFIC_BYTES_G2C,
+                        "traffic_source": TRAFFIC_SOURCE["g2c"]}
+        q3h, k3h, v3h = so.fmha_inputs(4, 32, 32, 1024, 1024, seed=42)
+        q3, k3, v3 = q3h.to(dev), k3h.to(dev), v3h.to(dev)
         o3 = torch.empty_like(q3)
-        ms3 = time_launches(lambda: lib.fmha_fwd_raw(q3.data_ptr(), k3.data_ptr(), v3.data_ptr(), o3.data_ptr(), None, 4, 32,
-                                                     32, 1024, 1024, 128, scale, 0, 1024, stream), 20, 3)
+        l3 = torch.empty((4, 32, 1024), dtype=torch.float32, device=dev)
+        t3 = time_launches(lambda: lib.fmha_fwd_raw(q3.data_ptr(), k3.data_ptr(), v3.data_ptr(), o3.data_ptr(), l3.data_ptr(), 4, 32,
+                                                    32, 1024, 1024, 128, scale, 0, 1024, stream), 50, 10, stats=True)
+        ms3 = t3["ms"]
         fl3 = 4.0 * 4 * 32 * 128 * 1024 * 1024
-        other["F3_fmha_noncausal_b4_h32_s1024"] = {"ms": ms3, "tflops": fl3 / ms3 / 1e9,
-                                                   "pct_of_fp16_mfma_peak": 100 * fl3 / ms3 / 1e9 / PEAK_FP16_TFLOPS}
-        del q3, k3, v3, o3
+        ok3 = True
+        for (bb, hh) in ((0, 0), (1, 17), (3, 31)):
+            orf, lrf = so.attention_ref(q3h[bb:bb + 1, hh:hh + 1], k3h[bb:bb + 1, hh:hh + 1], v3h[bb:bb + 1, hh:hh + 1])
+            ok3 = ok3 and so.fmha_tolerance_ok(o3[bb:bb + 1, hh:hh + 1], l3[bb:bb + 1, hh:hh + 1], orf, lrf)[0]
+        other["F3_fmha_noncausal_b4_h32_s1024"] = dict(t3, tflops=fl3 / ms3 / 1e9, within_tolerance=bool(ok3),
+                                                       pct_of_fp16_mfma_peak=100 * fl3 / ms3 / 1e9 / PEAK_FP16_TFLOPS)
+        del q3, k3, v3, o3, l3
         # the vendor libraries on the same box, same operands, same timing loop (context for the figures above; not this code)
         cv = torch.empty_like(c)
         ms_v = time_launches(lambda: torch.matmul(a, b, out=cv), 20, 3)
@@ -261,14 +293,16 @@ def main():
             other["fmha_decode_b%d_h32_8_sk%d" % (bd, skd)] = {"ms": ms_d, "gbs": by_d / ms_d / 1e6,
                                                                "pct_of_hbm_peak": 100 * by_d / ms_d / 1e6 / PEAK_HBM_GBS}
         del xd, wd_nt, od, qd, kd, vd, o_d
-        # L5: Llama-3-8B-shaped prefill layer at s = 8192, per stage
+        # L5: Llama-3-8B-shaped prefill layer at s = 8192, per stage; every stage is checked on sampled token rows against
+        # the oracle fed the GPU's own previous-stage output, and the chain's end against the pure fp32 chain
         S5, H5, F5 = 8192, 4096, 14336
-        x5 = so.randn_fp16((S5, H5), 0).to(dev)
-        wqkv, wo = so.randn_fp16((H5, 6144), 1, 0.02).to(dev), so.randn_fp16((H5, H5), 2, 0.02).to(dev)
-        wgu, wd = so.randn_fp16((H5, 2 * F5), 3, 0.02).to(dev), so.randn_fp16((F5, H5), 4, 0.02).to(dev)
+        x5h = so.randn_fp16((S5, H5), 0)
+        wqkv_h, wo_h = so.randn_fp16((H5, 6144), 1, 0.02), so.randn_fp16((H5, H5), 2, 0.02)
+        wgu_h, wd_h = so.randn_fp16((H5, 2 * F5), 3, 0.02), so.randn_fp16((F5, H5), 4, 0.02)
+        x5, wqkv, wo, wgu, wd = (t.to(dev) for t in (x5h, wqkv_h, wo_h, wgu_h, wd_h))
         st = {}
-        def stage(name, fn, flops, iters=5):
-            ms = time_launches(fn, iters, 1)
+        def stage(name, fn, flops, iters=10):
+            ms = time_launches(fn, iters, 3)
             st[name] = {"ms": ms, "tflops": flops / ms / 1e9}
         qkv5 = torch.empty((S5, 6144), dtype=torch.float16, device=dev)
         stage("qkv_gemm", lambda: lib.hgemm(x5, wqkv, out=qkv5), 2.0 * S5 * H5 * 6144)
@@ -276,8 +310,9 @@ def main():
         k5 = qkv5[:, 4096:5120].reshape(S5, 8, 128).permute(1, 0, 2)[None].contiguous()
         v5 = qkv5[:, 5120:].reshape(S5, 8, 128).permute(1, 0, 2)[None].contiguous()
         o5 = torch.empty_like(q5)
+        lse5 = torch.empty((1, 32, S5), dtype=torch.float32, device=dev)
         stage("fmha_causal_gqa_s8192", lambda: lib.fmha_fwd_raw(q5.data_ptr(), k5.data_ptr(), v5.data_ptr(), o5.data_ptr(),
-                                                                 None, 1, 32, 8, S5, S5, 128, scale, 1, S5, stream),
+                                                                 lse5.data_ptr(), 1, 32, 8, S5, S5, 128, scale, 1, S5, stream),
               4.0 * 32 * 128 * causal_pairs(S5, S5))
         a5 = o5[0].permute(1, 0, 2).reshape(S5, H5).contiguous()
         op5 = torch.empty((S5, H5), dtype=torch.float16, device=dev)
@@ -287,20 +322,46 @@ def main():
         act5 = (torch.nn.functional.silu(gu5[:, :F5].float()) * gu5[:, F5:].float()).half()
         dn5 = torch.empty((S5, H5), dtype=torch.float16, device=dev)
         stage("down_gemm", lambda: lib.hgemm(act5, wd, out=dn5), 2.0 * S5 * F5 * H5)
+        rows5 = torch.arange(0, S5, 61)
+        c5 = {"qkv": qkv5.cpu(), "attn": o5.cpu(), "attn_lse": lse5.cpu(), "oproj": op5.cpu(), "gate_up": gu5.cpu(),
+              "act": act5.cpu(), "down": dn5.cpu()}
+        ref5 = so.llama_layer_ref(x5h, wqkv_h, wo_h, wgu_h, wd_h, rows=rows5, stage_inputs={
+            "attn_in": c5["qkv"], "oproj_in": c5["attn"], "gu_in": c5["oproj"], "act_in": c5["gate_up"], "down_in": c5["act"]})
+        for sname, cname, kk in (("qkv_gemm", "qkv", H5), ("oproj_gemm", "oproj", H5), ("gate_up_gemm", "gate_up", H5),
+                                 ("down_gemm", "down", F5)):
+            st[sname]["within_tolerance"] = bool(so.gemm_tolerance_ok(c5[cname][rows5], ref5[cname], kk)[0])
+        st["fmha_causal_gqa_s8192"]["within_tolerance"] = bool(so.fmha_tolerance_ok(
+            c5["attn"][:, :, rows5], c5["attn_lse"][:, :, rows5], ref5["attn"], ref5["attn_lse"])[0])
+        full5 = so.llama_layer_ref(x5h, wqkv_h, wo_h, wgu_h, wd_h, rows=rows5)
+        rel5 = float((c5["down"][rows5].float() - full5["down"]).norm() / full5["down"].norm())
+        del c5, ref5, full5
         tot_ms = sum(s["ms"] for s in st.values())
         tot_fl = 2.0 * S5 * H5 * 6144 + 4.0 * 32 * 128 * causal_pairs(S5, S5) + 2.0 * S5 * H5 * H5 + 2.0 * S5 * H5 * 2 * F5 + 2.0 * S5 * F5 * H5
         other["L5_llama3_8b_layer_s8192"] = {"stages": st, "kernel_ms_total": tot_ms, "tflops_total": tot_fl / tot_ms / 1e9,
+                                             "within_tolerance": all(s_["within_tolerance"] for s_ in st.values()) and rel5 < 2e-2,
+                                             "end_to_end_relative_frobenius_error": rel5,
+                                             "parity": "every 61st token row of every stage against the fp32 oracle fed the GPU's previous "
+                                                       "stage; end to end against the pure fp32 chain",
                                              "note": "GEMM and attention stages only; reshapes and SiLU*up run in torch and are not timed; no RoPE/norm/residual"}
 
         # the same layer as the in-model adapter runs it: nn.Linear-layout weights, norms, RoPE, residuals, no layout copies
-        del x5, wqkv, wo, wgu, wd, qkv5, q5, k5, v5, o5, a5, op5, gu5, act5, dn5
+        del x5, wqkv, wo, wgu, wd, qkv5, q5, k5, v5, o5, lse5, a5, op5, gu5, act5, dn5, x5h, wqkv_h, wo_h, wgu_h, wd_h
         torch.cuda.empty_cache()
         from llama_layer import FineKVCache
-        layer, _ = llama3_8b_layer(torch, so, dev)
-        xl = so.randn_fp16((1, S5, H5), 18).to(dev)
-        ms_l = time_launches(lambda: layer(xl), 5, 2)
+        layer, _, wl_h = llama3_8b_layer(torch, so, dev, host_weights=True)
+        xl_h = so.randn_fp16((1, S5, H5), 18)
+        xl = xl_h.to(dev)
+        ms_l = time_launches(lambda: layer(xl), 10, 3)
+        out_l = layer(xl)[:, rows5.to(dev)].float().cpu()
+        ref_l, _, _ = so.llama_decoder_layer_ref(xl_h, wl_h, torch.arange(S5)[None], 32, 8, rows=rows5)
+        rel_l = float((out_l - ref_l).norm() / ref_l.norm())
+        worst_l = float((out_l - ref_l).abs().max() / ref_l.abs().max())
+        del wl_h, out_l, ref_l
         other["L5_decoder_layer_prefill_s8192"] = {
             "ms": ms_l, "tflops": tot_fl / ms_l / 1e9,
+            "within_tolerance": rel_l <= 2e-3 and worst_l <= 2e-2, "relative_frobenius_error": rel_l, "worst_relative_to_max": worst_l,
+            "parity": "every 61st token row against the fp32 oracle of the decoder layer with fp16 rounding between stages "
+                      "(bounds: 2e-3 relative Frobenius, 2e-2 of the largest output)",
             "note": "whole FineLlamaDecoderLayer.forward (8 launches: norms, fused QKV GEMM, RoPE, attention on strided operands, "
                     "O projection + residual, gate/up GEMM with SiLU*up epilogue, down GEMM + residual), flops of the GEMMs and attention only"}
         Bd = 8
@@ -392,14 +453,16 @@ def main():
     print(json.dumps(out))
 
 
-def llama3_8b_layer(torch, so, dev, S5=8192, H5=4096, F5=14336):
-    """FineLlamaDecoderLayer at Llama-3-8B shapes (32 q / 8 kv heads of 128) with seeded random weights."""
+def llama3_8b_layer(torch, so, dev, S5=8192, H5=4096, F5=14336, host_weights=False):
+    """FineLlamaDecoderLayer at Llama-3-8B shapes (32 q / 8 kv heads of 128) with seeded random weights; with
+    host_weights also the dict of CPU weights the oracle takes."""
     from llama_layer import FineLlamaDecoderLayer
-    gw = lambda shape, seed: so.randn_fp16(shape, seed, 0.02).to(dev)
-    wl = dict(q=gw((4096, H5), 11), k=gw((1024, H5), 12), v=gw((1024, H5), 13), o=gw((H5, 4096), 14), gate=gw((F5, H5), 15),
-              up=gw((F5, H5), 16), down=gw((H5, F5), 17), ln1=torch.ones(H5, dtype=torch.float16, device=dev),
-              ln2=torch.ones(H5, dtype=torch.float16, device=dev))
-    return FineLlamaDecoderLayer(wl, 32, 8, max_positions=S5 + 64), S5
+    gw = lambda shape, seed: so.randn_fp16(shape, seed, 0.02)
+    wh = dict(q=gw((4096, H5), 11), k=gw((1024, H5), 12), v=gw((1024, H5), 13), o=gw((H5, 4096), 14), gate=gw((F5, H5), 15),
+              up=gw((F5, H5), 16), down=gw((H5, F5), 17), ln1=torch.ones(H5, dtype=torch.float16),
+              ln2=torch.ones(H5, dtype=torch.float16))
+    layer = FineLlamaDecoderLayer({k: v.to(dev) for k, v in wh.items()}, 32, 8, max_positions=S5 + 64)
+    return (layer, S5, wh) if host_weights else (layer, S5)
 
 
 def _cpu_model():
