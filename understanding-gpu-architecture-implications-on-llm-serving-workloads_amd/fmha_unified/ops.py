@@ -17,6 +17,11 @@ def fine_fmha(q: Tensor, k: Tensor, v: Tensor, causal: bool, is_decode, kernel_i
 
     ``causal`` masks key j for query i when j > i + (Sk - Sq); ``is_decode`` (requires ``causal=False``) is the
     single-query generation step. GQA: query head h uses kv head h // (Hq // Hkv).
+
+    Difference from the reference for ``Sq != Sk``: its kernels mask key j when j > i (top-left alignment,
+    semi/fmha_2_amd.cpp:187-190); here the mask is aligned to the bottom-right corner (the KV-cache convention). The two
+    are the same mask when ``Sq == Sk``, the only causal case the reference's tests and drivers use. A query row with no
+    visible key (``Sq > Sk`` only) gives zeros. The result is a new contiguous [B, Hq, Sq, 128] tensor.
     """
     kernel = getattr(torch.ops.fmha_unified, f"finefmha_{int(kernel_index)}")
     decode_length = k.size(2)
