@@ -209,6 +209,20 @@ int mi355_fmha_fwd_ws(const void* Q, const void* K, const void* V, void* O, floa
                       int Sk, int D, float scale, int causal, int kv_valid_len, const int64_t* strides, int dtype,
                       void* workspace, size_t workspace_bytes, void* stream);
 
+/*
+ * mi355_fmha_fwd_strided (strides == NULL: contiguous [B, H, S, D] operands) for callers that cannot allocate device
+ * memory at all: code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc. It has no
+ * counterpart in the reference. It calls no hipMalloc / hipFree or any other allocating routine: the partial results of
+ * the split-KV path live in a fixed 16 MiB array in device memory that is part of the library's code object (one copy
+ * per GPU the library runs on, held until the process ends). A call whose partial results do not fit (more than
+ * 31775 = 16 MiB / 528 B (work unit, query column) pairs, i.e. B * Hkv * Hq/Hkv * Sq beyond ~31 k) returns
+ * MI355_ERR_UNSUPPORTED and launches nothing. Every call on a GPU shares that GPU's array: calls through this entry point
+ * that overlap on one GPU (different streams, or threads) race; order them on one stream. Shapes outside the split-KV path
+ * (prefill) do not touch the array and behave exactly like mi355_fmha_fwd_strided.
+ */
+int mi355_fmha_fwd_noalloc(const void* Q, const void* K, const void* V, void* O, float* LSE, int B, int Hq, int Hkv, int Sq,
+                           int Sk, int D, float scale, int causal, int kv_valid_len, const int64_t* strides, void* stream);
+
 /* Thread-local text for the last non-zero return of this thread ("" if none). */
 const char* mi355_last_error(void);
 

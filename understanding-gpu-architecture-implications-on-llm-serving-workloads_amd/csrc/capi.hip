@@ -181,6 +181,22 @@ int mi355_fmha_fwd_ws(const void* Q, const void* K, const void* V, void* O, floa
                         strides ? strides_from(strides) : contiguous_strides(Hq, Hkv, Sq, Sk, D), dtype, stream, 0, ws);
 }
 
+int mi355_fmha_fwd_noalloc(const void* Q, const void* K, const void* V, void* O, float* LSE, int B, int Hq, int Hkv, int Sq,
+                           int Sk, int D, float scale, int causal, int kv_valid_len, const int64_t* strides, void* stream) {
+    const char* fn = "mi355_fmha_fwd_noalloc";
+    if (B >= 1 && Hq >= 1 && Hkv >= 1 && Sq >= 1 && Sk >= 1 && Hq % Hkv == 0 && kv_valid_len >= 1 && kv_valid_len <= Sk) {
+        const size_t need = mi355::fmha_decode_workspace_bytes(B, Hq, Hkv, Sq, Sk, kv_valid_len);
+        if (need > mi355::fmha_decode_static_scratch_bytes())
+            return fail(MI355_ERR_UNSUPPORTED, "%s: the split-KV partial results of this call take %zu bytes, the static scratch "
+                        "holds %zu; use mi355_fmha_fwd_ws with a workspace of your own", fn, need,
+                        mi355::fmha_decode_static_scratch_bytes());
+    }
+    mi355::FmhaWorkspace ws;
+    ws.kind = mi355::FmhaWorkspace::kStatic;
+    return fmha_checked(fn, Q, K, V, O, LSE, B, Hq, Hkv, Sq, Sk, D, scale, causal, kv_valid_len,
+                        strides ? strides_from(strides) : contiguous_strides(Hq, Hkv, Sq, Sk, D), MI355_DTYPE_FP16, stream, 0, ws);
+}
+
 int mi355_internal_fmha_fwd_variant(const void* Q, const void* K, const void* V, void* O, float* LSE, int B, int Hq, int Hkv,
                                     int Sq, int Sk, int D, float scale, int causal, int kv_valid_len, const int64_t* strides,
                                     int dtype, int variant, void* stream) {

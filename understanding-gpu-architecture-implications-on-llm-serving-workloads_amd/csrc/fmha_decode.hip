@@ -371,6 +371,32 @@ static hipError_t decode_workspace(size_t bytes, hipStream_t stream, float** out
     return hipSuccess;
 }
 
+// Static scratch for callers that must not allocate (mi355_fmha_fwd_noalloc): a fixed array in device memory, one copy
+// per GPU the library is loaded on, held until the process ends. Host code never uses the symbol's name as an address:
+// the device address is looked up once per device with hipGetSymbolAddress and kept.
+constexpr size_t kStaticScratchBytes = size_t(16) << 20;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+size_t fmha_decode_static_scratch_bytes() { return kStaticScratchBytes; }
+
+static hipError_t static_scratch_ptr(float** out) {
+    constexpr int kMaxDevices = 64;
+    static std::atomic<void*> ptrs[kMaxDevices] = {};
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    if (dev < 0 || dev >= kMaxDevices) return hipErrorInvalidDevice;
+    void* p = ptrs[dev].load(std::memory_order_acquire);
+    if (p == nullptr) {   // threads may race here; every one of them gets the same address for this device
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return e;
+        if (p == nullptr) return hipErrorInvalidSymbol;
+        ptrs[dev].store(p, std::memory_order_release);
+    }
+    *out = static_cast<float*>(p);
+    return hipSuccess;
+}
+
 template <typename T>
 hipError_t fmha_decode_dispatch(const T* Q, const T* K, const T* V, T* O, float* LSE, int B, int Hq,
                                 int Hkv, int Sq, int Sk, float scale, int causal, int kv_valid, const FmhaStrides& sd,
@@ -388,6 +414,10 @@ hipError_t fmha_decode_dispatch(const T* Q, const T* K, const T* V, T* O, float*
         case FmhaWorkspace::kCaller:
             if (ws.ptr == nullptr || ws.bytes < plan.bytes || reinterpret_cast<uintptr_t>(ws.ptr) % 16 != 0) return hipErrorInvalidValue;
             part = static_cast<float*>(ws.ptr);
+            break;
+        case FmhaWorkspace::kStatic:
+            if (plan.bytes > kStaticScratchBytes) return hipErrorOutOfMemory;   // the entry point checks first and says why
+            e = static_scratch_ptr(&part);
             break;
         default:
             e = decode_workspace(plan.bytes, stream, &part);

@@ -43,10 +43,10 @@ hipError_t hgemm_silu_mul_dispatch(const void* A, const void* B, void* C, int M,
 
 // Where the split-KV attention path keeps its partial results.
 struct FmhaWorkspace {
-    enum Kind { kLibrary, kCaller };
+    enum Kind { kLibrary, kCaller, kStatic };
     Kind kind = kLibrary;     // kLibrary: the library's own grow-only buffer of (device, stream)
     void* ptr = nullptr;      // kCaller: device memory of the caller, `bytes` long
-    size_t bytes = 0;
+    size_t bytes = 0;         // kStatic: the fixed-size __device__ array of fmha_decode.hip (nothing is ever allocated)
 };
 
 // Launches the attention forward kernels; arguments as mi355_fmha_fwd_strided after validation.
@@ -59,6 +59,8 @@ hipError_t fmha_fwd_dispatch(const void* Q, const void* K, const void* V, void* 
 bool fmha_decode_applicable(int B, int Hq, int Hkv, int Sq, int Sk, int kv_valid_len);
 // Bytes of workspace a call with these sizes uses (0 when it does not take the split-KV path).
 size_t fmha_decode_workspace_bytes(int B, int Hq, int Hkv, int Sq, int Sk, int kv_valid_len);
+// Size of the static scratch array behind FmhaWorkspace::kStatic.
+size_t fmha_decode_static_scratch_bytes();
 template <typename T>
 hipError_t fmha_decode_dispatch(const T* Q, const T* K, const T* V, T* O, float* LSE, int B, int Hq, int Hkv, int Sq, int Sk,
                                 float scale, int causal, int kv_valid_len, const FmhaStrides& strides, const FmhaWorkspace& ws,

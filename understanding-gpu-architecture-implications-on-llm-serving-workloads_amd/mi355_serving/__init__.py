@@ -17,7 +17,7 @@ ERR_BAD_ARGUMENT, ERR_UNSUPPORTED = 10001, 10002
 
 EXPORTED_SYMBOLS = ("mi355_hgemm", "mi355_fmha_fwd", "mi355_fmha_fwd_strided", "mi355_fmha_fwd_bf16", "mi355_hgemm_silu_mul", "mi355_hgemm_add", "mi355_rmsnorm", "mi355_rope", "mi355_silu_mul",
                     "mi355_gemm_bf16", "mi355_gemm_silu_mul_bf16", "mi355_gemm_add_bf16", "mi355_rmsnorm_bf16", "mi355_rope_bf16", "mi355_silu_mul_bf16",
-                    "mi355_fmha_fwd_workspace_bytes", "mi355_fmha_fwd_ws",
+                    "mi355_fmha_fwd_workspace_bytes", "mi355_fmha_fwd_ws", "mi355_fmha_fwd_noalloc",
                     "mi355_last_error", "mi355_serving_version")
 # exported for tests and tuning runs, declared in csrc/mi355_serving_internal.h and not in the public header
 INTERNAL_SYMBOLS = ("mi355_internal_hgemm_variant", "mi355_internal_fmha_fwd_variant")
@@ -77,6 +77,8 @@ def load():
     lib.mi355_fmha_fwd_ws.argtypes = [vp, vp, vp, vp, vp, i32, i32, i32, i32, i32, i32, f32, i32, i32, ctypes.POINTER(i64), i32,
                                       vp, ctypes.c_size_t, vp]
     lib.mi355_fmha_fwd_ws.restype = i32
+    lib.mi355_fmha_fwd_noalloc.argtypes = lib.mi355_fmha_fwd_strided.argtypes
+    lib.mi355_fmha_fwd_noalloc.restype = i32
     lib.mi355_internal_hgemm_variant.argtypes = [vp, vp, vp, i32, i32, i32, i64, i64, i64, i32, i32, i32, vp]
     lib.mi355_internal_hgemm_variant.restype = i32
     lib.mi355_internal_fmha_fwd_variant.argtypes = [vp, vp, vp, vp, vp, i32, i32, i32, i32, i32, i32, f32, i32, i32,
@@ -166,6 +168,18 @@ def _bhs_strides(t):
 def fmha_workspace_bytes(B, Hq, Hkv, Sq, Sk, kv_valid_len=None):
     """Bytes of caller workspace mi355_fmha_fwd_ws needs for these sizes (0 outside the split-KV path)."""
     return int(load().mi355_fmha_fwd_workspace_bytes(B, Hq, Hkv, Sq, Sk, Sk if kv_valid_len is None else kv_valid_len))
+
+
+def fmha_fwd_noalloc(q, k, v, out, lse=None, causal=False, kv_valid_len=None, scale=None):
+    """mi355_fmha_fwd_noalloc on torch's current stream: fp16 [B, H, S, D] tensors or views with a contiguous last
+    dimension; `out` (and `lse`, if wanted) are the caller's. Neither this wrapper nor the library allocates."""
+    B, Hq, Sq, D = q.shape
+    _, Hkv, Sk, _ = k.shape
+    arr = (ctypes.c_int64 * 12)(*(_bhs_strides(q) + _bhs_strides(k) + _bhs_strides(v) + _bhs_strides(out)))
+    _check(load().mi355_fmha_fwd_noalloc(_ptr(q), _ptr(k), _ptr(v), _ptr(out), _ptr(lse), B, Hq, Hkv, Sq, Sk, D,
+                                         float(1.0 / (D ** 0.5) if scale is None else scale), int(bool(causal)),
+                                         int(Sk if kv_valid_len is None else kv_valid_len), arr, _stream_of(q)))
+    return out
 
 
 def fmha_fwd(q, k, v, causal=False, kv_valid_len=None, scale=None, return_lse=True, out=None, variant=0, workspace=None):
