@@ -5,7 +5,9 @@
 // "masked iff q_pos < k_pos" (:187-190), keys at or beyond the valid length masked (:191, with the off-by-one
 // of the reference corrected), scale 1/sqrt(d) supplied by the caller (:320).
 //
-// Shape of the computation (per wave, everything stays in registers between the two matrix products):
+// Two kernels: fmha_fwd_kernel (4 or 8 free-running waves, MFMA 32x32x16; shapes that do not fill the machine with
+// 256-query workgroups) and fmha_fwd_pingpong_kernel (8 phase-locked waves, MFMA 16x16x32; everything larger, see its own
+// comment). Shape of the computation in fmha_fwd_kernel (per wave, everything stays in registers between the two products):
 //   S^T = K * Q^T      MFMA 32x32x16, A operand = K fragment read from LDS (ds_read_b128),
 //                      B operand = Q fragment held in registers for the whole kernel.
 //                      A lane then owns ONE query column (q = lane % 32) and 16 of the 32 keys of the block,
@@ -16,6 +18,7 @@
 //                      ds_read_b64_tr_b16.
 // K and V tiles (64 keys x 128 d) are copied global -> LDS with 16-byte direct-to-LDS copies, double buffered,
 // 16-byte chunks XOR-swizzled so that both the b128 reads (K) and the transposing reads (V) are conflict free.
+#include <type_traits>
 #include "mi355_common.h"
 #include "mi355_serving_internal.h"
 
@@ -303,23 +306,56 @@ __global__ __launch_bounds__(NWAVES * 64, (NQ == 1 ? 2 : 1)) void fmha_fwd_kerne
 }
 
 // ---------------------------------------------------------------------------------------------------------
-// Ping-pong kernel: 8 waves x 32 queries per workgroup, two waves per SIMD that alternate roles.
-// Same mathematics and LDS layouts as fmha_fwd_kernel. A wave alternates between
-//     an M phase: 16 MFMAs of S(j+1) = K(j+1) Q^T and 16 MFMAs of O += V(j)^T P(j)   (matrix pipe + LDS reads)
-//     a  V phase: softmax of S(j+1) -> P(j+1)                                          (VALU only)
-// separated by workgroup barriers. Waves 4..7 run one phase behind waves 0..3, so on every SIMD one wave is in
-// its M phase while the other is in its V phase: the matrix pipe and the VALU are busy at the same time without
-// relying on the instruction scheduler to interleave them inside one wave. The phases of the workgroup are
-// numbered P0, P1, ...; waves 0..3 run M in the even ones, waves 4..7 in the odd ones.
-// K and V have separate double buffers: tile j lives in Kbuf[j&1] / Vbuf[j&1], is copied by all 8 waves at the
-// start of an even phase (K(i+1) and V(i) at P(2i)) and has two phases to land (waited for at the end of P(2i+1)).
+// Ping-pong kernel: 8 waves x 32 queries per workgroup, two waves per SIMD that alternate roles. A wave alternates between
+//     a matrix phase : S(j+1) = K(j+1) Q^T and O += V(j)^T P(j)      (matrix pipe + LDS reads)
+//     a softmax phase: S(j+1) -> P(j+1)                               (VALU only)
+// separated by workgroup barriers. Waves 4..7 run one phase behind waves 0..3, so on every SIMD one wave is in its matrix
+// phase while the other is in its softmax phase: the matrix pipe and the VALU are busy at the same time without relying on
+// the instruction scheduler to interleave them inside one wave. The phases of the workgroup are numbered P0, P1, ...; waves
+// 0..3 run the matrix phase in the even ones, waves 4..7 in the odd ones. K and V have separate double buffers: tile j lives
+// in Kbuf[j&1] / Vbuf[j&1], is copied by all 8 waves in an even phase (K(i+1) and V(i) at P(2i)) and has two phases to land
+// (waited for at the end of P(2i+1)).
+//
+// Every product is made of MFMA 16x16x32 blocks: under the board's power limit that instruction sustains a ~14 % higher
+// rate than 32x32x16 on random data (it also takes more VALU issue slots away from the partner wave's softmax, which is why
+// the softmax below is cut down to the fewest instructions). Per wave and key tile (64 keys):
+//   S^T[kb][qb] (16 keys x 16 queries) = K[kb] Q[qb]^T      4 key blocks x 2 query blocks x 4 steps of 32 d = 32 MFMAs
+//   O^T[db][qb] (16 d x 16 queries)   += V[j]^T[db] P[j][qb]^T   8 d blocks x 2 query blocks x 2 steps of 32 keys = 32 MFMAs
+//   l[qb]                             += 1 P[j][qb]^T            the softmax row sums, as a ninth all-ones "d block"  = 4 MFMAs
+// Lane l = 16 g + c holds, of S^T[kb][qb], keys 16 kb + 4 g + 0..3 of query 16 qb + c. The B operand of the second
+// product wants 8 keys of one query per lane: the four values of block 2j and the four of block 2j + 1 are taken as they
+// lie, i.e. contraction index 8 g + i of step j stands for key 32 j + 4 g + i (i < 4) or 32 j + 16 + 4 g + (i - 4); the
+// V^T fragment is gathered in that same order by two transposing LDS reads (key rows 32 j + 4 g .. and 32 j + 16 + 4 g ..),
+// so P never leaves the registers. The softmax statistics of a query live in the 4 lanes c, c + 16, c + 32, c + 48; they
+// only talk to each other when the running reference has to move (see the lazy rescaling below), which after the first
+// tile is rare: the common path has no cross-lane operation at all.
 // ---------------------------------------------------------------------------------------------------------
+namespace fmha {
+__device__ __forceinline__ int swz_v16(int row) { return (row & 7) << 1; }   // 8 key rows x 32 bytes on distinct bank groups
+// maximum / sum over the four lanes that share l % 16
+__device__ __forceinline__ float quad_max(float x) {
+    x = fmaxf(x, __shfl_xor(x, 16, 64));
+    return fmaxf(x, __shfl_xor(x, 32, 64));
+}
+__device__ __forceinline__ float quad_sum(float x) {
+    x += __shfl_xor(x, 16, 64);
+    return x + __shfl_xor(x, 32, 64);
+}
+// max(a, b, c) as one instruction. fmaxf() makes the compiler quiet possible signalling NaNs first (one extra
+// v_max_f32 x, x per input); scores are never NaN here, and v_max3_f32 returns the non-NaN operands anyway.
+__device__ __forceinline__ float max3(float a, float b, float c) {
+    float r;
+    asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+    return r;
+}
+}  // namespace fmha
+
 template <typename T>
 __global__ __launch_bounds__(512, 2) void fmha_fwd_pingpong_kernel(const T* __restrict__ Q, const T* __restrict__ K,
-                                                                   const T* __restrict__ V, T* __restrict__ O,
-                                                                   float* __restrict__ LSE, int B, int Hq, int Hkv, int Sq,
-                                                                   int Sk, float scale_log2, int causal, int kv_valid,
-                                                                   int q_tiles, FmhaStrides sd) {
+                                                               const T* __restrict__ V, T* __restrict__ O,
+                                                               float* __restrict__ LSE, int B, int Hq, int Hkv, int Sq,
+                                                               int Sk, float scale_log2, int causal, int kv_valid,
+                                                               int q_tiles, FmhaStrides sd) {
     using namespace fmha;
     using V8 = typename Elem<T>::v8;
     using V4 = typename Elem<T>::v4;
@@ -335,9 +371,9 @@ __global__ __launch_bounds__(512, 2) void fmha_fwd_pingpong_kernel(const T* __re
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int late = wave >> 2;  // 0: waves 0..3 (M in even phases), 1: waves 4..7 (one phase behind)
-    const int h = lane >> 5;
-    const int l32 = lane & 31;
+    const int late = wave >> 2;  // 0: waves 0..3 (matrix phase in even phases), 1: waves 4..7 (one phase behind)
+    const int g = lane >> 4;
+    const int c16 = lane & 15;
 
     int b, hq, q_tile;
     const int group = Hq / Hkv;
@@ -356,33 +392,29 @@ __global__ __launch_bounds__(512, 2) void fmha_fwd_pingpong_kernel(const T* __re
     if (causal) k_end = min(k_end, min(q_block0 + BM, Sq) - 1 + shift + 1);
     const int n_tiles = (k_end + BN - 1) / BN;  // may be <= 0: no visible key for the whole workgroup
 
-    V8 qf[8];
-    {
-        int qrow = min(q_wave0 + l32, Sq - 1);
-        const T* qp = Qh + qrow * sd.q_row + 8 * h;
+    // Q fragments (B operand of the first product): lane holds Q[16 qb + c][32 ks + 8 g .. +7]
+    V8 qf[2][4];
 #pragma unroll
-        for (int ks = 0; ks < 8; ++ks) qf[ks] = *(const V8*)(qp + ks * 16);
+    for (int qb = 0; qb < 2; ++qb) {
+        const int qrow = min(q_wave0 + qb * 16 + c16, Sq - 1);
+        const T* qp = Qh + qrow * sd.q_row + 8 * g;
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) qf[qb][ks] = *(const V8*)(qp + ks * 32);
     }
 
-    // copy i of this wave covers tile rows (i*NWAVES + wave)*4 + lane/16, 16-byte chunk position lane%16.
-    // Addresses = wave-uniform tile base (scalar registers) + 32-bit lane offset; rows past the last valid key are
-    // clamped onto it (they are masked later, but V must not feed NaNs into 0 * V).
-    int copy_row[COPIES];
-    uint32_t copy_kcol[COPIES], copy_vcol[COPIES];
-#pragma unroll
-    for (int i = 0; i < COPIES; ++i) {
-        int row = (i * NWAVES + wave) * 4 + (lane >> 4);
-        copy_row[i] = row;
-        copy_kcol[i] = ((lane & 15) ^ swz_k(row)) * 16;
-        copy_vcol[i] = ((lane & 15) ^ swz_v(row)) * 16;
-    }
+    // copy i of this wave covers tile rows 32 i + 4 wave + lane/16, 16-byte chunk position lane%16 (the swizzles depend on
+    // row % 16 only, so both copies of a lane share their column offsets); rows past the last valid key are clamped onto
+    // it (masked later, but V must not feed NaNs into 0 * V)
+    const int copy_row0 = wave * 4 + (lane >> 4);
+    const uint32_t copy_kcol = ((lane & 15) ^ swz_k(copy_row0)) * 16;
+    const uint32_t copy_vcol = ((lane & 15) ^ swz_v16(copy_row0)) * 16;
     const uint32_t k_row_bytes = (uint32_t)sd.k_row * 2, v_row_bytes = (uint32_t)sd.v_row * 2;
     auto issue_k = [&](int tile) {
         const char* base = (const char*)Kh + (long)tile * BN * sd.k_row * 2;
         const int last = kv_valid - 1 - tile * BN;
 #pragma unroll
         for (int i = 0; i < COPIES; ++i)
-            copy16_global_to_lds(base, (uint32_t)min(copy_row[i], last) * k_row_bytes + copy_kcol[i],
+            copy16_global_to_lds(base, (uint32_t)min(copy_row0 + 32 * i, last) * k_row_bytes + copy_kcol,
                                  kbuf + (tile & 1) * TILE_BYTES + (i * NWAVES + wave) * 1024);
     };
     auto issue_v = [&](int tile) {
@@ -390,179 +422,208 @@ __global__ __launch_bounds__(512, 2) void fmha_fwd_pingpong_kernel(const T* __re
         const int last = kv_valid - 1 - tile * BN;
 #pragma unroll
         for (int i = 0; i < COPIES; ++i)
-            copy16_global_to_lds(base, (uint32_t)min(copy_row[i], last) * v_row_bytes + copy_vcol[i],
+            copy16_global_to_lds(base, (uint32_t)min(copy_row0 + 32 * i, last) * v_row_bytes + copy_vcol,
                                  vbuf + (tile & 1) * TILE_BYTES + (i * NWAVES + wave) * 1024);
     };
 
-    const int k_base = l32 * ROW_BYTES + ((h ^ (lane & 15)) << 4);  // xor (ks << 5), + kb * 32 * ROW_BYTES
-    const int v_row = 4 * h + ((lane & 15) >> 2);
-    const int v_clow = 2 * ((lane >> 4) & 1) + ((lane & 3) >> 1);
-    const int v_base = v_row * ROW_BYTES + ((v_clow ^ swz_v(v_row)) << 4) + (lane & 1) * 8;  // xor (db << 6)
+    // K fragment (key block kb, d step ks): row 16 kb + c, chunk (4 ks + g) ^ (row & 15)
+    const int k_base = c16 * ROW_BYTES + ((g ^ c16) << 4);                 // xor (ks << 6), + kb * 16 * ROW_BYTES
+    // V^T fragment (key step j, d block db), transposing read t: input lane c of a 16-lane group supplies 4 d of key row
+    // 32 j + 16 t + 4 g + c / 4: d 16 db + 4 (c % 4) .. +3
+    const int v_row = 4 * g + (c16 >> 2);
+    const int v_base = v_row * ROW_BYTES + (((((c16 & 3) >> 1)) ^ swz_v16(v_row)) << 4) + (c16 & 1) * 8;   // xor (db << 5)
 
-    float16v o[4];
+    float4v o[8][2];
 #pragma unroll
-    for (int db = 0; db < 4; ++db)
+    for (int db = 0; db < 8; ++db)
 #pragma unroll
-        for (int e = 0; e < 16; ++e) o[db][e] = 0.f;
-    float m_run = -INFINITY, l_run = 0.f;
+        for (int qb = 0; qb < 2; ++qb) o[db][qb] = float4v{0.f, 0.f, 0.f, 0.f};
+    // Row sums of P ride on the matrix pipe: a ninth "d block" whose V^T rows are all ones, l[qb] += 1 P[j][qb]^T. Every
+    // row of that block (so all four elements of a lane) ends up holding the sum over all keys of the lane's query,
+    // accumulated from the same fp16-rounded P the output uses; no VALU additions and no cross-lane sum are needed.
+    // The rounding of P enters l with a relative error of at most 2^-12 for fp16, far inside the 1e-3 allowed on the
+    // log-sum-exp; for bfloat16 (2^-9) it would not be, so that type sums the unrounded fp32 values on the VALU instead
+    // (element 0 of l_acc then holds this lane's partial sum; the four lanes of a query are added at the end).
+    constexpr bool kSumOnMatrixPipe = std::is_same<T, half_t>::value;
+    float4v l_acc[2] = {float4v{0.f, 0.f, 0.f, 0.f}, float4v{0.f, 0.f, 0.f, 0.f}};
+    V8 ones;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) ones[e] = (T)1.0f;
+    float m_run[2] = {-INFINITY, -INFINITY};
 
-    // The compiler is free to move register-only work across s_barrier; these empty asm statements make a value
-    // "used" at a program point, which keeps the softmax in the V phase and the MFMAs in the M phase.
-    auto pin_s = [](float16v(&s)[2]) { asm volatile("" : "+v"(s[0]), "+v"(s[1])); };
+    // empty asm statements that make a value "used" at a program point: they keep the softmax in its phase and the MFMAs
+    // in theirs (the compiler is otherwise free to move register-only work across s_barrier)
+    auto pin_s = [](float4v(&s)[4][2]) {
+        asm volatile("" : "+v"(s[0][0]), "+v"(s[0][1]), "+v"(s[1][0]), "+v"(s[1][1]), "+v"(s[2][0]), "+v"(s[2][1]), "+v"(s[3][0]), "+v"(s[3][1]));
+    };
     auto pin_p = [](V8(&pf)[2][2]) { asm volatile("" : "+v"(pf[0][0]), "+v"(pf[0][1]), "+v"(pf[1][0]), "+v"(pf[1][1])); };
-    auto pin_o = [&]() { asm volatile("" : "+v"(o[0]), "+v"(o[1]), "+v"(o[2]), "+v"(o[3])); };
+    auto pin_o = [&]() {
+        asm volatile("" : "+v"(l_acc[0]), "+v"(l_acc[1]));
+#pragma unroll
+        for (int db = 0; db < 8; db += 4)
+            asm volatile("" : "+v"(o[db][0]), "+v"(o[db][1]), "+v"(o[db + 1][0]), "+v"(o[db + 1][1]), "+v"(o[db + 2][0]), "+v"(o[db + 2][1]),
+                              "+v"(o[db + 3][0]), "+v"(o[db + 3][1]));
+    };
 
-    // ---- phase bookkeeping -------------------------------------------------------------------------------------
     int phase = 0;  // index of the workgroup phase this wave is in
-    // ends the current phase and starts the next one
+    bool copies_due = false;
     auto next_phase = [&]() {
         if (phase & 1) wait_vmcnt<0>();  // copies issued at the start of the previous (even) phase have landed
         __syncthreads();
         ++phase;
         if (!(phase & 1)) {
+            if (!late) { copies_due = true; return; }   // a wave entering its matrix phase issues them behind its first reads
+            const int i = phase >> 1;
+            if (i + 1 < n_tiles) issue_k(i + 1);
+            if (i < n_tiles) issue_v(i);
+        }
+    };
+    auto due_copies = [&]() {
+        if (copies_due) {
+            copies_due = false;
             const int i = phase >> 1;
             if (i + 1 < n_tiles) issue_k(i + 1);
             if (i < n_tiles) issue_v(i);
         }
     };
 
-    // ---- building blocks ----------------------------------------------------------------------------------------
-    // LDS fragment reads, named so the M phase below can issue them long before their MFMA
-    auto read_k = [&](MI355_LDS char* kst, int kb, int ks) {
-        return Elem<T>::frag(lds_read_b128(kst + ((k_base ^ (ks << 5)) + kb * 32 * ROW_BYTES)));
-    };
-    auto read_v = [&](MI355_LDS char* vst, int step) {  // step = (kb*2 + tt)*4 + db, the order the MFMAs consume them
-        const int db = step & 3, tt = (step >> 2) & 1, kb = step >> 3;
-        const int off = (v_base ^ (db << 6)) + (kb * 32 + 16 * tt) * ROW_BYTES;
-        return Elem<T>::frag(concat(lds_read_tr16_b64(vst + off), lds_read_tr16_b64(vst + off + 8 * ROW_BYTES)));
-    };
-    // The M phase in the exact order it should issue: every fragment is read 8 MFMAs (256 cycles) before the MFMA
-    // that consumes it, into the register its predecessor has just released. sched_barrier pins that order.
-    //   MFMAs  0.. 7: S block 0 (K fragments read up front)        reads issued: K fragments of block 1
-    //   MFMAs  8..15: S block 1                                     reads issued: V fragments 0..7
-    //   MFMAs 16..23: O += V^T P, fragments 0..7                    reads issued: V fragments 8..15
-    //   MFMAs 24..31: O += V^T P, fragments 8..15
-    auto qk_tile = [&](int tile, float16v(&s)[2]) {  // S(tile) alone (first M phase of a wave)
-        MI355_LDS char* kst = kbuf + (tile & 1) * TILE_BYTES;
-        V8 kf[8];
-#pragma unroll
-        for (int i = 0; i < 8; ++i) kf[i] = read_k(kst, 0, i);
-#pragma unroll
-        for (int kb = 0; kb < 2; ++kb) {
-#pragma unroll
-            for (int e = 0; e < 16; ++e) s[kb][e] = 0.f;
-#pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                __builtin_amdgcn_sched_barrier(0);
-                s[kb] = Elem<T>::mfma32(kf[i], qf[i], s[kb]);
-                if (kb == 0) kf[i] = read_k(kst, 1, i);
-            }
+    // Fragment f of a matrix phase, in the order the MFMAs consume them: f < 16 is the K fragment (ks = f / 4, kb = f % 4),
+    // f >= 16 the V^T fragment (j = (f - 16) / 8, db = (f - 16) % 8). Each fragment feeds two MFMAs (the two query blocks).
+    auto read_frag = [&](MI355_LDS char* kst, MI355_LDS char* vst, int f) -> V8 {
+        if (f < 16) {
+            const int ks = f >> 2, kb = f & 3;
+            return Elem<T>::frag(lds_read_b128(kst + ((k_base ^ (ks << 6)) + kb * 16 * ROW_BYTES)));
         }
-        __builtin_amdgcn_sched_barrier(0);
+        const int j = (f - 16) >> 3, db = (f - 16) & 7;
+        const int off = (v_base ^ (db << 5)) + (32 * j) * ROW_BYTES;
+        return Elem<T>::frag(concat(lds_read_tr16_b64(vst + off), lds_read_tr16_b64(vst + off + 16 * ROW_BYTES)));
     };
-    auto pv_tile = [&](int tile, const V8(&pf)[2][2]) {  // O += V(tile)^T P alone (last M phase of a wave)
-        MI355_LDS char* vst = vbuf + (tile & 1) * TILE_BYTES;
-        V8 vf[8];
-#pragma unroll
-        for (int i = 0; i < 8; ++i) vf[i] = read_v(vst, i);
-#pragma unroll
-        for (int half = 0; half < 2; ++half)
-#pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                __builtin_amdgcn_sched_barrier(0);
-                const int step = half * 8 + i;
-                o[step & 3] = Elem<T>::mfma32(vf[i], pf[step >> 3][(step >> 2) & 1], o[step & 3]);
-                if (half == 0) vf[i] = read_v(vst, 8 + i);
-            }
-        __builtin_amdgcn_sched_barrier(0);
-    };
-    auto m_phase = [&](int tile_k, float16v(&s)[2], int tile_v, const V8(&pf)[2][2]) {  // S(tile_k) and O += V(tile_v)^T P
+    // The matrix phase over fragments [F0, F1): every fragment is read AHEAD fragments (12 MFMAs, 192 cycles) ahead of its
+    // MFMAs, into the register its predecessor has just released; sched_barrier pins that order.
+    auto mfma_phase = [&](auto f0c, auto f1c, int tile_k, float4v(&s)[4][2], int tile_v, const V8(&pf)[2][2]) {
+        constexpr int F0 = decltype(f0c)::value, F1 = decltype(f1c)::value;
         MI355_LDS char* kst = kbuf + (tile_k & 1) * TILE_BYTES;
         MI355_LDS char* vst = vbuf + (tile_v & 1) * TILE_BYTES;
-        V8 fr[8];
+        constexpr int AHEAD = 6;
+        V8 fr[AHEAD];
 #pragma unroll
-        for (int i = 0; i < 8; ++i) fr[i] = read_k(kst, 0, i);
+        for (int i = 0; i < AHEAD; ++i) fr[i] = read_frag(kst, vst, F0 + i);
+        due_copies();
+        if constexpr (F0 == 0) {
 #pragma unroll
-        for (int kb = 0; kb < 2; ++kb) {
+            for (int kb = 0; kb < 4; ++kb)
 #pragma unroll
-            for (int e = 0; e < 16; ++e) s[kb][e] = 0.f;
-#pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                __builtin_amdgcn_sched_barrier(0);
-                s[kb] = Elem<T>::mfma32(fr[i], qf[i], s[kb]);
-                fr[i] = (kb == 0) ? read_k(kst, 1, i) : read_v(vst, i);
-            }
+                for (int qb = 0; qb < 2; ++qb) s[kb][qb] = float4v{0.f, 0.f, 0.f, 0.f};
         }
 #pragma unroll
-        for (int half = 0; half < 2; ++half)
-#pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                __builtin_amdgcn_sched_barrier(0);
-                const int step = half * 8 + i;
-                o[step & 3] = Elem<T>::mfma32(fr[i], pf[step >> 3][(step >> 2) & 1], o[step & 3]);
-                if (half == 0) fr[i] = read_v(vst, 8 + i);
+        for (int f = F0; f < F1; ++f) {
+            __builtin_amdgcn_sched_barrier(0);
+            const int r = (f - F0) % AHEAD;
+            if (f < 16) {
+                const int ks = f >> 2, kb = f & 3;
+                s[kb][0] = Elem<T>::mfma16(fr[r], qf[0][ks], s[kb][0]);
+                s[kb][1] = Elem<T>::mfma16(fr[r], qf[1][ks], s[kb][1]);
+            } else {
+                const int j = (f - 16) >> 3, db = (f - 16) & 7;
+                o[db][0] = Elem<T>::mfma16(fr[r], pf[j][0], o[db][0]);
+                o[db][1] = Elem<T>::mfma16(fr[r], pf[j][1], o[db][1]);
+                if (kSumOnMatrixPipe && db == 3) {   // the row sums of this key step, in the middle of its eight d blocks
+                    l_acc[0] = Elem<T>::mfma16(ones, pf[j][0], l_acc[0]);
+                    l_acc[1] = Elem<T>::mfma16(ones, pf[j][1], l_acc[1]);
+                }
             }
+            if (f + AHEAD < F1) fr[r] = read_frag(kst, vst, f + AHEAD);
+        }
         __builtin_amdgcn_sched_barrier(0);
     };
-    auto softmax_tile = [&](float16v(&s)[2], int tile, V8(&pf)[2][2]) {
+    using I0 = std::integral_constant<int, 0>;
+    using I16 = std::integral_constant<int, 16>;
+    using I32 = std::integral_constant<int, 32>;
+
+    auto softmax_tile = [&](float4v(&s)[4][2], int tile, V8(&pf)[2][2]) {
         const int key0 = tile * BN;
         const bool need_mask = (key0 + BN > kv_valid) || (causal && (key0 + BN - 1 > q_wave0 + shift));
         if (need_mask) {
-            int qi = q_wave0 + l32;
-            int lim = causal ? min(kv_valid - 1, qi + shift) : kv_valid - 1;  // last visible key
 #pragma unroll
-            for (int kb = 0; kb < 2; ++kb)
+            for (int qb = 0; qb < 2; ++qb) {
+                const int qi = q_wave0 + qb * 16 + c16;
+                const int lim = causal ? min(kv_valid - 1, qi + shift) : kv_valid - 1;  // last visible key
 #pragma unroll
-                for (int e = 0; e < 16; ++e) {
-                    int key = key0 + kb * 32 + 8 * (e >> 2) + 4 * h + (e & 3);
-                    if (key > lim) s[kb][e] = -INFINITY;
-                }
+                for (int kb = 0; kb < 4; ++kb)
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        if (key0 + kb * 16 + 4 * g + e > lim) s[kb][qb][e] = -INFINITY;
+            }
         }
-        float mx = s[0][0];
+        // Lazy rescaling: m_run is the exponent reference of the running sums of a query (identical in its four lanes), not
+        // necessarily its running maximum. A lane only asks for it to move when one of ITS scores exceeds it by more than
+        // 2^kLazyLog2; then (any lane of the wave asked) the four lanes of every query agree on the tile's maximum and the
+        // reference is raised to the running maximum. Otherwise P = exp2((S - m_run) c) <= 2^kLazyLog2 everywhere and nothing
+        // crosses lanes.
+        float mx[2];
+        bool raise = false;
 #pragma unroll
-        for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-            for (int e = 0; e < 16; ++e) mx = fmaxf(mx, s[kb][e]);
-        mx = halves_max(mx);
-        const bool raise = (mx - m_run) * scale_log2 > kLazyLog2;  // lazy rescaling, see fmha_fwd_kernel
+        for (int qb = 0; qb < 2; ++qb) {
+            float a = max3(s[0][qb][0], s[0][qb][1], s[0][qb][2]);
+            float c = max3(s[0][qb][3], s[1][qb][0], s[1][qb][1]);
+            a = max3(a, s[1][qb][2], s[1][qb][3]);
+            c = max3(c, s[2][qb][0], s[2][qb][1]);
+            a = max3(a, s[2][qb][2], s[2][qb][3]);
+            c = max3(c, s[3][qb][0], s[3][qb][1]);
+            a = max3(a, s[3][qb][2], s[3][qb][3]);
+            a = max3(a, c, c);
+            mx[qb] = a;
+            raise = raise || ((a - m_run[qb]) * scale_log2 > kLazyLog2);  // -inf - -inf = NaN compares false
+        }
         if (__builtin_amdgcn_ballot_w64(raise) != 0) {
-            float m_new = fmaxf(m_run, mx);
-            float m_use = (m_new == -INFINITY) ? 0.f : m_new;
-            float alpha = fast_exp2((m_run - m_use) * scale_log2);
-            m_run = m_new;
-            l_run *= alpha;
 #pragma unroll
-            for (int db = 0; db < 4; ++db)
+            for (int qb = 0; qb < 2; ++qb) {
+                const float m_new = fmaxf(m_run[qb], quad_max(mx[qb]));
+                const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+                const float alpha = fast_exp2((m_run[qb] - m_use) * scale_log2);
+                m_run[qb] = m_new;
 #pragma unroll
-                for (int e = 0; e < 16; ++e) o[db][e] *= alpha;
+                for (int e = 0; e < 4; ++e) l_acc[qb][e] *= alpha;
+#pragma unroll
+                for (int db = 0; db < 8; ++db)
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) o[db][qb][e] *= alpha;
+            }
         }
-        const float neg_ms = (m_run == -INFINITY) ? 0.f : -m_run * scale_log2;
-        // In this phase the wave is the only one of its SIMD issuing VALU work, so dependent instructions must be
-        // kept apart: all 32 multiply-adds, then all 32 exponentials, then four independent partial sums.
+        // the wave is the only one of its SIMD issuing VALU work in this phase, so dependent instructions are kept apart:
+        // all multiply-adds, then all exponentials, then the sums and conversions
 #pragma unroll
-        for (int kb = 0; kb < 2; ++kb)
+        for (int qb = 0; qb < 2; ++qb) {
+            const float neg_ms = (m_run[qb] == -INFINITY) ? 0.f : -m_run[qb] * scale_log2;
 #pragma unroll
-            for (int e = 0; e < 16; ++e) s[kb][e] = __builtin_fmaf(s[kb][e], scale_log2, neg_ms);
+            for (int kb = 0; kb < 4; ++kb)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) s[kb][qb][e] = __builtin_fmaf(s[kb][qb][e], scale_log2, neg_ms);
+        }
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int kb = 0; kb < 2; ++kb)
+        for (int kb = 0; kb < 4; ++kb)
 #pragma unroll
-            for (int e = 0; e < 16; ++e) s[kb][e] = fast_exp2(s[kb][e]);
+            for (int qb = 0; qb < 2; ++qb)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) s[kb][qb][e] = fast_exp2(s[kb][qb][e]);
         __builtin_amdgcn_sched_barrier(0);
-        float ps[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int kb = 0; kb < 2; ++kb)
+        for (int qb = 0; qb < 2; ++qb) {
+            float ps[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-            for (int tt = 0; tt < 2; ++tt) {
+            for (int j = 0; j < 2; ++j) {
                 V8 pk;
 #pragma unroll
-                for (int j = 0; j < 8; ++j) {
-                    ps[j & 3] += s[kb][8 * tt + j];
-                    pk[j] = (T)s[kb][8 * tt + j];
+                for (int e = 0; e < 4; ++e) {
+                    if (!kSumOnMatrixPipe) ps[e] += s[2 * j][qb][e] + s[2 * j + 1][qb][e];
+                    pk[e] = (T)s[2 * j][qb][e];
+                    pk[4 + e] = (T)s[2 * j + 1][qb][e];
                 }
-                pf[kb][tt] = pk;
+                pf[j][qb] = pk;
             }
-        l_run += (ps[0] + ps[1]) + (ps[2] + ps[3]);
+            if (!kSumOnMatrixPipe) l_acc[qb][0] += (ps[0] + ps[1]) + (ps[2] + ps[3]);
+        }
     };
 
     if (n_tiles > 0) {
@@ -574,19 +635,19 @@ __global__ __launch_bounds__(512, 2) void fmha_fwd_pingpong_kernel(const T* __re
         issue_v(0);
         if (late) next_phase();  // waves 4..7 idle during P0
 
-        float16v s[2];
+        float4v s[4][2];
         V8 pf[2][2];
         __builtin_amdgcn_s_setprio(1);
-        qk_tile(0, s);
+        mfma_phase(I0{}, I16{}, 0, s, 0, pf);               // S(0) alone
         __builtin_amdgcn_s_setprio(0);
         pin_s(s);
         next_phase();
         for (int j = 0; j + 1 < n_tiles; ++j) {
-            softmax_tile(s, j, pf);  // V phase
+            softmax_tile(s, j, pf);
             pin_p(pf);
             next_phase();
             __builtin_amdgcn_s_setprio(1);
-            m_phase(j + 1, s, j, pf);
+            mfma_phase(I0{}, I32{}, j + 1, s, j, pf);        // S(j+1) and O += V(j)^T P(j)
             __builtin_amdgcn_s_setprio(0);
             pin_s(s);
             pin_o();
@@ -595,29 +656,30 @@ __global__ __launch_bounds__(512, 2) void fmha_fwd_pingpong_kernel(const T* __re
         softmax_tile(s, n_tiles - 1, pf);
         pin_p(pf);
         next_phase();
-        pv_tile(n_tiles - 1, pf);
+        mfma_phase(I16{}, I32{}, 0, s, n_tiles - 1, pf);     // O += V(last)^T P(last) alone
         next_phase();
         if (!late) next_phase();  // waves 0..3 idle while waves 4..7 finish
     }
 
-    // ---- finalize: O / l, LSE ---------------------------------------------------------------------------------
-    float l_tot = halves_sum(l_run);
-    float inv = (l_tot > 0.f) ? 1.f / l_tot : 0.f;
-    int qi = q_wave0 + l32;
-    if (qi < Sq) {
-        T* orow = Oh + qi * sd.o_row + 4 * h;
+    // ---- finalize: O / l, LSE: lane holds O[query 16 qb + c][d = 16 db + 4 g + 0..3] -----------------------------
 #pragma unroll
-        for (int db = 0; db < 4; ++db)
+    for (int qb = 0; qb < 2; ++qb) {
+        const float l_tot = kSumOnMatrixPipe ? l_acc[qb][0] : quad_sum(l_acc[qb][0]);
+        const float inv = (l_tot > 0.f) ? 1.f / l_tot : 0.f;
+        const int qi = q_wave0 + qb * 16 + c16;
+        if (qi < Sq) {
+            T* orow = Oh + qi * sd.o_row + 4 * g;
 #pragma unroll
-            for (int p = 0; p < 4; ++p) {
+            for (int db = 0; db < 8; ++db) {
                 V4 v;
 #pragma unroll
-                for (int q = 0; q < 4; ++q) v[q] = (T)(o[db][4 * p + q] * inv);
-                *(V4*)(orow + db * 32 + 8 * p) = v;
+                for (int e = 0; e < 4; ++e) v[e] = (T)(o[db][qb][e] * inv);
+                *(V4*)(orow + db * 16) = v;
             }
-        if (LSE != nullptr && h == 0) {
-            float lse = (l_tot > 0.f) ? (m_run * scale_log2 + __builtin_log2f(l_tot)) * 0.69314718055994531f : -INFINITY;
-            LSE[((long)b * Hq + hq) * (long)Sq + qi] = lse;
+            if (LSE != nullptr && g == 0) {
+                const float lse = (l_tot > 0.f) ? (m_run[qb] * scale_log2 + __builtin_log2f(l_tot)) * 0.69314718055994531f : -INFINITY;
+                LSE[((long)b * Hq + hq) * (long)Sq + qi] = lse;
+            }
         }
     }
 }
@@ -628,14 +690,15 @@ static hipError_t launch_fmha_pingpong(const T* Q, const T* K, const T* V, T* O,
                                        hipStream_t stream) {
     constexpr int BM = 256;
     constexpr int LDS = 4 * fmha::TILE_BYTES;
+    auto kern = fmha_fwd_pingpong_kernel<T>;
     static DynamicLdsOnce lds_once;
-    if (hipError_t e = lds_once.ensure(reinterpret_cast<const void*>(fmha_fwd_pingpong_kernel<T>), LDS); e != hipSuccess) return e;
+    if (hipError_t e = lds_once.ensure(reinterpret_cast<const void*>(kern), LDS); e != hipSuccess) return e;
     const int q_tiles = (Sq + BM - 1) / BM;
     const long blocks = (long)q_tiles * Hq * B;
     if (blocks > 0x7fffffffL) return hipErrorInvalidValue;
     const float scale_log2 = scale * 1.4426950408889634f;
-    fmha_fwd_pingpong_kernel<T><<<dim3((unsigned)blocks), dim3(512), LDS, stream>>>(Q, K, V, O, LSE, B, Hq, Hkv, Sq, Sk, scale_log2,
-                                                                                causal, kv_valid, q_tiles, sd);
+    kern<<<dim3((unsigned)blocks), dim3(512), LDS, stream>>>(Q, K, V, O, LSE, B, Hq, Hkv, Sq, Sk, scale_log2, causal, kv_valid,
+                                                             q_tiles, sd);
     return hipGetLastError();
 }
 
