@@ -161,7 +161,7 @@ def test_split_kv_workspace_outlives_growth_under_a_captured_graph(lib, gpu):
     # workspace than the one the graph's kernels hold the address of. The library must keep the old buffer alive (it
     # only ever adds buffers), so replays of the graph still write valid memory and still give the eager result.
     qs, ks, vs = (t.to(gpu) for t in so.fmha_inputs(1, 32, 8, 1, 4096, seed=31))
-    qb, kb, vb = (t.to(gpu) for t in so.fmha_inputs(8, 32, 1, 1, 16384, seed=32))     # 768 units x 32 columns: ~13 MB
+    qb, kb, vb = (t.to(gpu) for t in so.fmha_inputs(8, 32, 1, 1, 16384, seed=32))     # 256 workgroups x 32 columns: 4.3 MB
     assert lib.fmha_workspace_bytes(8, 32, 1, 1, 16384) > (4 << 20) > lib.fmha_workspace_bytes(1, 32, 8, 1, 4096) > 0
     ref_s = lib.fmha_fwd(qs, ks, vs)[0].clone()
     ref_b = lib.fmha_fwd(qb, kb, vb)[0].clone()
@@ -187,17 +187,21 @@ def test_split_kv_workspace_outlives_growth_under_a_captured_graph(lib, gpu):
 
 
 def test_split_kv_call_that_would_allocate_during_capture_is_refused(lib, gpu):
-    # The capture stream has no workspace large enough (this shape needs more than any other test's: torch hands out
-    # pooled streams, so "never used" cannot be relied on): the library must not allocate under capture; it reports an
-    # error and launches nothing. The same capture then succeeds with a caller-owned workspace.
-    B, Hq, Hkv, Sk = 1536, 32, 1, 512
+    # A stream the library has never seen (created through the HIP runtime directly: torch hands out pooled streams) has
+    # no workspace yet: the library must not allocate under capture; it reports an error and launches nothing. The same
+    # capture then succeeds with a caller-owned workspace.
+    import ctypes
+    hip = ctypes.CDLL("libamdhip64.so")
+    raw = ctypes.c_void_p()
+    assert hip.hipStreamCreate(ctypes.byref(raw)) == 0
+    fresh = torch.cuda.ExternalStream(raw.value)
+    B, Hq, Hkv, Sk = 1, 32, 8, 2048
     q, k, v = (t.to(gpu) for t in so.fmha_inputs(B, Hq, Hkv, 1, Sk, seed=33))
-    assert lib.fmha_workspace_bytes(B, Hq, Hkv, 1, Sk) > (24 << 20)
+    assert lib.fmha_workspace_bytes(B, Hq, Hkv, 1, Sk) > 0
     ref = lib.fmha_fwd(q, k, v)[0].clone()      # default stream (also sets the kernel attributes outside capture)
     ws = torch.empty(lib.fmha_workspace_bytes(B, Hq, Hkv, 1, Sk), dtype=torch.uint8, device=gpu)
     out_g = torch.zeros_like(q)
     torch.cuda.synchronize()
-    fresh = torch.cuda.Stream()
     graph = torch.cuda.CUDAGraph()
     refused = None
     with torch.cuda.graph(graph, stream=fresh):

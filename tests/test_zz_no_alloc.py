@@ -29,7 +29,7 @@ def both(lib, gpu, B, Hq, Hkv, Sq, Sk, causal, kvv, seed):
 
 
 def test_no_alloc_entry_point_matches_the_allocating_one_on_two_calls_in_a_row(lib, gpu):
-    # Llama-3-8B generation step at batch 4 over 8192 keys (768 work units x 4 columns), then a smaller call that leaves
+    # Llama-3-8B generation step at batch 4 over 8192 keys (256 workgroups x 4 columns), then a smaller call that leaves
     # most of the previous call's partials in the array untouched
     both(lib, gpu, 4, 32, 8, 1, 8192, False, None, seed=71)
     both(lib, gpu, 1, 8, 2, 3, 1000, True, 990, seed=72)
@@ -56,8 +56,8 @@ def test_no_alloc_entry_point_on_prefill_shapes_and_strided_operands(lib, gpu):
 
 
 def test_no_alloc_entry_point_rejects_what_does_not_fit(lib, gpu):
-    # 1536 work units x 32 columns x 528 B = 26 MB of partials > the 16 MiB array: refused before anything is launched
-    q, k, v = (t.to(gpu) for t in so.fmha_inputs(1536, 32, 1, 1, 512, seed=76))
+    # 256 workgroups x 32 columns x 528 B = 4.3 MB of partials > the 4 MiB array: refused before anything is launched
+    q, k, v = (t.to(gpu) for t in so.fmha_inputs(8, 32, 1, 1, 16384, seed=76))
     o = torch.empty_like(q)
     with pytest.raises(lib.Mi355Error, match="static scratch"):
         lib.fmha_fwd_noalloc(q, k, v, o)

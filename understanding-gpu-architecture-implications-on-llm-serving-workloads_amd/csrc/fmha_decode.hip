@@ -3,16 +3,19 @@
 // The reference runs its generation step (`is_decode`, one query row padded to 64 by ops.py:19-25) through the
 // prefill kernel, one workgroup per (batch, q head) walking all keys (semi/fmha_2_amd.cpp:341-356); that leaves
 // almost the whole GPU idle and is bound by one workgroup's memory rate. Here the step is a split-KV
-// ("flash-decoding") pass, HBM-bound by the single read of K and V:
+// ("flash-decoding") pass in ONE launch, HBM-bound by the single read of K and V:
 //
-//   pass 1  fmha_decode_split_kernel: a work unit is one wave = (batch, kv head, key range). The query rows of all
-//           q heads that share the kv head are packed side by side as the (up to 32) columns of the S^T = K Q^T
-//           product, so K and V are read once per kv head, not once per q head. The wave streams its key range in
-//           tiles of 32 keys through its own LDS pipeline (direct-to-LDS copies, no workgroup barriers), runs the
-//           same register-resident online softmax as the prefill kernel and writes unnormalised partial results
-//           (O~ [128], m, l per column, fp32) to a workspace.
-//   pass 2  fmha_decode_merge_kernel: one workgroup per query row combines the partials of all key ranges,
-//           O = sum_s 2^((m_s - m) c) O~_s / sum_s 2^((m_s - m) c) l_s, and writes O (fp16) and LSE.
+//   * a workgroup = (batch, kv head, key range); about one workgroup per CU. The query rows of all q heads that share
+//     the kv head are packed side by side as the (up to 32) columns of the S^T = K Q^T product, so K and V are read once
+//     per kv head, not once per q head.
+//   * the waves of a workgroup cut its key range into contiguous pieces; each wave streams its piece in tiles of 32 keys
+//     through a private LDS pipeline (direct-to-LDS copies, no workgroup barriers while streaming) and runs the
+//     register-resident online softmax of the prefill kernel.
+//   * the waves' results are combined through LDS and written as one unnormalised partial result per workgroup
+//     (O~ [128], m, l per column, fp32) to a workspace; the workgroup then takes a ticket from a counter of its
+//     (batch, kv head), and the one that draws the last ticket combines all partials of that pair,
+//     O = sum_s 2^((m_s - m) c) O~_s / sum_s 2^((m_s - m) c) l_s, writes O and LSE and puts the counter back to zero.
+//     With a single key range per (batch, kv head) the workgroup writes O and LSE directly and touches no workspace.
 //
 // Mask semantics are those of the prefill kernel (keys >= kv_valid_len masked; causal: key j visible to query i
 // iff j <= i + Sk - Sq).
@@ -32,13 +35,10 @@ constexpr int TK = 32;                       // keys per tile
 constexpr int ROW_BYTES = D * 2;             // 256
 constexpr int TILE_BYTES = TK * ROW_BYTES;   // 8 KiB
 constexpr int STAGE_BYTES = 2 * TILE_BYTES;  // K + V
-constexpr int NSTAGE = 3;
-constexpr int WAVES = 3;                     // work units per workgroup
-constexpr int WAVE_BYTES = NSTAGE * STAGE_BYTES;
-constexpr int LDS_BYTES = WAVES * WAVE_BYTES;  // 144 KiB
 constexpr float kLazyLog2 = 8.f;             // rescale only when a column maximum grows by more than 2^8
 constexpr int COPIES = 2 * (TILE_BYTES / 1024);  // 16 copy instructions per stage
-constexpr int PART_STRIDE = D + 4;           // floats per (unit, column): O~[128], m, l, 2 pad (keeps rows 16-byte aligned)
+constexpr int PART_STRIDE = D + 4;           // floats per (workgroup, column): O~[128], m, l, 2 pad (keeps rows 16-byte aligned)
+constexpr int kCounterAlign = 256;           // the counters in front of the partial results are padded to this many bytes
 
 __device__ __forceinline__ int swz_k(int row) { return row & 15; }
 __device__ __forceinline__ int swz_v(int row) {
@@ -51,73 +51,65 @@ __device__ __forceinline__ float other_half(float x) {
 }
 }  // namespace dec
 
-// units = B * Hkv * splits, unit u = (b * Hkv + hkv) * splits + s covers key tiles [s * tiles_per_split, ...)
-template <typename T>
-__global__ __launch_bounds__(dec::WAVES * 64) void fmha_decode_split_kernel(
-    const T* __restrict__ Q, const T* __restrict__ K, const T* __restrict__ V, float* __restrict__ part, int B,
-    int Hq, int Hkv, int Sq, int Sk, float scale_log2, int causal, int kv_valid, int splits, int tiles_per_split, int units, long q_batch,
-    long q_head, long q_rstride, long k_batch, long k_head, long k_rstride, long v_batch, long v_head, long v_rstride) {
+// Workgroup wg = (b * Hkv + hkv) * splits + s covers key tiles [s * tiles_per_split, (s + 1) * tiles_per_split).
+// WAVES waves with NSTAGE pipeline stages of 16 KiB each. <4, 2> (one wave per SIMD, one tile in flight behind the one
+// being consumed, 128 KiB of LDS) measured better than <3, 3> for short and for long key ranges alike.
+template <typename T, int WAVES, int NSTAGE>
+__global__ __launch_bounds__(WAVES * 64) void fmha_decode_kernel(
+    const T* __restrict__ Q, const T* __restrict__ K, const T* __restrict__ V, T* __restrict__ O, float* __restrict__ LSE,
+    float* part, unsigned* counters, int B, int Hq, int Hkv, int Sq, int Sk, float scale_log2, int causal, int kv_valid,
+    int splits, int tiles_per_split, FmhaStrides sd) {
     using namespace dec;
     using V8 = typename Elem<T>::v8;
+    constexpr int WAVE_BYTES = NSTAGE * STAGE_BYTES;
+    constexpr int NTHREADS = WAVES * 64;
     extern __shared__ __attribute__((aligned(1024))) char smem_raw[];
-    const int lane = threadIdx.x & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int unit = blockIdx.x * WAVES + wave;
-    if (unit >= units) return;  // no workgroup barrier is used anywhere in this kernel
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     MI355_LDS char* wbase = (MI355_LDS char*)smem_raw + wave * WAVE_BYTES;
 
     const int h = lane >> 5;
     const int l32 = lane & 31;
-    const int s_idx = unit % splits;
-    const int bh = unit / splits;
+    const int s_idx = blockIdx.x % splits;
+    const int bh = blockIdx.x / splits;
     const int hkv = bh % Hkv;
     const int b = bh / Hkv;
     const int group = Hq / Hkv;
     const int ncols = group * Sq;  // <= 32
     const int shift = Sk - Sq;
 
-    // column c of the packed query block = (q head hkv*group + c / Sq, query row c % Sq)
-    const int col = min(l32, ncols - 1);
-    const int hq = hkv * group + col / Sq;
-    const int qi = col % Sq;
-    const T* qp = Q + b * q_batch + hq * q_head + qi * q_rstride + 8 * h;
-    V8 qf[8];
-#pragma unroll
-    for (int ks = 0; ks < 8; ++ks) qf[ks] = *(const V8*)(qp + ks * 16);
-    const int lim = causal ? min(kv_valid - 1, qi + shift) : kv_valid - 1;  // last visible key of this column
-    // smallest such limit over the wave: tiles that end at or before it need no mask code
-    int lim_min = lim;
-#pragma unroll
-    for (int off = 32; off >= 1; off >>= 1) lim_min = min(lim_min, __shfl_xor(lim_min, off, 64));
-    lim_min = __builtin_amdgcn_readfirstlane(lim_min);
+    const T* Kh = K + b * sd.k_batch + hkv * sd.k_head;
+    const T* Vh = V + b * sd.v_batch + hkv * sd.v_head;
 
-    const T* Kh = K + b * k_batch + hkv * k_head;
-    const T* Vh = V + b * v_batch + hkv * v_head;
-
+    // this workgroup's tiles, and this wave's contiguous piece of them (possibly empty)
     const int tiles = (kv_valid + TK - 1) / TK;
-    const int t_begin = s_idx * tiles_per_split;
-    const int t_end = min(t_begin + tiles_per_split, tiles);
+    const int g_begin = s_idx * tiles_per_split;
+    const int g_end = min(g_begin + tiles_per_split, tiles);
+    const int per_wave = (max(g_end - g_begin, 0) + WAVES - 1) / WAVES;
+    const int t_begin = min(g_begin + wave * per_wave, g_end);
+    const int t_end = min(t_begin + per_wave, g_end);
 
-    // copy i (0..7) of a tile covers rows 4i + lane/16, chunk position lane%16
+    // copy i (0..7) of a tile covers rows 4i + lane/16, chunk position lane%16; addresses = wave-uniform tile base (scalar
+    // registers) + 32-bit lane offset; rows past the last valid key are clamped onto it (masked later, but V must not
+    // feed NaNs into 0 * V)
     const int c_row = lane >> 4;
-    // addresses = wave-uniform tile base (scalar registers) + 32-bit lane offset; rows past the last valid key are
-    // clamped onto it (masked later, but V must not feed NaNs into 0 * V)
-    const uint32_t k_row_bytes = (uint32_t)k_rstride * 2, v_row_bytes = (uint32_t)v_rstride * 2;
-    const uint32_t kcol = (lane & 15), c_row4 = c_row;
+    const uint32_t k_row_bytes = (uint32_t)sd.k_row * 2, v_row_bytes = (uint32_t)sd.v_row * 2;
+    const uint32_t kcol = (lane & 15);
     auto issue_stage = [&](int tile, int slot) {
         MI355_LDS char* st = wbase + slot * STAGE_BYTES;
         const int tile_u = __builtin_amdgcn_readfirstlane(tile);
-        const char* kb = (const char*)Kh + (long)tile_u * TK * k_rstride * 2;
-        const char* vb = (const char*)Vh + (long)tile_u * TK * v_rstride * 2;
+        const char* kb = (const char*)Kh + (long)tile_u * TK * sd.k_row * 2;
+        const char* vb = (const char*)Vh + (long)tile_u * TK * sd.v_row * 2;
         const int last = kv_valid - 1 - tile_u * TK;
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
-            int row = 4 * i + c_row4;
+            int row = 4 * i + c_row;
             copy16_global_to_lds(kb, (uint32_t)min(row, last) * k_row_bytes + ((kcol ^ swz_k(row)) << 4), st + i * 1024);
         }
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
-            int row = 4 * i + c_row4;
+            int row = 4 * i + c_row;
             copy16_global_to_lds(vb, (uint32_t)min(row, last) * v_row_bytes + ((kcol ^ swz_v(row)) << 4),
                                  st + TILE_BYTES + i * 1024);
         }
@@ -136,9 +128,9 @@ __global__ __launch_bounds__(dec::WAVES * 64) void fmha_decode_split_kernel(
     float m_run = -INFINITY, l_run = 0.f;
 
     const int n_loc = t_end - t_begin;
-    // each wave starts at a different tile of its range and wraps around (the online softmax does not care about the
-    // order): waves whose ranges lie a large power of two apart then do not walk the same memory channels in step
-    const int rot = n_loc > 0 ? (unit * 5) % n_loc : 0;
+    // each wave starts at a different tile of its piece and wraps around (the online softmax does not care about the
+    // order): waves whose pieces lie a large power of two apart then do not walk the same memory channels in step
+    const int rot = n_loc > 0 ? ((blockIdx.x * WAVES + wave) * 5) % n_loc : 0;
     auto tile_of = [&](int i) { int r = i + rot; return t_begin + (r >= n_loc ? r - n_loc : r); };
     int issued = t_begin;
 #pragma unroll
@@ -147,6 +139,22 @@ __global__ __launch_bounds__(dec::WAVES * 64) void fmha_decode_split_kernel(
             issue_stage(tile_of(issued - t_begin), i);
             ++issued;
         }
+    // Everything about the queries comes behind the first key / value copies, so that those leave as early as possible
+    // and the latency of the query fetch hides under theirs.
+    // column c of the packed query block = (q head hkv*group + c / Sq, query row c % Sq)
+    const int col = min(l32, ncols - 1);
+    const int hq = hkv * group + col / Sq;
+    const int qi = col % Sq;
+    const T* qp = Q + b * sd.q_batch + hq * sd.q_head + qi * sd.q_row + 8 * h;
+    const int lim = causal ? min(kv_valid - 1, qi + shift) : kv_valid - 1;  // last visible key of this column
+    // smallest such limit over the wave: tiles that end at or before it need no mask code
+    int lim_min = lim;
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) lim_min = min(lim_min, __shfl_xor(lim_min, off, 64));
+    lim_min = __builtin_amdgcn_readfirstlane(lim_min);
+    V8 qf[8];
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks) qf[ks] = *(const V8*)(qp + ks * 16);
     int slot = 0, fill = NSTAGE - 1;
     for (int tt0 = t_begin; tt0 < t_end; ++tt0) {
         const int t = tile_of(tt0 - t_begin);
@@ -223,83 +231,164 @@ __global__ __launch_bounds__(dec::WAVES * 64) void fmha_decode_split_kernel(
         wait_lgkmcnt<0>();  // the reads of this slot are complete before a later copy refills it
     }
 
-    // partial result of this unit: O~ (unnormalised), m (raw score units), l
+    // ---- combine the waves of the workgroup through LDS (the pipelines are drained: their memory is free) ------------
+    // per wave: O~ [ncols][128] floats, then m [32], l [32]
     const float l_tot = l_run + other_half(l_run);
-    if (l32 < ncols) {
-        float* pp = part + ((long)unit * ncols + l32) * PART_STRIDE;
+    __syncthreads();
+    MI355_LDS float* cmb = (MI355_LDS float*)smem_raw;
+    const int wave_floats = ncols * D + 64;
+    {
+        MI355_LDS float* mine = cmb + wave * wave_floats;
+        if (l32 < ncols) {
 #pragma unroll
-        for (int db = 0; db < 4; ++db)
+            for (int db = 0; db < 4; ++db)
 #pragma unroll
-            for (int p = 0; p < 4; ++p) {
-                float4v v;
+                for (int p = 0; p < 4; ++p) {
+                    float4v v;
 #pragma unroll
-                for (int q = 0; q < 4; ++q) v[q] = o[db][4 * p + q];
-                *(float4v*)(pp + db * 32 + 8 * p + 4 * h) = v;
+                    for (int q = 0; q < 4; ++q) v[q] = o[db][4 * p + q];
+                    *(MI355_LDS float4v*)(mine + l32 * D + db * 32 + 8 * p + 4 * h) = v;
+                }
+            if (h == 0) {
+                mine[ncols * D + l32] = m_run;
+                mine[ncols * D + 32 + l32] = l_tot;
             }
-        if (h == 0) {
-            pp[D] = m_run;
-            pp[D + 1] = l_tot;
         }
     }
+    __syncthreads();
+    const long row0 = ((long)b * Hq + (long)hkv * group) * Sq;   // LSE index of column 0 (columns are consecutive rows)
+    // element idx = (column, d) of the workgroup's result; weights 2^((m_w - m) c), 0 for waves without a visible key
+    auto combined = [&](int c, int d, float& m_out, float& l_out) {
+        float m = -INFINITY;
+#pragma unroll
+        for (int w = 0; w < WAVES; ++w) m = fmaxf(m, cmb[w * wave_floats + ncols * D + c]);
+        float acc = 0.f, l = 0.f;
+#pragma unroll
+        for (int w = 0; w < WAVES; ++w) {
+            const float mw = cmb[w * wave_floats + ncols * D + c];
+            const float wgt = (m == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f((mw - m) * scale_log2);
+            acc += wgt * cmb[w * wave_floats + c * D + d];
+            l += wgt * cmb[w * wave_floats + ncols * D + 32 + c];
+        }
+        m_out = m;
+        l_out = l;
+        return acc;
+    };
+    if (splits == 1) {   // the only key range of this (batch, kv head): the result is final
+        for (int idx = tid; idx < ncols * D; idx += NTHREADS) {
+            const int c = idx >> 7, d = idx & (D - 1);
+            float m, l;
+            const float acc = combined(c, d, m, l);
+            const int chq = hkv * group + c / Sq, cqi = c % Sq;
+            O[b * sd.o_batch + chq * sd.o_head + cqi * sd.o_row + d] = (T)((l > 0.f) ? acc / l : 0.f);
+            if (LSE != nullptr && d == 0)
+                LSE[row0 + c] = (l > 0.f) ? (m * scale_log2 + __builtin_log2f(l)) * 0.69314718055994531f : -INFINITY;
+        }
+        return;
+    }
+    // Partial results cross XCDs (each has its own L2), so they are written and read with device-scope relaxed atomic
+    // accesses, which go through to memory, instead of plain accesses bracketed by device-scope fences: such a fence
+    // writes back / invalidates a whole L2 and costs microseconds per workgroup here.
+    float* mypart = part + (long)blockIdx.x * ncols * PART_STRIDE;
+    for (int idx = tid; idx < ncols * D; idx += NTHREADS) {
+        const int c = idx >> 7, d = idx & (D - 1);
+        float m, l;
+        __hip_atomic_store(mypart + c * PART_STRIDE + d, combined(c, d, m, l), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (d == 0) {
+            __hip_atomic_store(mypart + c * PART_STRIDE + D, m, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(mypart + c * PART_STRIDE + D + 1, l, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+    }
+    // ---- ticket: the workgroup that completes the set of key ranges of (b, hkv) merges them ----------------------------
+    wait_vmcnt<0>();   // this thread's partial results have reached memory before the ticket is drawn
+    __syncthreads();
+    MI355_LDS unsigned* ticket_sh = (MI355_LDS unsigned*)(cmb + WAVES * wave_floats);
+    if (tid == 0) *ticket_sh = __hip_atomic_fetch_add(&counters[bh], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __syncthreads();
+    if (*ticket_sh != (unsigned)(splits - 1)) return;
+    // last ticket: every other workgroup of (b, hkv) drew its ticket after its partial results had reached memory.
+    // They are read back with device-coherent loads (sc1), many in flight per thread: one memory round trip for the
+    // statistics, then one per 16 key ranges for the outputs.
+    const float* base = part + (long)bh * splits * ncols * PART_STRIDE;
+    const long split_stride = (long)ncols * PART_STRIDE;
+    MI355_LDS float* st_m = cmb;                          // [splits][ncols]: m_s
+    MI355_LDS float* st_l = cmb + splits * ncols;         // [splits][ncols]: l_s
+    constexpr int BATCH = 32;
+    // BATCH loads of 16 bytes each: the outputs of key ranges sp0 .. sp0 + BATCH - 1 for 4 d of one column
+    auto load_batch = [&](float4v(&v)[BATCH], const float* pc, int sp0) {
+#pragma unroll
+        for (int u = 0; u < BATCH; ++u) {
+            const float* pa = pc + (long)min(sp0 + u, splits - 1) * split_stride;
+            asm volatile("global_load_dwordx4 %0, %1, off sc1" : "=v"(v[u]) : "v"(pa) : "memory");
+        }
+    };
+    auto wait_batch = [](float4v(&v)[BATCH]) {   // the loads above have landed; nothing that uses v moves in front of this
+        asm volatile("s_waitcnt vmcnt(0)"
+                     : "+v"(v[0]), "+v"(v[1]), "+v"(v[2]), "+v"(v[3]), "+v"(v[4]), "+v"(v[5]), "+v"(v[6]), "+v"(v[7]), "+v"(v[8]),
+                       "+v"(v[9]), "+v"(v[10]), "+v"(v[11]), "+v"(v[12]), "+v"(v[13]), "+v"(v[14]), "+v"(v[15])
+                     :: "memory");
+        asm volatile("" : "+v"(v[16]), "+v"(v[17]), "+v"(v[18]), "+v"(v[19]), "+v"(v[20]), "+v"(v[21]), "+v"(v[22]), "+v"(v[23]),
+                          "+v"(v[24]), "+v"(v[25]), "+v"(v[26]), "+v"(v[27]), "+v"(v[28]), "+v"(v[29]), "+v"(v[30]), "+v"(v[31]));
+    };
+    // the first batch of this thread's first output element goes out before the statistics are fetched: one memory
+    // round trip serves both
+    float4v v[BATCH];
+    const int n_out = ncols * (D / 4);   // output elements f = (column, group of 4 d)
+    if (tid < n_out) load_batch(v, base + (tid >> 5) * PART_STRIDE + (tid & 31) * 4, 0);
+    for (int i = tid; i < splits * ncols; i += NTHREADS) {
+        const float* ps = base + (long)(i / ncols) * split_stride + (i % ncols) * PART_STRIDE + D;
+        float ms, ls;
+        asm volatile("global_load_dword %0, %2, off sc1\n\tglobal_load_dword %1, %2, off offset:4 sc1\n\ts_waitcnt vmcnt(0)"
+                     : "=&v"(ms), "=&v"(ls) : "v"(ps) : "memory");
+        st_m[i] = ms;
+        st_l[i] = ls;
+    }
+    __syncthreads();
+    for (int f = tid; f < n_out; f += NTHREADS) {
+        const int c = f >> 5, d = (f & 31) * 4;
+        const float* pc = base + c * PART_STRIDE + d;
+        // every thread works out the statistics of its column itself (the lanes of a wave share one or two columns, so the
+        // LDS reads are broadcasts): cheaper than another pass and barrier with a few threads busy
+        float m = -INFINITY;
+        for (int sp = 0; sp < splits; ++sp) m = fmaxf(m, st_m[sp * ncols + c]);
+        float4v acc = float4v{0.f, 0.f, 0.f, 0.f};
+        float l = 0.f;
+        for (int sp0 = 0; sp0 < splits; sp0 += BATCH) {
+            if (f != tid || sp0 != 0) load_batch(v, pc, sp0);
+            // the weights of this batch, while its loads are in flight (all LDS reads first, so they overlap each other)
+            float wgt[BATCH], ls[BATCH];
+#pragma unroll
+            for (int u = 0; u < BATCH; ++u) {
+                const int sp = min(sp0 + u, splits - 1);
+                wgt[u] = st_m[sp * ncols + c];
+                ls[u] = st_l[sp * ncols + c];
+            }
+#pragma unroll
+            for (int u = 0; u < BATCH; ++u) {
+                wgt[u] = (m == -INFINITY || sp0 + u >= splits) ? 0.f : __builtin_amdgcn_exp2f((wgt[u] - m) * scale_log2);
+                l += wgt[u] * ls[u];
+            }
+            wait_batch(v);
+#pragma unroll
+            for (int u = 0; u < BATCH; ++u)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) acc[e] += wgt[u] * v[u][e];
+        }
+        const float inv = (l > 0.f) ? 1.f / l : 0.f;
+        const int chq = hkv * group + c / Sq, cqi = c % Sq;
+        typename Elem<T>::v4 ov;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) ov[e] = (T)(acc[e] * inv);
+        *(typename Elem<T>::v4*)(O + b * sd.o_batch + chq * sd.o_head + cqi * sd.o_row + d) = ov;
+        if (LSE != nullptr && d == 0)
+            LSE[row0 + c] = (l > 0.f) ? (m * scale_log2 + __builtin_log2f(l)) * 0.69314718055994531f : -INFINITY;
+    }
+    if (tid == 0) counters[bh] = 0u;   // ready for the next call that uses this workspace
 }
 
-// one workgroup of 128 threads per query row (b, hq, qi). The statistics of the key ranges are combined with the
-// ranges spread over the threads (so their loads are independent), then thread d merges element d of O.
-constexpr int kMaxSplits = 512;
-
-template <typename T>
-__global__ __launch_bounds__(128) void fmha_decode_merge_kernel(const float* __restrict__ part, T* __restrict__ O,
-                                                                float* __restrict__ LSE, int Hq, int Hkv, int Sq,
-                                                                float scale_log2, int splits, long o_batch, long o_head,
-                                                                long o_row) {
-    using namespace dec;
-    using V8 = typename Elem<T>::v8;
-    __shared__ float w_sh[kMaxSplits];
-    __shared__ float red[128];
-    const int tid = threadIdx.x;
-    const int row = blockIdx.x;  // (b * Hq + hq) * Sq + qi
-    const int qi = row % Sq;
-    const int hq = (row / Sq) % Hq;
-    const int b = row / (Sq * Hq);
-    const int group = Hq / Hkv;
-    const int hkv = hq / group;
-    const int ncols = group * Sq;
-    const int col = (hq - hkv * group) * Sq + qi;
-    const float* base = part + (((long)(b * Hkv + hkv) * splits) * ncols + col) * PART_STRIDE;
-    const long unit_stride = (long)ncols * PART_STRIDE;
-
-    // m = max over ranges
-    float m_loc = -INFINITY;
-    for (int s = tid; s < splits; s += 128) {
-        float ms = base[s * unit_stride + D];
-        w_sh[s] = ms;
-        m_loc = fmaxf(m_loc, ms);
-    }
-    red[tid] = m_loc;
-    __syncthreads();
-    float m = -INFINITY;
-#pragma unroll 8
-    for (int t = 0; t < 128; ++t) m = fmaxf(m, red[t]);
-    __syncthreads();
-    // weights 2^((m_s - m) c) (0 for ranges without a visible key) and l = sum_s w_s l_s
-    float l_loc = 0.f;
-    for (int s = tid; s < splits; s += 128) {
-        float w = (m == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f((w_sh[s] - m) * scale_log2);
-        w_sh[s] = w;
-        l_loc += w * base[s * unit_stride + D + 1];
-    }
-    red[tid] = l_loc;
-    __syncthreads();
-    float l = 0.f;
-#pragma unroll 8
-    for (int t = 0; t < 128; ++t) l += red[t];
-    // O[d] = sum_s w_s O~_s[d] / l
-    float acc = 0.f;
-#pragma unroll 8
-    for (int s = 0; s < splits; ++s) acc += w_sh[s] * base[s * unit_stride + tid];
-    O[b * o_batch + hq * o_head + qi * o_row + tid] = (T)((l > 0.f) ? acc / l : 0.f);
-    if (LSE != nullptr && tid == 0)
-        LSE[row] = (l > 0.f) ? (m * scale_log2 + __builtin_log2f(l)) * 0.69314718055994531f : -INFINITY;
+// Sets the counters of a workspace whose contents are unknown (a caller's) to zero.
+__global__ void fmha_decode_clear_kernel(unsigned* counters, int n) {
+    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < n; i += gridDim.x * blockDim.x) counters[i] = 0u;
 }
 
 bool fmha_decode_applicable(int B, int Hq, int Hkv, int Sq, int Sk, int kv_valid_len) {
@@ -307,27 +396,34 @@ bool fmha_decode_applicable(int B, int Hq, int Hkv, int Sq, int Sk, int kv_valid
     return (long)group * Sq <= 32 && kv_valid_len >= 512 && Sk >= kv_valid_len && B >= 1;
 }
 
-// How a call is cut into work units, and what its partial results occupy.
+namespace dec {
+constexpr int kMaxSplits = 256;   // key ranges per (batch, kv head)
+}   // up to this many tiles per wave: <4 waves, 2 stages>
+
+// How a call is cut into workgroups, and what its workspace holds: one counter per (batch, kv head), padded to
+// kCounterAlign bytes, then the partial results [workgroup][column][PART_STRIDE].
 struct DecodePlan {
     int splits, tiles_per_split;
-    long units;
-    size_t bytes;
+    long workgroups;
+    size_t counter_bytes, bytes;   // bytes == 0: a single key range per (batch, kv head), no workspace
 };
 static DecodePlan decode_plan(int B, int Hq, int Hkv, int Sq, int kv_valid) {
     using namespace dec;
     const int ncols = (Hq / Hkv) * Sq;
     const int tiles = (kv_valid + TK - 1) / TK;
-    // about three waves (one workgroup) per CU in flight, at least 4 key tiles (128 keys) per wave
-    int splits = (256 * WAVES) / (B * Hkv);
+    const long pairs = (long)B * Hkv;
+    // about one workgroup per CU; a key range is at least 8 tiles (two per wave)
+    long splits = (256 + pairs / 2) / pairs;
     splits = splits < 1 ? 1 : splits;
-    const int max_splits = (tiles + 3) / 4;
+    const long max_splits = (tiles + 7) / 8;
     if (splits > max_splits) splits = max_splits;
     if (splits > kMaxSplits) splits = kMaxSplits;
     DecodePlan p;
-    p.tiles_per_split = (tiles + splits - 1) / splits;
+    p.tiles_per_split = (int)((tiles + splits - 1) / splits);
     p.splits = (tiles + p.tiles_per_split - 1) / p.tiles_per_split;
-    p.units = (long)B * Hkv * p.splits;
-    p.bytes = (size_t)p.units * ncols * PART_STRIDE * sizeof(float);
+    p.workgroups = pairs * p.splits;
+    p.counter_bytes = p.splits > 1 ? ((size_t)pairs * sizeof(unsigned) + kCounterAlign - 1) / kCounterAlign * kCounterAlign : 0;
+    p.bytes = p.splits > 1 ? p.counter_bytes + (size_t)p.workgroups * ncols * PART_STRIDE * sizeof(float) : 0;
     return p;
 }
 
@@ -343,7 +439,7 @@ size_t fmha_decode_workspace_bytes(int B, int Hq, int Hkv, int Sq, int Sk, int k
 // buffer; calls on different streams get different ones. Nothing can be allocated while the stream is capturing: such a
 // call fails with hipErrorStreamCaptureUnsupported unless an earlier call on the same stream already made the buffer
 // large enough (run the step once before capturing it, or hand in a workspace of your own).
-static hipError_t decode_workspace(size_t bytes, hipStream_t stream, float** out) {
+static hipError_t decode_workspace(size_t bytes, hipStream_t stream, char** out) {
     struct Buf {
         void* ptr = nullptr;
         size_t size = 0;
@@ -364,22 +460,24 @@ static hipError_t decode_workspace(size_t bytes, hipStream_t stream, float** out
         void* fresh = nullptr;
         e = hipMalloc(&fresh, want);
         if (e != hipSuccess) return e;
+        e = hipMemset(fresh, 0, want);   // the ticket counters start at zero; every call leaves them at zero
+        if (e != hipSuccess) return e;
         b.ptr = fresh;   // the previous buffer, if any, stays allocated (see above)
         b.size = want;
     }
-    *out = static_cast<float*>(b.ptr);
+    *out = static_cast<char*>(b.ptr);
     return hipSuccess;
 }
 
 // Static scratch for callers that must not allocate (mi355_fmha_fwd_noalloc): a fixed array in device memory, one copy
-// per GPU the library is loaded on, held until the process ends. Host code never uses the symbol's name as an address:
+// per GPU the library is loaded on, held until the process ends; it starts out zeroed (so do its ticket counters). Host code never uses the symbol's name as an address:
 // the device address is looked up once per device with hipGetSymbolAddress and kept.
-constexpr size_t kStaticScratchBytes = size_t(16) << 20;
+constexpr size_t kStaticScratchBytes = size_t(4) << 20;
 static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
 
 size_t fmha_decode_static_scratch_bytes() { return kStaticScratchBytes; }
 
-static hipError_t static_scratch_ptr(float** out) {
+static hipError_t static_scratch_ptr(char** out) {
     constexpr int kMaxDevices = 64;
     static std::atomic<void*> ptrs[kMaxDevices] = {};
     int dev = 0;
@@ -393,8 +491,24 @@ static hipError_t static_scratch_ptr(float** out) {
         if (p == nullptr) return hipErrorInvalidSymbol;
         ptrs[dev].store(p, std::memory_order_release);
     }
-    *out = static_cast<float*>(p);
+    *out = static_cast<char*>(p);
     return hipSuccess;
+}
+
+template <typename T, int WAVES, int NSTAGE>
+static hipError_t launch_decode(const T* Q, const T* K, const T* V, T* O, float* LSE, float* part, unsigned* counters, int B,
+                                int Hq, int Hkv, int Sq, int Sk, float scale_log2, int causal, int kv_valid, int splits,
+                                int tiles_per_split, long workgroups, const FmhaStrides& sd, hipStream_t stream) {
+    constexpr int LDS = WAVES * NSTAGE * dec::STAGE_BYTES;
+    static_assert(LDS >= WAVES * (32 * dec::D + 64) * 4 + 64, "the combine step reuses the pipeline memory");
+    static_assert(LDS >= (2 * dec::kMaxSplits * 32 + 64) * 4, "so does the merge of the key ranges");
+    auto kern = fmha_decode_kernel<T, WAVES, NSTAGE>;
+    static DynamicLdsOnce lds_once;
+    if (hipError_t e = lds_once.ensure(reinterpret_cast<const void*>(kern), LDS); e != hipSuccess) return e;
+    if (workgroups > 0x7fffffffL) return hipErrorInvalidValue;
+    kern<<<dim3((unsigned)workgroups), dim3(WAVES * 64), LDS, stream>>>(Q, K, V, O, LSE, part, counters, B, Hq, Hkv, Sq, Sk, scale_log2,
+                                                                         causal, kv_valid, splits, tiles_per_split, sd);
+    return hipGetLastError();
 }
 
 template <typename T>
@@ -402,38 +516,35 @@ hipError_t fmha_decode_dispatch(const T* Q, const T* K, const T* V, T* O, float*
                                 int Hkv, int Sq, int Sk, float scale, int causal, int kv_valid, const FmhaStrides& sd,
                                 const FmhaWorkspace& ws, hipStream_t stream) {
     using namespace dec;
-    static DynamicLdsOnce lds_once;
-    if (hipError_t e = lds_once.ensure(reinterpret_cast<const void*>(fmha_decode_split_kernel<T>), LDS_BYTES); e != hipSuccess) return e;
     const DecodePlan plan = decode_plan(B, Hq, Hkv, Sq, kv_valid);
-    const int splits = plan.splits, tiles_per_split = plan.tiles_per_split;
-    const long units = plan.units;
-
-    float* part = nullptr;
+    char* wsp = nullptr;
     hipError_t e = hipSuccess;
-    switch (ws.kind) {
-        case FmhaWorkspace::kCaller:
-            if (ws.ptr == nullptr || ws.bytes < plan.bytes || reinterpret_cast<uintptr_t>(ws.ptr) % 16 != 0) return hipErrorInvalidValue;
-            part = static_cast<float*>(ws.ptr);
-            break;
-        case FmhaWorkspace::kStatic:
-            if (plan.bytes > kStaticScratchBytes) return hipErrorOutOfMemory;   // the entry point checks first and says why
-            e = static_scratch_ptr(&part);
-            break;
-        default:
-            e = decode_workspace(plan.bytes, stream, &part);
-            break;
+    if (plan.bytes > 0) {
+        switch (ws.kind) {
+            case FmhaWorkspace::kCaller:
+                if (ws.ptr == nullptr || ws.bytes < plan.bytes || reinterpret_cast<uintptr_t>(ws.ptr) % 16 != 0) return hipErrorInvalidValue;
+                wsp = static_cast<char*>(ws.ptr);
+                // a caller's memory holds anything: zero its counters first (the library's own buffers and the static array
+                // start at zero and every call leaves them at zero)
+                fmha_decode_clear_kernel<<<dim3(1), dim3(256), 0, stream>>>(reinterpret_cast<unsigned*>(wsp),
+                                                                            (int)(plan.counter_bytes / sizeof(unsigned)));
+                e = hipGetLastError();
+                break;
+            case FmhaWorkspace::kStatic:
+                if (plan.bytes > kStaticScratchBytes) return hipErrorOutOfMemory;   // the entry point checks first and says why
+                e = static_scratch_ptr(&wsp);
+                break;
+            default:
+                e = decode_workspace(plan.bytes, stream, &wsp);
+                break;
+        }
+        if (e != hipSuccess) return e;
     }
-    if (e != hipSuccess) return e;
+    float* part = reinterpret_cast<float*>(wsp + plan.counter_bytes);
+    unsigned* counters = reinterpret_cast<unsigned*>(wsp);
     const float scale_log2 = scale * 1.4426950408889634f;
-    const unsigned blocks = (unsigned)((units + WAVES - 1) / WAVES);
-    fmha_decode_split_kernel<T><<<dim3(blocks), dim3(WAVES * 64), LDS_BYTES, stream>>>(
-        Q, K, V, part, B, Hq, Hkv, Sq, Sk, scale_log2, causal, kv_valid, splits, tiles_per_split, (int)units, sd.q_batch,
-        sd.q_head, sd.q_row, sd.k_batch, sd.k_head, sd.k_row, sd.v_batch, sd.v_head, sd.v_row);
-    e = hipGetLastError();
-    if (e != hipSuccess) return e;
-    fmha_decode_merge_kernel<T><<<dim3((unsigned)((long)B * Hq * Sq)), dim3(128), 0, stream>>>(
-        part, O, LSE, Hq, Hkv, Sq, scale_log2, splits, sd.o_batch, sd.o_head, sd.o_row);
-    return hipGetLastError();
+    return launch_decode<T, 4, 2>(Q, K, V, O, LSE, part, counters, B, Hq, Hkv, Sq, Sk, scale_log2, causal, kv_valid, plan.splits,
+                                  plan.tiles_per_split, plan.workgroups, sd, stream);
 }
 
 template hipError_t fmha_decode_dispatch<half_t>(const half_t*, const half_t*, const half_t*, half_t*, float*, int, int, int, int,
