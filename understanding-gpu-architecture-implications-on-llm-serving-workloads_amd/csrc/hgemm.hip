@@ -80,14 +80,19 @@ struct MNContigTile {
     static constexpr int kRowsPerPass = kRowsPerInst * NWAVES;
     static constexpr int kInsts = BK / kRowsPerPass;
     static constexpr int kBytes = BK * kRowBytes;
-    static_assert(COLS == 256 || COLS == 128, "swizzle below needs at least 16 chunks per row");
+    static_assert(COLS == 256 || COLS == 128 || COLS == 64, "the swizzles below are written for these row lengths");
     static_assert(kRowsPerPass % 16 == 0, "copy i of a lane is 16 rows or a multiple further down: same swizzle for all i");
     static_assert(BK % kRowsPerPass == 0, "tile depth must be a multiple of one pass of the workgroup");
 
     // A transposing read touches, per 16 lanes, 4 k-rows x 32 bytes (two neighbouring chunks); lanes 0..31 of a
     // fragment read cover rows {0..3} and {8..11} (+ a multiple of 4 that does not change what follows). XOR-ing the
     // chunk index with an even number that differs for those 8 rows keeps their 8 chunk pairs on distinct banks.
-    __device__ static __forceinline__ int swz(int row) { return ((row & 3) | (((row >> 3) & 1) << 2)) << 1; }
+    // Rows of 128 bytes (COLS == 64) fill only half of the 256-byte bank window: rows of equal parity share a half, so
+    // it is the 4 rows of one parity among those 8 that need distinct chunk pairs (bits 1 and 3 of the row tell them apart).
+    __device__ static __forceinline__ int swz(int row) {
+        if constexpr (COLS == 64) return (((row >> 1) & 1) | (((row >> 3) & 1) << 1)) << 1;
+        else return ((row & 3) | (((row >> 3) & 1) << 2)) << 1;
+    }
     __device__ static __forceinline__ long first_copy_offset(int wave, int lane, long ld) {
         int row = wave * kRowsPerInst + lane / kChunksPerRow;
         int chunk = (lane % kChunksPerRow) ^ swz(row);
@@ -126,8 +131,10 @@ struct MainCfg {
     static constexpr int B_BYTES = BN * BK * 2;
     static constexpr int STAGE_BYTES = A_BYTES + B_BYTES;
     // 64 KiB stages: two of them fit; the 32 KiB stages of the 128x128 tile get a third, which gives every copy one more
-    // K tile of time to land (small problems run few tiles per workgroup and are bound by that latency)
-    static constexpr int NSTAGE = STAGE_BYTES > 48 * 1024 ? 2 : 3;
+    // K tile of time to land (small problems run few tiles per workgroup and are bound by that latency). The narrow tiles
+    // serve products with few rows, which are bound by the stream of the weight matrix from HBM: their ring is as deep
+    // as 128 KiB of LDS allow (5 stages of 24 KiB, 8 of 16 KiB), so that a CU keeps ~50 KiB of that stream in flight.
+    static constexpr int NSTAGE = STAGE_BYTES > 48 * 1024 ? 2 : STAGE_BYTES > 24 * 1024 ? 3 : STAGE_BYTES > 16 * 1024 ? 5 : 8;
     static constexpr int LDS_BYTES = STAGE_BYTES * NSTAGE;
     static constexpr int A_INSTS = A_BYTES / (NWAVES * 1024);  // 16-byte copies per lane per K tile
     static constexpr int B_INSTS = B_BYTES / (NWAVES * 1024);
@@ -848,16 +855,34 @@ static hipError_t launch_main(const T* A, const T* B, T* C, const T* R, int M, i
 // 17..64 rows: the small-M kernels stream B once per 16 rows (the L2 catches part of the repeats), the 128x128 tiles
 // stream it once but run K / 64 dependent tile steps of ~0.4 us on at most one workgroup per 128 columns. Cost models
 // from measurements of both at Llama projection shapes; true = the tiles are expected to be faster.
-static bool few_rows_prefer_tiles(int M, int N, int K, bool nt) {
-    if (M <= 16) return false;
-    const double small_us = (double)((M + 15) / 16) * (double)N * (double)K * 2.0 / 6.5e6;
+static double small_m_us(int M, int N, int K, bool nn) {
+    return (double)((M + 15) / 16) * (double)N * (double)K * 2.0 / 6.5e6 + (nn ? 2.3 : 4.0);
+}
+static double few_row_tiles_us(int M, int N, int K, bool nt) {
     long tiles = (long)((M + 127) / 128) * ((N + 127) / 128);
     double step_us = 0.42;
     if (nt && tiles < 192) {   // layout NT runs 128x64 tiles then
         tiles = (long)((M + 127) / 128) * ((N + 63) / 64);
         step_us = 0.34;
     }
-    return (double)(K / 64) * step_us * (double)((tiles + 255) / 256) < small_us;
+    return (double)(K / 64) * step_us * (double)((tiles + 255) / 256);
+}
+static bool few_rows_prefer_tiles(int M, int N, int K, bool nt) {
+    if (M <= 16) return false;
+    return few_row_tiles_us(M, N, K, nt) < small_m_us(M, N, K, false) - 4.0;
+}
+// Up to 64 rows on 64x64 tiles with an 8-deep ring: the second operand is streamed once whatever M is, by N / 64
+// workgroups that each sustain ~38 GB/s until HBM saturates (~6.3 TB/s); layout NN pays ~10 % for its 128-byte row
+// segments. True when that is expected to beat both alternatives above (measured at Llama projection shapes:
+// 16 x 14336 x 4096 NT 19 us against 22, 64 rows NN 22 against 31, 64 x 4096 x 4096 NT 15 against 17; but
+// 16 x 4096 x 14336 NT 41 against 19 on the split-K small-M kernel, and 16 x 14336 x 4096 NN 21 against 20).
+static bool few_rows_prefer_deep_ring(int M, int N, int K, bool nn, bool nt) {
+    const double bytes = (double)N * (double)K * 2.0;
+    const double rate = fmin(6.3e6, (double)((N + 63) / 64) * 38e3);   // bytes per microsecond
+    const double deep_us = (bytes / rate + 1.0) * (nn ? 1.1 : 1.0);
+    double other_us = small_m_us(M, N, K, nn);
+    if (M > 16) other_us = fmin(other_us, few_row_tiles_us(M, N, K, nt) + 4.0);
+    return deep_us < other_us;
 }
 
 template <typename T, bool A_KC, bool B_KC>
@@ -872,6 +897,12 @@ static hipError_t launch_layout(const T* A, const T* B, T* C, const T* R, int M,
     const bool fits128 = k_ok && M % 128 == 0 && N % 128 == 0;
     const bool ragged_ok = k_ok && N % 8 == 0 && N >= 8 && (A_KC || (M % 8 == 0 && M >= 8));
     const bool small_m = M <= 64 && !(ragged_ok && few_rows_prefer_tiles(M, N, K, A_KC && B_KC));
+    // Up to 64 rows (generation-step projections): 64x64 tiles with an 8-deep ring stream the second operand once, on
+    // N / 64 workgroups with ~50 KiB each in flight, where the split-K small-M kernels below stream it once per 16 rows.
+    if (ragged_ok && M <= 64 && variant == 0 && few_rows_prefer_deep_ring(M, N, K, A_KC && !B_KC, A_KC && B_KC)) {
+        if (M == 64 && N % 64 == 0) return launch_main<T, A_KC, B_KC, 64, 64, 2, 2>(A, B, C, R, M, N, K, lda, ldb, ldc, ldr, stream);
+        return launch_main<T, A_KC, B_KC, 64, 64, 2, 2, 0, true>(A, B, C, R, M, N, K, lda, ldb, ldc, ldr, stream);
+    }
     if constexpr (!B_KC) {   // NN, and TN with M a multiple of 8 (its A slab is copied in 8-row chunks)
         if (aligned && small_m && K % 32 == 0 && K >= 32 && N % 8 == 0 && ldc % 2 == 0 && (A_KC || M % 8 == 0))
             return launch_smallm_nn<T, A_KC>(A, B, C, R, M, N, K, lda, ldb, ldc, ldr, stream);
