@@ -85,6 +85,9 @@ def main():
     ap.add_argument("--layer-only", choices=["prefill", "step"], default=None,
                     help="run only the Llama-3-8B-shaped decoder layer (prefill at s=8192, or a generation step at batch 8 over "
                          "8192 cached tokens) for --steps iterations and print its timing; for per-kernel profiles")
+    ap.add_argument("--kernel-config", default=None, choices=sorted(KERNEL_CONFIGS),
+                    help="launch one named kernel configuration --steps times (after --warmup) and print its timing; the "
+                         "workload of the per-kernel rocprofv3 summaries in profiles/")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also launch one 1 GiB device-to-device copy, so FETCH_SIZE / WRITE_SIZE read under rocprofv3 "
                          "--pmc can be scaled by what the same counter reports for a transfer of known size")
@@ -102,6 +105,10 @@ def main():
     lib.load()
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+
+    if args.kernel_config:
+        run_kernel_config(args, torch, lib, so, dev)
+        return
 
     if args.layer_only:
         layer, S5 = llama3_8b_layer(torch, so, dev)
@@ -451,6 +458,60 @@ def main():
         "other_configs": other, "parity": checks,
     }
     print(json.dumps(out))
+
+
+# name -> ("gemm", M, N, K, layout) or ("fmha", B, Hq, Hkv, Sq, Sk, causal); each runs one kernel of the library
+KERNEL_CONFIGS = {
+    "g1_gemm_1024_nn": ("gemm", 1024, 1024, 1024, "NN"),                    # 64x128 tiles
+    "g2a_gemm_4096_nn": ("gemm", 4096, 4096, 4096, "NN"),                   # 256x256 tiles, one per CU
+    "g2b_gemm_8192_nn": ("gemm", 8192, 8192, 8192, "NN"),                   # 256x256 tiles
+    "g2b_gemm_8192_nt": ("gemm", 8192, 8192, 8192, "NT"),
+    "gemm_2048x2048x4096_nn": ("gemm", 2048, 2048, 4096, "NN"),             # 128x128 tiles
+    "g2c_gemm_16x14336x4096_nn": ("gemm", 16, 14336, 4096, "NN"),           # split-K small-M kernel
+    "gemm_16x14336x4096_nt": ("gemm", 16, 14336, 4096, "NT"),               # 64x64 tiles, 8-deep ring
+    "gemm_64x14336x4096_nt": ("gemm", 64, 14336, 4096, "NT"),               # 64x64 tiles, 8-deep ring
+    "gemm_16x4096x14336_nt": ("gemm", 16, 4096, 14336, "NT"),               # split-K small-M kernel (NT)
+    "gemm_1024x4096x4096_nt": ("gemm", 1024, 4096, 4096, "NT"),             # 128x64 tiles
+    "f3_fmha_noncausal_b4_h32_s1024": ("fmha", 4, 32, 32, 1024, 1024, False),   # ping-pong kernel
+    "f4_fmha_causal_gqa_s4096": ("fmha", 1, 32, 8, 4096, 4096, True),           # ping-pong kernel
+    "l5_fmha_causal_gqa_s8192": ("fmha", 1, 32, 8, 8192, 8192, True),           # ping-pong kernel
+    "fmha_causal_gqa_s1024": ("fmha", 1, 32, 8, 1024, 1024, True),              # 4-wave kernel (128 workgroups of 256 queries would not fill the CUs)
+    "fmha_decode_b1_sk8192": ("fmha", 1, 32, 8, 1, 8192, False),                # split-KV kernel
+    "fmha_decode_b8_sk8192": ("fmha", 8, 32, 8, 1, 8192, False),
+    "fmha_decode_b64_sk8192": ("fmha", 64, 32, 8, 1, 8192, False),              # one key range per (batch, kv head)
+}
+
+
+def run_kernel_config(args, torch, lib, so, dev):
+    cfg = KERNEL_CONFIGS[args.kernel_config]
+    stream = torch.cuda.current_stream().cuda_stream
+    if cfg[0] == "gemm":
+        _, M, N, K, lay = cfg
+        a_h, b_h = so.gemm_inputs(M, N, K, seed=0, a_std=1.0, b_std=0.02)
+        if lay == "NT":
+            b_h = b_h.t().contiguous()
+        a, b = a_h.to(dev), b_h.to(dev)
+        c = torch.empty((M, N), dtype=torch.float16, device=dev)
+        fn = lambda: lib.hgemm_raw(a.data_ptr(), b.data_ptr(), c.data_ptr(), M, N, K, a.shape[1], b.shape[1], N, lib.LAYOUTS[lay], stream)
+        flops, nbytes = 2.0 * M * N * K, 2.0 * (M * K + K * N + M * N)
+    else:
+        _, B, Hq, Hkv, Sq, Sk, causal = cfg
+        q, k, v = (t.to(dev) for t in so.fmha_inputs(B, Hq, Hkv, Sq, Sk, seed=42))
+        o = torch.empty_like(q)
+        lse = torch.empty((B, Hq, Sq), dtype=torch.float32, device=dev)
+        fn = lambda: lib.fmha_fwd_raw(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), lse.data_ptr(), B, Hq, Hkv, Sq, Sk,
+                                      128, 1.0 / math.sqrt(128), int(causal), Sk, stream)
+        flops = 4.0 * B * Hq * 128 * (causal_pairs(Sq, Sk) if causal else Sq * Sk)
+        nbytes = 2.0 * (2 * B * Hq * Sq * 128 + 2 * B * Hkv * Sk * 128) + 4.0 * B * Hq * Sq
+    if args.calibrate_copy:
+        src = torch.empty(1 << 30, dtype=torch.uint8, device=dev).fill_(1)
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
+    t = time_launches(fn, args.steps, args.warmup, stats=True)
+    print(json.dumps(dict(t, kernel_config=args.kernel_config, tflops=flops / t["ms"] / 1e9, gbs=nbytes / t["ms"] / 1e6,
+                          algorithmic_flop=flops, algorithmic_bytes=nbytes)))
 
 
 def llama3_8b_layer(torch, so, dev, S5=8192, H5=4096, F5=14336, host_weights=False):
