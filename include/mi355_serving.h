@@ -117,7 +117,8 @@ int mi355_fmha_fwd(const void* Q, const void* K, const void* V, void* O, float* 
  * mi355_fmha_fwd for operands that are not contiguous [B, H, S, D] tensors: element [b][h][s][d] of each operand
  * lives at b*batch + h*head + s*row + d, with d contiguous. `strides` holds 12 element strides in the order
  *   q_batch, q_head, q_row,  k_batch, k_head, k_row,  v_batch, v_head, v_row,  o_batch, o_head, o_row
- * each a non-negative multiple of 8 (16 bytes); rows of O must not overlap. LSE stays [B, Hq, Sq] contiguous.
+ * each a non-negative multiple of 8 (16 bytes), k_row and v_row below 2^24; rows of O must not overlap. LSE stays
+ * [B, Hq, Sq] contiguous.
  *
  * Replaces the copies the reference makes before its kernel: its callers hand over transposed views of
  * [B, S, H, D] projections (benchmarks/flashattn-cuda/modeling_llama.py:658-660) which

@@ -107,6 +107,8 @@ static int fmha_checked(const char* fn, const void* Q, const void* K, const void
     }
     hipError_t e = mi355::fmha_fwd_dispatch(Q, K, V, O, LSE, B, Hq, Hkv, Sq, Sk, scale, causal != 0, kv_valid_len, sd, dtype,
                                             variant, ws, static_cast<hipStream_t>(stream));
+    if (e == hipErrorNotSupported)
+        return fail(MI355_ERR_UNSUPPORTED, "%s: row strides of K and V must be below 2^24 elements (got %ld, %ld)", fn, sd.k_row, sd.v_row);
     if (e == hipErrorStreamCaptureUnsupported)
         return fail(static_cast<int>(e), "%s: the split-KV workspace of this stream would have to be allocated or enlarged while "
                     "the stream is capturing; run the call once before capture, or use mi355_fmha_fwd_ws", fn);

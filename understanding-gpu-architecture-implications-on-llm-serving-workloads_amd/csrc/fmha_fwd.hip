@@ -5,17 +5,16 @@
 // "masked iff q_pos < k_pos" (:187-190), keys at or beyond the valid length masked (:191, with the off-by-one
 // of the reference corrected), scale 1/sqrt(d) supplied by the caller (:320).
 //
-// Two kernels: fmha_fwd_kernel (4 or 8 free-running waves, MFMA 32x32x16; shapes that do not fill the machine with
-// 256-query workgroups) and fmha_fwd_pingpong_kernel (8 phase-locked waves, MFMA 16x16x32; everything larger, see its own
-// comment). Shape of the computation in fmha_fwd_kernel (per wave, everything stays in registers between the two products):
-//   S^T = K * Q^T      MFMA 32x32x16, A operand = K fragment read from LDS (ds_read_b128),
-//                      B operand = Q fragment held in registers for the whole kernel.
-//                      A lane then owns ONE query column (q = lane % 32) and 16 of the 32 keys of the block,
-//                      so the softmax statistics m, l and the rescale factor are per-lane scalars.
-//   P^T                exp2((S - m) * scale*log2e) in fp32, rounded to fp16; the accumulator layout of S^T is
-//                      already the B-operand layout of the second product, so P never leaves the registers.
+// One kernel family, fmha_fwd_pingpong_kernel<T, QB> (8 phase-locked waves per workgroup, MFMA 16x16x32; 256 or 128 queries
+// per workgroup), described at its definition. Everything stays in registers between the two matrix products:
+//   S^T = K * Q^T      A operand = K fragment read from LDS (ds_read_b128), B operand = Q fragment held in registers for the
+//                      whole kernel. A lane then owns ONE query column per 16-query block and 4 of the 16 keys of a key
+//                      block, so the softmax statistics m, l and the rescale factor are per-lane scalars.
+//   P^T                exp2((S - m) * scale*log2e) in fp32, rounded to fp16; the accumulator layout of S^T is (up to a
+//                      fixed permutation of the keys) the B-operand layout of the second product, so P never leaves the
+//                      registers.
 //   O^T += V^T * P^T   A operand = V^T fragment, read from the row-major V tile in LDS with the transposing
-//                      ds_read_b64_tr_b16.
+//                      ds_read_b64_tr_b16 in that same key order.
 // K and V tiles (64 keys x 128 d) are copied global -> LDS with 16-byte direct-to-LDS copies, double buffered,
 // 16-byte chunks XOR-swizzled so that both the b128 reads (K) and the transposing reads (V) are conflict free.
 #include <type_traits>
@@ -30,26 +29,29 @@ constexpr int D = 128;            // head dim
 constexpr int BN = 64;            // keys per tile
 constexpr int ROW_BYTES = D * 2;  // 256
 constexpr int TILE_BYTES = BN * ROW_BYTES;  // 16 KiB
-constexpr int STAGE_BYTES = 2 * TILE_BYTES; // K + V
-constexpr int NSTAGE = 2;
 constexpr float kLazyLog2 = 8.f;  // rescale only when a row maximum grows by more than 2^8
 
 __device__ __forceinline__ int swz_k(int row) { return row & 15; }
-__device__ __forceinline__ int swz_v(int row) {
-    int r = row & 3;
-    return (r << 1) | ((r & 1) << 3);  // 0, 10, 4, 14
-}
+__device__ __forceinline__ int swz_v16(int row) { return (row & 7) << 1; }   // 8 key rows x 32 bytes on distinct bank groups
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
-// value held by the lane 32 positions away (lane ^ 32)
-__device__ __forceinline__ float other_half(float x) {
-    int idx = ((int)(threadIdx.x & 63) ^ 32) << 2;
-    return __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute(idx, __builtin_bit_cast(int, x)));
+// maximum / sum over the four lanes that share l % 16
+__device__ __forceinline__ float quad_max(float x) {
+    x = fmaxf(x, __shfl_xor(x, 16, 64));
+    return fmaxf(x, __shfl_xor(x, 32, 64));
 }
-// max / sum over the two 32-lane halves of the wave; result valid in all 64 lanes
-__device__ __forceinline__ float halves_max(float x) { return fmaxf(x, other_half(x)); }
-__device__ __forceinline__ float halves_sum(float x) { return x + other_half(x); }
+__device__ __forceinline__ float quad_sum(float x) {
+    x += __shfl_xor(x, 16, 64);
+    return x + __shfl_xor(x, 32, 64);
+}
+// max(a, b, c) as one instruction. fmaxf() makes the compiler quiet possible signalling NaNs first (one extra
+// v_max_f32 x, x per input); scores are never NaN here, and v_max3_f32 returns the non-NaN operands anyway.
+__device__ __forceinline__ float max3(float a, float b, float c) {
+    float r;
+    asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+    return r;
+}
 
 }  // namespace fmha
 
@@ -69,240 +71,6 @@ __device__ __forceinline__ void fmha_decode_block(int bid, int q_tiles, int grou
     q_tile = q_tiles - 1 - qt;
     b = g / Hkv;
     hq = (g - b * Hkv) * group + hin;
-}
-
-template <typename T, int NQ, int NWAVES>
-__global__ __launch_bounds__(NWAVES * 64, (NQ == 1 ? 2 : 1)) void fmha_fwd_kernel(const T* __restrict__ Q, const T* __restrict__ K,
-                                                               const T* __restrict__ V, T* __restrict__ O,
-                                                               float* __restrict__ LSE, int B, int Hq, int Hkv, int Sq,
-                                                               int Sk, float scale_log2, int causal, int kv_valid,
-                                                               int q_tiles, FmhaStrides sd) {
-    using namespace fmha;
-    using V8 = typename Elem<T>::v8;
-    using V4 = typename Elem<T>::v4;
-    constexpr int BM = NWAVES * NQ * 32;
-    constexpr int COPIES = (BN * ROW_BYTES / 1024) / NWAVES;  // wave-instructions per tile per wave
-    static_assert(COPIES >= 1, "too many waves for the tile");
-
-    extern __shared__ __attribute__((aligned(1024))) char smem_raw[];
-    MI355_LDS char* smem = (MI355_LDS char*)smem_raw;
-
-    const int tid = threadIdx.x;
-    const int lane = tid & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int h = lane >> 5;
-    const int l32 = lane & 31;
-
-    int b, hq, q_tile;
-    const int group = Hq / Hkv;
-    fmha_decode_block(blockIdx.x, q_tiles, group, Hkv, B, b, hq, q_tile);
-    const int hkv = hq / group;
-
-    const int q_block0 = q_tile * BM;            // first query row of the workgroup
-    const int q_wave0 = q_block0 + wave * NQ * 32;  // first query row of this wave
-    const int shift = Sk - Sq;
-
-    const T* Qh = Q + b * sd.q_batch + hq * sd.q_head;
-    const T* Kh = K + b * sd.k_batch + hkv * sd.k_head;
-    const T* Vh = V + b * sd.v_batch + hkv * sd.v_head;
-    T* Oh = O + b * sd.o_batch + hq * sd.o_head;
-
-    // ---- number of key tiles this workgroup has to visit ----------------------------------------------
-    int k_end = kv_valid;
-    if (causal) {
-        int last_q = min(q_block0 + BM, Sq) - 1;
-        k_end = min(k_end, last_q + shift + 1);
-    }
-    const int n_tiles = (k_end + BN - 1) / BN;  // may be <= 0: no visible key for the whole tile
-
-    // ---- Q fragments: lane holds Q[q = l32][d = 16*ks + 8*h .. +7] ---------------------------------------
-    V8 qf[NQ][8];
-#pragma unroll
-    for (int qb = 0; qb < NQ; ++qb) {
-        int qrow = min(q_wave0 + qb * 32 + l32, Sq - 1);
-        const T* qp = Qh + qrow * sd.q_row + 8 * h;
-#pragma unroll
-        for (int ks = 0; ks < 8; ++ks) qf[qb][ks] = *(const V8*)(qp + ks * 16);
-    }
-
-    // ---- global -> LDS copy bookkeeping ----------------------------------------------------------------
-    // copy i of this wave covers tile rows (i*NWAVES + wave)*4 + lane/16, 16-byte chunk position lane%16
-    int copy_row[COPIES];
-    int copy_kcol[COPIES], copy_vcol[COPIES];
-#pragma unroll
-    for (int i = 0; i < COPIES; ++i) {
-        int row = (i * NWAVES + wave) * 4 + (lane >> 4);
-        copy_row[i] = row;
-        copy_kcol[i] = ((lane & 15) ^ swz_k(row)) * 8;
-        copy_vcol[i] = ((lane & 15) ^ swz_v(row)) * 8;
-    }
-    auto issue_copies = [&](int tile, int stage) {
-        MI355_LDS char* sk = smem + stage * STAGE_BYTES;
-        MI355_LDS char* sv = sk + TILE_BYTES;
-#pragma unroll
-        for (int i = 0; i < COPIES; ++i) {
-            int krow = min(tile * BN + copy_row[i], kv_valid - 1);
-            copy16_global_to_lds(Kh + krow * sd.k_row + copy_kcol[i], sk + (i * NWAVES + wave) * 1024);
-        }
-#pragma unroll
-        for (int i = 0; i < COPIES; ++i) {
-            int krow = min(tile * BN + copy_row[i], kv_valid - 1);
-            copy16_global_to_lds(Vh + krow * sd.v_row + copy_vcol[i], sv + (i * NWAVES + wave) * 1024);
-        }
-    };
-
-    // ---- LDS fragment offsets ----------------------------------------------------------------------------
-    // K fragment (key block kb, k-step ks): row kb*32 + l32, chunk (2ks + h) ^ (row & 15)
-    const int k_base = l32 * ROW_BYTES + ((h ^ (lane & 15)) << 4);  // xor (ks << 5), + kb * 32 * ROW_BYTES
-    // V^T fragment (d block db): rows 4h + (lane%16)/4 (+ kb*32 + 16t + 8u), chunk (4db + clow) ^ swz_v(row)
-    const int v_row = 4 * h + ((lane & 15) >> 2);
-    const int v_clow = 2 * ((lane >> 4) & 1) + ((lane & 3) >> 1);
-    const int v_base = TILE_BYTES + v_row * ROW_BYTES + ((v_clow ^ swz_v(v_row)) << 4) + (lane & 1) * 8;  // xor (db << 6)
-
-    float16v o[NQ][4];
-    float m_run[NQ], l_run[NQ];
-#pragma unroll
-    for (int qb = 0; qb < NQ; ++qb) {
-        m_run[qb] = -INFINITY;
-        l_run[qb] = 0.f;
-#pragma unroll
-        for (int db = 0; db < 4; ++db)
-#pragma unroll
-            for (int e = 0; e < 16; ++e) o[qb][db][e] = 0.f;
-    }
-
-    if (n_tiles > 0) issue_copies(0, 0);
-
-    for (int t = 0; t < n_tiles; ++t) {
-        wait_vmcnt<0>();
-        __syncthreads();
-        if (t + 1 < n_tiles) issue_copies(t + 1, (t + 1) & 1);
-        MI355_LDS char* st = smem + (t & 1) * STAGE_BYTES;
-        const int key0 = t * BN;
-
-        // ---- S^T = K Q^T ---------------------------------------------------------------------------------
-        float16v s[NQ][2];
-#pragma unroll
-        for (int qb = 0; qb < NQ; ++qb)
-#pragma unroll
-            for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-                for (int e = 0; e < 16; ++e) s[qb][kb][e] = 0.f;
-#pragma unroll
-        for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-            for (int ks = 0; ks < 8; ++ks) {
-                V8 kf = Elem<T>::frag(lds_read_b128(st + ((k_base ^ (ks << 5)) + kb * 32 * ROW_BYTES)));
-#pragma unroll
-                for (int qb = 0; qb < NQ; ++qb)
-                    s[qb][kb] = Elem<T>::mfma32(kf, qf[qb][ks], s[qb][kb]);
-            }
-
-        // ---- mask (only tiles that touch the diagonal or the end of the valid keys) ----------------------
-        const bool need_mask = (key0 + BN > kv_valid) || (causal && (key0 + BN - 1 > q_wave0 + shift));
-        if (need_mask) {
-#pragma unroll
-            for (int qb = 0; qb < NQ; ++qb) {
-                int qi = q_wave0 + qb * 32 + l32;
-                int lim = causal ? min(kv_valid - 1, qi + shift) : kv_valid - 1;  // last visible key
-#pragma unroll
-                for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-                    for (int e = 0; e < 16; ++e) {
-                        int key = key0 + kb * 32 + 8 * (e >> 2) + 4 * h + (e & 3);
-                        if (key > lim) s[qb][kb][e] = -INFINITY;
-                    }
-            }
-        }
-
-        // ---- online softmax with lazy rescaling --------------------------------------------------------------
-        // m_run is the exponent reference of the running sums, not necessarily the running maximum: it is only
-        // raised (and O, l rescaled) when some row of the wave exceeds it by more than 2^kLazyLog2, which after the
-        // first tiles almost never happens; until then P = exp2((S - m_run) * c) is at most 2^kLazyLog2, exact in
-        // fp16/fp32 terms, and the final O / l and LSE do not depend on the choice of reference.
-        V8 pf[NQ][2][2];
-#pragma unroll
-        for (int qb = 0; qb < NQ; ++qb) {
-            float mx = s[qb][0][0];
-#pragma unroll
-            for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-                for (int e = 0; e < 16; ++e) mx = fmaxf(mx, s[qb][kb][e]);
-            mx = halves_max(mx);
-            const bool raise = (mx - m_run[qb]) * scale_log2 > kLazyLog2;  // -inf - -inf = NaN compares false
-            if (__builtin_amdgcn_ballot_w64(raise) != 0) {
-                float m_new = fmaxf(m_run[qb], mx);
-                float m_use = (m_new == -INFINITY) ? 0.f : m_new;
-                float alpha = fast_exp2((m_run[qb] - m_use) * scale_log2);
-                m_run[qb] = m_new;
-                l_run[qb] *= alpha;
-#pragma unroll
-                for (int db = 0; db < 4; ++db)
-#pragma unroll
-                    for (int e = 0; e < 16; ++e) o[qb][db][e] *= alpha;
-            }
-            const float neg_ms = (m_run[qb] == -INFINITY) ? 0.f : -m_run[qb] * scale_log2;
-            float psum = 0.f;
-#pragma unroll
-            for (int kb = 0; kb < 2; ++kb) {
-#pragma unroll
-                for (int e = 0; e < 16; ++e) {
-                    float p = fast_exp2(__builtin_fmaf(s[qb][kb][e], scale_log2, neg_ms));
-                    s[qb][kb][e] = p;
-                    psum += p;
-                }
-#pragma unroll
-                for (int tt = 0; tt < 2; ++tt) {
-                    V8 pk;
-#pragma unroll
-                    for (int j = 0; j < 8; ++j) pk[j] = (T)s[qb][kb][8 * tt + j];
-                    pf[qb][kb][tt] = pk;
-                }
-            }
-            l_run[qb] += psum;
-        }
-
-        // ---- O^T += V^T P^T ----------------------------------------------------------------------------------
-#pragma unroll
-        for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-            for (int tt = 0; tt < 2; ++tt)
-#pragma unroll
-                for (int db = 0; db < 4; ++db) {
-                    int off = (v_base ^ (db << 6)) + (kb * 32 + 16 * tt) * ROW_BYTES;
-                    half4 lo = lds_read_tr16_b64(st + off);
-                    half4 hi = lds_read_tr16_b64(st + off + 8 * ROW_BYTES);
-                    V8 vf = Elem<T>::frag(concat(lo, hi));
-#pragma unroll
-                    for (int qb = 0; qb < NQ; ++qb)
-                        o[qb][db] = Elem<T>::mfma32(vf, pf[qb][kb][tt], o[qb][db]);
-                }
-    }
-
-    // ---- finalize: O / l, LSE ---------------------------------------------------------------------------------
-#pragma unroll
-    for (int qb = 0; qb < NQ; ++qb) {
-        float l_tot = halves_sum(l_run[qb]);
-        float inv = (l_tot > 0.f) ? 1.f / l_tot : 0.f;
-        int qi = q_wave0 + qb * 32 + l32;
-        if (qi < Sq) {
-            T* orow = Oh + qi * sd.o_row + 4 * h;
-#pragma unroll
-            for (int db = 0; db < 4; ++db)
-#pragma unroll
-                for (int p = 0; p < 4; ++p) {
-                    V4 v;
-#pragma unroll
-                    for (int q = 0; q < 4; ++q) v[q] = (T)(o[qb][db][4 * p + q] * inv);
-                    *(V4*)(orow + db * 32 + 8 * p) = v;
-                }
-            if (LSE != nullptr && h == 0) {
-                float lse = (l_tot > 0.f) ? (m_run[qb] * scale_log2 + __builtin_log2f(l_tot)) * 0.69314718055994531f
-                                          : -INFINITY;
-                LSE[((long)b * Hq + hq) * (long)Sq + qi] = lse;
-            }
-        }
-    }
 }
 
 // ---------------------------------------------------------------------------------------------------------
@@ -330,28 +98,11 @@ __global__ __launch_bounds__(NWAVES * 64, (NQ == 1 ? 2 : 1)) void fmha_fwd_kerne
 // only talk to each other when the running reference has to move (see the lazy rescaling below), which after the first
 // tile is rare: the common path has no cross-lane operation at all.
 // ---------------------------------------------------------------------------------------------------------
-namespace fmha {
-__device__ __forceinline__ int swz_v16(int row) { return (row & 7) << 1; }   // 8 key rows x 32 bytes on distinct bank groups
-// maximum / sum over the four lanes that share l % 16
-__device__ __forceinline__ float quad_max(float x) {
-    x = fmaxf(x, __shfl_xor(x, 16, 64));
-    return fmaxf(x, __shfl_xor(x, 32, 64));
-}
-__device__ __forceinline__ float quad_sum(float x) {
-    x += __shfl_xor(x, 16, 64);
-    return x + __shfl_xor(x, 32, 64);
-}
-// max(a, b, c) as one instruction. fmaxf() makes the compiler quiet possible signalling NaNs first (one extra
-// v_max_f32 x, x per input); scores are never NaN here, and v_max3_f32 returns the non-NaN operands anyway.
-__device__ __forceinline__ float max3(float a, float b, float c) {
-    float r;
-    asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
-    return r;
-}
-}  // namespace fmha
-
-template <typename T>
-__global__ __launch_bounds__(512, 2) void fmha_fwd_pingpong_kernel(const T* __restrict__ Q, const T* __restrict__ K,
+// QB = query blocks of 16 per wave: 2 (256 queries per workgroup) or 1 (128 queries, for shapes with too few 256-query
+// workgroups to fill the machine and for short sequences; every K / V fragment then feeds one MFMA instead of two, and
+// the kernel is held to 128 registers so that two workgroups share a CU).
+template <typename T, int QB>
+__global__ __launch_bounds__(512, (QB == 1 ? 4 : 2)) void fmha_fwd_pingpong_kernel(const T* __restrict__ Q, const T* __restrict__ K,
                                                                const T* __restrict__ V, T* __restrict__ O,
                                                                float* __restrict__ LSE, int B, int Hq, int Hkv, int Sq,
                                                                int Sk, float scale_log2, int causal, int kv_valid,
@@ -360,7 +111,8 @@ __global__ __launch_bounds__(512, 2) void fmha_fwd_pingpong_kernel(const T* __re
     using V8 = typename Elem<T>::v8;
     using V4 = typename Elem<T>::v4;
     constexpr int NWAVES = 8;
-    constexpr int BM = NWAVES * 32;
+    constexpr int WQ = 16 * QB;          // queries per wave
+    constexpr int BM = NWAVES * WQ;
     constexpr int COPIES = (BN * ROW_BYTES / 1024) / NWAVES;  // 2 wave-instructions per tile per wave
 
     extern __shared__ __attribute__((aligned(1024))) char smem_raw[];
@@ -380,7 +132,7 @@ __global__ __launch_bounds__(512, 2) void fmha_fwd_pingpong_kernel(const T* __re
     fmha_decode_block(blockIdx.x, q_tiles, group, Hkv, B, b, hq, q_tile);
     const int hkv = hq / group;
     const int q_block0 = q_tile * BM;
-    const int q_wave0 = q_block0 + wave * 32;
+    const int q_wave0 = q_block0 + wave * WQ;
     const int shift = Sk - Sq;
 
     const T* Qh = Q + b * sd.q_batch + hq * sd.q_head;
@@ -393,9 +145,9 @@ __global__ __launch_bounds__(512, 2) void fmha_fwd_pingpong_kernel(const T* __re
     const int n_tiles = (k_end + BN - 1) / BN;  // may be <= 0: no visible key for the whole workgroup
 
     // Q fragments (B operand of the first product): lane holds Q[16 qb + c][32 ks + 8 g .. +7]
-    V8 qf[2][4];
+    V8 qf[QB][4];
 #pragma unroll
-    for (int qb = 0; qb < 2; ++qb) {
+    for (int qb = 0; qb < QB; ++qb) {
         const int qrow = min(q_wave0 + qb * 16 + c16, Sq - 1);
         const T* qp = Qh + qrow * sd.q_row + 8 * g;
 #pragma unroll
@@ -433,11 +185,11 @@ __global__ __launch_bounds__(512, 2) void fmha_fwd_pingpong_kernel(const T* __re
     const int v_row = 4 * g + (c16 >> 2);
     const int v_base = v_row * ROW_BYTES + (((((c16 & 3) >> 1)) ^ swz_v16(v_row)) << 4) + (c16 & 1) * 8;   // xor (db << 5)
 
-    float4v o[8][2];
+    float4v o[8][QB];
 #pragma unroll
     for (int db = 0; db < 8; ++db)
 #pragma unroll
-        for (int qb = 0; qb < 2; ++qb) o[db][qb] = float4v{0.f, 0.f, 0.f, 0.f};
+        for (int qb = 0; qb < QB; ++qb) o[db][qb] = float4v{0.f, 0.f, 0.f, 0.f};
     // Row sums of P ride on the matrix pipe: a ninth "d block" whose V^T rows are all ones, l[qb] += 1 P[j][qb]^T. Every
     // row of that block (so all four elements of a lane) ends up holding the sum over all keys of the lane's query,
     // accumulated from the same fp16-rounded P the output uses; no VALU additions and no cross-lane sum are needed.
@@ -445,24 +197,39 @@ __global__ __launch_bounds__(512, 2) void fmha_fwd_pingpong_kernel(const T* __re
     // log-sum-exp; for bfloat16 (2^-9) it would not be, so that type sums the unrounded fp32 values on the VALU instead
     // (element 0 of l_acc then holds this lane's partial sum; the four lanes of a query are added at the end).
     constexpr bool kSumOnMatrixPipe = std::is_same<T, half_t>::value;
-    float4v l_acc[2] = {float4v{0.f, 0.f, 0.f, 0.f}, float4v{0.f, 0.f, 0.f, 0.f}};
+    float4v l_acc[QB];
+#pragma unroll
+    for (int qb = 0; qb < QB; ++qb) l_acc[qb] = float4v{0.f, 0.f, 0.f, 0.f};
     V8 ones;
 #pragma unroll
     for (int e = 0; e < 8; ++e) ones[e] = (T)1.0f;
-    float m_run[2] = {-INFINITY, -INFINITY};
+    float m_run[QB];
+#pragma unroll
+    for (int qb = 0; qb < QB; ++qb) m_run[qb] = -INFINITY;
 
     // empty asm statements that make a value "used" at a program point: they keep the softmax in its phase and the MFMAs
     // in theirs (the compiler is otherwise free to move register-only work across s_barrier)
-    auto pin_s = [](float4v(&s)[4][2]) {
-        asm volatile("" : "+v"(s[0][0]), "+v"(s[0][1]), "+v"(s[1][0]), "+v"(s[1][1]), "+v"(s[2][0]), "+v"(s[2][1]), "+v"(s[3][0]), "+v"(s[3][1]));
+    auto pin_s = [](float4v(&s)[4][QB]) {
+        if constexpr (QB == 2)
+            asm volatile("" : "+v"(s[0][0]), "+v"(s[0][1]), "+v"(s[1][0]), "+v"(s[1][1]), "+v"(s[2][0]), "+v"(s[2][1]), "+v"(s[3][0]), "+v"(s[3][1]));
+        else
+            asm volatile("" : "+v"(s[0][0]), "+v"(s[1][0]), "+v"(s[2][0]), "+v"(s[3][0]));
     };
-    auto pin_p = [](V8(&pf)[2][2]) { asm volatile("" : "+v"(pf[0][0]), "+v"(pf[0][1]), "+v"(pf[1][0]), "+v"(pf[1][1])); };
+    auto pin_p = [](V8(&pf)[2][QB]) {
+        if constexpr (QB == 2) asm volatile("" : "+v"(pf[0][0]), "+v"(pf[0][1]), "+v"(pf[1][0]), "+v"(pf[1][1]));
+        else asm volatile("" : "+v"(pf[0][0]), "+v"(pf[1][0]));
+    };
     auto pin_o = [&]() {
-        asm volatile("" : "+v"(l_acc[0]), "+v"(l_acc[1]));
+        if constexpr (QB == 2) {
+            asm volatile("" : "+v"(l_acc[0]), "+v"(l_acc[1]));
 #pragma unroll
-        for (int db = 0; db < 8; db += 4)
-            asm volatile("" : "+v"(o[db][0]), "+v"(o[db][1]), "+v"(o[db + 1][0]), "+v"(o[db + 1][1]), "+v"(o[db + 2][0]), "+v"(o[db + 2][1]),
-                              "+v"(o[db + 3][0]), "+v"(o[db + 3][1]));
+            for (int db = 0; db < 8; db += 4)
+                asm volatile("" : "+v"(o[db][0]), "+v"(o[db][1]), "+v"(o[db + 1][0]), "+v"(o[db + 1][1]), "+v"(o[db + 2][0]), "+v"(o[db + 2][1]),
+                                  "+v"(o[db + 3][0]), "+v"(o[db + 3][1]));
+        } else {
+            asm volatile("" : "+v"(l_acc[0]), "+v"(o[0][0]), "+v"(o[1][0]), "+v"(o[2][0]), "+v"(o[3][0]), "+v"(o[4][0]), "+v"(o[5][0]), "+v"(o[6][0]),
+                              "+v"(o[7][0]));
+        }
     };
 
     int phase = 0;  // index of the workgroup phase this wave is in
@@ -500,11 +267,11 @@ __global__ __launch_bounds__(512, 2) void fmha_fwd_pingpong_kernel(const T* __re
     };
     // The matrix phase over fragments [F0, F1): every fragment is read AHEAD fragments (12 MFMAs, 192 cycles) ahead of its
     // MFMAs, into the register its predecessor has just released; sched_barrier pins that order.
-    auto mfma_phase = [&](auto f0c, auto f1c, int tile_k, float4v(&s)[4][2], int tile_v, const V8(&pf)[2][2]) {
+    auto mfma_phase = [&](auto f0c, auto f1c, int tile_k, float4v(&s)[4][QB], int tile_v, const V8(&pf)[2][QB]) {
         constexpr int F0 = decltype(f0c)::value, F1 = decltype(f1c)::value;
         MI355_LDS char* kst = kbuf + (tile_k & 1) * TILE_BYTES;
         MI355_LDS char* vst = vbuf + (tile_v & 1) * TILE_BYTES;
-        constexpr int AHEAD = 6;
+        constexpr int AHEAD = QB == 1 ? 5 : 6;
         V8 fr[AHEAD];
 #pragma unroll
         for (int i = 0; i < AHEAD; ++i) fr[i] = read_frag(kst, vst, F0 + i);
@@ -513,7 +280,7 @@ __global__ __launch_bounds__(512, 2) void fmha_fwd_pingpong_kernel(const T* __re
 #pragma unroll
             for (int kb = 0; kb < 4; ++kb)
 #pragma unroll
-                for (int qb = 0; qb < 2; ++qb) s[kb][qb] = float4v{0.f, 0.f, 0.f, 0.f};
+                for (int qb = 0; qb < QB; ++qb) s[kb][qb] = float4v{0.f, 0.f, 0.f, 0.f};
         }
 #pragma unroll
         for (int f = F0; f < F1; ++f) {
@@ -521,15 +288,15 @@ __global__ __launch_bounds__(512, 2) void fmha_fwd_pingpong_kernel(const T* __re
             const int r = (f - F0) % AHEAD;
             if (f < 16) {
                 const int ks = f >> 2, kb = f & 3;
-                s[kb][0] = Elem<T>::mfma16(fr[r], qf[0][ks], s[kb][0]);
-                s[kb][1] = Elem<T>::mfma16(fr[r], qf[1][ks], s[kb][1]);
+#pragma unroll
+                for (int qb = 0; qb < QB; ++qb) s[kb][qb] = Elem<T>::mfma16(fr[r], qf[qb][ks], s[kb][qb]);
             } else {
                 const int j = (f - 16) >> 3, db = (f - 16) & 7;
-                o[db][0] = Elem<T>::mfma16(fr[r], pf[j][0], o[db][0]);
-                o[db][1] = Elem<T>::mfma16(fr[r], pf[j][1], o[db][1]);
+#pragma unroll
+                for (int qb = 0; qb < QB; ++qb) o[db][qb] = Elem<T>::mfma16(fr[r], pf[j][qb], o[db][qb]);
                 if (kSumOnMatrixPipe && db == 3) {   // the row sums of this key step, in the middle of its eight d blocks
-                    l_acc[0] = Elem<T>::mfma16(ones, pf[j][0], l_acc[0]);
-                    l_acc[1] = Elem<T>::mfma16(ones, pf[j][1], l_acc[1]);
+#pragma unroll
+                    for (int qb = 0; qb < QB; ++qb) l_acc[qb] = Elem<T>::mfma16(ones, pf[j][qb], l_acc[qb]);
                 }
             }
             if (f + AHEAD < F1) fr[r] = read_frag(kst, vst, f + AHEAD);
@@ -540,12 +307,12 @@ __global__ __launch_bounds__(512, 2) void fmha_fwd_pingpong_kernel(const T* __re
     using I16 = std::integral_constant<int, 16>;
     using I32 = std::integral_constant<int, 32>;
 
-    auto softmax_tile = [&](float4v(&s)[4][2], int tile, V8(&pf)[2][2]) {
+    auto softmax_tile = [&](float4v(&s)[4][QB], int tile, V8(&pf)[2][QB]) {
         const int key0 = tile * BN;
         const bool need_mask = (key0 + BN > kv_valid) || (causal && (key0 + BN - 1 > q_wave0 + shift));
         if (need_mask) {
 #pragma unroll
-            for (int qb = 0; qb < 2; ++qb) {
+            for (int qb = 0; qb < QB; ++qb) {
                 const int qi = q_wave0 + qb * 16 + c16;
                 const int lim = causal ? min(kv_valid - 1, qi + shift) : kv_valid - 1;  // last visible key
 #pragma unroll
@@ -560,10 +327,10 @@ __global__ __launch_bounds__(512, 2) void fmha_fwd_pingpong_kernel(const T* __re
         // 2^kLazyLog2; then (any lane of the wave asked) the four lanes of every query agree on the tile's maximum and the
         // reference is raised to the running maximum. Otherwise P = exp2((S - m_run) c) <= 2^kLazyLog2 everywhere and nothing
         // crosses lanes.
-        float mx[2];
+        float mx[QB];
         bool raise = false;
 #pragma unroll
-        for (int qb = 0; qb < 2; ++qb) {
+        for (int qb = 0; qb < QB; ++qb) {
             float a = max3(s[0][qb][0], s[0][qb][1], s[0][qb][2]);
             float c = max3(s[0][qb][3], s[1][qb][0], s[1][qb][1]);
             a = max3(a, s[1][qb][2], s[1][qb][3]);
@@ -577,7 +344,7 @@ __global__ __launch_bounds__(512, 2) void fmha_fwd_pingpong_kernel(const T* __re
         }
         if (__builtin_amdgcn_ballot_w64(raise) != 0) {
 #pragma unroll
-            for (int qb = 0; qb < 2; ++qb) {
+            for (int qb = 0; qb < QB; ++qb) {
                 const float m_new = fmaxf(m_run[qb], quad_max(mx[qb]));
                 const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
                 const float alpha = fast_exp2((m_run[qb] - m_use) * scale_log2);
@@ -593,7 +360,7 @@ __global__ __launch_bounds__(512, 2) void fmha_fwd_pingpong_kernel(const T* __re
         // the wave is the only one of its SIMD issuing VALU work in this phase, so dependent instructions are kept apart:
         // all multiply-adds, then all exponentials, then the sums and conversions
 #pragma unroll
-        for (int qb = 0; qb < 2; ++qb) {
+        for (int qb = 0; qb < QB; ++qb) {
             const float neg_ms = (m_run[qb] == -INFINITY) ? 0.f : -m_run[qb] * scale_log2;
 #pragma unroll
             for (int kb = 0; kb < 4; ++kb)
@@ -604,12 +371,12 @@ __global__ __launch_bounds__(512, 2) void fmha_fwd_pingpong_kernel(const T* __re
 #pragma unroll
         for (int kb = 0; kb < 4; ++kb)
 #pragma unroll
-            for (int qb = 0; qb < 2; ++qb)
+            for (int qb = 0; qb < QB; ++qb)
 #pragma unroll
                 for (int e = 0; e < 4; ++e) s[kb][qb][e] = fast_exp2(s[kb][qb][e]);
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int qb = 0; qb < 2; ++qb) {
+        for (int qb = 0; qb < QB; ++qb) {
             float ps[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int j = 0; j < 2; ++j) {
@@ -635,8 +402,8 @@ __global__ __launch_bounds__(512, 2) void fmha_fwd_pingpong_kernel(const T* __re
         issue_v(0);
         if (late) next_phase();  // waves 4..7 idle during P0
 
-        float4v s[4][2];
-        V8 pf[2][2];
+        float4v s[4][QB];
+        V8 pf[2][QB];
         __builtin_amdgcn_s_setprio(1);
         mfma_phase(I0{}, I16{}, 0, s, 0, pf);               // S(0) alone
         __builtin_amdgcn_s_setprio(0);
@@ -663,7 +430,7 @@ __global__ __launch_bounds__(512, 2) void fmha_fwd_pingpong_kernel(const T* __re
 
     // ---- finalize: O / l, LSE: lane holds O[query 16 qb + c][d = 16 db + 4 g + 0..3] -----------------------------
 #pragma unroll
-    for (int qb = 0; qb < 2; ++qb) {
+    for (int qb = 0; qb < QB; ++qb) {
         const float l_tot = kSumOnMatrixPipe ? l_acc[qb][0] : quad_sum(l_acc[qb][0]);
         const float inv = (l_tot > 0.f) ? 1.f / l_tot : 0.f;
         const int qi = q_wave0 + qb * 16 + c16;
@@ -684,13 +451,13 @@ __global__ __launch_bounds__(512, 2) void fmha_fwd_pingpong_kernel(const T* __re
     }
 }
 
-template <typename T>
+template <typename T, int QB>
 static hipError_t launch_fmha_pingpong(const T* Q, const T* K, const T* V, T* O, float* LSE, int B, int Hq,
                                        int Hkv, int Sq, int Sk, float scale, int causal, int kv_valid, const FmhaStrides& sd,
                                        hipStream_t stream) {
-    constexpr int BM = 256;
+    constexpr int BM = 128 * QB;
     constexpr int LDS = 4 * fmha::TILE_BYTES;
-    auto kern = fmha_fwd_pingpong_kernel<T>;
+    auto kern = fmha_fwd_pingpong_kernel<T, QB>;
     static DynamicLdsOnce lds_once;
     if (hipError_t e = lds_once.ensure(reinterpret_cast<const void*>(kern), LDS); e != hipSuccess) return e;
     const int q_tiles = (Sq + BM - 1) / BM;
@@ -702,24 +469,6 @@ static hipError_t launch_fmha_pingpong(const T* Q, const T* K, const T* V, T* O,
     return hipGetLastError();
 }
 
-template <typename T, int NQ, int NWAVES>
-static hipError_t launch_fmha(const T* Q, const T* K, const T* V, T* O, float* LSE, int B, int Hq,
-                              int Hkv, int Sq, int Sk, float scale, int causal, int kv_valid, const FmhaStrides& sd,
-                                       hipStream_t stream) {
-    constexpr int BM = NWAVES * NQ * 32;
-    constexpr int LDS = fmha::STAGE_BYTES * fmha::NSTAGE;
-    auto kern = fmha_fwd_kernel<T, NQ, NWAVES>;
-    static DynamicLdsOnce lds_once;
-    if (hipError_t e = lds_once.ensure(reinterpret_cast<const void*>(kern), LDS); e != hipSuccess) return e;
-    const int q_tiles = (Sq + BM - 1) / BM;
-    const long blocks = (long)q_tiles * Hq * B;
-    if (blocks > 0x7fffffffL) return hipErrorInvalidValue;
-    const float scale_log2 = scale * 1.4426950408889634f;
-    kern<<<dim3((unsigned)blocks), dim3(NWAVES * 64), LDS, stream>>>(Q, K, V, O, LSE, B, Hq, Hkv, Sq, Sk, scale_log2,
-                                                                    causal, kv_valid, q_tiles, sd);
-    return hipGetLastError();
-}
-
 template <typename T>
 static hipError_t fmha_fwd_dispatch_t(const void* Q, const void* K, const void* V, void* O, float* LSE, int B, int Hq, int Hkv,
                                       int Sq, int Sk, float scale, int causal, int kv_valid_len, const FmhaStrides& sd,
@@ -728,21 +477,21 @@ static hipError_t fmha_fwd_dispatch_t(const void* Q, const void* K, const void* 
     const T* k = static_cast<const T*>(K);
     const T* v = static_cast<const T*>(V);
     T* o = static_cast<T*>(O);
-    // the split-KV and ping-pong kernels address a K/V tile with 32-bit byte offsets from its first row
-    const bool rows_fit_32bit = sd.k_row < (1L << 24) && sd.v_row < (1L << 24);
-    if ((variant == 0 || variant == 4) && rows_fit_32bit && fmha_decode_applicable(B, Hq, Hkv, Sq, Sk, kv_valid_len))
+    // the kernels address a K/V tile with 32-bit byte offsets from its first row
+    if (sd.k_row >= (1L << 24) || sd.v_row >= (1L << 24)) return hipErrorNotSupported;
+    if (variant == 0 && fmha_decode_applicable(B, Hq, Hkv, Sq, Sk, kv_valid_len))
         return fmha_decode_dispatch<T>(q, k, v, o, LSE, B, Hq, Hkv, Sq, Sk, scale, causal, kv_valid_len, sd, ws, stream);
-    if (variant == 0 || variant == 4) {
-        // 256-query ping-pong workgroups once there are enough of them to fill the 256 CUs, otherwise 128-query ones
+    if (variant == 0) {
+        // 256-query workgroups once there are clearly more of them than CUs (with exactly one per CU a causal problem runs
+        // as long as its heaviest tile; 128-query workgroups then balance better and still fill the machine) and the
+        // sequences are long enough to amortise their longer prologue. Measured (b, heads 32/8, s, 128- vs 256-query):
+        // 1 x 1024 causal 25 / 35 us, 1 x 2048 57 / 65, 8 x 512 43 / 50, 1 x 3000 108 / 94, 1 x 4096 182 / 144,
+        // 4 x 1024 (32 kv heads, non-causal) 100 / 82.
         const long wg256 = (long)((Sq + 255) / 256) * Hq * B;
-        variant = (wg256 >= 256) ? 3 : 1;
+        variant = (wg256 >= 320 && Sq > 512) ? 2 : 1;
     }
-    if (variant == 3 && !rows_fit_32bit) variant = 1;
-    switch (variant) {
-        case 2: return launch_fmha<T, 1, 8>(q, k, v, o, LSE, B, Hq, Hkv, Sq, Sk, scale, causal, kv_valid_len, sd, stream);
-        case 3: return launch_fmha_pingpong<T>(q, k, v, o, LSE, B, Hq, Hkv, Sq, Sk, scale, causal, kv_valid_len, sd, stream);
-        default: return launch_fmha<T, 1, 4>(q, k, v, o, LSE, B, Hq, Hkv, Sq, Sk, scale, causal, kv_valid_len, sd, stream);
-    }
+    if (variant == 2) return launch_fmha_pingpong<T, 2>(q, k, v, o, LSE, B, Hq, Hkv, Sq, Sk, scale, causal, kv_valid_len, sd, stream);
+    return launch_fmha_pingpong<T, 1>(q, k, v, o, LSE, B, Hq, Hkv, Sq, Sk, scale, causal, kv_valid_len, sd, stream);
 }
 
 hipError_t fmha_fwd_dispatch(const void* Q, const void* K, const void* V, void* O, float* LSE, int B, int Hq, int Hkv,

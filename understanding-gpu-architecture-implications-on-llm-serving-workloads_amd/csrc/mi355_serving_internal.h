@@ -80,8 +80,8 @@ hipError_t silu_mul_dispatch(const void* in, void* out, long rows, int inter, in
 // Test and tuning hooks: exported from the shared library but not part of its public header. They take the kernel
 // variant as an argument (no process-wide state): variants that do not fit the shape fall back to the choice by shape.
 //   gemm: 0 = by shape, 1 = 256x256 tiles, 2 = 128x128 tiles
-//   fmha: 0 = by shape, 1 = 4 waves x 32 queries, 2 = 8 waves x 32 queries, 3 = 8 waves x 32 queries ping-pong
-//         (1..3 also keep generation-step shapes off the split-KV path)
+//   fmha: 0 = by shape, 1 = 128-query workgroups, 2 = 256-query workgroups (1 and 2 also keep generation-step shapes off
+//         the split-KV path)
 extern "C" {
 int mi355_internal_hgemm_variant(const void* A, const void* B, void* C, int M, int N, int K, int64_t lda, int64_t ldb,
                                  int64_t ldc, int layout, int dtype, int variant, void* stream);
