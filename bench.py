@@ -44,6 +44,33 @@ def log(*a):
     print(*a, file=sys.stderr, flush=True)
 
 
+def time_graph(fn, iters, warmup):
+    """Mean duration (ms) of `iters` launches replayed from ONE HIP graph (captured after `warmup` eager launches on the
+    capture stream): the kernels run back to back without the ~3 us the runtime takes between two dependent eager launches,
+    which is a sizeable part of a 20 us kernel. HIP events around the replay, on the stream it runs on."""
+    import torch
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(warmup):
+            fn()
+    side.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        for _ in range(iters):
+            fn()
+    graph.replay()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    graph.replay()
+    e1.record()
+    e1.synchronize()
+    ms = e0.elapsed_time(e1) / iters
+    del graph
+    return ms
+
+
 def time_launches(fn, iters, warmup, stats=False):
     """Mean duration (ms) of `iters` back-to-back launches after `warmup` untimed ones: two HIP events on the current
     stream around the whole batch. With stats=True a second batch is timed with an event after every launch, for the
@@ -223,8 +250,11 @@ def main():
             x_h, w_h = so.randn_fp16((m, kk), 1), so.randn_fp16((kk, n), 2, 0.02)
             x, w = x_h.to(dev), w_h.to(dev)
             out = torch.empty((m, n), dtype=torch.float16, device=dev)
-            t = time_launches(lambda: lib.hgemm_raw(x.data_ptr(), w.data_ptr(), out.data_ptr(), m, n, kk, kk, n, n,
-                                                    lib.GEMM_NN, stream), iters, 10, stats=True)
+            fn_ = lambda: lib.hgemm_raw(x.data_ptr(), w.data_ptr(), out.data_ptr(), m, n, kk, kk, n, n, lib.GEMM_NN,
+                                        torch.cuda.current_stream().cuda_stream)
+            t = time_launches(fn_, iters, 10, stats=True)
+            t["ms_eager"] = t["ms"]
+            t["ms"] = time_graph(fn_, iters, 10)   # replayed from one HIP graph: without the runtime's gap between eager launches
             ms = t["ms"]
             fl, by = 2.0 * m * n * kk, 2.0 * (m * kk + kk * n + m * n)
             rows_ = torch.arange(0, m, max(1, m // 64))
@@ -488,7 +518,7 @@ KERNEL_CONFIGS = {
 
 def run_kernel_config(args, torch, lib, so, dev):
     cfg = KERNEL_CONFIGS[args.kernel_config]
-    stream = torch.cuda.current_stream().cuda_stream
+    cur = lambda: torch.cuda.current_stream().cuda_stream   # at call time: graph capture runs on a stream of its own
     if cfg[0] == "gemm":
         _, M, N, K, lay = cfg
         a_h, b_h = so.gemm_inputs(M, N, K, seed=0, a_std=1.0, b_std=0.02)
@@ -496,7 +526,7 @@ def run_kernel_config(args, torch, lib, so, dev):
             b_h = b_h.t().contiguous()
         a, b = a_h.to(dev), b_h.to(dev)
         c = torch.empty((M, N), dtype=torch.float16, device=dev)
-        fn = lambda: lib.hgemm_raw(a.data_ptr(), b.data_ptr(), c.data_ptr(), M, N, K, a.shape[1], b.shape[1], N, lib.LAYOUTS[lay], stream)
+        fn = lambda: lib.hgemm_raw(a.data_ptr(), b.data_ptr(), c.data_ptr(), M, N, K, a.shape[1], b.shape[1], N, lib.LAYOUTS[lay], cur())
         flops, nbytes = 2.0 * M * N * K, 2.0 * (M * K + K * N + M * N)
     else:
         _, B, Hq, Hkv, Sq, Sk, causal = cfg
@@ -504,7 +534,7 @@ def run_kernel_config(args, torch, lib, so, dev):
         o = torch.empty_like(q)
         lse = torch.empty((B, Hq, Sq), dtype=torch.float32, device=dev)
         fn = lambda: lib.fmha_fwd_raw(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), lse.data_ptr(), B, Hq, Hkv, Sq, Sk,
-                                      128, 1.0 / math.sqrt(128), int(causal), Sk, stream)
+                                      128, 1.0 / math.sqrt(128), int(causal), Sk, cur())
         flops = 4.0 * B * Hq * 128 * (causal_pairs(Sq, Sk) if causal else Sq * Sk)
         nbytes = 2.0 * (2 * B * Hq * Sq * 128 + 2 * B * Hkv * Sk * 128) + 4.0 * B * Hq * Sq
     if args.calibrate_copy:
@@ -514,7 +544,9 @@ def run_kernel_config(args, torch, lib, so, dev):
         torch.cuda.synchronize()
         del src, dst
     t = time_launches(fn, args.steps, args.warmup, stats=True)
+    t["ms_graph_replay"] = time_graph(fn, args.steps, args.warmup)
     print(json.dumps(dict(t, kernel_config=args.kernel_config, tflops=flops / t["ms"] / 1e9, gbs=nbytes / t["ms"] / 1e6,
+                          tflops_graph_replay=flops / t["ms_graph_replay"] / 1e9, gbs_graph_replay=nbytes / t["ms_graph_replay"] / 1e6,
                           algorithmic_flop=flops, algorithmic_bytes=nbytes)))
 
 
