@@ -38,7 +38,17 @@ constexpr int STAGE_BYTES = 2 * TILE_BYTES;  // K + V
 constexpr float kLazyLog2 = 8.f;             // rescale only when a column maximum grows by more than 2^8
 constexpr int COPIES = 2 * (TILE_BYTES / 1024);  // 16 copy instructions per stage
 constexpr int PART_STRIDE = D + 4;           // floats per (workgroup, column): O~[128], m, l, 2 pad (keeps rows 16-byte aligned)
-constexpr int kCounterAlign = 256;           // the counters in front of the partial results are padded to this many bytes
+// Ticket counters lie this many 32-bit words (256 bytes) apart. Device-scope atomics of workgroups on different XCDs are
+// carried out at the memory side, one after the other per address range: with the counters of all (batch, kv head)
+// pairs in one 64-byte line, the 256 tickets of a call queued up behind each other (~12 ns each, 3 us from the first to
+// the last at batch 1); 256 bytes apart they proceed side by side (a larger stride brought nothing more).
+constexpr int kCounterStride = 64;
+// The counters occupy a region of FIXED size at the start of every workspace, whatever the call: a workspace is shared by
+// calls of different shapes, each of which leaves its counters at zero, and a region that grew and shrank with the number
+// of (batch, kv head) pairs would let one call's partial results land where the next call keeps its counters. A call is
+// cut into several key ranges only while it has at most kMaxSplitPairs pairs.
+constexpr int kMaxSplitPairs = 255;
+constexpr size_t kCounterBytes = size_t(kMaxSplitPairs + 1) * kCounterStride * sizeof(unsigned);   // 64 KiB
 
 __device__ __forceinline__ int swz_k(int row) { return row & 15; }
 __device__ __forceinline__ int swz_v(int row) {
@@ -303,7 +313,7 @@ __global__ __launch_bounds__(WAVES * 64) void fmha_decode_kernel(
     wait_vmcnt<0>();   // this thread's partial results have reached memory before the ticket is drawn
     __syncthreads();
     MI355_LDS unsigned* ticket_sh = (MI355_LDS unsigned*)(cmb + WAVES * wave_floats);
-    if (tid == 0) *ticket_sh = __hip_atomic_fetch_add(&counters[bh], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (tid == 0) *ticket_sh = __hip_atomic_fetch_add(&counters[(long)bh * kCounterStride], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     __syncthreads();
     if (*ticket_sh != (unsigned)(splits - 1)) return;
     // last ticket: every other workgroup of (b, hkv) drew its ticket after its partial results had reached memory.
@@ -344,29 +354,47 @@ __global__ __launch_bounds__(WAVES * 64) void fmha_decode_kernel(
         st_l[i] = ls;
     }
     __syncthreads();
+    // The weight of key range s for column c, 2^((m_s - m_c) scale), is worked out once, by thread s * ncols + c, and left in
+    // LDS together with its share of the row sum; the accumulation loop below then is two LDS reads and four
+    // multiply-adds per key range.
+    MI355_LDS float* st_w = cmb + 2 * splits * ncols;     // [splits][ncols]: weight of key range s
+    MI355_LDS float* st_mc = cmb + 3 * splits * ncols;    // [ncols]: m_c
+    for (int i = tid; i < splits * ncols; i += NTHREADS) {
+        const int c = i % ncols;
+        float m = -INFINITY;
+        for (int sp0 = 0; sp0 < splits; sp0 += 8) {   // 8 independent LDS reads at a time
+            float ms[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) ms[u] = st_m[min(sp0 + u, splits - 1) * ncols + c];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) m = fmaxf(m, ms[u]);
+        }
+        const float w = (m == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f((st_m[i] - m) * scale_log2);
+        st_w[i] = w;
+        st_l[i] *= w;
+        if (i < ncols) st_mc[c] = m;
+    }
+    __syncthreads();
     for (int f = tid; f < n_out; f += NTHREADS) {
         const int c = f >> 5, d = (f & 31) * 4;
         const float* pc = base + c * PART_STRIDE + d;
-        // every thread works out the statistics of its column itself (the lanes of a wave share one or two columns, so the
-        // LDS reads are broadcasts): cheaper than another pass and barrier with a few threads busy
-        float m = -INFINITY;
-        for (int sp = 0; sp < splits; ++sp) m = fmaxf(m, st_m[sp * ncols + c]);
         float4v acc = float4v{0.f, 0.f, 0.f, 0.f};
         float l = 0.f;
         for (int sp0 = 0; sp0 < splits; sp0 += BATCH) {
             if (f != tid || sp0 != 0) load_batch(v, pc, sp0);
-            // the weights of this batch, while its loads are in flight (all LDS reads first, so they overlap each other)
+            // the weights of this batch, while its loads are in flight (all LDS reads first, so they overlap each other);
+            // key ranges past the last one repeat it with weight zero
             float wgt[BATCH], ls[BATCH];
 #pragma unroll
             for (int u = 0; u < BATCH; ++u) {
                 const int sp = min(sp0 + u, splits - 1);
-                wgt[u] = st_m[sp * ncols + c];
+                wgt[u] = st_w[sp * ncols + c];
                 ls[u] = st_l[sp * ncols + c];
             }
 #pragma unroll
             for (int u = 0; u < BATCH; ++u) {
-                wgt[u] = (m == -INFINITY || sp0 + u >= splits) ? 0.f : __builtin_amdgcn_exp2f((wgt[u] - m) * scale_log2);
-                l += wgt[u] * ls[u];
+                if (sp0 + u >= splits) wgt[u] = ls[u] = 0.f;
+                l += ls[u];
             }
             wait_batch(v);
 #pragma unroll
@@ -381,9 +409,9 @@ __global__ __launch_bounds__(WAVES * 64) void fmha_decode_kernel(
         for (int e = 0; e < 4; ++e) ov[e] = (T)(acc[e] * inv);
         *(typename Elem<T>::v4*)(O + b * sd.o_batch + chq * sd.o_head + cqi * sd.o_row + d) = ov;
         if (LSE != nullptr && d == 0)
-            LSE[row0 + c] = (l > 0.f) ? (m * scale_log2 + __builtin_log2f(l)) * 0.69314718055994531f : -INFINITY;
+            LSE[row0 + c] = (l > 0.f) ? (st_mc[c] * scale_log2 + __builtin_log2f(l)) * 0.69314718055994531f : -INFINITY;
     }
-    if (tid == 0) counters[bh] = 0u;   // ready for the next call that uses this workspace
+    if (tid == 0) counters[(long)bh * kCounterStride] = 0u;   // ready for the next call that uses this workspace
 }
 
 // Sets the counters of a workspace whose contents are unknown (a caller's) to zero.
@@ -400,8 +428,8 @@ namespace dec {
 constexpr int kMaxSplits = 256;   // key ranges per (batch, kv head)
 }   // up to this many tiles per wave: <4 waves, 2 stages>
 
-// How a call is cut into workgroups, and what its workspace holds: one counter per (batch, kv head), padded to
-// kCounterAlign bytes, then the partial results [workgroup][column][PART_STRIDE].
+// How a call is cut into workgroups, and what its workspace holds: one counter per (batch, kv head), kCounterStride
+// words apart, then the partial results [workgroup][column][PART_STRIDE].
 struct DecodePlan {
     int splits, tiles_per_split;
     long workgroups;
@@ -414,7 +442,7 @@ static DecodePlan decode_plan(int B, int Hq, int Hkv, int Sq, int kv_valid) {
     const long pairs = (long)B * Hkv;
     // about one workgroup per CU; a key range is at least 8 tiles (two per wave)
     long splits = (256 + pairs / 2) / pairs;
-    splits = splits < 1 ? 1 : splits;
+    splits = (splits < 1 || pairs > kMaxSplitPairs) ? 1 : splits;
     const long max_splits = (tiles + 7) / 8;
     if (splits > max_splits) splits = max_splits;
     if (splits > kMaxSplits) splits = kMaxSplits;
@@ -422,7 +450,7 @@ static DecodePlan decode_plan(int B, int Hq, int Hkv, int Sq, int kv_valid) {
     p.tiles_per_split = (int)((tiles + splits - 1) / splits);
     p.splits = (tiles + p.tiles_per_split - 1) / p.tiles_per_split;
     p.workgroups = pairs * p.splits;
-    p.counter_bytes = p.splits > 1 ? ((size_t)pairs * sizeof(unsigned) + kCounterAlign - 1) / kCounterAlign * kCounterAlign : 0;
+    p.counter_bytes = p.splits > 1 ? kCounterBytes : 0;
     p.bytes = p.splits > 1 ? p.counter_bytes + (size_t)p.workgroups * ncols * PART_STRIDE * sizeof(float) : 0;
     return p;
 }
@@ -501,7 +529,7 @@ static hipError_t launch_decode(const T* Q, const T* K, const T* V, T* O, float*
                                 int tiles_per_split, long workgroups, const FmhaStrides& sd, hipStream_t stream) {
     constexpr int LDS = WAVES * NSTAGE * dec::STAGE_BYTES;
     static_assert(LDS >= WAVES * (32 * dec::D + 64) * 4 + 64, "the combine step reuses the pipeline memory");
-    static_assert(LDS >= (2 * dec::kMaxSplits * 32 + 64) * 4, "so does the merge of the key ranges");
+    static_assert(LDS >= (3 * dec::kMaxSplits * 32 + 32 + 64) * 4, "so does the merge of the key ranges");
     auto kern = fmha_decode_kernel<T, WAVES, NSTAGE>;
     static DynamicLdsOnce lds_once;
     if (hipError_t e = lds_once.ensure(reinterpret_cast<const void*>(kern), LDS); e != hipSuccess) return e;
@@ -527,7 +555,7 @@ hipError_t fmha_decode_dispatch(const T* Q, const T* K, const T* V, T* O, float*
                 // a caller's memory holds anything: zero its counters first (the library's own buffers and the static array
                 // start at zero and every call leaves them at zero)
                 fmha_decode_clear_kernel<<<dim3(1), dim3(256), 0, stream>>>(reinterpret_cast<unsigned*>(wsp),
-                                                                            (int)(plan.counter_bytes / sizeof(unsigned)));
+                                                                            (int)((long)B * Hkv * kCounterStride));   // this call's counters
                 e = hipGetLastError();
                 break;
             case FmhaWorkspace::kStatic:
