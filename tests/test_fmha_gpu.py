@@ -138,6 +138,15 @@ def test_generation_step_split_kv_path(lib, gpu, B, Hq, Hkv, Sq, Sk, causal, kvv
     assert (o.float() - o1.float()).abs().max() <= 2e-3 and (lse - lse1).abs().max() <= 1e-3
 
 
+def test_generation_step_workspace_shared_by_calls_of_different_shapes(lib, gpu):
+    # One workspace per stream serves every call. The ticket counters sit in a region of fixed size in front of the partial
+    # results: calls with 8, then 4, then 64, then 8 (batch, kv head) pairs must all find their counters at zero (with a
+    # counter region sized by the call, the partial results of the second call lay on counters of the fourth).
+    for B, Hq, Hkv, Sk in ((1, 32, 8, 4096), (2, 8, 2, 1500), (8, 32, 8, 2048), (1, 32, 8, 4096), (170, 1, 1, 640), (3, 8, 4, 1024)):
+        q, k, v = so.fmha_inputs(B, Hq, Hkv, 1, Sk, seed=B + Sk)
+        check(lib, gpu, q, k, v, False, None)
+
+
 def test_generation_step_on_two_streams(lib, gpu):
     # the split-KV workspace is per stream: interleaved calls on two streams must not disturb each other
     qa, ka, va = (t.to(gpu) for t in so.fmha_inputs(1, 32, 8, 1, 4096, seed=1))

@@ -325,11 +325,18 @@ __global__ __launch_bounds__(WAVES * 64) void fmha_decode_kernel(
     MI355_LDS float* st_l = cmb + splits * ncols;         // [splits][ncols]: l_s
     constexpr int BATCH = 32;
     // BATCH loads of 16 bytes each: the outputs of key ranges sp0 .. sp0 + BATCH - 1 for 4 d of one column
+    // (in groups of 8 key ranges, a group only when it holds a key range that exists: a call with 4 key ranges issues 8
+    // loads per thread, not 32; within a group, key ranges past the last one repeat it and get weight zero)
     auto load_batch = [&](float4v(&v)[BATCH], const float* pc, int sp0) {
 #pragma unroll
-        for (int u = 0; u < BATCH; ++u) {
-            const float* pa = pc + (long)min(sp0 + u, splits - 1) * split_stride;
-            asm volatile("global_load_dwordx4 %0, %1, off sc1" : "=v"(v[u]) : "v"(pa) : "memory");
+        for (int g8 = 0; g8 < BATCH; g8 += 8) {
+            if (sp0 + g8 < splits) {
+#pragma unroll
+                for (int u = g8; u < g8 + 8; ++u) {
+                    const float* pa = pc + (long)min(sp0 + u, splits - 1) * split_stride;
+                    asm volatile("global_load_dwordx4 %0, %1, off sc1" : "=v"(v[u]) : "v"(pa) : "memory");
+                }
+            }
         }
     };
     auto wait_batch = [](float4v(&v)[BATCH]) {   // the loads above have landed; nothing that uses v moves in front of this
@@ -386,21 +393,31 @@ __global__ __launch_bounds__(WAVES * 64) void fmha_decode_kernel(
             // key ranges past the last one repeat it with weight zero
             float wgt[BATCH], ls[BATCH];
 #pragma unroll
-            for (int u = 0; u < BATCH; ++u) {
-                const int sp = min(sp0 + u, splits - 1);
-                wgt[u] = st_w[sp * ncols + c];
-                ls[u] = st_l[sp * ncols + c];
-            }
+            for (int g8 = 0; g8 < BATCH; g8 += 8) {
+                if (sp0 + g8 < splits) {
 #pragma unroll
-            for (int u = 0; u < BATCH; ++u) {
-                if (sp0 + u >= splits) wgt[u] = ls[u] = 0.f;
-                l += ls[u];
+                    for (int u = g8; u < g8 + 8; ++u) {
+                        const int sp = min(sp0 + u, splits - 1);
+                        wgt[u] = st_w[sp * ncols + c];
+                        ls[u] = st_l[sp * ncols + c];
+                    }
+#pragma unroll
+                    for (int u = g8; u < g8 + 8; ++u) {
+                        if (sp0 + u >= splits) wgt[u] = ls[u] = 0.f;
+                        l += ls[u];
+                    }
+                }
             }
             wait_batch(v);
 #pragma unroll
-            for (int u = 0; u < BATCH; ++u)
+            for (int g8 = 0; g8 < BATCH; g8 += 8) {
+                if (sp0 + g8 < splits) {
 #pragma unroll
-                for (int e = 0; e < 4; ++e) acc[e] += wgt[u] * v[u][e];
+                    for (int u = g8; u < g8 + 8; ++u)
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) acc[e] += wgt[u] * v[u][e];
+                }
+            }
         }
         const float inv = (l > 0.f) ? 1.f / l : 0.f;
         const int chq = hkv * group + c / Sq, cqi = c % Sq;
