@@ -199,7 +199,7 @@ int mi355_silu_mul_bf16(const void* gate_up, void* out, int64_t rows, int inter,
  * The attention forward with a workspace owned by the caller, for callers that manage all device memory themselves
  * (HIP graph capture, arena allocators). mi355_fmha_fwd_workspace_bytes returns how many bytes a call with these sizes
  * needs: 0 for every shape outside the split-KV path and when B * Hkv is large enough for one key range per (batch, kv
- * head) (then `workspace` may be NULL), otherwise the size of its partial results (at most ~9 MiB). mi355_fmha_fwd_ws is mi355_fmha_fwd_strided (strides == NULL:
+ * head) (then `workspace` may be NULL), otherwise 64 KiB of ticket counters plus the size of its partial results (at most ~9 MiB). mi355_fmha_fwd_ws is mi355_fmha_fwd_strided (strides == NULL:
  * contiguous [B, H, S, D] operands) for dtype MI355_DTYPE_FP16 or MI355_DTYPE_BF16 that keeps those partial results in
  * `workspace` (16-byte aligned, at least that many bytes, contents irrelevant before and after the call: a small kernel
  * clears the part that must start at zero) and never allocates. Calls that share a workspace must be ordered on one stream. No counterpart in the reference, whose
@@ -215,8 +215,8 @@ int mi355_fmha_fwd_ws(const void* Q, const void* K, const void* V, void* O, floa
  * memory at all: code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc. It has no
  * counterpart in the reference. It calls no hipMalloc / hipFree or any other allocating routine: the partial results of
  * the split-KV path live in a fixed 4 MiB array in device memory that is part of the library's code object (one copy
- * per GPU the library runs on, held until the process ends). A call whose partial results do not fit (more than about
- * 7900 = 4 MiB / 528 B (workgroup, query column) pairs; a call runs about 256 workgroups, so this means more than ~30 query
+ * per GPU the library runs on, held until the process ends; its first 64 KiB hold the ticket counters). A call whose partial results do not fit (more than about
+ * 7800 = (4 MiB - 64 KiB) / 528 B (workgroup, query column) pairs; a call runs about 256 workgroups, so this means more than ~30 query
  * rows per kv head at small batch; a Llama generation step has 4) returns MI355_ERR_UNSUPPORTED and launches nothing. Every call on a GPU shares that GPU's array: calls through this entry point
  * that overlap on one GPU (different streams, or threads) race; order them on one stream. Shapes outside the split-KV path
  * (prefill) do not touch the array and behave exactly like mi355_fmha_fwd_strided.
