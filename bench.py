@@ -120,6 +120,13 @@ def main():
     ap.add_argument("--kernel-config", default=None, choices=sorted(KERNEL_CONFIGS),
                     help="launch one named kernel configuration --steps times (after --warmup) and print its timing; the "
                          "workload of the per-kernel rocprofv3 summaries in profiles/")
+    ap.add_argument("--timeline", action="store_true",
+                    help="with --kernel-config: load the profiling twin of the library (libmi355_serving_timeline.so), whose "
+                         "tiled GEMM and attention kernels record wall-clock and cycle stamps per workgroup, and print a "
+                         "summary of the last launch (configurations on the small-M GEMM kernels leave no records)")
+    ap.add_argument("--zero-inputs", action="store_true",
+                    help="with --kernel-config: all-zero operands instead of the seeded random ones (the arithmetic and its "
+                         "cycle count stay the same, the switching power does not: shows what the board's power limit costs)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also launch one 1 GiB device-to-device copy, so FETCH_SIZE / WRITE_SIZE read under rocprofv3 "
                          "--pmc can be scaled by what the same counter reports for a transfer of known size")
@@ -134,6 +141,10 @@ def main():
 
     if not torch.cuda.is_available():
         sys.exit("bench.py: no GPU visible; the kernels have no CPU fallback")
+    if args.timeline:
+        if not args.kernel_config:
+            sys.exit("bench.py: --timeline needs --kernel-config")
+        lib.LIB_PATH = os.path.join(os.path.dirname(lib.LIB_PATH), "libmi355_serving_timeline.so")
     lib.load()
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
@@ -516,6 +527,50 @@ KERNEL_CONFIGS = {
 }
 
 
+def timeline_summary(lib, cfg):
+    """Summary of the per-workgroup stamps the profiling twin of the library recorded in its last attention launch
+    (csrc/mi355_timeline.h): microseconds from the first workgroup's entry, 100 MHz wall clock; cycles = shader clock."""
+    import ctypes
+    import numpy as np
+    gemm = cfg[0] == "gemm"
+    decode = (not gemm) and cfg[4] == 1
+    buf = np.zeros(4096 * 8, dtype=np.uint64)
+    read = (lib.load().mi355_timeline_read_hgemm if gemm else
+            lib.load().mi355_timeline_read_fmha_decode if decode else lib.load().mi355_timeline_read_fmha_fwd)
+    read.argtypes = [ctypes.c_void_p, ctypes.c_size_t]
+    rc = read(buf.ctypes.data_as(ctypes.c_void_p), buf.nbytes)
+    if rc != 0:
+        raise RuntimeError("timeline read failed: %d" % rc)
+    rec = buf.reshape(4096, 8).astype(np.float64)
+    rec = rec[rec[:, 0] > 0]
+    t0 = rec[:, 0].min()
+    us = lambda col: (col[col > 0] - t0) / 100.0
+    stat = lambda x: {"workgroups": int(x.size), "min": round(float(x.min()), 2), "mean": round(float(x.mean()), 2), "max": round(float(x.max()), 2)} if x.size else None
+    if decode:
+        names = ["entry", "first_tile_landed", "key_range_done", "partials_stored", "ticket_drawn", "merge_partials_landed",
+                 "merge_summed", "exit"]
+        return {"unit": "us after the first workgroup's entry", **{n: stat(us(rec[:, i])) for i, n in enumerate(names)}}
+    tiles = np.maximum(rec[:, 6], 1.0)
+    loop_us = (rec[:, 2] - rec[:, 1]) / 100.0
+    loop_cycles = rec[:, 5] - rec[:, 4]
+    big = rec[:, 6] >= 0.75 * rec[:, 6].max()    # pipeline fill and drain weigh on workgroups with few tiles
+    if gemm:   # a K tile of 64 is 64 MFMA 16x16x32 per wave of the 256x256 tile, 2 waves per SIMD
+        return {"unit": "us after the first workgroup's entry", "workgroups_recorded": int(rec.shape[0]),
+                "kernel_span_us": round(float((rec[:, 3].max() - t0) / 100.0), 2),
+                "prologue_us": stat((rec[:, 1] - rec[:, 0]) / 100.0), "epilogue_us": stat((rec[:, 3] - rec[:, 2]) / 100.0),
+                "k_tiles_per_workgroup": stat(rec[:, 6]), "loop_cycles_per_k_tile": stat(loop_cycles / tiles),
+                "loop_clock_ghz": stat(loop_cycles / (loop_us * 1e3)),
+                "note": "MFMA cycles per K tile and SIMD: 2048 for 256x256 tiles (8 waves), 1024 for 128x128 tiles (4 waves)"}
+    return {"unit": "us after the first workgroup's entry", "workgroups": int(rec.shape[0]),
+            "kernel_span_us": round(float((rec[:, 3].max() - t0) / 100.0), 2),
+            "prologue_us": stat((rec[:, 1] - rec[:, 0]) / 100.0), "epilogue_us": stat((rec[:, 3] - rec[:, 2]) / 100.0),
+            "key_tiles_per_workgroup": stat(rec[:, 6]),
+            "loop_us_per_key_tile": stat(loop_us / tiles),
+            "long_workgroups": {"loop_cycles_per_key_tile": stat((loop_cycles / tiles)[big]),
+                                "loop_clock_ghz": stat((loop_cycles / (loop_us * 1e3))[big])},
+            "mfma_cycles_per_key_tile_per_simd": 2 * 68 * 16}
+
+
 def run_kernel_config(args, torch, lib, so, dev):
     cfg = KERNEL_CONFIGS[args.kernel_config]
     cur = lambda: torch.cuda.current_stream().cuda_stream   # at call time: graph capture runs on a stream of its own
@@ -525,12 +580,16 @@ def run_kernel_config(args, torch, lib, so, dev):
         if lay == "NT":
             b_h = b_h.t().contiguous()
         a, b = a_h.to(dev), b_h.to(dev)
+        if args.zero_inputs:
+            a.zero_(), b.zero_()
         c = torch.empty((M, N), dtype=torch.float16, device=dev)
         fn = lambda: lib.hgemm_raw(a.data_ptr(), b.data_ptr(), c.data_ptr(), M, N, K, a.shape[1], b.shape[1], N, lib.LAYOUTS[lay], cur())
         flops, nbytes = 2.0 * M * N * K, 2.0 * (M * K + K * N + M * N)
     else:
         _, B, Hq, Hkv, Sq, Sk, causal = cfg
         q, k, v = (t.to(dev) for t in so.fmha_inputs(B, Hq, Hkv, Sq, Sk, seed=42))
+        if args.zero_inputs:
+            q.zero_(), k.zero_(), v.zero_()
         o = torch.empty_like(q)
         lse = torch.empty((B, Hq, Sq), dtype=torch.float32, device=dev)
         fn = lambda: lib.fmha_fwd_raw(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), lse.data_ptr(), B, Hq, Hkv, Sq, Sk,
@@ -544,6 +603,11 @@ def run_kernel_config(args, torch, lib, so, dev):
         torch.cuda.synchronize()
         del src, dst
     t = time_launches(fn, args.steps, args.warmup, stats=True)
+    if args.timeline:
+        fn()
+        torch.cuda.synchronize()
+        print(json.dumps(dict(t, kernel_config=args.kernel_config, zero_inputs=bool(args.zero_inputs), timeline=timeline_summary(lib, cfg))))
+        return
     t["ms_graph_replay"] = time_graph(fn, args.steps, args.warmup)
     print(json.dumps(dict(t, kernel_config=args.kernel_config, tflops=flops / t["ms"] / 1e9, gbs=nbytes / t["ms"] / 1e6,
                           tflops_graph_replay=flops / t["ms_graph_replay"] / 1e9, gbs_graph_replay=nbytes / t["ms_graph_replay"] / 1e6,

@@ -2,6 +2,7 @@
 
 Produces, inside the three packages:
     mi355_serving/libmi355_serving.so   HIP kernels + C ABI (include/mi355_serving.h); no torch dependency
+    mi355_serving/libmi355_serving_timeline.so   profiling twin: the attention kernels also record per-workgroup time stamps
     gemm_unified/_C.so                  torch operators gemm_unified::finegemm_N, linked against the library above
     fmha_unified/_C.so                  torch operators fmha_unified::finefmha_N
 Each _C.so finds the library through RUNPATH $ORIGIN/../mi355_serving: the packages sit side by side both in the source
@@ -65,8 +66,16 @@ def _run(cmd, quiet_patterns=("is not a recognized feature for this target",)):
         print(out)
 
 
+TIMELINE_LIB_NAME = "libmi355_serving_timeline.so"
+TIMELINE_LIB_PATH = os.path.join(LIB_DIR, TIMELINE_LIB_NAME)
+# Sources that carry per-workgroup time stamps when compiled with -DMI355_TIMELINE (csrc/mi355_timeline.h).
+TIMELINE_SOURCES = ("csrc/hgemm.hip", "csrc/fmha_fwd.hip", "csrc/fmha_decode.hip")
+
+
 def build_library(verbose=True):
-    """Compile the HIP kernels and the C ABI into libmi355_serving.so (one object per source, compiled side by side)."""
+    """Compile the HIP kernels and the C ABI into libmi355_serving.so (one object per source, compiled side by side), and
+    the profiling twin libmi355_serving_timeline.so: the same objects, except that the GEMM and attention sources are compiled a
+    second time with -DMI355_TIMELINE (`bench.py --timeline` loads it; nothing else does)."""
     import tempfile
     from concurrent.futures import ThreadPoolExecutor
 
@@ -76,15 +85,24 @@ def build_library(verbose=True):
         for src in KERNEL_SOURCES:
             obj = os.path.join(tmp, os.path.basename(src) + ".o")
             cmd = [HIPCC] + DEVICE_FLAGS + SOURCE_FLAGS.get(src, []) + ["-I", INCLUDE, "-c", src, "-o", obj]
-            if verbose:
-                print("[build] " + " ".join(cmd))
             jobs.append((cmd, obj))
+        tl_objs = {}
+        for src in TIMELINE_SOURCES:
+            obj = os.path.join(tmp, os.path.basename(src) + ".timeline.o")
+            cmd = [HIPCC] + DEVICE_FLAGS + SOURCE_FLAGS.get(src, []) + ["-DMI355_TIMELINE", "-I", INCLUDE, "-c", src, "-o", obj]
+            jobs.append((cmd, obj))
+            tl_objs[src] = obj
+        if verbose:
+            for cmd, _ in jobs:
+                print("[build] " + " ".join(cmd))
         with ThreadPoolExecutor(max_workers=max_jobs(len(jobs))) as pool:
             list(pool.map(lambda job: _run(job[0]), jobs))
-        link = [HIPCC, "--offload-arch=gfx950", "-fPIC", "-shared"] + [obj for _, obj in jobs] + ["-o", LIB_PATH]
-        if verbose:
-            print("[build] " + " ".join(link))
-        _run(link)
+        objs = [os.path.join(tmp, os.path.basename(src) + ".o") for src in KERNEL_SOURCES]
+        for out, these in ((LIB_PATH, objs), (TIMELINE_LIB_PATH, [tl_objs.get(src, o) for src, o in zip(KERNEL_SOURCES, objs)])):
+            link = [HIPCC, "--offload-arch=gfx950", "-fPIC", "-shared"] + these + ["-o", out]
+            if verbose:
+                print("[build] " + " ".join(link))
+            _run(link)
     return LIB_PATH
 
 

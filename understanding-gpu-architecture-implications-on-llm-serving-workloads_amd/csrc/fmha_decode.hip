@@ -26,8 +26,13 @@
 
 #include "mi355_common.h"
 #include "mi355_serving_internal.h"
+#include "mi355_timeline.h"
 
 namespace mi355 {
+
+// profiling build: per workgroup, wall clock at [entry, first tile landed, key range done, partial results stored, ticket
+// drawn, merge: partial results landed, merge: summed, exit] (0 = the workgroup did not get there)
+MI355_TL(static __device__ unsigned long long fmha_decode_stamps[timeline::kMaxWorkgroups * timeline::kSlots];)
 
 namespace dec {
 constexpr int D = 128;
@@ -71,6 +76,11 @@ __global__ __launch_bounds__(WAVES * 64) void fmha_decode_kernel(
     int splits, int tiles_per_split, FmhaStrides sd) {
     using namespace dec;
     using V8 = typename Elem<T>::v8;
+    MI355_TL(unsigned long long tl[8] = {timeline::wall_clock(), 0, 0, 0, 0, 0, 0, 0};
+             auto tl_dump = [&]() {
+                 if (threadIdx.x == 0 && blockIdx.x < timeline::kMaxWorkgroups)
+                     for (int i = 0; i < 8; ++i) fmha_decode_stamps[(long)blockIdx.x * timeline::kSlots + i] = tl[i];
+             };)
     constexpr int WAVE_BYTES = NSTAGE * STAGE_BYTES;
     constexpr int NTHREADS = WAVES * 64;
     extern __shared__ __attribute__((aligned(1024))) char smem_raw[];
@@ -176,6 +186,7 @@ __global__ __launch_bounds__(WAVES * 64) void fmha_decode_kernel(
         } else {
             wait_vmcnt<0>();
         }
+        MI355_TL(if (tt0 == t_begin) tl[1] = timeline::wall_clock();)
         MI355_LDS char* st = wbase + slot * STAGE_BYTES;
         slot = (slot + 1 == NSTAGE) ? 0 : slot + 1;
 
@@ -244,6 +255,7 @@ __global__ __launch_bounds__(WAVES * 64) void fmha_decode_kernel(
     // ---- combine the waves of the workgroup through LDS (the pipelines are drained: their memory is free) ------------
     // per wave: O~ [ncols][128] floats, then m [32], l [32]
     const float l_tot = l_run + other_half(l_run);
+    MI355_TL(tl[2] = timeline::wall_clock();)
     __syncthreads();
     MI355_LDS float* cmb = (MI355_LDS float*)smem_raw;
     const int wave_floats = ncols * D + 64;
@@ -294,6 +306,7 @@ __global__ __launch_bounds__(WAVES * 64) void fmha_decode_kernel(
             if (LSE != nullptr && d == 0)
                 LSE[row0 + c] = (l > 0.f) ? (m * scale_log2 + __builtin_log2f(l)) * 0.69314718055994531f : -INFINITY;
         }
+        MI355_TL(wait_vmcnt<0>(); tl[7] = timeline::wall_clock(); tl_dump();)
         return;
     }
     // Partial results cross XCDs (each has its own L2), so they are written and read with device-scope relaxed atomic
@@ -311,11 +324,16 @@ __global__ __launch_bounds__(WAVES * 64) void fmha_decode_kernel(
     }
     // ---- ticket: the workgroup that completes the set of key ranges of (b, hkv) merges them ----------------------------
     wait_vmcnt<0>();   // this thread's partial results have reached memory before the ticket is drawn
+    MI355_TL(tl[3] = timeline::wall_clock();)
     __syncthreads();
     MI355_LDS unsigned* ticket_sh = (MI355_LDS unsigned*)(cmb + WAVES * wave_floats);
     if (tid == 0) *ticket_sh = __hip_atomic_fetch_add(&counters[(long)bh * kCounterStride], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     __syncthreads();
-    if (*ticket_sh != (unsigned)(splits - 1)) return;
+    MI355_TL(tl[4] = timeline::wall_clock();)
+    if (*ticket_sh != (unsigned)(splits - 1)) {
+        MI355_TL(tl[7] = tl[4]; tl_dump();)
+        return;
+    }
     // last ticket: every other workgroup of (b, hkv) drew its ticket after its partial results had reached memory.
     // They are read back with device-coherent loads (sc1), many in flight per thread: one memory round trip for the
     // statistics, then one per 16 key ranges for the outputs.
@@ -360,6 +378,7 @@ __global__ __launch_bounds__(WAVES * 64) void fmha_decode_kernel(
         st_m[i] = ms;
         st_l[i] = ls;
     }
+    MI355_TL(tl[5] = timeline::wall_clock();)
     __syncthreads();
     // The weight of key range s for column c, 2^((m_s - m_c) scale), is worked out once, by thread s * ncols + c, and left in
     // LDS together with its share of the row sum; the accumulation loop below then is two LDS reads and four
@@ -419,6 +438,7 @@ __global__ __launch_bounds__(WAVES * 64) void fmha_decode_kernel(
                 }
             }
         }
+        MI355_TL(tl[6] = timeline::wall_clock();)
         const float inv = (l > 0.f) ? 1.f / l : 0.f;
         const int chq = hkv * group + c / Sq, cqi = c % Sq;
         typename Elem<T>::v4 ov;
@@ -429,6 +449,7 @@ __global__ __launch_bounds__(WAVES * 64) void fmha_decode_kernel(
             LSE[row0 + c] = (l > 0.f) ? (st_mc[c] * scale_log2 + __builtin_log2f(l)) * 0.69314718055994531f : -INFINITY;
     }
     if (tid == 0) counters[(long)bh * kCounterStride] = 0u;   // ready for the next call that uses this workspace
+    MI355_TL(wait_vmcnt<0>(); tl[7] = timeline::wall_clock(); tl_dump();)
 }
 
 // Sets the counters of a workspace whose contents are unknown (a caller's) to zero.
@@ -598,3 +619,11 @@ template hipError_t fmha_decode_dispatch<bf16_t>(const bf16_t*, const bf16_t*, c
                                                  int, float, int, int, const FmhaStrides&, const FmhaWorkspace&, hipStream_t);
 
 }  // namespace mi355
+
+#ifdef MI355_TIMELINE
+// profiling build: copies the records of the last generation-step attention launch to the host
+extern "C" int mi355_timeline_read_fmha_decode(void* dst, size_t bytes) {
+    const size_t all = sizeof(unsigned long long) * mi355::timeline::kMaxWorkgroups * mi355::timeline::kSlots;
+    return (int)hipMemcpyFromSymbol(dst, HIP_SYMBOL(mi355::fmha_decode_stamps), bytes < all ? bytes : all);
+}
+#endif

@@ -20,8 +20,12 @@
 #include <type_traits>
 #include "mi355_common.h"
 #include "mi355_serving_internal.h"
+#include "mi355_timeline.h"
 
 namespace mi355 {
+
+// profiling build: per workgroup [wall: entry, loop start, loop end, exit; cycles: loop start, loop end; key tiles; 0]
+MI355_TL(static __device__ unsigned long long fmha_fwd_stamps[timeline::kMaxWorkgroups * timeline::kSlots];)
 
 namespace fmha {
 
@@ -115,6 +119,7 @@ __global__ __launch_bounds__(512, (QB == 1 ? 4 : 2)) void fmha_fwd_pingpong_kern
     constexpr int BM = NWAVES * WQ;
     constexpr int COPIES = (BN * ROW_BYTES / 1024) / NWAVES;  // 2 wave-instructions per tile per wave
 
+    MI355_TL(unsigned long long tl_w[4] = {timeline::wall_clock(), 0, 0, 0}; unsigned long long tl_c[2] = {0, 0};)
     extern __shared__ __attribute__((aligned(1024))) char smem_raw[];
     MI355_LDS char* smem = (MI355_LDS char*)smem_raw;
     MI355_LDS char* kbuf = smem;                   // 2 x TILE_BYTES
@@ -404,6 +409,7 @@ __global__ __launch_bounds__(512, (QB == 1 ? 4 : 2)) void fmha_fwd_pingpong_kern
 
         float4v s[4][QB];
         V8 pf[2][QB];
+        MI355_TL(tl_w[1] = timeline::wall_clock(); tl_c[0] = timeline::shader_cycles();)
         __builtin_amdgcn_s_setprio(1);
         mfma_phase(I0{}, I16{}, 0, s, 0, pf);               // S(0) alone
         __builtin_amdgcn_s_setprio(0);
@@ -427,6 +433,7 @@ __global__ __launch_bounds__(512, (QB == 1 ? 4 : 2)) void fmha_fwd_pingpong_kern
         next_phase();
         if (!late) next_phase();  // waves 0..3 idle while waves 4..7 finish
     }
+    MI355_TL(tl_w[2] = timeline::wall_clock(); tl_c[1] = timeline::shader_cycles();)
 
     // ---- finalize: O / l, LSE: lane holds O[query 16 qb + c][d = 16 db + 4 g + 0..3] -----------------------------
 #pragma unroll
@@ -449,6 +456,14 @@ __global__ __launch_bounds__(512, (QB == 1 ? 4 : 2)) void fmha_fwd_pingpong_kern
             }
         }
     }
+    MI355_TL(
+        wait_vmcnt<0>();   // the stores of this wave have been accepted
+        tl_w[3] = timeline::wall_clock();
+        if (tid == 0 && blockIdx.x < timeline::kMaxWorkgroups) {
+            unsigned long long* rec = fmha_fwd_stamps + (long)blockIdx.x * timeline::kSlots;
+            rec[0] = tl_w[0]; rec[1] = tl_w[1]; rec[2] = tl_w[2]; rec[3] = tl_w[3];
+            rec[4] = tl_c[0]; rec[5] = tl_c[1]; rec[6] = (unsigned long long)max(n_tiles, 0); rec[7] = 0;
+        })
 }
 
 template <typename T, int QB>
@@ -503,3 +518,11 @@ hipError_t fmha_fwd_dispatch(const void* Q, const void* K, const void* V, void* 
 }
 
 }  // namespace mi355
+
+#ifdef MI355_TIMELINE
+// profiling build: copies the records of the last attention forward launch (kMaxWorkgroups x kSlots 64-bit values) to the host
+extern "C" int mi355_timeline_read_fmha_fwd(void* dst, size_t bytes) {
+    const size_t all = sizeof(unsigned long long) * mi355::timeline::kMaxWorkgroups * mi355::timeline::kSlots;
+    return (int)hipMemcpyFromSymbol(dst, HIP_SYMBOL(mi355::fmha_fwd_stamps), bytes < all ? bytes : all);
+}
+#endif

@@ -24,8 +24,13 @@
 #include <type_traits>
 #include "mi355_common.h"
 #include "mi355_serving_internal.h"
+#include "mi355_timeline.h"
 
 namespace mi355 {
+
+// profiling build: per workgroup of hgemm_main_kernel [wall: entry, loop start, loop end, exit; cycles: loop start, loop
+// end; K tiles; 0]
+MI355_TL(static __device__ unsigned long long hgemm_stamps[timeline::kMaxWorkgroups * timeline::kSlots];)
 
 // ---------------------------------------------------------------------------------------------------------
 // LDS tile descriptions
@@ -195,6 +200,7 @@ void hgemm_main_kernel(const T* __restrict__ A, const T* __restrict__ B,
     using BTN = typename Cfg::BTileN;
     constexpr int TM = Cfg::TM, TN = Cfg::TN, BK = Cfg::BK;
 
+    MI355_TL(unsigned long long tl_w[4] = {timeline::wall_clock(), 0, 0, 0}; unsigned long long tl_c[2] = {0, 0};)
     extern __shared__ __attribute__((aligned(1024))) char smem_raw[];
     MI355_LDS char* smem = (MI355_LDS char*)smem_raw;
 
@@ -430,6 +436,7 @@ void hgemm_main_kernel(const T* __restrict__ A, const T* __restrict__ B,
         stage = next;
     };
     int kt = 0;
+    MI355_TL(tl_w[1] = timeline::wall_clock(); tl_c[0] = timeline::shader_cycles();)
     for (; kt + NSTAGE < ktiles; ++kt) tile(std::true_type{});
     for (; kt + 1 < ktiles; ++kt) tile(std::false_type{});
     {  // last tile: nothing left to fetch
@@ -437,6 +444,7 @@ void hgemm_main_kernel(const T* __restrict__ A, const T* __restrict__ B,
         substep(af[0], bf[0], reads_of(st, 1, af[1], bf[1]));
         substep(af[1], bf[1], [](auto) {});
     }
+    MI355_TL(tl_w[2] = timeline::wall_clock(); tl_c[1] = timeline::shader_cycles();)
 
     // ---- epilogue ------------------------------------------------------------------------------------------------
     // A lane holds C[m][n .. n+3] for m = l%16, n = 4*(l/16) of every 16x16 block. Storing that directly would write
@@ -502,6 +510,14 @@ void hgemm_main_kernel(const T* __restrict__ A, const T* __restrict__ B,
             }
         }
     }
+    MI355_TL(
+        wait_vmcnt<0>();   // the stores of this wave have been accepted
+        tl_w[3] = timeline::wall_clock();
+        if (tid == 0 && blockIdx.x < timeline::kMaxWorkgroups) {
+            unsigned long long* rec = hgemm_stamps + (long)blockIdx.x * timeline::kSlots;
+            rec[0] = tl_w[0]; rec[1] = tl_w[1]; rec[2] = tl_w[2]; rec[3] = tl_w[3];
+            rec[4] = tl_c[0]; rec[5] = tl_c[1]; rec[6] = (unsigned long long)ktiles; rec[7] = 0;
+        })
 }
 
 // ---------------------------------------------------------------------------------------------------------
@@ -1019,3 +1035,11 @@ hipError_t hgemm_dispatch(const void* A, const void* B, void* C, const void* R, 
 }
 
 }  // namespace mi355
+
+#ifdef MI355_TIMELINE
+// profiling build: copies the records of the last tiled GEMM launch (kMaxWorkgroups x kSlots 64-bit values) to the host
+extern "C" int mi355_timeline_read_hgemm(void* dst, size_t bytes) {
+    const size_t all = sizeof(unsigned long long) * mi355::timeline::kMaxWorkgroups * mi355::timeline::kSlots;
+    return (int)hipMemcpyFromSymbol(dst, HIP_SYMBOL(mi355::hgemm_stamps), bytes < all ? bytes : all);
+}
+#endif
