@@ -175,6 +175,13 @@ __global__ __launch_bounds__(WAVES * 64) void fmha_decode_kernel(
     V8 qf[8];
 #pragma unroll
     for (int ks = 0; ks < 8; ++ks) qf[ks] = *(const V8*)(qp + ks * 16);
+    // A use of the query fragments in front of the loop: the compiler waits for their loads where they are first used,
+    // and it does not count the tile copies (inline assembly) among the loads in flight. With the first use inside the
+    // loop that wait, "everything I know of has landed", came back on every iteration as vmcnt(0) in front of the S^T
+    // products and held each tile's arithmetic until the NEXT tile's copies had landed too: no copy ever overlapped
+    // arithmetic. Out here it waits once, for the first tile and the queries, which the first iteration needs anyway.
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks) asm volatile("" : "+v"(qf[ks]));
     int slot = 0, fill = NSTAGE - 1;
     for (int tt0 = t_begin; tt0 < t_end; ++tt0) {
         const int t = tile_of(tt0 - t_begin);
