@@ -579,13 +579,15 @@ __global__ __launch_bounds__(256) void hgemm_edge_kernel(const T* __restrict__ A
 //   * layout TN (A stored [K,M], A_KC = false): the A slab of a k-step is 32 rows (k) x 16 m, copied as it lies and read
 //     with the transposing read like B; M must be a multiple of 8.
 // ---------------------------------------------------------------------------------------------------------
+constexpr int kSmallMWaves = 8;
 constexpr int kSmallMStages = 3;
 constexpr int kSmallMStageBytes = 5 * 1024;  // 4 KiB of B + 1 KiB of A
 constexpr int kSmallMWaveBytes = kSmallMStages * kSmallMStageBytes;
-constexpr int kSmallMLdsBytes = 8 * kSmallMWaveBytes;
+constexpr int kSmallMLdsBytes = kSmallMWaves * kSmallMWaveBytes;
+static_assert(kSmallMLdsBytes >= kSmallMWaves * 1024 * 4, "the reduction reuses the pipeline memory");
 
 template <typename T, bool A_KC>
-__global__ __launch_bounds__(512) void hgemm_smallm_nn_kernel(const T* __restrict__ A, const T* __restrict__ B,
+__global__ __launch_bounds__(kSmallMWaves * 64) void hgemm_smallm_nn_kernel(const T* __restrict__ A, const T* __restrict__ B,
                                                               T* C, const T* R, int M, int N, int K, long lda,
                                                               long ldb, long ldc, long ldr, int n_tiles) {
     using V8 = typename Elem<T>::v8;
@@ -604,8 +606,8 @@ __global__ __launch_bounds__(512) void hgemm_smallm_nn_kernel(const T* __restric
     const int m0 = blockIdx.y * 16;
 
     const int ksteps = K / 32;
-    const int s_begin = (int)((long)wave * ksteps / 8);
-    const int s_end = (int)((long)(wave + 1) * ksteps / 8);
+    const int s_begin = (int)((long)wave * ksteps / kSmallMWaves);
+    const int s_end = (int)((long)(wave + 1) * ksteps / kSmallMWaves);
 
     MI355_LDS char* wbase = smem + wave * kSmallMWaveBytes;
 
@@ -701,25 +703,26 @@ __global__ __launch_bounds__(512) void hgemm_smallm_nn_kernel(const T* __restric
 #pragma unroll
         for (int q = 0; q < 4; ++q) red[wave * 1024 + (4 * (lane >> 4) + q) * 64 + 16 * j + (lane & 15)] = acc[j][q];
     __syncthreads();
-    const int o = tid * 2;  // two neighbouring columns of one row
-    float s0 = 0.f, s1 = 0.f;
+    for (int o = tid * 2; o < 1024; o += kSmallMWaves * 128) {  // two neighbouring columns of one row
+        float s0 = 0.f, s1 = 0.f;
 #pragma unroll
-    for (int w = 0; w < 8; ++w) {
-        s0 += red[w * 1024 + o];
-        s1 += red[w * 1024 + o + 1];
-    }
-    const int m = m0 + (o >> 6);
-    const int n = n0 + (o & 63);
-    if (m < M && n < N) {
-        V2 v;
-        v[0] = (T)s0;
-        v[1] = (T)s1;
-        if (R != nullptr) {
-            const V2 r = *(const V2*)(R + (long)m * ldr + n);
-            v[0] = (T)((float)v[0] + (float)r[0]);
-            v[1] = (T)((float)v[1] + (float)r[1]);
+        for (int w = 0; w < kSmallMWaves; ++w) {
+            s0 += red[w * 1024 + o];
+            s1 += red[w * 1024 + o + 1];
         }
-        *(V2*)(C + (long)m * ldc + n) = v;
+        const int m = m0 + (o >> 6);
+        const int n = n0 + (o & 63);
+        if (m < M && n < N) {
+            V2 v;
+            v[0] = (T)s0;
+            v[1] = (T)s1;
+            if (R != nullptr) {
+                const V2 r = *(const V2*)(R + (long)m * ldr + n);
+                v[0] = (T)((float)v[0] + (float)r[0]);
+                v[1] = (T)((float)v[1] + (float)r[1]);
+            }
+            *(V2*)(C + (long)m * ldc + n) = v;
+        }
     }
 }
 
@@ -730,24 +733,30 @@ static hipError_t launch_smallm_nn(const T* A, const T* B, T* C, const T* R, int
     if (hipError_t e = lds_once.ensure(reinterpret_cast<const void*>(hgemm_smallm_nn_kernel<T, A_KC>), kSmallMLdsBytes); e != hipSuccess) return e;
     const int n_tiles = (N + 63) / 64;
     dim3 grid(n_tiles, (M + 15) / 16);
-    hgemm_smallm_nn_kernel<T, A_KC><<<grid, dim3(512), kSmallMLdsBytes, stream>>>(A, B, C, R, M, N, K, lda, ldb, ldc, ldr, n_tiles);
+    hgemm_smallm_nn_kernel<T, A_KC><<<grid, dim3(kSmallMWaves * 64), kSmallMLdsBytes, stream>>>(A, B, C, R, M, N, K, lda, ldb, ldc, ldr, n_tiles);
     return hipGetLastError();
 }
 
 // ---------------------------------------------------------------------------------------------------------
 // Small-M kernel for layout NT (B stored [N,K]: the nn.Linear weight layout of decode-time projections), M <= 16
 // rows per workgroup row. HBM-bound like hgemm_smallm_nn_kernel and built the same way: a workgroup owns 16
-// columns of C (16 rows of B), its 8 waves split K and are reduced through LDS; every wave runs a private,
+// columns of C (16 rows of B), its waves split K and are reduced through LDS; every wave runs a private,
 // barrier-free copy pipeline of 64-deep k-steps (16x64 of B and 16x64 of A, 2 KiB each, direct-to-LDS), both
 // operands are K-contiguous so both fragments are plain ds_read_b128, the product is MFMA 16x16x32.
+// Four waves with four stages each = 64 KiB of LDS, so that two or three workgroups share a CU and one's start-up
+// and reduction hide under the others' streaming: with weights that come from HBM (not from the memory-side cache, as
+// when one weight matrix is launched on again and again) that beats eight waves on 128 KiB, one workgroup per CU, by
+// 7-15 % (8 x 4096 x 14336: 21.7 us against 23.3, 8 x 6144 x 4096: 11.9 against 13.4).
 // ---------------------------------------------------------------------------------------------------------
+constexpr int kSmallMNtWaves = 4;
 constexpr int kSmallMNtStages = 4;
 constexpr int kSmallMNtStageBytes = 4 * 1024;  // 2 KiB of B + 2 KiB of A
 constexpr int kSmallMNtWaveBytes = kSmallMNtStages * kSmallMNtStageBytes;
-constexpr int kSmallMNtLdsBytes = 8 * kSmallMNtWaveBytes;
+constexpr int kSmallMNtLdsBytes = kSmallMNtWaves * kSmallMNtWaveBytes;
+static_assert(kSmallMNtLdsBytes >= kSmallMNtWaves * 256 * 4, "the reduction reuses the pipeline memory");
 
-template <typename T>
-__global__ __launch_bounds__(512) void hgemm_smallm_nt_kernel(const T* __restrict__ A, const T* __restrict__ B,
+template <typename T, bool HALF_A>
+__global__ __launch_bounds__(kSmallMNtWaves * 64) void hgemm_smallm_nt_kernel(const T* __restrict__ A, const T* __restrict__ B,
                                                               T* C, const T* R, int M, int N, int K, long lda,
                                                               long ldb, long ldc, long ldr, int n_tiles) {
     using V8 = typename Elem<T>::v8;
@@ -765,8 +774,8 @@ __global__ __launch_bounds__(512) void hgemm_smallm_nt_kernel(const T* __restric
     const int m0 = blockIdx.y * 16;
 
     const int ksteps = K / 64;
-    const int s_begin = (int)((long)wave * ksteps / 8);
-    const int s_end = (int)((long)(wave + 1) * ksteps / 8);
+    const int s_begin = (int)((long)wave * ksteps / kSmallMNtWaves);
+    const int s_end = (int)((long)(wave + 1) * ksteps / kSmallMNtWaves);
     MI355_LDS char* wbase = smem + wave * kSmallMNtWaveBytes;
 
     // slab = 16 rows x 128 bytes; a copy instruction covers 8 rows (row lane/8, chunk position lane%8);
@@ -778,12 +787,15 @@ __global__ __launch_bounds__(512) void hgemm_smallm_nt_kernel(const T* __restric
     const T* a_src0 = A + (long)min(m0 + c_row, M - 1) * lda + (long)s_begin * 64 + c_chunk * 8;
     const T* a_src1 = A + (long)min(m0 + c_row + 8, M - 1) * lda + (long)s_begin * 64 + c_chunk * 8;
 
+    // HALF_A (M <= 8): rows 8..15 of the A slab are not copied; the fragment rows read from there hold whatever the
+    // memory held, and so do rows 8..15 of the product, which are never stored (an output row depends on its own A row only)
+    constexpr int kCopies = HALF_A ? 3 : 4;
     auto issue_stage = [&](int slot) {
         MI355_LDS char* st = wbase + slot * kSmallMNtStageBytes;
         copy16_global_to_lds(b_src0, st);
         copy16_global_to_lds(b_src1, st + 1024);
         copy16_global_to_lds(a_src0, st + 2048);
-        copy16_global_to_lds(a_src1, st + 3072);
+        if constexpr (!HALF_A) copy16_global_to_lds(a_src1, st + 3072);
         b_src0 += 64;
         b_src1 += 64;
         a_src0 += 64;
@@ -811,7 +823,7 @@ __global__ __launch_bounds__(512) void hgemm_smallm_nt_kernel(const T* __restric
             issue_stage(fill);
             ++issued;
             fill = (fill + 1 == kSmallMNtStages) ? 0 : fill + 1;
-            wait_vmcnt<4 * (kSmallMNtStages - 1)>();  // everything but the newest kSmallMNtStages-1 steps has landed
+            wait_vmcnt<kCopies * (kSmallMNtStages - 1)>();  // everything but the newest kSmallMNtStages-1 steps has landed
         } else {
             wait_vmcnt<0>();
         }
@@ -832,12 +844,12 @@ __global__ __launch_bounds__(512) void hgemm_smallm_nt_kernel(const T* __restric
 #pragma unroll
     for (int q = 0; q < 4; ++q) red[wave * 256 + (4 * (lane >> 4) + q) * 16 + (lane & 15)] = acc[q];
     __syncthreads();
-    if (tid < 256) {
+    for (int o = tid; o < 256; o += kSmallMNtWaves * 64) {
         float sum = 0.f;
 #pragma unroll
-        for (int w = 0; w < 8; ++w) sum += red[w * 256 + tid];
-        const int m = m0 + (tid >> 4);
-        const int n = n0 + (tid & 15);
+        for (int w = 0; w < kSmallMNtWaves; ++w) sum += red[w * 256 + o];
+        const int m = m0 + (o >> 4);
+        const int n = n0 + (o & 15);
         if (m < M && n < N) {
             T v = (T)sum;
             if (R != nullptr) v = (T)((float)v + (float)R[(long)m * ldr + n]);
@@ -849,11 +861,16 @@ __global__ __launch_bounds__(512) void hgemm_smallm_nt_kernel(const T* __restric
 template <typename T>
 static hipError_t launch_smallm_nt(const T* A, const T* B, T* C, const T* R, int M, int N, int K, long lda, long ldb,
                                    long ldc, long ldr, hipStream_t stream) {
-    static DynamicLdsOnce lds_once;
-    if (hipError_t e = lds_once.ensure(reinterpret_cast<const void*>(hgemm_smallm_nt_kernel<T>), kSmallMNtLdsBytes); e != hipSuccess) return e;
+    static DynamicLdsOnce lds_once, lds_once_half;
     const int n_tiles = (N + 15) / 16;
     dim3 grid(n_tiles, (M + 15) / 16);
-    hgemm_smallm_nt_kernel<T><<<grid, dim3(512), kSmallMNtLdsBytes, stream>>>(A, B, C, R, M, N, K, lda, ldb, ldc, ldr, n_tiles);
+    if (M <= 8) {
+        if (hipError_t e = lds_once_half.ensure(reinterpret_cast<const void*>(hgemm_smallm_nt_kernel<T, true>), kSmallMNtLdsBytes); e != hipSuccess) return e;
+        hgemm_smallm_nt_kernel<T, true><<<grid, dim3(kSmallMNtWaves * 64), kSmallMNtLdsBytes, stream>>>(A, B, C, R, M, N, K, lda, ldb, ldc, ldr, n_tiles);
+    } else {
+        if (hipError_t e = lds_once.ensure(reinterpret_cast<const void*>(hgemm_smallm_nt_kernel<T, false>), kSmallMNtLdsBytes); e != hipSuccess) return e;
+        hgemm_smallm_nt_kernel<T, false><<<grid, dim3(kSmallMNtWaves * 64), kSmallMNtLdsBytes, stream>>>(A, B, C, R, M, N, K, lda, ldb, ldc, ldr, n_tiles);
+    }
     return hipGetLastError();
 }
 
@@ -895,7 +912,11 @@ static bool few_rows_prefer_tiles(int M, int N, int K, bool nt) {
 // segments. True when that is expected to beat both alternatives above (measured at Llama projection shapes:
 // 16 x 14336 x 4096 NT 19 us against 22, 64 rows NN 22 against 31, 64 x 4096 x 4096 NT 15 against 17; but
 // 16 x 4096 x 14336 NT 41 against 19 on the split-K small-M kernel, and 16 x 14336 x 4096 NN 21 against 20).
+// Layout NT with up to 16 rows always takes the split-K small-M kernel: with weights that are in no cache (a different
+// weight matrix on every launch, as in a decoder stack) it is the faster one at every Llama projection shape
+// (8 x 28672 x 4096: 39 us against 46, 8 x 14336 x 4096: 23 against 26, 16 x 14336 x 4096: 24.6 against 25.8).
 static bool few_rows_prefer_deep_ring(int M, int N, int K, bool nn, bool nt) {
+    if (nt && M <= 16) return false;
     const double bytes = (double)N * (double)K * 2.0;
     const double rate = fmin(6.3e6, (double)((N + 63) / 64) * 38e3);   // bytes per microsecond
     const double deep_us = (bytes / rate + 1.0) * (nn ? 1.1 : 1.0);
