@@ -71,9 +71,10 @@ int mi355_hgemm(const void* A, const void* B, void* C, int M, int N, int K, int6
  * gate and up projections of a Llama MLP computed by one GEMM on an interleaved weight matrix, with the activation
  * applied to the accumulators before the single rounding to fp16. Replaces `self.act_fn(self.gate_proj(x)) * self.up_proj(x)`
  * (benchmarks/flashattn-cuda/modeling_llama.py:227): two GEMMs, a SiLU kernel and a multiply kernel in the reference.
- * Layouts NN and NT. Only shapes the tiled kernels cover have the fused form (M > 64, or M > 16 when the product is wide enough for
- * the tiled kernels to beat the small-M kernels; N a multiple of 32, K a multiple of 64,
- * 16-byte aligned operands and leading dimensions); others return MI355_ERR_UNSUPPORTED and nothing is launched: run
+ * Layouts NN and NT. The fused form exists for M <= 16 in layout NT (the generation step: the split-K small-M kernel with
+ * the same epilogue) and for the shapes the tiled kernels cover (M > 64, or M > 16 when the product is wide enough for
+ * the tiled kernels to beat the small-M kernels); N a multiple of 32, K a multiple of 64, 16-byte aligned operands and
+ * leading dimensions. Other shapes return MI355_ERR_UNSUPPORTED and nothing is launched: run
  * mi355_hgemm on the same operands followed by mi355_silu_mul with interleave = 32.
  */
 int mi355_hgemm_silu_mul(const void* A, const void* B, void* C, int M, int N, int K, int64_t lda, int64_t ldb, int64_t ldc,

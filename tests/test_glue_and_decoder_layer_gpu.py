@@ -100,9 +100,12 @@ def test_silu_mul(lib, gpu, rows, inter):
 @pytest.mark.parametrize("M,F,K,layout", [(256, 256, 128, "NT"), (2048, 4096, 512, "NT"), (1024, 14336, 256, "NT"),
                                           (384, 192, 64, "NT"), (512, 1024, 256, "NN"), (8, 512, 256, "NT"), (100, 96, 72, "NT"),
                                           (300, 160, 128, "NT"), (1000, 14336, 128, "NT"), (4100, 4096, 64, "NN"),
-                                          (32, 14336, 256, "NT"), (64, 14336, 128, "NN"), (24, 7168, 512, "NT")])
+                                          (32, 14336, 256, "NT"), (64, 14336, 128, "NN"), (24, 7168, 512, "NT"),
+                                          (1, 32, 64, "NT"), (8, 14336, 512, "NT"), (16, 2048, 1024, "NT"), (13, 96, 128, "NT"),
+                                          (9, 4096, 4096, "NT"), (16, 512, 256, "NN")])
 def test_gemm_with_gate_up_epilogue(lib, gpu, M, F, K, layout):
-    # silu(x Wg^T) * (x Wu^T) from one launch on the interleaved weight (tiled shapes) or from the two-step fallback;
+    # silu(x Wg^T) * (x Wu^T) from one launch on the interleaved weight (tiled shapes; up to 16 rows in layout NT on the
+    # split-K kernel, with and without the second half of the A slab) or from the two-step fallback;
     # compared with the fp32 oracle. One rounding of an fp32 value: |err| <= 2^-10 |ref| + the GEMM's accumulation slack.
     x = so.randn_fp16((M, K), 1)
     wg, wu = so.randn_fp16((F, K), 2, 0.05), so.randn_fp16((F, K), 3, 0.05)

@@ -129,7 +129,7 @@ static int hgemm_silu_mul_impl(const char* fn, int dtype, const void* A, const v
     hipError_t e = mi355::hgemm_silu_mul_dispatch(A, B, C, M, 2 * N, K, lda, ldb, ldc, layout, dtype, static_cast<hipStream_t>(stream));
     if (e == hipErrorNotSupported)
         return fail(MI355_ERR_UNSUPPORTED,
-                    "%s: needs M > 64 (or M > 16 with enough columns to fill the machine), N a multiple of 32, K a multiple of 64 and 16-byte aligned operands; "
+                    "%s: needs M <= 16 with layout NT, or M > 64 (or M > 16 with enough columns to fill the machine), N a multiple of 32, K a multiple of 64 and 16-byte aligned operands; "
                     "run mi355_hgemm and mi355_silu_mul(interleave = 32) instead", fn);
     if (e != hipSuccess) return hip_fail(e, fn);
     return 0;

@@ -755,7 +755,10 @@ constexpr int kSmallMNtWaveBytes = kSmallMNtStages * kSmallMNtStageBytes;
 constexpr int kSmallMNtLdsBytes = kSmallMNtWaves * kSmallMNtWaveBytes;
 static_assert(kSmallMNtLdsBytes >= kSmallMNtWaves * 256 * 4, "the reduction reuses the pipeline memory");
 
-template <typename T, bool HALF_A>
+// GATE_UP: the rows of B come in groups of [32 gate | 32 up] (the operand of the tiled kernels' gate/up epilogue) and C is
+// silu(gate) * up, half as wide. Workgroup t then takes the 8 gate rows 64 (t / 4) + 8 (t % 4) .. +7 and the 8 up rows 32
+// further on, and stores the 8 columns 32 (t / 4) + 8 (t % 4) .. +7 of C.
+template <typename T, bool HALF_A, bool GATE_UP>
 __global__ __launch_bounds__(kSmallMNtWaves * 64) void hgemm_smallm_nt_kernel(const T* __restrict__ A, const T* __restrict__ B,
                                                               T* C, const T* R, int M, int N, int K, long lda,
                                                               long ldb, long ldc, long ldr, int n_tiles) {
@@ -782,8 +785,10 @@ __global__ __launch_bounds__(kSmallMNtWaves * 64) void hgemm_smallm_nt_kernel(co
     // chunk c of row r is stored at position c ^ (r & 7)
     const int c_row = lane >> 3;  // + 8*i
     const int c_chunk = (lane & 7) ^ (c_row & 7);
-    const T* b_src0 = B + (long)min(n0 + c_row, N - 1) * ldb + (long)s_begin * 64 + c_chunk * 8;
-    const T* b_src1 = B + (long)min(n0 + c_row + 8, N - 1) * ldb + (long)s_begin * 64 + c_chunk * 8;
+    const int b_row0 = GATE_UP ? 64 * (tile >> 2) + 8 * (tile & 3) + c_row : n0 + c_row;
+    const int b_row1 = GATE_UP ? b_row0 + 32 : b_row0 + 8;
+    const T* b_src0 = B + (long)min(b_row0, N - 1) * ldb + (long)s_begin * 64 + c_chunk * 8;
+    const T* b_src1 = B + (long)min(b_row1, N - 1) * ldb + (long)s_begin * 64 + c_chunk * 8;
     const T* a_src0 = A + (long)min(m0 + c_row, M - 1) * lda + (long)s_begin * 64 + c_chunk * 8;
     const T* a_src1 = A + (long)min(m0 + c_row + 8, M - 1) * lda + (long)s_begin * 64 + c_chunk * 8;
 
@@ -849,6 +854,16 @@ __global__ __launch_bounds__(kSmallMNtWaves * 64) void hgemm_smallm_nt_kernel(co
 #pragma unroll
         for (int w = 0; w < kSmallMNtWaves; ++w) sum += red[w * 256 + o];
         const int m = m0 + (o >> 4);
+        if constexpr (GATE_UP) {
+            if ((o & 15) < 8 && m < M) {   // column o % 16 is a gate, the one 8 further on its up
+                float up = 0.f;
+#pragma unroll
+                for (int w = 0; w < kSmallMNtWaves; ++w) up += red[w * 256 + o + 8];
+                const float sig = __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(-sum * 1.4426950408889634f));
+                C[(long)m * ldc + 32 * (tile >> 2) + 8 * (tile & 3) + (o & 15)] = (T)(sum * sig * up);
+            }
+            continue;
+        }
         const int n = n0 + (o & 15);
         if (m < M && n < N) {
             T v = (T)sum;
@@ -865,11 +880,29 @@ static hipError_t launch_smallm_nt(const T* A, const T* B, T* C, const T* R, int
     const int n_tiles = (N + 15) / 16;
     dim3 grid(n_tiles, (M + 15) / 16);
     if (M <= 8) {
-        if (hipError_t e = lds_once_half.ensure(reinterpret_cast<const void*>(hgemm_smallm_nt_kernel<T, true>), kSmallMNtLdsBytes); e != hipSuccess) return e;
-        hgemm_smallm_nt_kernel<T, true><<<grid, dim3(kSmallMNtWaves * 64), kSmallMNtLdsBytes, stream>>>(A, B, C, R, M, N, K, lda, ldb, ldc, ldr, n_tiles);
+        if (hipError_t e = lds_once_half.ensure(reinterpret_cast<const void*>(hgemm_smallm_nt_kernel<T, true, false>), kSmallMNtLdsBytes); e != hipSuccess) return e;
+        hgemm_smallm_nt_kernel<T, true, false><<<grid, dim3(kSmallMNtWaves * 64), kSmallMNtLdsBytes, stream>>>(A, B, C, R, M, N, K, lda, ldb, ldc, ldr, n_tiles);
     } else {
-        if (hipError_t e = lds_once.ensure(reinterpret_cast<const void*>(hgemm_smallm_nt_kernel<T, false>), kSmallMNtLdsBytes); e != hipSuccess) return e;
-        hgemm_smallm_nt_kernel<T, false><<<grid, dim3(kSmallMNtWaves * 64), kSmallMNtLdsBytes, stream>>>(A, B, C, R, M, N, K, lda, ldb, ldc, ldr, n_tiles);
+        if (hipError_t e = lds_once.ensure(reinterpret_cast<const void*>(hgemm_smallm_nt_kernel<T, false, false>), kSmallMNtLdsBytes); e != hipSuccess) return e;
+        hgemm_smallm_nt_kernel<T, false, false><<<grid, dim3(kSmallMNtWaves * 64), kSmallMNtLdsBytes, stream>>>(A, B, C, R, M, N, K, lda, ldb, ldc, ldr, n_tiles);
+    }
+    return hipGetLastError();
+}
+
+// silu(A gate^T) * (A up^T) for up to 16 rows: N counts the rows of B ([32 gate | 32 up] groups, a multiple of 64), C is
+// [M, N / 2].
+template <typename T>
+static hipError_t launch_smallm_nt_gate_up(const T* A, const T* B, T* C, int M, int N, int K, long lda, long ldb, long ldc,
+                                           hipStream_t stream) {
+    static DynamicLdsOnce lds_once, lds_once_half;
+    const int n_tiles = N / 16;
+    dim3 grid(n_tiles, 1);
+    if (M <= 8) {
+        if (hipError_t e = lds_once_half.ensure(reinterpret_cast<const void*>(hgemm_smallm_nt_kernel<T, true, true>), kSmallMNtLdsBytes); e != hipSuccess) return e;
+        hgemm_smallm_nt_kernel<T, true, true><<<grid, dim3(kSmallMNtWaves * 64), kSmallMNtLdsBytes, stream>>>(A, B, C, nullptr, M, N, K, lda, ldb, ldc, 0, n_tiles);
+    } else {
+        if (hipError_t e = lds_once.ensure(reinterpret_cast<const void*>(hgemm_smallm_nt_kernel<T, false, true>), kSmallMNtLdsBytes); e != hipSuccess) return e;
+        hgemm_smallm_nt_kernel<T, false, true><<<grid, dim3(kSmallMNtWaves * 64), kSmallMNtLdsBytes, stream>>>(A, B, C, nullptr, M, N, K, lda, ldb, ldc, 0, n_tiles);
     }
     return hipGetLastError();
 }
@@ -1003,6 +1036,9 @@ static hipError_t launch_silu_mul(const T* A, const T* B, T* C, int M, int N, in
                          (reinterpret_cast<uintptr_t>(C) % 16 == 0) && (lda % 8 == 0) && (ldb % 8 == 0) && (ldc % 8 == 0);
     // N = columns of op(B); gate/up pairs are 64 columns wide. Few rows are better served by the small-M product.
     if (!aligned || K % 64 != 0 || K < 64 || N % 64 != 0 || lda >= (1L << 22) || ldb >= (1L << 22)) return hipErrorNotSupported;
+    if constexpr (A_KC && B_KC) {   // generation step: the split-K small-M kernel with the same epilogue
+        if (M <= 16) return launch_smallm_nt_gate_up<T>(A, B, C, M, N, K, lda, ldb, ldc, stream);
+    }
     if (M <= 64 && !few_rows_prefer_tiles(M, N, K, false)) return hipErrorNotSupported;   // the small-M product + silu_mul is faster
     const bool fits128 = M % 128 == 0 && N % 128 == 0;
     const bool fits256 = M % 256 == 0 && N % 256 == 0;
