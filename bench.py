@@ -156,6 +156,10 @@ def main():
     ap.add_argument("--zero-inputs", action="store_true",
                     help="with --kernel-config: all-zero operands instead of the seeded random ones (the arithmetic and its "
                          "cycle count stay the same, the switching power does not: shows what the board's power limit costs)")
+    ap.add_argument("--rotate-operands", action="store_true",
+                    help="with --kernel-config: every launch reads a different copy of the big operand (the weight matrix of a "
+                         "GEMM, K and V of attention), enough copies to exceed the 256 MB memory-side cache three times: the "
+                         "rate with operands that come from HBM, as in a decoder stack, not from a cache warmed by the launch before")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also launch one 1 GiB device-to-device copy, so FETCH_SIZE / WRITE_SIZE read under rocprofv3 "
                          "--pmc can be scaled by what the same counter reports for a transfer of known size")
@@ -570,7 +574,8 @@ KERNEL_CONFIGS = {
     "g2b_gemm_8192_nt": ("gemm", 8192, 8192, 8192, "NT"),
     "gemm_2048x2048x4096_nn": ("gemm", 2048, 2048, 4096, "NN"),             # 128x128 tiles
     "g2c_gemm_16x14336x4096_nn": ("gemm", 16, 14336, 4096, "NN"),           # split-K small-M kernel
-    "gemm_16x14336x4096_nt": ("gemm", 16, 14336, 4096, "NT"),               # 64x64 tiles, 8-deep ring
+    "gemm_16x14336x4096_nt": ("gemm", 16, 14336, 4096, "NT"),               # split-K small-M kernel (NT)
+    "gemm_8x28672x4096_nt": ("gemm", 8, 28672, 4096, "NT"),                 # split-K small-M kernel (NT), A rows 0..7 only
     "gemm_64x14336x4096_nt": ("gemm", 64, 14336, 4096, "NT"),               # 64x64 tiles, 8-deep ring
     "gemm_16x4096x14336_nt": ("gemm", 16, 4096, 14336, "NT"),               # split-K small-M kernel (NT)
     "gemm_1024x4096x4096_nt": ("gemm", 1024, 4096, 4096, "NT"),             # 128x64 tiles
@@ -642,6 +647,10 @@ def run_kernel_config(args, torch, lib, so, dev):
         c = torch.empty((M, N), dtype=torch.float16, device=dev)
         fn = lambda: lib.hgemm_raw(a.data_ptr(), b.data_ptr(), c.data_ptr(), M, N, K, a.shape[1], b.shape[1], N, lib.LAYOUTS[lay], cur())
         flops, nbytes = 2.0 * M * N * K, 2.0 * (M * K + K * N + M * N)
+        if args.rotate_operands:
+            bs = [b] + [b.clone() for _ in range(copies_to_defeat_cache(2.0 * K * N) - 1)]
+            fn = rotating(lambda j: lib.hgemm_raw(a.data_ptr(), bs[j].data_ptr(), c.data_ptr(), M, N, K, a.shape[1], b.shape[1], N,
+                                                  lib.LAYOUTS[lay], cur()), len(bs))
     else:
         _, B, Hq, Hkv, Sq, Sk, causal = cfg
         q, k, v = (t.to(dev) for t in so.fmha_inputs(B, Hq, Hkv, Sq, Sk, seed=42))
@@ -653,6 +662,11 @@ def run_kernel_config(args, torch, lib, so, dev):
                                       128, 1.0 / math.sqrt(128), int(causal), Sk, cur())
         flops = 4.0 * B * Hq * 128 * (causal_pairs(Sq, Sk) if causal else Sq * Sk)
         nbytes = 2.0 * (2 * B * Hq * Sq * 128 + 2 * B * Hkv * Sk * 128) + 4.0 * B * Hq * Sq
+        if args.rotate_operands:
+            kvs = [(k, v)] + [(k.clone(), v.clone()) for _ in range(copies_to_defeat_cache(4.0 * B * Hkv * Sk * 128) - 1)]
+            fn = rotating(lambda j: lib.fmha_fwd_raw(q.data_ptr(), kvs[j][0].data_ptr(), kvs[j][1].data_ptr(), o.data_ptr(),
+                                                     lse.data_ptr(), B, Hq, Hkv, Sq, Sk, 128, 1.0 / math.sqrt(128), int(causal), Sk,
+                                                     cur()), len(kvs))
     if args.calibrate_copy:
         src = torch.empty(1 << 30, dtype=torch.uint8, device=dev).fill_(1)
         dst = torch.empty_like(src)
@@ -666,7 +680,8 @@ def run_kernel_config(args, torch, lib, so, dev):
         print(json.dumps(dict(t, kernel_config=args.kernel_config, zero_inputs=bool(args.zero_inputs), timeline=timeline_summary(lib, cfg))))
         return
     t["ms_graph_replay"] = time_graph(fn, args.steps, args.warmup)
-    print(json.dumps(dict(t, kernel_config=args.kernel_config, tflops=flops / t["ms"] / 1e9, gbs=nbytes / t["ms"] / 1e6,
+    print(json.dumps(dict(t, kernel_config=args.kernel_config, rotate_operands=bool(args.rotate_operands),
+                          tflops=flops / t["ms"] / 1e9, gbs=nbytes / t["ms"] / 1e6,
                           tflops_graph_replay=flops / t["ms_graph_replay"] / 1e9, gbs_graph_replay=nbytes / t["ms_graph_replay"] / 1e6,
                           algorithmic_flop=flops, algorithmic_bytes=nbytes)))
 

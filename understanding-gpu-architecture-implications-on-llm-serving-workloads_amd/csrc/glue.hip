@@ -5,6 +5,8 @@
 // calls of fine_fmha (benchmarks/flashattn-cuda/modeling_llama.py): LlamaRMSNorm.forward (:95-100), rotate_half /
 // apply_rotary_pos_emb (:164-195), LlamaMLP.forward's act_fn(gate) * up (:227) and the residual adds of
 // LlamaDecoderLayer.forward (:776-781). Each kernel moves every byte once with 16-byte accesses.
+#include <type_traits>
+
 #include "mi355_common.h"
 #include "mi355_serving_internal.h"
 
@@ -31,8 +33,12 @@ __device__ __forceinline__ float block_sum(float x, float* scratch) {
 // One workgroup per row. ADD: h = residual + x is rounded to fp16, written to `res_out` (which may be `residual`
 // itself), and normalised (the rounded value is what the next layer sees, so it is also what gets normalised).
 // Otherwise h = x.
-// out = weight * h * rsqrt(mean(h^2) + eps). The second pass re-reads the row (it is still in L2).
-template <typename T, bool ADD>
+// out = weight * h * rsqrt(mean(h^2) + eps).
+// REGS > 0: hidden <= REGS * 2048, the row and the weight stay in registers (REGS 16-byte pieces per thread each): every
+// load of the kernel is issued up front, so a row costs one memory round trip, the sum and the store. On the 8 rows of a
+// generation step the kernel is nothing but its chain of round trips (4.5 us with the weight fetched behind the sum and
+// the row read a second time). REGS == 0: any hidden; the second pass re-reads the row (it is still in L2).
+template <typename T, bool ADD, int REGS>
 __global__ __launch_bounds__(glue::THREADS) void rmsnorm_kernel(const T* x, const T* residual, T* res_out,
                                                                 const T* __restrict__ weight, T* out,
                                                                 int hidden, long ldx, long ldr, long ldro, long ldo,
@@ -45,6 +51,44 @@ __global__ __launch_bounds__(glue::THREADS) void rmsnorm_kernel(const T* x, cons
     T* ro = ADD ? res_out + row * ldro : nullptr;
     T* orow = out + row * ldo;
     float ss = 0.f;
+    if constexpr (REGS > 0) {
+        V8 v[REGS], r[REGS], w[REGS];
+#pragma unroll
+        for (int i = 0; i < REGS; ++i) {
+            const int c = (i * glue::THREADS + threadIdx.x) * 8;
+            if (c < hidden) {
+                v[i] = *(const V8*)(xr + c);
+                if (ADD) r[i] = *(const V8*)(rr + c);
+                w[i] = *(const V8*)(weight + c);
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < REGS; ++i) {
+            const int c = (i * glue::THREADS + threadIdx.x) * 8;
+            if (c < hidden) {
+                if (ADD) {
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) v[i][j] = (T)((float)v[i][j] + (float)r[i][j]);
+                    *(V8*)(ro + c) = v[i];
+                }
+#pragma unroll
+                for (int j = 0; j < 8; ++j) ss += (float)v[i][j] * (float)v[i][j];
+            }
+        }
+        const float total = glue::block_sum(ss, scratch);
+        const float inv = __builtin_amdgcn_rsqf(total / (float)hidden + eps);
+#pragma unroll
+        for (int i = 0; i < REGS; ++i) {
+            const int c = (i * glue::THREADS + threadIdx.x) * 8;
+            if (c < hidden) {
+                V8 o;
+#pragma unroll
+                for (int j = 0; j < 8; ++j) o[j] = (T)((float)w[i][j] * ((float)v[i][j] * inv));
+                *(V8*)(orow + c) = o;
+            }
+        }
+        return;
+    }
     for (int c = threadIdx.x * 8; c < hidden; c += glue::THREADS * 8) {
         V8 v = *(const V8*)(xr + c);
         if (ADD) {
@@ -143,12 +187,18 @@ static hipError_t rmsnorm_t(const void* x, const void* residual, void* res_out, 
                             int hidden, long ldx, long ldr, long ldro, long ldo, float eps, hipStream_t stream) {
     if (rows > 0x7fffffffL) return hipErrorInvalidValue;
     const dim3 grid((unsigned)rows), block(glue::THREADS);
-    if (residual != nullptr)
-        rmsnorm_kernel<T, true><<<grid, block, 0, stream>>>((const T*)x, (const T*)residual, (T*)res_out, (const T*)weight,
-                                                            (T*)out, hidden, ldx, ldr, ldro, ldo, eps);
-    else
-        rmsnorm_kernel<T, false><<<grid, block, 0, stream>>>((const T*)x, nullptr, nullptr, (const T*)weight, (T*)out, hidden,
-                                                             ldx, 0, 0, ldo, eps);
+    auto launch = [&](auto regs) {
+        constexpr int REGS = decltype(regs)::value;
+        if (residual != nullptr)
+            rmsnorm_kernel<T, true, REGS><<<grid, block, 0, stream>>>((const T*)x, (const T*)residual, (T*)res_out, (const T*)weight,
+                                                                      (T*)out, hidden, ldx, ldr, ldro, ldo, eps);
+        else
+            rmsnorm_kernel<T, false, REGS><<<grid, block, 0, stream>>>((const T*)x, nullptr, nullptr, (const T*)weight, (T*)out,
+                                                                       hidden, ldx, 0, 0, ldo, eps);
+    };
+    if (hidden <= 2 * 2048) launch(std::integral_constant<int, 2>{});
+    else if (hidden <= 4 * 2048) launch(std::integral_constant<int, 4>{});
+    else launch(std::integral_constant<int, 0>{});
     return hipGetLastError();
 }
 
