@@ -586,6 +586,13 @@ KERNEL_CONFIGS = {
     "fmha_decode_b1_sk8192": ("fmha", 1, 32, 8, 1, 8192, False),                # split-KV kernel
     "fmha_decode_b8_sk8192": ("fmha", 8, 32, 8, 1, 8192, False),
     "fmha_decode_b64_sk8192": ("fmha", 64, 32, 8, 1, 8192, False),              # one key range per (batch, kv head)
+    # a kernel that only reads (profiling twin of the library, --timeline): the yardstick of the bandwidth-bound kernels, at
+    # the sizes of the big operands of a Llama-3-8B generation step at batch 8 (O, QKV, down, gate/up weights; K + V)
+    "stream_read_34mb": ("read", 4096 * 4096 * 2),
+    "stream_read_50mb": ("read", 6144 * 4096 * 2),
+    "stream_read_117mb": ("read", 14336 * 4096 * 2),
+    "stream_read_235mb": ("read", 28672 * 4096 * 2),
+    "stream_read_268mb": ("read", 2 * 8 * 8 * 8192 * 128 * 2),
 }
 
 
@@ -636,6 +643,26 @@ def timeline_summary(lib, cfg):
 def run_kernel_config(args, torch, lib, so, dev):
     cfg = KERNEL_CONFIGS[args.kernel_config]
     cur = lambda: torch.cuda.current_stream().cuda_stream   # at call time: graph capture runs on a stream of its own
+    if cfg[0] == "read":
+        import ctypes
+        if not args.timeline:
+            sys.exit("bench.py: the stream_read configurations live in the profiling twin of the library: add --timeline")
+        read = lib.load().mi355_timeline_stream_read
+        read.argtypes = [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p, ctypes.c_void_p]
+        read.restype = ctypes.c_int
+        nbytes = cfg[1]
+        n_copies = copies_to_defeat_cache(nbytes) if args.rotate_operands else 1
+        bufs = [torch.full((nbytes // 2,), 1.0, dtype=torch.float16, device=dev) for _ in range(n_copies)]
+        sink = torch.zeros(4, dtype=torch.float32, device=dev)
+
+        def call(j):
+            rc = read(bufs[j].data_ptr(), nbytes, sink.data_ptr(), cur())
+            if rc != 0:
+                raise RuntimeError("mi355_timeline_stream_read failed: %d" % rc)
+        t = time_launches(rotating(call, n_copies), args.steps, args.warmup, stats=True)
+        print(json.dumps(dict(t, kernel_config=args.kernel_config, rotate_operands=bool(args.rotate_operands), copies=n_copies,
+                              gbs=nbytes / t["ms"] / 1e6, algorithmic_bytes=float(nbytes))))
+        return
     if cfg[0] == "gemm":
         _, M, N, K, lay = cfg
         a_h, b_h = so.gemm_inputs(M, N, K, seed=0, a_std=1.0, b_std=0.02)

@@ -32,6 +32,22 @@ def test_library_exports_every_declared_symbol(lib):
     assert not hasattr(cdll, "mi355_debug_set_gemm_variant") and not hasattr(cdll, "mi355_debug_set_fmha_variant")
 
 
+def test_profiling_twin_exports_the_library_plus_its_readers(lib):
+    # libmi355_serving_timeline.so (bench.py --timeline) is the same library with time stamps compiled into the tiled GEMM and the
+    # attention kernels: every public symbol, plus the readers of the records and the read-only yardstick kernel; the product
+    # library carries none of those
+    twin = ctypes.CDLL(os.path.join(os.path.dirname(lib.LIB_PATH), "libmi355_serving_timeline.so"))
+    for n in declared_functions():
+        assert getattr(twin, n) is not None
+    extra = ("mi355_timeline_read_hgemm", "mi355_timeline_read_fmha_fwd", "mi355_timeline_read_fmha_decode",
+             "mi355_timeline_stream_read")
+    cdll = lib.load()
+    for n in extra:
+        assert getattr(twin, n) is not None
+        assert not hasattr(cdll, n)
+    assert twin.mi355_timeline_stream_read(None, ctypes.c_size_t(64), None, None) != 0   # null pointers: refused, nothing launched
+
+
 def test_capi_rejects_bad_arguments_without_a_gpu(lib):
     cdll = lib.load()
     assert cdll.mi355_hgemm(None, None, None, 4, 4, 4, 4, 4, 4, 0, None) == 10001
