@@ -6,8 +6,9 @@ calls, transposes to [B, H, S, D], applies RoPE, expands K/V with repeat_kv (:67
 ``fmha_unified.ops.fine_fmha`` (:687-690), transposes back with a copy (:700) and projects; LlamaDecoderLayer.forward
 (:755-781) wraps it in RMSNorm, residual adds and the gate/up/down MLP (:227), all as separate PyTorch kernels.
 
-Here one layer is nine launches with a KV cache (ten on a generation step, whose split attention ends in a merge
-kernel; one more where the gate/up epilogue does not apply and SiLU*up runs on its own) with no layout copies:
+Here one layer is nine launches with a KV cache, prefill and generation step alike (eight without a cache: one RoPE launch
+instead of two; one more for 17..64 token rows, where the gate/up epilogue does not apply and SiLU*up runs on its own),
+with no layout copies:
     rmsnorm -> QKV GEMM (one fused NT GEMM on the nn.Linear weights) -> RoPE in place on the q and k heads of the
     projection (k goes straight into the KV cache when there is one) -> attention reading q, k, v where they lie
     (strided operands, GQA inside the kernel, output written as [B, S, Hq*D]) -> O projection with the residual
