@@ -169,6 +169,20 @@ int mi355_rope(const void* x, void* out, int B, int S, int heads, int copy_heads
                int64_t pos_batch, int n_positions, void* stream);
 
 /*
+ * mi355_rope_qkv: the two mi355_rope calls of a decoder layer with a KV cache in one launch. Token (b, t) of the fused
+ *   projection lies at qkv + b*x_batch + t*x_row as [q_heads | kv_heads key heads | kv_heads value heads] of 128; the query
+ *   heads are rotated in place, the rotated key heads and the value heads are written to kv_out + b*out_batch + t*out_row as
+ *   [kv_heads keys | kv_heads values] (the new rows of a cache tensor that holds K and V of a token side by side). Same
+ *   tables, positions and arithmetic as mi355_rope: the results are bit-identical to
+ *   mi355_rope(qkv, qkv, .., q_heads, 0, ..) followed by mi355_rope(qkv + q_heads*128, kv_out, .., kv_heads, kv_heads, ..).
+ *   (`query_states, key_states = apply_rotary_pos_emb(..)` and `past_key_value.update(key_states, value_states, ..)`,
+ *   modeling_llama.py:664-668.)
+ */
+int mi355_rope_qkv(void* qkv, void* kv_out, int B, int S, int q_heads, int kv_heads, int D, int64_t x_batch, int64_t x_row,
+                   int64_t out_batch, int64_t out_row, const float* cos_table, const float* sin_table, const int32_t* positions,
+                   int64_t pos_batch, int n_positions, void* stream);
+
+/*
  * mi355_silu_mul: out[r][j] = silu(g[r][j]) * u[r][j] (`act_fn(gate_proj(x)) * up_proj(x)`, modeling_llama.py:227, for gate
  *   and up computed by one GEMM). interleave == 0: g = gate_up[r][0 .. inter), u = gate_up[r][inter .. 2 inter).
  *   interleave == b > 0 (a multiple of 8 dividing inter): g and u alternate in groups of b columns, the layout
@@ -193,6 +207,9 @@ int mi355_rmsnorm_bf16(const void* x, const void* residual, void* residual_out, 
 int mi355_rope_bf16(const void* x, void* out, int B, int S, int heads, int copy_heads, int D, int64_t x_batch, int64_t x_row,
                     int64_t out_batch, int64_t out_row, const float* cos_table, const float* sin_table,
                     const int32_t* positions, int64_t pos_batch, int n_positions, void* stream);
+int mi355_rope_qkv_bf16(void* qkv, void* kv_out, int B, int S, int q_heads, int kv_heads, int D, int64_t x_batch, int64_t x_row,
+                        int64_t out_batch, int64_t out_row, const float* cos_table, const float* sin_table,
+                        const int32_t* positions, int64_t pos_batch, int n_positions, void* stream);
 int mi355_silu_mul_bf16(const void* gate_up, void* out, int64_t rows, int inter, int interleave, int64_t ld_in, int64_t ld_out,
                         void* stream);
 

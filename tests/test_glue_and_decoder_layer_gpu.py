@@ -72,6 +72,34 @@ def test_rope_in_place_and_into_a_cache(lib, gpu, B, S, heads):
     assert float(cache[:, :4].abs().max()) == 0.0 and float(cache[:, 4 + S:].abs().max()) == 0.0
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("B,S,n_q,n_kv,shared_positions", [(2, 5, 4, 1, True), (8, 1, 32, 8, True), (1, 37, 32, 8, False),
+                                                           (3, 2, 40, 5, False)])
+def test_rope_qkv_equals_the_two_rope_calls_it_replaces(lib, gpu, dtype, B, S, n_q, n_kv, shared_positions):
+    # q in place, k rotated + v copied into a cache tensor: one launch, bit-identical to mi355_rope on the q heads followed by
+    # mi355_rope(copy_heads = n_kv) on the k and v heads (itself checked against the oracle above); everything around the new
+    # rows of the cache, and the k / v heads of the projection, stay untouched
+    cos, sin = so.rope_tables(128, 128, 10000.0)
+    cos, sin = cos.to(gpu), sin.to(gpu)
+    qkv = so.randn_fp16((B, S, n_q + 2 * n_kv, 128), 5).to(gpu).to(dtype)
+    if shared_positions:
+        pos = (torch.arange(S, dtype=torch.int32) + 60).to(gpu)
+    else:
+        pos = ((torch.arange(B * S, dtype=torch.int32) * 7) % 128).reshape(B, S).to(gpu)
+    past, max_len = 11, 11 + S + 3
+    cache_a = torch.full((B, max_len, 2 * n_kv, 128), 3.0, dtype=dtype, device=gpu)
+    cache_b = cache_a.clone()
+    two = qkv.clone()
+    lib.rope(two[:, :, :n_q], cos, sin, pos)
+    lib.rope(two[:, :, n_q:], cos, sin, pos, out=cache_a[:, past:past + S], copy_heads=n_kv)
+    one = qkv.clone()
+    lib.rope_qkv(one, cache_b[:, past:past + S], cos, sin, pos, n_q, n_kv)
+    assert torch.equal(one, two) and torch.equal(cache_a, cache_b)
+    assert torch.equal(one[:, :, n_q:], qkv[:, :, n_q:]) and not torch.equal(one[:, :, :n_q], qkv[:, :, :n_q])
+    assert bool((cache_b[:, :past] == 3.0).all()) and bool((cache_b[:, past + S:] == 3.0).all())
+    assert torch.equal(cache_b[:, past:past + S, n_kv:], qkv[:, :, n_q + n_kv:])
+
+
 def test_rope_copies_value_heads_and_shares_one_position_table(lib, gpu):
     # k heads rotated and v heads copied into a fused K|V cache row by one launch; one [S] position table for all batch rows
     B, S, n_kv = 3, 17, 5

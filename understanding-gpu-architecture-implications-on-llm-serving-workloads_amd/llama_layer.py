@@ -6,9 +6,8 @@ calls, transposes to [B, H, S, D], applies RoPE, expands K/V with repeat_kv (:67
 ``fmha_unified.ops.fine_fmha`` (:687-690), transposes back with a copy (:700) and projects; LlamaDecoderLayer.forward
 (:755-781) wraps it in RMSNorm, residual adds and the gate/up/down MLP (:227), all as separate PyTorch kernels.
 
-Here one layer is nine launches with a KV cache, prefill and generation step alike (eight without a cache: one RoPE launch
-instead of two; one more for 17..64 token rows, where the gate/up epilogue does not apply and SiLU*up runs on its own),
-with no layout copies:
+Here one layer is eight launches, with or without a KV cache, prefill and generation step alike (one more for 17..64 token
+rows, where the gate/up epilogue does not apply and SiLU*up runs on its own), with no layout copies:
     rmsnorm -> QKV GEMM (one fused NT GEMM on the nn.Linear weights) -> RoPE in place on the q and k heads of the
     projection (k goes straight into the KV cache when there is one) -> attention reading q, k, v where they lie
     (strided operands, GQA inside the kernel, output written as [B, S, Hq*D]) -> O projection with the residual
@@ -111,9 +110,8 @@ class FineLlamaDecoderLayer:
         else:
             if past + S > kv_cache.max_len:
                 raise ValueError("KV cache of %d tokens cannot take %d more after %d" % (kv_cache.max_len, S, past))
-            lib.rope(q, self.cos, self.sin, pos)
-            # rotated keys and plain values of the new tokens go into the cache in one launch
-            lib.rope(qkv[:, :, Hq:], self.cos, self.sin, pos, out=kv_cache.kv[:, past:past + S], copy_heads=Hkv)
+            # one launch: q rotated in place, rotated keys and plain values of the new tokens into the cache
+            lib.rope_qkv(qkv, kv_cache.kv[:, past:past + S], self.cos, self.sin, pos, Hq, Hkv)
             kv_cache.length = past + S
             k, v = kv_cache.k[:, :past + S], kv_cache.v[:, :past + S]
         attn = torch.empty((B, S, Hq, D), dtype=self.dtype, device=x.device)

@@ -15,8 +15,8 @@ GEMM_NN, GEMM_NT, GEMM_TN = 0, 1, 2
 LAYOUTS = {"NN": GEMM_NN, "NT": GEMM_NT, "TN": GEMM_TN}
 ERR_BAD_ARGUMENT, ERR_UNSUPPORTED = 10001, 10002
 
-EXPORTED_SYMBOLS = ("mi355_hgemm", "mi355_fmha_fwd", "mi355_fmha_fwd_strided", "mi355_fmha_fwd_bf16", "mi355_hgemm_silu_mul", "mi355_hgemm_add", "mi355_rmsnorm", "mi355_rope", "mi355_silu_mul",
-                    "mi355_gemm_bf16", "mi355_gemm_silu_mul_bf16", "mi355_gemm_add_bf16", "mi355_rmsnorm_bf16", "mi355_rope_bf16", "mi355_silu_mul_bf16",
+EXPORTED_SYMBOLS = ("mi355_hgemm", "mi355_fmha_fwd", "mi355_fmha_fwd_strided", "mi355_fmha_fwd_bf16", "mi355_hgemm_silu_mul", "mi355_hgemm_add", "mi355_rmsnorm", "mi355_rope", "mi355_rope_qkv", "mi355_silu_mul",
+                    "mi355_gemm_bf16", "mi355_gemm_silu_mul_bf16", "mi355_gemm_add_bf16", "mi355_rmsnorm_bf16", "mi355_rope_bf16", "mi355_rope_qkv_bf16", "mi355_silu_mul_bf16",
                     "mi355_fmha_fwd_workspace_bytes", "mi355_fmha_fwd_ws", "mi355_fmha_fwd_noalloc",
                     "mi355_last_error", "mi355_serving_version")
 # exported for tests and tuning runs, declared in csrc/mi355_serving_internal.h and not in the public header
@@ -56,6 +56,8 @@ def load():
     lib.mi355_rmsnorm.restype = i32
     lib.mi355_rope.argtypes = [vp, vp, i32, i32, i32, i32, i32, i64, i64, i64, i64, vp, vp, vp, i64, i32, vp]
     lib.mi355_rope.restype = i32
+    lib.mi355_rope_qkv.argtypes = lib.mi355_rope.argtypes
+    lib.mi355_rope_qkv.restype = i32
     lib.mi355_silu_mul.argtypes = [vp, vp, i64, i32, i32, i64, i64, vp]
     lib.mi355_hgemm_silu_mul.argtypes = lib.mi355_hgemm.argtypes
     lib.mi355_hgemm_silu_mul.restype = i32
@@ -65,6 +67,7 @@ def load():
     for fp16_name, bf16_name in (("mi355_hgemm", "mi355_gemm_bf16"), ("mi355_hgemm_silu_mul", "mi355_gemm_silu_mul_bf16"),
                                  ("mi355_hgemm_add", "mi355_gemm_add_bf16"),
                                  ("mi355_rmsnorm", "mi355_rmsnorm_bf16"), ("mi355_rope", "mi355_rope_bf16"),
+                                 ("mi355_rope_qkv", "mi355_rope_qkv_bf16"),
                                  ("mi355_silu_mul", "mi355_silu_mul_bf16")):
         getattr(lib, bf16_name).argtypes = getattr(lib, fp16_name).argtypes
         getattr(lib, bf16_name).restype = i32
@@ -271,6 +274,23 @@ def rope(x, cos, sin, positions, out=None, copy_heads=0):
                              out.stride(0), out.stride(1), _ptr(cos), _ptr(sin), _ptr(positions), pos_batch, cos.shape[0],
                              _stream_of(x)))
     return out
+
+
+def rope_qkv(qkv, kv_out, cos, sin, positions, q_heads, kv_heads):
+    """One launch for a fused projection qkv [B, S, q_heads + 2 kv_heads, 128]: query heads rotated in place, rotated key heads
+    and plain value heads written to kv_out [B, S, 2 kv_heads, 128] (own batch / token strides: the new rows of a KV cache)."""
+    import torch
+    B, S, heads, D = qkv.shape
+    assert heads == q_heads + 2 * kv_heads and kv_out.shape == (B, S, 2 * kv_heads, D)
+    assert qkv.dtype in (torch.float16, torch.bfloat16) and kv_out.dtype == qkv.dtype
+    assert qkv.stride(3) == 1 and qkv.stride(2) == D and kv_out.stride(3) == 1 and kv_out.stride(2) == D
+    assert cos.dtype == torch.float32 and cos.is_contiguous() and sin.is_contiguous() and cos.shape == sin.shape
+    assert positions.dtype == torch.int32 and positions.is_contiguous() and positions.numel() in (S, B * S)
+    pos_batch = S if (positions.numel() == B * S and B > 1) else 0
+    entry = load().mi355_rope_qkv_bf16 if qkv.dtype == torch.bfloat16 else load().mi355_rope_qkv
+    _check(entry(_ptr(qkv), _ptr(kv_out), B, S, q_heads, kv_heads, D, qkv.stride(0), qkv.stride(1), kv_out.stride(0),
+                 kv_out.stride(1), _ptr(cos), _ptr(sin), _ptr(positions), pos_batch, cos.shape[0], _stream_of(qkv)))
+    return kv_out
 
 
 def silu_mul(gate_up, out=None, interleave=0):
