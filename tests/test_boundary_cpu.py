@@ -92,11 +92,13 @@ def test_capi_rejects_bad_arguments_without_a_gpu(lib):
     assert cdll.mi355_rope(p, p, 1, 4, 2, 0, 64, 1024, 256, 1024, 256, p, p, p, 0, 16, None) == 10002    # head_dim != 128
     assert cdll.mi355_rope(p, p, 1, 4, 1, 1, 128, 1024, 128, 1024, 256, p, p, p, 0, 16, None) == 10001   # row stride < heads * 128
     assert cdll.mi355_rope(p, p, 1, 4, 2, 0, 128, 1024, 256, 1024, 256, p, p, None, 0, 16, None) == 10001
-    assert cdll.mi355_rope_qkv(p, p, 1, 4, 4, 1, 128, 4096, 512, 1024, 256, p, p, p, 0, 16, None) == 10001   # x_row < (4 + 2) * 128
-    assert cdll.mi355_rope_qkv(p, p, 1, 4, 4, 1, 128, 4096, 768, 1024, 128, p, p, p, 0, 16, None) == 10001   # out_row < 2 * 128
-    assert cdll.mi355_rope_qkv(p, p, 1, 4, 4, 0, 128, 4096, 768, 1024, 256, p, p, p, 0, 16, None) == 10001   # no kv heads
-    assert cdll.mi355_rope_qkv(p, None, 1, 4, 4, 1, 128, 4096, 768, 1024, 256, p, p, p, 0, 16, None) == 10001
-    assert cdll.mi355_rope_qkv_bf16(p, p, 1, 4, 4, 1, 64, 4096, 768, 1024, 256, p, p, p, 0, 16, None) == 10002   # head_dim != 128
+    assert cdll.mi355_rope_qkv(p, p, 1, 4, 4, 1, 128, 4096, 512, 1024, 256, 128, p, p, p, 0, 16, None) == 10001   # x_row < (4 + 2) * 128
+    assert cdll.mi355_rope_qkv(p, p, 1, 4, 4, 1, 128, 4096, 768, 1024, 128, 128, p, p, p, 0, 16, None) == 10001   # token-major row too short for k | v
+    assert cdll.mi355_rope_qkv(p, p, 1, 4, 4, 1, 128, 4096, 768, 1024, 128, 256, p, p, p, 0, 16, None) == 10001   # head-major: head stride < 4 rows
+    assert cdll.mi355_rope_qkv(p, p, 1, 4, 4, 1, 128, 4096, 768, 1024, 256, 64, p, p, p, 0, 16, None) == 10001    # out_head < 128
+    assert cdll.mi355_rope_qkv(p, p, 1, 4, 4, 0, 128, 4096, 768, 1024, 256, 128, p, p, p, 0, 16, None) == 10001   # no kv heads
+    assert cdll.mi355_rope_qkv(p, None, 1, 4, 4, 1, 128, 4096, 768, 1024, 256, 128, p, p, p, 0, 16, None) == 10001
+    assert cdll.mi355_rope_qkv_bf16(p, p, 1, 4, 4, 1, 64, 4096, 768, 1024, 256, 128, p, p, p, 0, 16, None) == 10002   # head_dim != 128
     assert cdll.mi355_silu_mul(p, p, 4, 64, 0, 64, 64, None) == 10001                               # ld_in < 2 * inter
     assert cdll.mi355_silu_mul(p, p, 0, 64, 0, 128, 64, None) == 10001
     assert cdll.mi355_silu_mul(p, p, 4, 64, 12, 128, 64, None) == 10001                             # interleave % 8

@@ -98,6 +98,11 @@ def test_rope_qkv_equals_the_two_rope_calls_it_replaces(lib, gpu, dtype, B, S, n
     assert torch.equal(one[:, :, n_q:], qkv[:, :, n_q:]) and not torch.equal(one[:, :, :n_q], qkv[:, :, :n_q])
     assert bool((cache_b[:, :past] == 3.0).all()) and bool((cache_b[:, past + S:] == 3.0).all())
     assert torch.equal(cache_b[:, past:past + S, n_kv:], qkv[:, :, n_q + n_kv:])
+    # the same rows into a head-major cache [B, 2 n_kv, max_len, 128]
+    cache_h = torch.full((B, 2 * n_kv, max_len, 128), 3.0, dtype=dtype, device=gpu)
+    one_h = qkv.clone()
+    lib.rope_qkv(one_h, cache_h[:, :, past:past + S].transpose(1, 2), cos, sin, pos, n_q, n_kv)
+    assert torch.equal(one_h, two) and torch.equal(cache_h.transpose(1, 2), cache_a)
 
 
 def test_rope_copies_value_heads_and_shares_one_position_table(lib, gpu):

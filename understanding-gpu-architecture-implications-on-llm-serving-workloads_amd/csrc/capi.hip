@@ -256,41 +256,46 @@ static int rope_impl(const char* fn, int dtype, const void* x, void* out, int B,
         return fail(MI355_ERR_BAD_ARGUMENT, "%s: strides must be multiples of 8, row strides >= (heads + copy_heads) * 128", fn);
     if (!aligned16(x) || !aligned16(out) || !aligned16(cos_table) || !aligned16(sin_table))
         return fail(MI355_ERR_BAD_ARGUMENT, "%s: pointers must be 16-byte aligned", fn);
-    hipError_t e = mi355::rope_dispatch(x, out, B, S, 0, heads, copy_heads, x_batch, x_row, out_batch, out_row, cos_table, sin_table,
+    hipError_t e = mi355::rope_dispatch(x, out, B, S, 0, heads, copy_heads, x_batch, x_row, out_batch, out_row, D, cos_table, sin_table,
                                         positions, pos_batch, n_positions, dtype, static_cast<hipStream_t>(stream));
     if (e != hipSuccess) return hip_fail(e, fn);
     return 0;
 }
 
 static int rope_qkv_impl(const char* fn, int dtype, void* qkv, void* kv_out, int B, int S, int q_heads, int kv_heads, int D,
-                         int64_t x_batch, int64_t x_row, int64_t out_batch, int64_t out_row, const float* cos_table,
+                         int64_t x_batch, int64_t x_row, int64_t out_batch, int64_t out_row, int64_t out_head, const float* cos_table,
                          const float* sin_table, const int32_t* positions, int64_t pos_batch, int n_positions, void* stream) {
     if (!qkv || !kv_out || !cos_table || !sin_table || !positions) return fail(MI355_ERR_BAD_ARGUMENT, "%s: null pointer", fn);
     if (D != 128) return fail(MI355_ERR_UNSUPPORTED, "%s: head_dim must be 128 (got %d)", fn, D);
     if (B < 1 || S < 1 || q_heads < 1 || kv_heads < 1 || n_positions < 1 || pos_batch < 0)
         return fail(MI355_ERR_BAD_ARGUMENT, "%s: B, S, q_heads, kv_heads, n_positions must be >= 1, pos_batch >= 0", fn);
-    const int64_t in_width = ((int64_t)q_heads + 2 * (int64_t)kv_heads) * D, out_width = 2 * (int64_t)kv_heads * D;
-    if (x_row < in_width || out_row < out_width || x_row % 8 || out_row % 8 || x_batch % 8 || out_batch % 8 || x_batch < 0 || out_batch < 0)
+    const int64_t in_width = ((int64_t)q_heads + 2 * (int64_t)kv_heads) * D;
+    if (x_row < in_width || out_row < D || out_head < D || x_row % 8 || out_row % 8 || out_head % 8 || x_batch % 8 || out_batch % 8 ||
+        x_batch < 0 || out_batch < 0)
         return fail(MI355_ERR_BAD_ARGUMENT,
-                    "%s: strides must be multiples of 8, x_row >= (q_heads + 2 kv_heads) * 128, out_row >= 2 kv_heads * 128", fn);
+                    "%s: strides must be multiples of 8, x_row >= (q_heads + 2 kv_heads) * 128, out_row >= 128, out_head >= 128", fn);
+    // heads side by side in a token row (out_head == 128) need a row that holds them all; a head-major cache (out_head >= a
+    // head's whole sequence) needs rows of 128
+    if (out_head < (int64_t)S * out_row && out_row < 2 * (int64_t)kv_heads * out_head)
+        return fail(MI355_ERR_BAD_ARGUMENT, "%s: out_row / out_head make the heads of a token overlap those of the next", fn);
     if (!aligned16(qkv) || !aligned16(kv_out) || !aligned16(cos_table) || !aligned16(sin_table))
         return fail(MI355_ERR_BAD_ARGUMENT, "%s: pointers must be 16-byte aligned", fn);
     hipError_t e = mi355::rope_dispatch(qkv, kv_out, B, S, q_heads, q_heads + kv_heads, kv_heads, x_batch, x_row, out_batch, out_row,
-                                        cos_table, sin_table, positions, pos_batch, n_positions, dtype, static_cast<hipStream_t>(stream));
+                                        out_head, cos_table, sin_table, positions, pos_batch, n_positions, dtype, static_cast<hipStream_t>(stream));
     if (e != hipSuccess) return hip_fail(e, fn);
     return 0;
 }
 
 int mi355_rope_qkv(void* qkv, void* kv_out, int B, int S, int q_heads, int kv_heads, int D, int64_t x_batch, int64_t x_row,
-                   int64_t out_batch, int64_t out_row, const float* cos_table, const float* sin_table, const int32_t* positions,
+                   int64_t out_batch, int64_t out_row, int64_t out_head, const float* cos_table, const float* sin_table, const int32_t* positions,
                    int64_t pos_batch, int n_positions, void* stream) {
-    return rope_qkv_impl("mi355_rope_qkv", MI355_DTYPE_FP16, qkv, kv_out, B, S, q_heads, kv_heads, D, x_batch, x_row, out_batch, out_row, cos_table, sin_table, positions, pos_batch, n_positions, stream);
+    return rope_qkv_impl("mi355_rope_qkv", MI355_DTYPE_FP16, qkv, kv_out, B, S, q_heads, kv_heads, D, x_batch, x_row, out_batch, out_row, out_head, cos_table, sin_table, positions, pos_batch, n_positions, stream);
 }
 
 int mi355_rope_qkv_bf16(void* qkv, void* kv_out, int B, int S, int q_heads, int kv_heads, int D, int64_t x_batch, int64_t x_row,
-                        int64_t out_batch, int64_t out_row, const float* cos_table, const float* sin_table, const int32_t* positions,
+                        int64_t out_batch, int64_t out_row, int64_t out_head, const float* cos_table, const float* sin_table, const int32_t* positions,
                         int64_t pos_batch, int n_positions, void* stream) {
-    return rope_qkv_impl("mi355_rope_qkv_bf16", MI355_DTYPE_BF16, qkv, kv_out, B, S, q_heads, kv_heads, D, x_batch, x_row, out_batch, out_row, cos_table, sin_table, positions, pos_batch, n_positions, stream);
+    return rope_qkv_impl("mi355_rope_qkv_bf16", MI355_DTYPE_BF16, qkv, kv_out, B, S, q_heads, kv_heads, D, x_batch, x_row, out_batch, out_row, out_head, cos_table, sin_table, positions, pos_batch, n_positions, stream);
 }
 
 int mi355_rope(const void* x, void* out, int B, int S, int heads, int copy_heads, int D, int64_t x_batch, int64_t x_row,

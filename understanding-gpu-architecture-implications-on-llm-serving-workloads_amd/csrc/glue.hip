@@ -118,12 +118,13 @@ __global__ __launch_bounds__(glue::THREADS) void rmsnorm_kernel(const T* x, cons
 // (rotate_half convention, modeling_llama.py:164-168,193-194), cos/sin rows of 64 fp32 selected by the token's position.
 // The `copy_heads` heads that follow are moved unrotated (the value heads on their way into a KV cache).
 // The first `inplace_heads` heads are written back where they were read (the query heads of a fused QKV projection); the
-// others go to `out`, whose head 0 is head `inplace_heads` of x (the key and value heads on their way into the cache).
+// others go to `out`, whose head 0 is head `inplace_heads` of x (the key and value heads on their way into the cache),
+// `o_head` elements from one head to the next (128 for heads side by side; a whole head's sequence for a head-major cache).
 // A thread owns 8 values of the lower half and their 8 partners; 8 threads per head, 32 heads per workgroup.
 template <typename T>
 __global__ __launch_bounds__(glue::THREADS) void rope_kernel(const T* x, T* out, int S, int inplace_heads,
                                                              int heads, int copy_heads, long x_batch, long x_row, long o_batch,
-                                                             long o_row, const float* __restrict__ cos_t,
+                                                             long o_row, long o_head, const float* __restrict__ cos_t,
                                                              const float* __restrict__ sin_t, const int* __restrict__ positions,
                                                              long pos_batch, int n_pos) {
     using V8 = typename Elem<T>::v8;
@@ -133,7 +134,7 @@ __global__ __launch_bounds__(glue::THREADS) void rope_kernel(const T* x, T* out,
     const int i0 = (threadIdx.x & 7) * 8;
     const long b = token / S, s = token - b * S;
     const T* xp = x + b * x_batch + s * x_row + (long)head * 128 + i0;
-    T* op = head < inplace_heads ? const_cast<T*>(xp) : out + b * o_batch + s * o_row + (long)(head - inplace_heads) * 128 + i0;
+    T* op = head < inplace_heads ? const_cast<T*>(xp) : out + b * o_batch + s * o_row + (long)(head - inplace_heads) * o_head + i0;
     const V8 lo = *(const V8*)xp;
     const V8 hi = *(const V8*)(xp + 64);
     if (head >= heads) {
@@ -211,7 +212,7 @@ hipError_t rmsnorm_dispatch(const void* x, const void* residual, void* res_out, 
 }
 
 hipError_t rope_dispatch(const void* x, void* out, int B, int S, int inplace_heads, int heads, int copy_heads, long x_batch,
-                         long x_row, long o_batch, long o_row, const float* cos_t, const float* sin_t, const int* positions, long pos_batch,
+                         long x_row, long o_batch, long o_row, long o_head, const float* cos_t, const float* sin_t, const int* positions, long pos_batch,
                          int n_pos, int dtype, hipStream_t stream) {
     const long tokens = (long)B * S;
     const int groups = (heads + copy_heads + 31) / 32;
@@ -219,10 +220,10 @@ hipError_t rope_dispatch(const void* x, void* out, int B, int S, int inplace_hea
     const dim3 grid((unsigned)tokens, (unsigned)groups), block(glue::THREADS);
     if (dtype == MI355_DTYPE_BF16)
         rope_kernel<bf16_t><<<grid, block, 0, stream>>>((const bf16_t*)x, (bf16_t*)out, S, inplace_heads, heads, copy_heads, x_batch, x_row,
-                                                        o_batch, o_row, cos_t, sin_t, positions, pos_batch, n_pos);
+                                                        o_batch, o_row, o_head, cos_t, sin_t, positions, pos_batch, n_pos);
     else
         rope_kernel<half_t><<<grid, block, 0, stream>>>((const half_t*)x, (half_t*)out, S, inplace_heads, heads, copy_heads, x_batch, x_row,
-                                                        o_batch, o_row, cos_t, sin_t, positions, pos_batch, n_pos);
+                                                        o_batch, o_row, o_head, cos_t, sin_t, positions, pos_batch, n_pos);
     return hipGetLastError();
 }
 

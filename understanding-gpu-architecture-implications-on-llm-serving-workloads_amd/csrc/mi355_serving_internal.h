@@ -69,9 +69,10 @@ hipError_t fmha_decode_dispatch(const T* Q, const T* K, const T* V, T* O, float*
 // Layer glue (glue.hip); arguments as the mi355_rmsnorm / mi355_rope / mi355_silu_mul entry points after validation.
 hipError_t rmsnorm_dispatch(const void* x, const void* residual, void* res_out, const void* weight, void* out, long rows,
                             int hidden, long ldx, long ldr, long ldro, long ldo, float eps, int dtype, hipStream_t stream);
-// rope_dispatch: `heads` heads are rotated, the first `inplace_heads` of them in place, `copy_heads` more are copied.
+// rope_dispatch: `heads` heads are rotated, the first `inplace_heads` of them in place, `copy_heads` more are copied;
+// consecutive heads of `out` lie o_head elements apart.
 hipError_t rope_dispatch(const void* x, void* out, int B, int S, int inplace_heads, int heads, int copy_heads, long x_batch,
-                         long x_row, long o_batch, long o_row, const float* cos_t, const float* sin_t, const int* positions, long pos_batch,
+                         long x_row, long o_batch, long o_row, long o_head, const float* cos_t, const float* sin_t, const int* positions, long pos_batch,
                          int n_pos, int dtype, hipStream_t stream);
 hipError_t silu_mul_dispatch(const void* in, void* out, long rows, int inter, int block, long ld_in, long ld_out, int dtype,
                              hipStream_t stream);

@@ -56,7 +56,7 @@ def load():
     lib.mi355_rmsnorm.restype = i32
     lib.mi355_rope.argtypes = [vp, vp, i32, i32, i32, i32, i32, i64, i64, i64, i64, vp, vp, vp, i64, i32, vp]
     lib.mi355_rope.restype = i32
-    lib.mi355_rope_qkv.argtypes = lib.mi355_rope.argtypes
+    lib.mi355_rope_qkv.argtypes = [vp, vp, i32, i32, i32, i32, i32, i64, i64, i64, i64, i64, vp, vp, vp, i64, i32, vp]
     lib.mi355_rope_qkv.restype = i32
     lib.mi355_silu_mul.argtypes = [vp, vp, i64, i32, i32, i64, i64, vp]
     lib.mi355_hgemm_silu_mul.argtypes = lib.mi355_hgemm.argtypes
@@ -278,18 +278,19 @@ def rope(x, cos, sin, positions, out=None, copy_heads=0):
 
 def rope_qkv(qkv, kv_out, cos, sin, positions, q_heads, kv_heads):
     """One launch for a fused projection qkv [B, S, q_heads + 2 kv_heads, 128]: query heads rotated in place, rotated key heads
-    and plain value heads written to kv_out [B, S, 2 kv_heads, 128] (own batch / token strides: the new rows of a KV cache)."""
+    and plain value heads written to kv_out [B, S, 2 kv_heads, 128] (own batch / token / head strides: the new rows of a KV
+    cache, token-major or head-major)."""
     import torch
     B, S, heads, D = qkv.shape
     assert heads == q_heads + 2 * kv_heads and kv_out.shape == (B, S, 2 * kv_heads, D)
     assert qkv.dtype in (torch.float16, torch.bfloat16) and kv_out.dtype == qkv.dtype
-    assert qkv.stride(3) == 1 and qkv.stride(2) == D and kv_out.stride(3) == 1 and kv_out.stride(2) == D
+    assert qkv.stride(3) == 1 and qkv.stride(2) == D and kv_out.stride(3) == 1
     assert cos.dtype == torch.float32 and cos.is_contiguous() and sin.is_contiguous() and cos.shape == sin.shape
     assert positions.dtype == torch.int32 and positions.is_contiguous() and positions.numel() in (S, B * S)
     pos_batch = S if (positions.numel() == B * S and B > 1) else 0
     entry = load().mi355_rope_qkv_bf16 if qkv.dtype == torch.bfloat16 else load().mi355_rope_qkv
     _check(entry(_ptr(qkv), _ptr(kv_out), B, S, q_heads, kv_heads, D, qkv.stride(0), qkv.stride(1), kv_out.stride(0),
-                 kv_out.stride(1), _ptr(cos), _ptr(sin), _ptr(positions), pos_batch, cos.shape[0], _stream_of(qkv)))
+                 kv_out.stride(1), kv_out.stride(2), _ptr(cos), _ptr(sin), _ptr(positions), pos_batch, cos.shape[0], _stream_of(qkv)))
     return kv_out
 
 
