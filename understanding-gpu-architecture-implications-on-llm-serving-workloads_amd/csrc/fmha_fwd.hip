@@ -502,8 +502,13 @@ static hipError_t fmha_fwd_dispatch_t(const void* Q, const void* K, const void* 
         // sequences are long enough to amortise their longer prologue. Measured (b, heads 32/8, s, 128- vs 256-query):
         // 1 x 1024 causal 25 / 35 us, 1 x 2048 57 / 65, 8 x 512 43 / 50, 1 x 3000 108 / 94, 1 x 4096 182 / 144,
         // 4 x 1024 (32 kv heads, non-causal) 100 / 82.
+        // A causal problem whose keys are its own queries computes every diagonal block in full: with 256-query workgroups
+        // that is 1 / (2 Sq / 256) more work than with 128-query ones, which outweighs their cheaper inner loop below
+        // ~1400 queries (many workgroups either way; 128- / 256-query: 16 x 768 127 / 136 us, 8 x 1024 101 / 108,
+        // 8 x 1280 142 / 146, 4 x 1536 101 / 99, 4 x 2048 169 / 153).
         const long wg256 = (long)((Sq + 255) / 256) * Hq * B;
-        variant = (wg256 >= 320 && Sq > 512) ? 2 : 1;
+        const bool diagonal_heavy = causal && Sk < 2L * Sq;
+        variant = (wg256 >= 320 && Sq > (diagonal_heavy ? 1408 : 512)) ? 2 : 1;
     }
     if (variant == 2) return launch_fmha_pingpong<T, 2>(q, k, v, o, LSE, B, Hq, Hkv, Sq, Sk, scale, causal, kv_valid_len, sd, stream);
     return launch_fmha_pingpong<T, 1>(q, k, v, o, LSE, B, Hq, Hkv, Sq, Sk, scale, causal, kv_valid_len, sd, stream);
