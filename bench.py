@@ -593,6 +593,17 @@ KERNEL_CONFIGS = {
     "stream_read_117mb": ("read", 14336 * 4096 * 2),
     "stream_read_235mb": ("read", 28672 * 4096 * 2),
     "stream_read_268mb": ("read", 2 * 8 * 8 * 8192 * 128 * 2),
+    # matrix instructions back to back on register operands, two waves per SIMD on every CU (profiling twin, --timeline): what
+    # the matrix pipes sustain on N(0,1) operands under the board's power limit, and on zeros (--zero-inputs)
+    "mfma_only_16x16x32": ("mfma", 16),
+    "mfma_only_32x32x16": ("mfma", 32),
+    # one wave per SIMD issues the matrix instructions of an attention key tile while the other runs the softmax's
+    # instruction mix (profiling twin, --timeline): each alone, then side by side
+    "mfma_valu_16x16x32": ("mfma_valu", 16),
+    "mfma_valu_32x32x16": ("mfma_valu", 32),
+    # the vendor library on the same box, same operands and timing loop (torch.matmul = hipBLASLt); not this code
+    "vendor_gemm_8192_nn": ("vendor_gemm", 8192, 8192, 8192, "NN"),
+    "vendor_gemm_8192_nt": ("vendor_gemm", 8192, 8192, 8192, "NT"),
 }
 
 
@@ -662,6 +673,75 @@ def run_kernel_config(args, torch, lib, so, dev):
         t = time_launches(rotating(call, n_copies), args.steps, args.warmup, stats=True)
         print(json.dumps(dict(t, kernel_config=args.kernel_config, rotate_operands=bool(args.rotate_operands), copies=n_copies,
                               gbs=nbytes / t["ms"] / 1e6, algorithmic_bytes=float(nbytes))))
+        return
+    if cfg[0] in ("mfma", "mfma_valu"):
+        import ctypes
+        import numpy as np
+        if not args.timeline:
+            sys.exit("bench.py: the mfma_* configurations live in the profiling twin of the library: add --timeline")
+        L = lib.load()
+        shape = cfg[1]
+        fill = so.randn_fp16((8192,), 5).to(dev)
+        if args.zero_inputs:
+            fill.zero_()
+        out = torch.empty(256 * 512, dtype=torch.float32, device=dev)
+        vp, i32 = ctypes.c_void_p, ctypes.c_int
+        if cfg[0] == "mfma":
+            f = L.mi355_timeline_mfma_only
+            f.argtypes, f.restype = [i32, vp, vp, i32, vp], i32
+            iters = 2000
+            def fn():
+                rc = f(shape, fill.data_ptr(), out.data_ptr(), iters, cur())
+                if rc != 0:
+                    raise RuntimeError("mi355_timeline_mfma_only failed: %d" % rc)
+            t = time_launches(fn, args.steps, args.warmup, stats=True)
+            flops = 256.0 * 8 * iters * 32 * (2.0 * 16 * 16 * 32 if shape == 16 else 2.0 * 32 * 32 * 16)
+            print(json.dumps(dict(t, kernel_config=args.kernel_config, zero_inputs=bool(args.zero_inputs), tflops=flops / t["ms"] / 1e9,
+                                  pct_of_fp16_mfma_peak=100 * flops / t["ms"] / 1e9 / PEAK_FP16_TFLOPS,
+                                  note="256 workgroups x 8 waves, %d x 32 MFMA %s per wave, operands in registers" % (
+                                      iters, "16x16x32" if shape == 16 else "32x32x16"))))
+            return
+        f = L.mi355_timeline_mfma_valu
+        f.argtypes, f.restype = [i32, vp, vp, i32, i32, vp], i32
+        rd = L.mi355_timeline_read_mfma_valu
+        rd.argtypes, rd.restype = [vp, ctypes.c_size_t], i32
+        iters = 400
+        res = {}
+        modes = [(1, "matrix_wave_alone"), (2, "valu_wave_alone"), (3, "side_by_side")]
+        if shape == 16:
+            modes += [(5, "matrix_wave_with_lds_fragment_reads_alone"), (7, "side_by_side_with_lds_fragment_reads")]
+        for mode, tag in modes:
+            for _ in range(3):
+                rc = f(shape, fill.data_ptr(), out.data_ptr(), iters, mode, cur())
+                if rc != 0:
+                    raise RuntimeError("mi355_timeline_mfma_valu failed: %d" % rc)
+            torch.cuda.synchronize()
+            buf = np.zeros(512, dtype=np.uint64)
+            if rd(buf.ctypes.data_as(vp), buf.nbytes) != 0:
+                raise RuntimeError("mi355_timeline_read_mfma_valu failed")
+            cyc = buf.reshape(256, 2).astype(np.float64) / iters
+            res[tag] = {"matrix_wave_cycles_per_tile": round(float(cyc[:, 0].mean()), 1) if mode & 1 else None,
+                        "valu_wave_cycles_per_tile": round(float(cyc[:, 1].mean()), 1) if mode & 2 else None}
+        print(json.dumps({"kernel_config": args.kernel_config, "zero_inputs": bool(args.zero_inputs), "cycles": res,
+                          "matrix_pipe_cycles_per_tile": 68 * 16,
+                          "note": "per key tile of a 32-query wave: matrix wave = 68 MFMA 16x16x32 (34 MFMA 32x32x16) on registers, "
+                                  "VALU wave = 16 v_max3 + 32 v_fma + 32 v_exp + 16 v_cvt_pk; the two waves share one SIMD, no barriers, "
+                                  "no memory traffic"}))
+        return
+    if cfg[0] == "vendor_gemm":
+        _, M, N, K, lay = cfg
+        a_h, b_h = so.gemm_inputs(M, N, K, seed=0, a_std=1.0, b_std=0.02)
+        a, b = a_h.to(dev), b_h.to(dev)
+        if lay == "NT":
+            b = b.t().contiguous().t()   # stored [N, K], passed as its transposed view
+        if args.zero_inputs:
+            a.zero_(), b.zero_()
+        c = torch.empty((M, N), dtype=torch.float16, device=dev)
+        t = time_launches(lambda: torch.matmul(a, b, out=c), args.steps, args.warmup, stats=True)
+        flops = 2.0 * M * N * K
+        print(json.dumps(dict(t, kernel_config=args.kernel_config, zero_inputs=bool(args.zero_inputs), tflops=flops / t["ms"] / 1e9,
+                              pct_of_fp16_mfma_peak=100 * flops / t["ms"] / 1e9 / PEAK_FP16_TFLOPS,
+                              note="torch.matmul (hipBLASLt) on the operands of the g2b configuration; the vendor library, not this code")))
         return
     if cfg[0] == "gemm":
         _, M, N, K, lay = cfg

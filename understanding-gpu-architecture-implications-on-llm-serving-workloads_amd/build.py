@@ -70,6 +70,9 @@ TIMELINE_LIB_NAME = "libmi355_serving_timeline.so"
 TIMELINE_LIB_PATH = os.path.join(LIB_DIR, TIMELINE_LIB_NAME)
 # Sources that carry per-workgroup time stamps when compiled with -DMI355_TIMELINE (csrc/mi355_timeline.h).
 TIMELINE_SOURCES = ("csrc/hgemm.hip", "csrc/fmha_fwd.hip", "csrc/fmha_decode.hip")
+# Yardstick kernels that exist in the profiling twin only (a read-only kernel, matrix instructions on registers, matrix and
+# VALU instructions side by side on one SIMD).
+TIMELINE_ONLY_SOURCES = ("csrc/timeline_probes.hip",)
 
 
 def build_library(verbose=True):
@@ -92,13 +95,18 @@ def build_library(verbose=True):
             cmd = [HIPCC] + DEVICE_FLAGS + SOURCE_FLAGS.get(src, []) + ["-DMI355_TIMELINE", "-I", INCLUDE, "-c", src, "-o", obj]
             jobs.append((cmd, obj))
             tl_objs[src] = obj
+        tl_extra = []
+        for src in TIMELINE_ONLY_SOURCES:
+            obj = os.path.join(tmp, os.path.basename(src) + ".timeline.o")
+            jobs.append(([HIPCC] + DEVICE_FLAGS + ["-DMI355_TIMELINE", "-I", INCLUDE, "-c", src, "-o", obj], obj))
+            tl_extra.append(obj)
         if verbose:
             for cmd, _ in jobs:
                 print("[build] " + " ".join(cmd))
         with ThreadPoolExecutor(max_workers=max_jobs(len(jobs))) as pool:
             list(pool.map(lambda job: _run(job[0]), jobs))
         objs = [os.path.join(tmp, os.path.basename(src) + ".o") for src in KERNEL_SOURCES]
-        for out, these in ((LIB_PATH, objs), (TIMELINE_LIB_PATH, [tl_objs.get(src, o) for src, o in zip(KERNEL_SOURCES, objs)])):
+        for out, these in ((LIB_PATH, objs), (TIMELINE_LIB_PATH, [tl_objs.get(src, o) for src, o in zip(KERNEL_SOURCES, objs)] + tl_extra)):
             link = [HIPCC, "--offload-arch=gfx950", "-fPIC", "-shared"] + these + ["-o", out]
             if verbose:
                 print("[build] " + " ".join(link))

@@ -15,8 +15,8 @@
 //                      registers.
 //   O^T += V^T * P^T   A operand = V^T fragment, read from the row-major V tile in LDS with the transposing
 //                      ds_read_b64_tr_b16 in that same key order.
-// K and V tiles (64 keys x 128 d) are copied global -> LDS with 16-byte direct-to-LDS copies, double buffered,
-// 16-byte chunks XOR-swizzled so that both the b128 reads (K) and the transposing reads (V) are conflict free.
+// K and V tiles (64 keys x 128 d) are copied global -> LDS with 16-byte direct-to-LDS copies into a ring of four slots
+// per operand, 16-byte chunks XOR-swizzled so that both the b128 reads (K) and the transposing reads (V) are conflict free.
 #include <type_traits>
 #include "mi355_common.h"
 #include "mi355_serving_internal.h"
@@ -78,19 +78,16 @@ __device__ __forceinline__ void fmha_decode_block(int bid, int q_tiles, int grou
 }
 
 // ---------------------------------------------------------------------------------------------------------
-// Ping-pong kernel: 8 waves x 32 queries per workgroup, two waves per SIMD that alternate roles. A wave alternates between
+// Ping-pong kernel: 8 waves x 16 QB queries per workgroup, two waves per SIMD that alternate roles. A wave alternates between
 //     a matrix phase : S(j+1) = K(j+1) Q^T and O += V(j)^T P(j)      (matrix pipe + LDS reads)
-//     a softmax phase: S(j+1) -> P(j+1)                               (VALU only)
+//     a softmax phase: S(j+1) -> P(j+1)                               (VALU; the tile copies ride along)
 // separated by workgroup barriers. Waves 4..7 run one phase behind waves 0..3, so on every SIMD one wave is in its matrix
 // phase while the other is in its softmax phase: the matrix pipe and the VALU are busy at the same time without relying on
 // the instruction scheduler to interleave them inside one wave. The phases of the workgroup are numbered P0, P1, ...; waves
-// 0..3 run the matrix phase in the even ones, waves 4..7 in the odd ones. K and V have separate double buffers: tile j lives
-// in Kbuf[j&1] / Vbuf[j&1], is copied by all 8 waves in an even phase (K(i+1) and V(i) at P(2i)) and has two phases to land
-// (waited for at the end of P(2i+1)).
+// 0..3 run the matrix phase in the even ones, waves 4..7 in the odd ones.
 //
 // Every product is made of MFMA 16x16x32 blocks: under the board's power limit that instruction sustains a ~14 % higher
-// rate than 32x32x16 on random data (it also takes more VALU issue slots away from the partner wave's softmax, which is why
-// the softmax below is cut down to the fewest instructions). Per wave and key tile (64 keys):
+// rate than 32x32x16 on random data. Per wave and key tile (64 keys), QB = 2:
 //   S^T[kb][qb] (16 keys x 16 queries) = K[kb] Q[qb]^T      4 key blocks x 2 query blocks x 4 steps of 32 d = 32 MFMAs
 //   O^T[db][qb] (16 d x 16 queries)   += V[j]^T[db] P[j][qb]^T   8 d blocks x 2 query blocks x 2 steps of 32 keys = 32 MFMAs
 //   l[qb]                             += 1 P[j][qb]^T            the softmax row sums, as a ninth all-ones "d block"  = 4 MFMAs
@@ -99,14 +96,43 @@ __device__ __forceinline__ void fmha_decode_block(int bid, int q_tiles, int grou
 // lie, i.e. contraction index 8 g + i of step j stands for key 32 j + 4 g + i (i < 4) or 32 j + 16 + 4 g + (i - 4); the
 // V^T fragment is gathered in that same order by two transposing LDS reads (key rows 32 j + 4 g .. and 32 j + 16 + 4 g ..),
 // so P never leaves the registers. The softmax statistics of a query live in the 4 lanes c, c + 16, c + 32, c + 48; they
-// only talk to each other when the running reference has to move (see the lazy rescaling below), which after the first
-// tile is rare: the common path has no cross-lane operation at all.
-// ---------------------------------------------------------------------------------------------------------
+// only talk to each other when the running reference has to move (lazy rescaling, below), which after the first tile is
+// rare: the common path has no cross-lane operation at all.
+//
+// A wave issues about one instruction per 5 cycles when it has its SIMD to itself and one per 10-12 next to the partner
+// wave's MFMAs, whatever the instruction is (scalar bookkeeping included): the phases are bound by their instruction
+// COUNT, and the loop is built to need few:
+//   * The K / V tiles live in a ring of NBUF = 4 slots per operand and the main loop is unrolled four times, so every LDS
+//     address of a fragment read is a loop-invariant register plus an immediate offset (no address arithmetic in the
+//     matrix phase), and the LDS destination of a copy is an immediate added into M0.
+//   * A tile pair {K(q), V(q-1)} (read in the phases P(2q) and P(2q+1)) is copied by every wave during its softmax phase
+//     three tile steps earlier, one copy instruction between two blocks of VALU work (issued together right behind a
+//     barrier, the 32 copy instructions of a pair queue up in the CU's memory pipeline and hold every wave at its issue for
+//     ~450 cycles). In the unrolled loop all 64 rows of the tile exist, so a copy is three instructions (M0, wait state,
+//     load: the tile base is a scalar pointer that advances once per tile, the lane offset a loop-invariant register); the
+//     last few tiles of a workgroup run a general loop whose copies clamp the tile index and the row.
+//   * The pair is published (s_waitcnt vmcnt + barrier) at the end of P(2q-2), a whole phase before its first use, so a
+//     wave reads the first fragments of its next matrix phase at the end of its softmax phase, in front of the barrier, and
+//     the matrix pipe starts on operands that are already in registers.
+//   * The softmax keeps, per query, the threshold that makes the exponent reference move and the negated scaled reference
+//     as state (recomputed only when the reference moves): the common path is max tree, one compare, fma, exp2, pack.
 // QB = query blocks of 16 per wave: 2 (256 queries per workgroup) or 1 (128 queries, for shapes with too few 256-query
-// workgroups to fill the machine and for short sequences; every K / V fragment then feeds one MFMA instead of two, and
-// the kernel is held to 128 registers so that two workgroups share a CU).
+// workgroups to fill the machine and for short sequences; every K / V fragment then feeds one MFMA instead of two).
+// ---------------------------------------------------------------------------------------------------------
+// 16-byte global -> LDS copy whose LDS address is a scalar register plus a compile-time constant (added straight into M0)
+template <int IMM>
+__device__ __forceinline__ void copy16_global_to_lds_at(const void* uniform_base, uint32_t lane_byte_offset, uint32_t lds_wave_base) {
+    asm volatile(
+        "s_add_u32 m0, %2, %3\n\t"
+        "s_nop 0\n\t"
+        "global_load_lds_dwordx4 %0, %1"
+        :
+        : "v"(lane_byte_offset), "s"(uniform_base), "s"(lds_wave_base), "n"(IMM)
+        : "memory", "m0", "scc");
+}
+
 template <typename T, int QB>
-__global__ __launch_bounds__(512, (QB == 1 ? 4 : 2)) void fmha_fwd_pingpong_kernel(const T* __restrict__ Q, const T* __restrict__ K,
+__global__ __launch_bounds__(512, 2) void fmha_fwd_pingpong_kernel(const T* __restrict__ Q, const T* __restrict__ K,
                                                                const T* __restrict__ V, T* __restrict__ O,
                                                                float* __restrict__ LSE, int B, int Hq, int Hkv, int Sq,
                                                                int Sk, float scale_log2, int causal, int kv_valid,
@@ -115,15 +141,15 @@ __global__ __launch_bounds__(512, (QB == 1 ? 4 : 2)) void fmha_fwd_pingpong_kern
     using V8 = typename Elem<T>::v8;
     using V4 = typename Elem<T>::v4;
     constexpr int NWAVES = 8;
+    constexpr int NBUF = 4;
     constexpr int WQ = 16 * QB;          // queries per wave
     constexpr int BM = NWAVES * WQ;
-    constexpr int COPIES = (BN * ROW_BYTES / 1024) / NWAVES;  // 2 wave-instructions per tile per wave
+    constexpr int VBUF0 = NBUF * TILE_BYTES;   // LDS: NBUF K slots, then NBUF V slots; slot q % NBUF holds K(q) and V(q - 1)
+    static_assert(BN * ROW_BYTES / 1024 / NWAVES == 2, "the softmax phase carries four copy slots: two of K, two of V");
 
     MI355_TL(unsigned long long tl_w[4] = {timeline::wall_clock(), 0, 0, 0}; unsigned long long tl_c[2] = {0, 0};)
     extern __shared__ __attribute__((aligned(1024))) char smem_raw[];
     MI355_LDS char* smem = (MI355_LDS char*)smem_raw;
-    MI355_LDS char* kbuf = smem;                   // 2 x TILE_BYTES
-    MI355_LDS char* vbuf = smem + 2 * TILE_BYTES;  // 2 x TILE_BYTES
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -148,8 +174,8 @@ __global__ __launch_bounds__(512, (QB == 1 ? 4 : 2)) void fmha_fwd_pingpong_kern
     int k_end = kv_valid;
     if (causal) k_end = min(k_end, min(q_block0 + BM, Sq) - 1 + shift + 1);
     const int n_tiles = (k_end + BN - 1) / BN;  // may be <= 0: no visible key for the whole workgroup
+    const int n_full = min(n_tiles, kv_valid / BN);   // tiles 0 .. n_full-1 have all 64 rows
 
-    // Q fragments (B operand of the first product): lane holds Q[16 qb + c][32 ks + 8 g .. +7]
     V8 qf[QB][4];
 #pragma unroll
     for (int qb = 0; qb < QB; ++qb) {
@@ -159,48 +185,58 @@ __global__ __launch_bounds__(512, (QB == 1 ? 4 : 2)) void fmha_fwd_pingpong_kern
         for (int ks = 0; ks < 4; ++ks) qf[qb][ks] = *(const V8*)(qp + ks * 32);
     }
 
-    // copy i of this wave covers tile rows 32 i + 4 wave + lane/16, 16-byte chunk position lane%16 (the swizzles depend on
-    // row % 16 only, so both copies of a lane share their column offsets); rows past the last valid key are clamped onto
-    // it (masked later, but V must not feed NaNs into 0 * V)
+    // copy i of this wave covers tile rows 32 i + 4 wave + lane/16, 16-byte chunk position lane%16
     const int copy_row0 = wave * 4 + (lane >> 4);
     const uint32_t copy_kcol = ((lane & 15) ^ swz_k(copy_row0)) * 16;
     const uint32_t copy_vcol = ((lane & 15) ^ swz_v16(copy_row0)) * 16;
     const uint32_t k_row_bytes = (uint32_t)sd.k_row * 2, v_row_bytes = (uint32_t)sd.v_row * 2;
-    auto issue_k = [&](int tile) {
-        const char* base = (const char*)Kh + (long)tile * BN * sd.k_row * 2;
+    const long k_tile_bytes = (long)BN * sd.k_row * 2, v_tile_bytes = (long)BN * sd.v_row * 2;
+    const int last_tile = n_tiles - 1;
+    const uint32_t lds_wave = (uint32_t)(uintptr_t)smem + (uint32_t)wave * 1024u;
+    // general copies: the tile index is clamped to the last tile (past the end a copy re-reads that tile into a slot nobody
+    // reads any more) and rows past the last valid key onto it (masked later, but V must not feed NaNs into 0 * V)
+    auto issue_k1 = [&](int q, int i) {   // half i of K(q) into slot q % NBUF
+        const int tile = min(q, last_tile);
         const int last = kv_valid - 1 - tile * BN;
-#pragma unroll
-        for (int i = 0; i < COPIES; ++i)
-            copy16_global_to_lds(base, (uint32_t)min(copy_row0 + 32 * i, last) * k_row_bytes + copy_kcol,
-                                 kbuf + (tile & 1) * TILE_BYTES + (i * NWAVES + wave) * 1024);
+        copy16_global_to_lds((const char*)Kh + tile * k_tile_bytes, (uint32_t)min(copy_row0 + 32 * i, last) * k_row_bytes + copy_kcol,
+                             smem + (q & (NBUF - 1)) * TILE_BYTES + (i * NWAVES + wave) * 1024);
     };
-    auto issue_v = [&](int tile) {
-        const char* base = (const char*)Vh + (long)tile * BN * sd.v_row * 2;
+    auto issue_v1 = [&](int q, int i) {   // half i of V(q - 1) into slot q % NBUF
+        const int tile = max(min(q - 1, last_tile), 0);
         const int last = kv_valid - 1 - tile * BN;
-#pragma unroll
-        for (int i = 0; i < COPIES; ++i)
-            copy16_global_to_lds(base, (uint32_t)min(copy_row0 + 32 * i, last) * v_row_bytes + copy_vcol,
-                                 vbuf + (tile & 1) * TILE_BYTES + (i * NWAVES + wave) * 1024);
+        copy16_global_to_lds((const char*)Vh + tile * v_tile_bytes, (uint32_t)min(copy_row0 + 32 * i, last) * v_row_bytes + copy_vcol,
+                             smem + VBUF0 + (q & (NBUF - 1)) * TILE_BYTES + (i * NWAVES + wave) * 1024);
     };
+    // copies of the unrolled loop: tile base pointers of K(j + 3) and V(j + 2), advanced once per tile step
+    uint32_t k_lane_off[2], v_lane_off[2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        k_lane_off[i] = (uint32_t)(copy_row0 + 32 * i) * k_row_bytes + copy_kcol;
+        v_lane_off[i] = (uint32_t)(copy_row0 + 32 * i) * v_row_bytes + copy_vcol;
+    }
+    const char* k_next = (const char*)Kh + 3 * k_tile_bytes;
+    const char* v_next = (const char*)Vh + 2 * v_tile_bytes;
 
-    // K fragment (key block kb, d step ks): row 16 kb + c, chunk (4 ks + g) ^ (row & 15)
-    const int k_base = c16 * ROW_BYTES + ((g ^ c16) << 4);                 // xor (ks << 6), + kb * 16 * ROW_BYTES
-    // V^T fragment (key step j, d block db), transposing read t: input lane c of a 16-lane group supplies 4 d of key row
-    // 32 j + 16 t + 4 g + c / 4: d 16 db + 4 (c % 4) .. +3
-    const int v_row = 4 * g + (c16 >> 2);
-    const int v_base = v_row * ROW_BYTES + (((((c16 & 3) >> 1)) ^ swz_v16(v_row)) << 4) + (c16 & 1) * 8;   // xor (db << 5)
+    // fragment addresses: loop-invariant registers, the slot and the block inside the tile are immediate offsets
+    //   K fragment (key block kb, d step ks): row 16 kb + c, chunk (4 ks + g) ^ (row & 15)
+    //   V^T fragment (key step j, d block db), transposing read t: key row 32 j + 16 t + 4 g + c / 4, d 16 db + 4 (c % 4) .. +3
+    MI355_LDS char* k_ptr[4];
+    MI355_LDS char* v_ptr[8];
+    {
+        const int k_base = c16 * ROW_BYTES + ((g ^ c16) << 4);
+        const int v_row = 4 * g + (c16 >> 2);
+        const int v_base = v_row * ROW_BYTES + (((((c16 & 3) >> 1)) ^ swz_v16(v_row)) << 4) + (c16 & 1) * 8;
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) k_ptr[ks] = smem + (k_base ^ (ks << 6));
+#pragma unroll
+        for (int db = 0; db < 8; ++db) v_ptr[db] = smem + VBUF0 + (v_base ^ (db << 5));
+    }
 
     float4v o[8][QB];
 #pragma unroll
     for (int db = 0; db < 8; ++db)
 #pragma unroll
         for (int qb = 0; qb < QB; ++qb) o[db][qb] = float4v{0.f, 0.f, 0.f, 0.f};
-    // Row sums of P ride on the matrix pipe: a ninth "d block" whose V^T rows are all ones, l[qb] += 1 P[j][qb]^T. Every
-    // row of that block (so all four elements of a lane) ends up holding the sum over all keys of the lane's query,
-    // accumulated from the same fp16-rounded P the output uses; no VALU additions and no cross-lane sum are needed.
-    // The rounding of P enters l with a relative error of at most 2^-12 for fp16, far inside the 1e-3 allowed on the
-    // log-sum-exp; for bfloat16 (2^-9) it would not be, so that type sums the unrounded fp32 values on the VALU instead
-    // (element 0 of l_acc then holds this lane's partial sum; the four lanes of a query are added at the end).
     constexpr bool kSumOnMatrixPipe = std::is_same<T, half_t>::value;
     float4v l_acc[QB];
 #pragma unroll
@@ -208,12 +244,16 @@ __global__ __launch_bounds__(512, (QB == 1 ? 4 : 2)) void fmha_fwd_pingpong_kern
     V8 ones;
 #pragma unroll
     for (int e = 0; e < 8; ++e) ones[e] = (T)1.0f;
-    float m_run[QB];
+    // per query: exponent reference of the running sums, the score above which it has to move, and -reference * scale
+    float m_run[QB], m_thr[QB], neg_ms[QB];
+    const float lazy_margin = kLazyLog2 / scale_log2;
 #pragma unroll
-    for (int qb = 0; qb < QB; ++qb) m_run[qb] = -INFINITY;
+    for (int qb = 0; qb < QB; ++qb) {
+        m_run[qb] = -INFINITY;
+        m_thr[qb] = -INFINITY;
+        neg_ms[qb] = 0.f;
+    }
 
-    // empty asm statements that make a value "used" at a program point: they keep the softmax in its phase and the MFMAs
-    // in theirs (the compiler is otherwise free to move register-only work across s_barrier)
     auto pin_s = [](float4v(&s)[4][QB]) {
         if constexpr (QB == 2)
             asm volatile("" : "+v"(s[0][0]), "+v"(s[0][1]), "+v"(s[1][0]), "+v"(s[1][1]), "+v"(s[2][0]), "+v"(s[2][1]), "+v"(s[3][0]), "+v"(s[3][1]));
@@ -237,50 +277,40 @@ __global__ __launch_bounds__(512, (QB == 1 ? 4 : 2)) void fmha_fwd_pingpong_kern
         }
     };
 
-    int phase = 0;  // index of the workgroup phase this wave is in
-    bool copies_due = false;
-    auto next_phase = [&]() {
-        if (phase & 1) wait_vmcnt<0>();  // copies issued at the start of the previous (even) phase have landed
-        __syncthreads();
-        ++phase;
-        if (!(phase & 1)) {
-            if (!late) { copies_due = true; return; }   // a wave entering its matrix phase issues them behind its first reads
-            const int i = phase >> 1;
-            if (i + 1 < n_tiles) issue_k(i + 1);
-            if (i < n_tiles) issue_v(i);
-        }
-    };
-    auto due_copies = [&]() {
-        if (copies_due) {
-            copies_due = false;
-            const int i = phase >> 1;
-            if (i + 1 < n_tiles) issue_k(i + 1);
-            if (i < n_tiles) issue_v(i);
-        }
-    };
+    // s_barrier as inline assembly: in front of a barrier it recognises the compiler waits for every LDS read it knows of,
+    // and the fragments read ahead for the next matrix phase are meant to stay in flight across this one. Nothing else
+    // crosses: the reads of a matrix phase have been consumed by its MFMAs, the copies are waited for explicitly.
+    auto phase_barrier = []() { asm volatile("s_barrier" ::: "memory"); };
+    // At the end of an even phase the pair of the step after next must have landed (all but this wave's four newest
+    // copies), so that the barrier publishes it a whole phase ahead of its first reader. Waves 0..3 end matrix phases
+    // there, waves 4..7 softmax phases.
+    auto end_even_phase = [&]() { wait_vmcnt<4>(); phase_barrier(); };
+    auto end_odd_phase = [&]() { phase_barrier(); };
+    auto end_m = [&]() { if (late) end_odd_phase(); else end_even_phase(); };
+    auto end_s = [&]() { if (late) end_even_phase(); else end_odd_phase(); };
 
-    // Fragment f of a matrix phase, in the order the MFMAs consume them: f < 16 is the K fragment (ks = f / 4, kb = f % 4),
-    // f >= 16 the V^T fragment (j = (f - 16) / 8, db = (f - 16) % 8). Each fragment feeds two MFMAs (the two query blocks).
-    auto read_frag = [&](MI355_LDS char* kst, MI355_LDS char* vst, int f) -> V8 {
+    constexpr int AHEAD = QB == 1 ? 5 : 6;   // fragments in flight ahead of their MFMAs
+    // fragment f of the matrix phase on the pair in ring slot `slot`: f < 16 K (ks = f / 4, kb = f % 4), f >= 16 V^T
+    // (j = (f - 16) / 8, db = (f - 16) % 8); SLOT >= 0: compile-time slot, the whole offset is an immediate
+    auto read_frag = [&](auto slot_c, int slot, int f) -> V8 {
+        constexpr int SLOT = decltype(slot_c)::value;
+        const int so = (SLOT >= 0 ? SLOT : slot) * TILE_BYTES;
         if (f < 16) {
             const int ks = f >> 2, kb = f & 3;
-            return Elem<T>::frag(lds_read_b128(kst + ((k_base ^ (ks << 6)) + kb * 16 * ROW_BYTES)));
+            return Elem<T>::frag(lds_read_b128(k_ptr[ks] + (so + kb * 16 * ROW_BYTES)));
         }
         const int j = (f - 16) >> 3, db = (f - 16) & 7;
-        const int off = (v_base ^ (db << 5)) + (32 * j) * ROW_BYTES;
-        return Elem<T>::frag(concat(lds_read_tr16_b64(vst + off), lds_read_tr16_b64(vst + off + 16 * ROW_BYTES)));
+        MI355_LDS char* p = v_ptr[db] + (so + (32 * j) * ROW_BYTES);
+        return Elem<T>::frag(concat(lds_read_tr16_b64(p), lds_read_tr16_b64(p + 16 * ROW_BYTES)));
     };
-    // The matrix phase over fragments [F0, F1): every fragment is read AHEAD fragments (12 MFMAs, 192 cycles) ahead of its
-    // MFMAs, into the register its predecessor has just released; sched_barrier pins that order.
-    auto mfma_phase = [&](auto f0c, auto f1c, int tile_k, float4v(&s)[4][QB], int tile_v, const V8(&pf)[2][QB]) {
-        constexpr int F0 = decltype(f0c)::value, F1 = decltype(f1c)::value;
-        MI355_LDS char* kst = kbuf + (tile_k & 1) * TILE_BYTES;
-        MI355_LDS char* vst = vbuf + (tile_v & 1) * TILE_BYTES;
-        constexpr int AHEAD = QB == 1 ? 5 : 6;
-        V8 fr[AHEAD];
+    auto preload = [&](auto f0c, auto slot_c, int slot, V8(&fr)[AHEAD]) {
+        constexpr int F0 = decltype(f0c)::value;
 #pragma unroll
-        for (int i = 0; i < AHEAD; ++i) fr[i] = read_frag(kst, vst, F0 + i);
-        due_copies();
+        for (int i = 0; i < AHEAD; ++i) fr[i] = read_frag(slot_c, slot, F0 + i);
+    };
+    // matrix phase over fragments [F0, F1): S = K Q^T (f < 16) and O += V^T P (f >= 16); fr holds the first AHEAD fragments
+    auto mfma_phase = [&](auto f0c, auto f1c, auto slot_c, int slot, float4v(&s)[4][QB], const V8(&pf)[2][QB], V8(&fr)[AHEAD]) {
+        constexpr int F0 = decltype(f0c)::value, F1 = decltype(f1c)::value;
         if constexpr (F0 == 0) {
 #pragma unroll
             for (int kb = 0; kb < 4; ++kb)
@@ -299,22 +329,37 @@ __global__ __launch_bounds__(512, (QB == 1 ? 4 : 2)) void fmha_fwd_pingpong_kern
                 const int j = (f - 16) >> 3, db = (f - 16) & 7;
 #pragma unroll
                 for (int qb = 0; qb < QB; ++qb) o[db][qb] = Elem<T>::mfma16(fr[r], pf[j][qb], o[db][qb]);
-                if (kSumOnMatrixPipe && db == 3) {   // the row sums of this key step, in the middle of its eight d blocks
+                if (kSumOnMatrixPipe && db == 3) {
 #pragma unroll
                     for (int qb = 0; qb < QB; ++qb) l_acc[qb] = Elem<T>::mfma16(ones, pf[j][qb], l_acc[qb]);
                 }
             }
-            if (f + AHEAD < F1) fr[r] = read_frag(kst, vst, f + AHEAD);
+            if (f + AHEAD < F1) fr[r] = read_frag(slot_c, slot, f + AHEAD);
         }
         __builtin_amdgcn_sched_barrier(0);
     };
     using I0 = std::integral_constant<int, 0>;
     using I16 = std::integral_constant<int, 16>;
     using I32 = std::integral_constant<int, 32>;
+    using Dyn = std::integral_constant<int, -1>;
 
-    auto softmax_tile = [&](float4v(&s)[4][QB], int tile, V8(&pf)[2][QB]) {
+    // softmax of tile `tile`. CSLOT >= 0: the four copies of the pair in ring slot CSLOT ride along, full tiles from the
+    // running pointers; CSLOT == -1: general copies of pair cq; CSLOT == -2: none.
+    auto softmax_tile = [&](float4v(&s)[4][QB], int tile, V8(&pf)[2][QB], auto cslot_c, int cq) {
+        constexpr int CSLOT = decltype(cslot_c)::value;
+        auto copy = [&](auto which_c) {
+            constexpr int W = decltype(which_c)::value;   // 0, 1: halves of K; 2, 3: halves of V
+            if constexpr (CSLOT >= 0) {
+                if constexpr (W < 2) copy16_global_to_lds_at<CSLOT * TILE_BYTES + W * NWAVES * 1024>(k_next, k_lane_off[W], lds_wave);
+                else copy16_global_to_lds_at<VBUF0 + CSLOT * TILE_BYTES + (W - 2) * NWAVES * 1024>(v_next, v_lane_off[W - 2], lds_wave);
+            } else if constexpr (CSLOT == -1) {
+                if constexpr (W < 2) issue_k1(cq, W);
+                else issue_v1(cq, W - 2);
+            }
+        };
         const int key0 = tile * BN;
         const bool need_mask = (key0 + BN > kv_valid) || (causal && (key0 + BN - 1 > q_wave0 + shift));
+        copy(std::integral_constant<int, 0>{});
         if (need_mask) {
 #pragma unroll
             for (int qb = 0; qb < QB; ++qb) {
@@ -328,10 +373,9 @@ __global__ __launch_bounds__(512, (QB == 1 ? 4 : 2)) void fmha_fwd_pingpong_kern
             }
         }
         // Lazy rescaling: m_run is the exponent reference of the running sums of a query (identical in its four lanes), not
-        // necessarily its running maximum. A lane only asks for it to move when one of ITS scores exceeds it by more than
-        // 2^kLazyLog2; then (any lane of the wave asked) the four lanes of every query agree on the tile's maximum and the
-        // reference is raised to the running maximum. Otherwise P = exp2((S - m_run) c) <= 2^kLazyLog2 everywhere and nothing
-        // crosses lanes.
+        // necessarily its running maximum. A lane asks for it to move when one of ITS scores exceeds m_thr = m_run +
+        // 2^kLazyLog2 / scale; then (any lane of the wave asked) the four lanes of every query agree on the tile's maximum
+        // and the reference is raised to the running maximum. Otherwise P = exp2((S - m_run) c) <= 2^kLazyLog2 everywhere.
         float mx[QB];
         bool raise = false;
 #pragma unroll
@@ -345,7 +389,7 @@ __global__ __launch_bounds__(512, (QB == 1 ? 4 : 2)) void fmha_fwd_pingpong_kern
             a = max3(a, s[3][qb][2], s[3][qb][3]);
             a = max3(a, c, c);
             mx[qb] = a;
-            raise = raise || ((a - m_run[qb]) * scale_log2 > kLazyLog2);  // -inf - -inf = NaN compares false
+            raise = raise || (a > m_thr[qb]);
         }
         if (__builtin_amdgcn_ballot_w64(raise) != 0) {
 #pragma unroll
@@ -354,31 +398,39 @@ __global__ __launch_bounds__(512, (QB == 1 ? 4 : 2)) void fmha_fwd_pingpong_kern
                 const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
                 const float alpha = fast_exp2((m_run[qb] - m_use) * scale_log2);
                 m_run[qb] = m_new;
+                m_thr[qb] = m_new + lazy_margin;
+                neg_ms[qb] = -m_use * scale_log2;
+                // in place, as assembly: left to itself the compiler writes the products to other registers, and the common
+                // path (no rescale) then pays for 72 register moves to meet it at the join
+                l_acc[qb] *= alpha;
 #pragma unroll
-                for (int e = 0; e < 4; ++e) l_acc[qb][e] *= alpha;
-#pragma unroll
-                for (int db = 0; db < 8; ++db)
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) o[db][qb][e] *= alpha;
+                for (int db = 0; db < 8; ++db) o[db][qb] *= alpha;
             }
         }
-        // the wave is the only one of its SIMD issuing VALU work in this phase, so dependent instructions are kept apart:
-        // all multiply-adds, then all exponentials, then the sums and conversions
+        __builtin_amdgcn_sched_barrier(0);
+        copy(std::integral_constant<int, 1>{});
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int qb = 0; qb < QB; ++qb) {
-            const float neg_ms = (m_run[qb] == -INFINITY) ? 0.f : -m_run[qb] * scale_log2;
+        for (int qb = 0; qb < QB; ++qb)
 #pragma unroll
             for (int kb = 0; kb < 4; ++kb)
 #pragma unroll
-                for (int e = 0; e < 4; ++e) s[kb][qb][e] = __builtin_fmaf(s[kb][qb][e], scale_log2, neg_ms);
-        }
+                for (int e = 0; e < 4; ++e) s[kb][qb][e] = __builtin_fmaf(s[kb][qb][e], scale_log2, neg_ms[qb]);
+        __builtin_amdgcn_sched_barrier(0);
+        copy(std::integral_constant<int, 2>{});
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int kb = 0; kb < 4; ++kb)
+        for (int kb = 0; kb < 4; ++kb) {
 #pragma unroll
             for (int qb = 0; qb < QB; ++qb)
 #pragma unroll
                 for (int e = 0; e < 4; ++e) s[kb][qb][e] = fast_exp2(s[kb][qb][e]);
+            if (kb == 1) {
+                __builtin_amdgcn_sched_barrier(0);
+                copy(std::integral_constant<int, 3>{});
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int qb = 0; qb < QB; ++qb) {
@@ -396,46 +448,70 @@ __global__ __launch_bounds__(512, (QB == 1 ? 4 : 2)) void fmha_fwd_pingpong_kern
             }
             if (!kSumOnMatrixPipe) l_acc[qb][0] += (ps[0] + ps[1]) + (ps[2] + ps[3]);
         }
+        if constexpr (CSLOT >= 0) {
+            k_next += k_tile_bytes;
+            v_next += v_tile_bytes;
+        }
     };
 
     if (n_tiles > 0) {
-        // before P0: K(0) must be in LDS
-        issue_k(0);
-        wait_vmcnt<0>();
+        // pairs 0 and 1 (K(0), K(1), V(0)) must be in LDS before P0; pair 2 is on its way
+        issue_k1(0, 0); issue_k1(0, 1);
+        issue_k1(1, 0); issue_k1(1, 1);
+        issue_v1(1, 0); issue_v1(1, 1);
+        issue_k1(2, 0); issue_k1(2, 1);
+        issue_v1(2, 0); issue_v1(2, 1);
+        wait_vmcnt<4>();
         __syncthreads();
-        if (1 < n_tiles) issue_k(1);  // start of P0
-        issue_v(0);
-        if (late) next_phase();  // waves 4..7 idle during P0
+        if (late) end_even_phase();   // waves 4..7 idle during P0
 
         float4v s[4][QB];
         V8 pf[2][QB];
+        V8 fr[AHEAD];
         MI355_TL(tl_w[1] = timeline::wall_clock(); tl_c[0] = timeline::shader_cycles();)
+        preload(I0{}, std::integral_constant<int, 0>{}, 0, fr);
         __builtin_amdgcn_s_setprio(1);
-        mfma_phase(I0{}, I16{}, 0, s, 0, pf);               // S(0) alone
+        mfma_phase(I0{}, I16{}, std::integral_constant<int, 0>{}, 0, s, pf, fr);               // S(0) alone
         __builtin_amdgcn_s_setprio(0);
         pin_s(s);
-        next_phase();
-        for (int j = 0; j + 1 < n_tiles; ++j) {
-            softmax_tile(s, j, pf);
+        end_m();
+        // tile step j: softmax(j) (with the copies of pair j + 3), then S(j+1) and O += V(j)^T P(j) on pair j + 1
+        auto step = [&](auto u_c, int j) {
+            constexpr int U = decltype(u_c)::value;   // j % NBUF in the unrolled loop, -1 in the general one
+            using CopySlot = std::integral_constant<int, (U >= 0 ? (U + 3) % NBUF : -1)>;
+            using ReadSlot = std::integral_constant<int, (U >= 0 ? (U + 1) % NBUF : -1)>;
+            softmax_tile(s, j, pf, CopySlot{}, j + 3);
             pin_p(pf);
-            next_phase();
+            preload(I0{}, ReadSlot{}, (j + 1) & (NBUF - 1), fr);
+            end_s();
             __builtin_amdgcn_s_setprio(1);
-            mfma_phase(I0{}, I32{}, j + 1, s, j, pf);        // S(j+1) and O += V(j)^T P(j)
+            mfma_phase(I0{}, I32{}, ReadSlot{}, (j + 1) & (NBUF - 1), s, pf, fr);
             __builtin_amdgcn_s_setprio(0);
             pin_s(s);
             pin_o();
-            next_phase();
+            end_m();
+        };
+        // unrolled loop: while the pair copied in step j (tiles j + 3 and j + 2) is made of full tiles
+        const int j_fast = max(0, min(n_full - 3, n_tiles - 1)) & ~(NBUF - 1);
+        int j = 0;
+        for (; j < j_fast; j += NBUF) {
+            step(std::integral_constant<int, 0>{}, j);
+            step(std::integral_constant<int, 1>{}, j + 1);
+            step(std::integral_constant<int, 2>{}, j + 2);
+            step(std::integral_constant<int, 3>{}, j + 3);
         }
-        softmax_tile(s, n_tiles - 1, pf);
+        for (; j + 1 < n_tiles; ++j) step(Dyn{}, j);
+        softmax_tile(s, n_tiles - 1, pf, std::integral_constant<int, -2>{}, 0);
         pin_p(pf);
-        next_phase();
-        mfma_phase(I16{}, I32{}, 0, s, n_tiles - 1, pf);     // O += V(last)^T P(last) alone
-        next_phase();
-        if (!late) next_phase();  // waves 0..3 idle while waves 4..7 finish
+        preload(I16{}, Dyn{}, n_tiles & (NBUF - 1), fr);
+        end_s();
+        mfma_phase(I16{}, I32{}, Dyn{}, n_tiles & (NBUF - 1), s, pf, fr);     // O += V(last)^T P(last) alone
+        end_m();
+        if (!late) end_odd_phase();  // waves 0..3 idle while waves 4..7 finish
+        wait_vmcnt<0>();   // no copy may still be on its way into LDS when the workgroup gives the memory back
     }
     MI355_TL(tl_w[2] = timeline::wall_clock(); tl_c[1] = timeline::shader_cycles();)
 
-    // ---- finalize: O / l, LSE: lane holds O[query 16 qb + c][d = 16 db + 4 g + 0..3] -----------------------------
 #pragma unroll
     for (int qb = 0; qb < QB; ++qb) {
         const float l_tot = kSumOnMatrixPipe ? l_acc[qb][0] : quad_sum(l_acc[qb][0]);
@@ -468,10 +544,10 @@ __global__ __launch_bounds__(512, (QB == 1 ? 4 : 2)) void fmha_fwd_pingpong_kern
 
 template <typename T, int QB>
 static hipError_t launch_fmha_pingpong(const T* Q, const T* K, const T* V, T* O, float* LSE, int B, int Hq,
-                                       int Hkv, int Sq, int Sk, float scale, int causal, int kv_valid, const FmhaStrides& sd,
-                                       hipStream_t stream) {
+                                   int Hkv, int Sq, int Sk, float scale, int causal, int kv_valid, const FmhaStrides& sd,
+                                   hipStream_t stream) {
     constexpr int BM = 128 * QB;
-    constexpr int LDS = 4 * fmha::TILE_BYTES;
+    constexpr int LDS = 8 * fmha::TILE_BYTES;
     auto kern = fmha_fwd_pingpong_kernel<T, QB>;
     static DynamicLdsOnce lds_once;
     if (hipError_t e = lds_once.ensure(reinterpret_cast<const void*>(kern), LDS); e != hipSuccess) return e;
@@ -497,18 +573,16 @@ static hipError_t fmha_fwd_dispatch_t(const void* Q, const void* K, const void* 
     if (variant == 0 && fmha_decode_applicable(B, Hq, Hkv, Sq, Sk, kv_valid_len))
         return fmha_decode_dispatch<T>(q, k, v, o, LSE, B, Hq, Hkv, Sq, Sk, scale, causal, kv_valid_len, sd, ws, stream);
     if (variant == 0) {
-        // 256-query workgroups once there are clearly more of them than CUs (with exactly one per CU a causal problem runs
-        // as long as its heaviest tile; 128-query workgroups then balance better and still fill the machine) and the
-        // sequences are long enough to amortise their longer prologue. Measured (b, heads 32/8, s, 128- vs 256-query):
-        // 1 x 1024 causal 25 / 35 us, 1 x 2048 57 / 65, 8 x 512 43 / 50, 1 x 3000 108 / 94, 1 x 4096 182 / 144,
-        // 4 x 1024 (32 kv heads, non-causal) 100 / 82.
-        // A causal problem whose keys are its own queries computes every diagonal block in full: with 256-query workgroups
-        // that is 1 / (2 Sq / 256) more work than with 128-query ones, which outweighs their cheaper inner loop below
-        // ~1400 queries (many workgroups either way; 128- / 256-query: 16 x 768 127 / 136 us, 8 x 1024 101 / 108,
-        // 8 x 1280 142 / 146, 4 x 1536 101 / 99, 4 x 2048 169 / 153).
+        // 256-query workgroups (every K / V fragment feeds two MFMAs) once they fill the machine: clearly more of them than
+        // CUs for a causal problem (with about one per CU it runs as long as its heaviest tile, and 128-query workgroups
+        // balance better), one per CU otherwise; never for sequences of a tile or two. Measured (b x heads q/kv x s, 128-
+        // / 256-query workgroups, us): causal 1 x 32/8 x 1024 21 / 31, 1 x 32/8 x 2048 48 / 54, 2 x 32/8 x 1024 31 / 34,
+        // 1 x 16/16 x 4096 84 / 94, 1 x 8/8 x 8192 149 / 173, 32 x 32/8 x 256 71 / 74, but 8 x 32/8 x 512 46 / 45,
+        // 1 x 32/8 x 3000 99 / 83, 2 x 32/8 x 1536 62 / 53, 4 x 32/8 x 1024 62 / 59, 1 x 32/8 x 4096 160 / 134,
+        // 16 x 32/8 x 768 152 / 137, 4 x 32/8 x 2048 189 / 155; not causal 2 x 32/8 x 1024 47 / 38, 1 x 32/8 x 2048 81 / 65,
+        // 4 x 32/32 x 1024 93 / 75.
         const long wg256 = (long)((Sq + 255) / 256) * Hq * B;
-        const bool diagonal_heavy = causal && Sk < 2L * Sq;
-        variant = (wg256 >= 320 && Sq > (diagonal_heavy ? 1408 : 512)) ? 2 : 1;
+        variant = (Sq >= 512 && wg256 >= (causal ? 320 : 256)) ? 2 : 1;
     }
     if (variant == 2) return launch_fmha_pingpong<T, 2>(q, k, v, o, LSE, B, Hq, Hkv, Sq, Sk, scale, causal, kv_valid_len, sd, stream);
     return launch_fmha_pingpong<T, 1>(q, k, v, o, LSE, B, Hq, Hkv, Sq, Sk, scale, causal, kv_valid_len, sd, stream);

@@ -1100,30 +1100,4 @@ extern "C" int mi355_timeline_read_hgemm(void* dst, size_t bytes) {
     const size_t all = sizeof(unsigned long long) * mi355::timeline::kMaxWorkgroups * mi355::timeline::kSlots;
     return (int)hipMemcpyFromSymbol(dst, HIP_SYMBOL(mi355::hgemm_stamps), bytes < all ? bytes : all);
 }
-
-// profiling build: a kernel that only reads `bytes` (a multiple of 16) with 16-byte loads, eight in flight per thread, one
-// 256-thread workgroup per CU walking the buffer side by side -- what the memory system delivers to a kernel that does
-// nothing else, launch and tail included; the yardstick of the bandwidth-bound kernels.
-namespace mi355 {
-__global__ __launch_bounds__(256) void stream_read_kernel(const float4v* __restrict__ p, long n16, float* sink) {
-    float4v acc = {0.f, 0.f, 0.f, 0.f};
-    const long stride = (long)gridDim.x * blockDim.x;
-    long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
-    for (; i + 7 * stride < n16; i += 8 * stride) {
-        float4v v[8];
-#pragma unroll
-        for (int u = 0; u < 8; ++u) v[u] = __builtin_nontemporal_load(p + i + u * stride);
-#pragma unroll
-        for (int u = 0; u < 8; ++u) acc += v[u];
-    }
-    for (; i < n16; i += stride) acc += p[i];
-    if (acc[0] + acc[1] + acc[2] + acc[3] == 12345.678f) sink[0] = 1.f;   // keeps the loads alive; never true for the bench's data
-}
-}  // namespace mi355
-extern "C" int mi355_timeline_stream_read(const void* src, size_t bytes, void* sink, void* stream) {
-    if (src == nullptr || sink == nullptr || bytes % 16 != 0 || reinterpret_cast<uintptr_t>(src) % 16 != 0) return (int)hipErrorInvalidValue;
-    mi355::stream_read_kernel<<<dim3(256), dim3(256), 0, static_cast<hipStream_t>(stream)>>>(
-        static_cast<const mi355::float4v*>(src), (long)(bytes / 16), static_cast<float*>(sink));
-    return (int)hipGetLastError();
-}
 #endif
