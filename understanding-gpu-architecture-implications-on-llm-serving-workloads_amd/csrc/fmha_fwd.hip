@@ -56,6 +56,16 @@ __device__ __forceinline__ float max3(float a, float b, float c) {
     asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
     return r;
 }
+// Register (index into the AHEAD fragment registers) of the i-th fragment of a matrix phase when fragments are read in
+// order and consumed pairwise swapped (1, 0, 3, 2, ..): fragment i >= AHEAD goes where the fragment consumed just before its
+// read was, i.e. where fragment (i - AHEAD) ^ 1 lived.
+__device__ __forceinline__ constexpr int frag_reg(int i, int ahead) { return i < ahead ? i : frag_reg((i - ahead) ^ 1, ahead); }
+// the same, kept in program order relative to its like
+__device__ __forceinline__ float max3v(float a, float b, float c) {
+    float r;
+    asm volatile("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+    return r;
+}
 
 }  // namespace fmha
 
@@ -282,14 +292,11 @@ __global__ __launch_bounds__(512, 2) void fmha_fwd_pingpong_kernel(const T* __re
     // crosses: the reads of a matrix phase have been consumed by its MFMAs, the copies are waited for explicitly.
     auto phase_barrier = []() { asm volatile("s_barrier" ::: "memory"); };
     // At the end of an even phase the pair of the step after next must have landed (all but this wave's four newest
-    // copies), so that the barrier publishes it a whole phase ahead of its first reader. Waves 0..3 end matrix phases
-    // there, waves 4..7 softmax phases.
-    auto end_even_phase = [&]() { wait_vmcnt<4>(); phase_barrier(); };
-    auto end_odd_phase = [&]() { phase_barrier(); };
-    auto end_m = [&]() { if (late) end_odd_phase(); else end_even_phase(); };
-    auto end_s = [&]() { if (late) end_even_phase(); else end_odd_phase(); };
-
-    constexpr int AHEAD = QB == 1 ? 5 : 6;   // fragments in flight ahead of their MFMAs
+    // copies), so that the barrier publishes it a whole phase ahead of its first reader. The same wait at the end of an odd
+    // phase finds nothing to wait for (a wave's newest four copies are all that is outstanding there), so every phase ends
+    // the same way and no wave has to know which half of the workgroup it belongs to.
+    auto end_phase = [&]() { wait_vmcnt<4>(); phase_barrier(); };
+    constexpr int AHEAD = 6;   // fragments in flight ahead of their MFMAs
     // fragment f of the matrix phase on the pair in ring slot `slot`: f < 16 K (ks = f / 4, kb = f % 4), f >= 16 V^T
     // (j = (f - 16) / 8, db = (f - 16) % 8); SLOT >= 0: compile-time slot, the whole offset is an immediate
     auto read_frag = [&](auto slot_c, int slot, int f) -> V8 {
@@ -317,10 +324,11 @@ __global__ __launch_bounds__(512, 2) void fmha_fwd_pingpong_kernel(const T* __re
 #pragma unroll
                 for (int qb = 0; qb < QB; ++qb) s[kb][qb] = float4v{0.f, 0.f, 0.f, 0.f};
         }
-#pragma unroll
-        for (int f = F0; f < F1; ++f) {
-            __builtin_amdgcn_sched_barrier(0);
-            const int r = (f - F0) % AHEAD;
+        // Fragments are read in the order f = F0, F0 + 1, .. and consumed in pairs, the later-read one first: LDS reads complete
+        // in order, so the wait for it covers its predecessor and a pair costs one s_waitcnt instead of two. The register a
+        // fragment frees takes the next fragment in read order (frag_reg).
+        auto use = [&](int f) {
+            const int r = frag_reg(f - F0, AHEAD);
             if (f < 16) {
                 const int ks = f >> 2, kb = f & 3;
 #pragma unroll
@@ -334,7 +342,16 @@ __global__ __launch_bounds__(512, 2) void fmha_fwd_pingpong_kernel(const T* __re
                     for (int qb = 0; qb < QB; ++qb) l_acc[qb] = Elem<T>::mfma16(ones, pf[j][qb], l_acc[qb]);
                 }
             }
-            if (f + AHEAD < F1) fr[r] = read_frag(slot_c, slot, f + AHEAD);
+        };
+        static_assert((F1 - F0) % 2 == 0 && AHEAD % 2 == 0, "fragments come in pairs");
+#pragma unroll
+        for (int f = F0; f < F1; f += 2) {
+            __builtin_amdgcn_sched_barrier(0);
+            use(f + 1);
+            if (f + AHEAD < F1) fr[frag_reg(f + AHEAD - F0, AHEAD)] = read_frag(slot_c, slot, f + AHEAD);
+            __builtin_amdgcn_sched_barrier(0);
+            use(f);
+            if (f + 1 + AHEAD < F1) fr[frag_reg(f + 1 + AHEAD - F0, AHEAD)] = read_frag(slot_c, slot, f + 1 + AHEAD);
         }
         __builtin_amdgcn_sched_barrier(0);
     };
@@ -376,21 +393,28 @@ __global__ __launch_bounds__(512, 2) void fmha_fwd_pingpong_kernel(const T* __re
         // necessarily its running maximum. A lane asks for it to move when one of ITS scores exceeds m_thr = m_run +
         // 2^kLazyLog2 / scale; then (any lane of the wave asked) the four lanes of every query agree on the tile's maximum
         // and the reference is raised to the running maximum. Otherwise P = exp2((S - m_run) c) <= 2^kLazyLog2 everywhere.
-        float mx[QB];
+        // maximum of the 16 scores a lane holds of a query: two chains of v_max3 per query, the chains of both queries
+        // interleaved (written in the order they are to run: between an instruction of an assembly statement and a
+        // dependent one right behind it the compiler puts a wait state, an issue slot each)
+        float mx[QB], mc[QB];
+#pragma unroll
+        for (int qb = 0; qb < QB; ++qb) mx[qb] = max3v(s[0][qb][0], s[0][qb][1], s[0][qb][2]);
+#pragma unroll
+        for (int qb = 0; qb < QB; ++qb) mc[qb] = max3v(s[0][qb][3], s[1][qb][0], s[1][qb][1]);
+#pragma unroll
+        for (int kb = 1; kb < 4; ++kb) {
+#pragma unroll
+            for (int qb = 0; qb < QB; ++qb) mx[qb] = max3v(mx[qb], s[kb][qb][2], s[kb][qb][3]);
+            if (kb < 3) {
+#pragma unroll
+                for (int qb = 0; qb < QB; ++qb) mc[qb] = max3v(mc[qb], s[kb + 1][qb][0], s[kb + 1][qb][1]);
+            }
+        }
+#pragma unroll
+        for (int qb = 0; qb < QB; ++qb) mx[qb] = max3v(mx[qb], mc[qb], mc[qb]);
         bool raise = false;
 #pragma unroll
-        for (int qb = 0; qb < QB; ++qb) {
-            float a = max3(s[0][qb][0], s[0][qb][1], s[0][qb][2]);
-            float c = max3(s[0][qb][3], s[1][qb][0], s[1][qb][1]);
-            a = max3(a, s[1][qb][2], s[1][qb][3]);
-            c = max3(c, s[2][qb][0], s[2][qb][1]);
-            a = max3(a, s[2][qb][2], s[2][qb][3]);
-            c = max3(c, s[3][qb][0], s[3][qb][1]);
-            a = max3(a, s[3][qb][2], s[3][qb][3]);
-            a = max3(a, c, c);
-            mx[qb] = a;
-            raise = raise || (a > m_thr[qb]);
-        }
+        for (int qb = 0; qb < QB; ++qb) raise = raise || (mx[qb] > m_thr[qb]);
         if (__builtin_amdgcn_ballot_w64(raise) != 0) {
 #pragma unroll
             for (int qb = 0; qb < QB; ++qb) {
@@ -463,7 +487,7 @@ __global__ __launch_bounds__(512, 2) void fmha_fwd_pingpong_kernel(const T* __re
         issue_v1(2, 0); issue_v1(2, 1);
         wait_vmcnt<4>();
         __syncthreads();
-        if (late) end_even_phase();   // waves 4..7 idle during P0
+        if (late) end_phase();   // waves 4..7 idle during P0
 
         float4v s[4][QB];
         V8 pf[2][QB];
@@ -474,7 +498,7 @@ __global__ __launch_bounds__(512, 2) void fmha_fwd_pingpong_kernel(const T* __re
         mfma_phase(I0{}, I16{}, std::integral_constant<int, 0>{}, 0, s, pf, fr);               // S(0) alone
         __builtin_amdgcn_s_setprio(0);
         pin_s(s);
-        end_m();
+        end_phase();
         // tile step j: softmax(j) (with the copies of pair j + 3), then S(j+1) and O += V(j)^T P(j) on pair j + 1
         auto step = [&](auto u_c, int j) {
             constexpr int U = decltype(u_c)::value;   // j % NBUF in the unrolled loop, -1 in the general one
@@ -483,13 +507,13 @@ __global__ __launch_bounds__(512, 2) void fmha_fwd_pingpong_kernel(const T* __re
             softmax_tile(s, j, pf, CopySlot{}, j + 3);
             pin_p(pf);
             preload(I0{}, ReadSlot{}, (j + 1) & (NBUF - 1), fr);
-            end_s();
+            end_phase();
             __builtin_amdgcn_s_setprio(1);
             mfma_phase(I0{}, I32{}, ReadSlot{}, (j + 1) & (NBUF - 1), s, pf, fr);
             __builtin_amdgcn_s_setprio(0);
             pin_s(s);
             pin_o();
-            end_m();
+            end_phase();
         };
         // unrolled loop: while the pair copied in step j (tiles j + 3 and j + 2) is made of full tiles
         const int j_fast = max(0, min(n_full - 3, n_tiles - 1)) & ~(NBUF - 1);
@@ -504,10 +528,10 @@ __global__ __launch_bounds__(512, 2) void fmha_fwd_pingpong_kernel(const T* __re
         softmax_tile(s, n_tiles - 1, pf, std::integral_constant<int, -2>{}, 0);
         pin_p(pf);
         preload(I16{}, Dyn{}, n_tiles & (NBUF - 1), fr);
-        end_s();
+        end_phase();
         mfma_phase(I16{}, I32{}, Dyn{}, n_tiles & (NBUF - 1), s, pf, fr);     // O += V(last)^T P(last) alone
-        end_m();
-        if (!late) end_odd_phase();  // waves 0..3 idle while waves 4..7 finish
+        end_phase();
+        if (!late) end_phase();  // waves 0..3 idle while waves 4..7 finish
         wait_vmcnt<0>();   // no copy may still be on its way into LDS when the workgroup gives the memory back
     }
     MI355_TL(tl_w[2] = timeline::wall_clock(); tl_c[1] = timeline::shader_cycles();)
