@@ -69,22 +69,32 @@ __device__ __forceinline__ float max3v(float a, float b, float c) {
 
 }  // namespace fmha
 
-// Decode the linear workgroup id into (batch, q head, q tile). Workgroups with ids congruent mod 8 share an
-// XCD (and its L2): give each XCD whole (batch, kv head) groups so K/V are fetched from HBM once per XCD,
-// and inside a group hand out the q tiles with the most keys (causal) first.
-__device__ __forceinline__ void fmha_decode_block(int bid, int q_tiles, int group, int Hkv, int B, int& b, int& hq,
-                                                  int& q_tile) {
-    const int per_group = group * q_tiles;
-    const int total = per_group * Hkv * B;
-    int v = bid;
-    if (total % 8 == 0) v = (bid % 8) * (total / 8) + bid / 8;
-    int g = v / per_group;
-    int r = v - g * per_group;
-    int qt = r / group;
-    int hin = r - qt * group;
-    q_tile = q_tiles - 1 - qt;
-    b = g / Hkv;
-    hq = (g - b * Hkv) * group + hin;
+// Work item `round` of workgroup `wg` out of `n_wg`: a (batch, q head, q tile), or false when the workgroup has none left.
+// A launch has at most one workgroup per CU; each walks its own list of items (no global counter: nothing to reset, nothing
+// two launches could share). Workgroups with ids congruent mod 8 share an XCD (and its L2): when the (batch, kv head)
+// groups divide evenly every XCD gets whole groups, so K and V are fetched from HBM once. On an XCD the items are ranked
+// with the q tiles that see the most keys (causal) first and dealt out in rounds that run forwards and backwards in turn:
+// the workgroup that got the heaviest item of one round gets the lightest of the next.
+__device__ __forceinline__ bool fmha_work_item(int wg, int n_wg, int round, int q_tiles, int group, int Hkv, int B, int& b,
+                                               int& hq, int& q_tile) {
+    const int kv_groups = Hkv * B;
+    int x = 0, n_x = 1;
+    if (kv_groups % 8 == 0 && n_wg % 8 == 0) {
+        x = wg % 8;
+        n_x = 8;
+    }
+    const int wl = wg / n_x, wgs = n_wg / n_x;   // workgroup index on its XCD, workgroups per XCD
+    const int gpx = kv_groups / n_x;             // (batch, kv head) groups per XCD
+    const int per_rank = gpx * group;            // items of one q tile on this XCD
+    const int u = round * wgs + ((round & 1) ? wgs - 1 - wl : wl);
+    if (u >= per_rank * q_tiles) return false;
+    const int rank = u / per_rank, rem = u - rank * per_rank;
+    const int gl = rem / group, hin = rem - gl * group;
+    q_tile = q_tiles - 1 - rank;
+    const int kvg = x * gpx + gl;
+    b = kvg / Hkv;
+    hq = (kvg - b * Hkv) * group + hin;
+    return true;
 }
 
 // ---------------------------------------------------------------------------------------------------------
@@ -168,32 +178,43 @@ __global__ __launch_bounds__(512, 2) void fmha_fwd_pingpong_kernel(const T* __re
     const int g = lane >> 4;
     const int c16 = lane & 15;
 
-    int b, hq, q_tile;
+    // ---- the work item this workgroup is on (set_item) --------------------------------------------------------------
     const int group = Hq / Hkv;
-    fmha_decode_block(blockIdx.x, q_tiles, group, Hkv, B, b, hq, q_tile);
-    const int hkv = hq / group;
-    const int q_block0 = q_tile * BM;
-    const int q_wave0 = q_block0 + wave * WQ;
     const int shift = Sk - Sq;
+    int b = 0, hq = 0, q_wave0 = 0, n_tiles = 0, n_full = 0, last_tile = 0;
+    const T* Qh = Q;
+    const T* Kh = K;
+    const T* Vh = V;
+    T* Oh = O;
+    auto set_item = [&](int round) -> bool {
+        int q_tile;
+        if (!fmha_work_item(blockIdx.x, gridDim.x, round, q_tiles, group, Hkv, B, b, hq, q_tile)) return false;
+        const int hkv = hq / group;
+        const int q_block0 = q_tile * BM;
+        q_wave0 = q_block0 + wave * WQ;
+        Qh = Q + b * sd.q_batch + hq * sd.q_head;
+        Kh = K + b * sd.k_batch + hkv * sd.k_head;
+        Vh = V + b * sd.v_batch + hkv * sd.v_head;
+        Oh = O + b * sd.o_batch + hq * sd.o_head;
+        int k_end = kv_valid;
+        if (causal) k_end = min(k_end, min(q_block0 + BM, Sq) - 1 + shift + 1);
+        n_tiles = (k_end + BN - 1) / BN;            // may be <= 0: no visible key for the whole work item
+        n_full = min(n_tiles, kv_valid / BN);       // tiles 0 .. n_full-1 have all 64 rows
+        last_tile = n_tiles - 1;
+        return true;
+    };
 
-    const T* Qh = Q + b * sd.q_batch + hq * sd.q_head;
-    const T* Kh = K + b * sd.k_batch + hkv * sd.k_head;
-    const T* Vh = V + b * sd.v_batch + hkv * sd.v_head;
-    T* Oh = O + b * sd.o_batch + hq * sd.o_head;
-
-    int k_end = kv_valid;
-    if (causal) k_end = min(k_end, min(q_block0 + BM, Sq) - 1 + shift + 1);
-    const int n_tiles = (k_end + BN - 1) / BN;  // may be <= 0: no visible key for the whole workgroup
-    const int n_full = min(n_tiles, kv_valid / BN);   // tiles 0 .. n_full-1 have all 64 rows
-
+    // Q fragments (B operand of the first product): lane holds Q[16 qb + c][32 ks + 8 g .. +7]
     V8 qf[QB][4];
+    auto load_q = [&]() {
 #pragma unroll
-    for (int qb = 0; qb < QB; ++qb) {
-        const int qrow = min(q_wave0 + qb * 16 + c16, Sq - 1);
-        const T* qp = Qh + qrow * sd.q_row + 8 * g;
+        for (int qb = 0; qb < QB; ++qb) {
+            const int qrow = min(q_wave0 + qb * 16 + c16, Sq - 1);
+            const T* qp = Qh + qrow * sd.q_row + 8 * g;
 #pragma unroll
-        for (int ks = 0; ks < 4; ++ks) qf[qb][ks] = *(const V8*)(qp + ks * 32);
-    }
+            for (int ks = 0; ks < 4; ++ks) qf[qb][ks] = *(const V8*)(qp + ks * 32);
+        }
+    };
 
     // copy i of this wave covers tile rows 32 i + 4 wave + lane/16, 16-byte chunk position lane%16
     const int copy_row0 = wave * 4 + (lane >> 4);
@@ -201,7 +222,6 @@ __global__ __launch_bounds__(512, 2) void fmha_fwd_pingpong_kernel(const T* __re
     const uint32_t copy_vcol = ((lane & 15) ^ swz_v16(copy_row0)) * 16;
     const uint32_t k_row_bytes = (uint32_t)sd.k_row * 2, v_row_bytes = (uint32_t)sd.v_row * 2;
     const long k_tile_bytes = (long)BN * sd.k_row * 2, v_tile_bytes = (long)BN * sd.v_row * 2;
-    const int last_tile = n_tiles - 1;
     const uint32_t lds_wave = (uint32_t)(uintptr_t)smem + (uint32_t)wave * 1024u;
     // general copies: the tile index is clamped to the last tile (past the end a copy re-reads that tile into a slot nobody
     // reads any more) and rows past the last valid key onto it (masked later, but V must not feed NaNs into 0 * V)
@@ -224,8 +244,18 @@ __global__ __launch_bounds__(512, 2) void fmha_fwd_pingpong_kernel(const T* __re
         k_lane_off[i] = (uint32_t)(copy_row0 + 32 * i) * k_row_bytes + copy_kcol;
         v_lane_off[i] = (uint32_t)(copy_row0 + 32 * i) * v_row_bytes + copy_vcol;
     }
-    const char* k_next = (const char*)Kh + 3 * k_tile_bytes;
-    const char* v_next = (const char*)Vh + 2 * v_tile_bytes;
+    const char* k_next = nullptr;
+    const char* v_next = nullptr;
+    // the first pairs of the current item: K(0), K(1), V(0), K(2), V(1)
+    auto issue_first_pairs = [&]() {
+        issue_k1(0, 0); issue_k1(0, 1);
+        issue_k1(1, 0); issue_k1(1, 1);
+        issue_v1(1, 0); issue_v1(1, 1);
+        issue_k1(2, 0); issue_k1(2, 1);
+        issue_v1(2, 0); issue_v1(2, 1);
+        k_next = (const char*)Kh + 3 * k_tile_bytes;
+        v_next = (const char*)Vh + 2 * v_tile_bytes;
+    };
 
     // fragment addresses: loop-invariant registers, the slot and the block inside the tile are immediate offsets
     //   K fragment (key block kb, d step ks): row 16 kb + c, chunk (4 ks + g) ^ (row & 15)
@@ -243,26 +273,15 @@ __global__ __launch_bounds__(512, 2) void fmha_fwd_pingpong_kernel(const T* __re
     }
 
     float4v o[8][QB];
-#pragma unroll
-    for (int db = 0; db < 8; ++db)
-#pragma unroll
-        for (int qb = 0; qb < QB; ++qb) o[db][qb] = float4v{0.f, 0.f, 0.f, 0.f};
     constexpr bool kSumOnMatrixPipe = std::is_same<T, half_t>::value;
     float4v l_acc[QB];
-#pragma unroll
-    for (int qb = 0; qb < QB; ++qb) l_acc[qb] = float4v{0.f, 0.f, 0.f, 0.f};
     V8 ones;
 #pragma unroll
     for (int e = 0; e < 8; ++e) ones[e] = (T)1.0f;
+    asm volatile("" : "+v"(ones));   // in vector registers for good (the compiler would re-materialise it in every matrix phase)
     // per query: exponent reference of the running sums, the score above which it has to move, and -reference * scale
     float m_run[QB], m_thr[QB], neg_ms[QB];
     const float lazy_margin = kLazyLog2 / scale_log2;
-#pragma unroll
-    for (int qb = 0; qb < QB; ++qb) {
-        m_run[qb] = -INFINITY;
-        m_thr[qb] = -INFINITY;
-        neg_ms[qb] = 0.f;
-    }
 
     auto pin_s = [](float4v(&s)[4][QB]) {
         if constexpr (QB == 2)
@@ -412,6 +431,11 @@ __global__ __launch_bounds__(512, 2) void fmha_fwd_pingpong_kernel(const T* __re
         }
 #pragma unroll
         for (int qb = 0; qb < QB; ++qb) mx[qb] = max3v(mx[qb], mc[qb], mc[qb]);
+        // the second copy sits between the max tree and the compare that reads its result: the compiler puts wait states
+        // between an assembly statement and a dependent instruction, and these instructions take their place
+        __builtin_amdgcn_sched_barrier(0);
+        copy(std::integral_constant<int, 1>{});
+        __builtin_amdgcn_sched_barrier(0);
         bool raise = false;
 #pragma unroll
         for (int qb = 0; qb < QB; ++qb) raise = raise || (mx[qb] > m_thr[qb]);
@@ -431,8 +455,6 @@ __global__ __launch_bounds__(512, 2) void fmha_fwd_pingpong_kernel(const T* __re
                 for (int db = 0; db < 8; ++db) o[db][qb] *= alpha;
             }
         }
-        __builtin_amdgcn_sched_barrier(0);
-        copy(std::integral_constant<int, 1>{});
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int qb = 0; qb < QB; ++qb)
@@ -478,83 +500,109 @@ __global__ __launch_bounds__(512, 2) void fmha_fwd_pingpong_kernel(const T* __re
         }
     };
 
-    if (n_tiles > 0) {
-        // pairs 0 and 1 (K(0), K(1), V(0)) must be in LDS before P0; pair 2 is on its way
-        issue_k1(0, 0); issue_k1(0, 1);
-        issue_k1(1, 0); issue_k1(1, 1);
-        issue_v1(1, 0); issue_v1(1, 1);
-        issue_k1(2, 0); issue_k1(2, 1);
-        issue_v1(2, 0); issue_v1(2, 1);
-        wait_vmcnt<4>();
-        __syncthreads();
-        if (late) end_phase();   // waves 4..7 idle during P0
+    // ---- persistent loop over the work items of this workgroup ----------------------------------------------------------
+    // The first pairs and the Q fragments of the NEXT item are requested as soon as the last barrier of the current one is
+    // passed (every wave has finished reading LDS, and the Q registers are free), in front of the current item's epilogue:
+    // normalising and storing O runs while those loads are on their way, and the workgroup never goes back to the
+    // dispatcher between items.
+    MI355_TL(unsigned long long tl_tiles = 0;)
+    set_item(0);   // a launch has no more workgroups than items
+    load_q();
+    if (n_tiles > 0) issue_first_pairs();
+    for (int round = 0;;) {
+#pragma unroll
+        for (int qb = 0; qb < QB; ++qb) {
+            m_run[qb] = -INFINITY;
+            m_thr[qb] = -INFINITY;
+            neg_ms[qb] = 0.f;
+            l_acc[qb] = float4v{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int db = 0; db < 8; ++db) o[db][qb] = float4v{0.f, 0.f, 0.f, 0.f};
+        }
+        if (n_tiles > 0) {
+            // pairs 0, 1, 2 and Q have landed (and the stores of the previous item's epilogue have been accepted)
+            wait_vmcnt<0>();
+            __syncthreads();
+            if (late) end_phase();   // waves 4..7 idle during P0
 
-        float4v s[4][QB];
-        V8 pf[2][QB];
-        V8 fr[AHEAD];
-        MI355_TL(tl_w[1] = timeline::wall_clock(); tl_c[0] = timeline::shader_cycles();)
-        preload(I0{}, std::integral_constant<int, 0>{}, 0, fr);
-        __builtin_amdgcn_s_setprio(1);
-        mfma_phase(I0{}, I16{}, std::integral_constant<int, 0>{}, 0, s, pf, fr);               // S(0) alone
-        __builtin_amdgcn_s_setprio(0);
-        pin_s(s);
-        end_phase();
-        // tile step j: softmax(j) (with the copies of pair j + 3), then S(j+1) and O += V(j)^T P(j) on pair j + 1
-        auto step = [&](auto u_c, int j) {
-            constexpr int U = decltype(u_c)::value;   // j % NBUF in the unrolled loop, -1 in the general one
-            using CopySlot = std::integral_constant<int, (U >= 0 ? (U + 3) % NBUF : -1)>;
-            using ReadSlot = std::integral_constant<int, (U >= 0 ? (U + 1) % NBUF : -1)>;
-            softmax_tile(s, j, pf, CopySlot{}, j + 3);
-            pin_p(pf);
-            preload(I0{}, ReadSlot{}, (j + 1) & (NBUF - 1), fr);
-            end_phase();
+            float4v s[4][QB];
+            V8 pf[2][QB];
+            V8 fr[AHEAD];
+            MI355_TL(if (round == 0) tl_w[1] = timeline::wall_clock(); const unsigned long long tl_c0 = timeline::shader_cycles();)
+            preload(I0{}, std::integral_constant<int, 0>{}, 0, fr);
             __builtin_amdgcn_s_setprio(1);
-            mfma_phase(I0{}, I32{}, ReadSlot{}, (j + 1) & (NBUF - 1), s, pf, fr);
+            mfma_phase(I0{}, I16{}, std::integral_constant<int, 0>{}, 0, s, pf, fr);               // S(0) alone
             __builtin_amdgcn_s_setprio(0);
             pin_s(s);
-            pin_o();
             end_phase();
-        };
-        // unrolled loop: while the pair copied in step j (tiles j + 3 and j + 2) is made of full tiles
-        const int j_fast = max(0, min(n_full - 3, n_tiles - 1)) & ~(NBUF - 1);
-        int j = 0;
-        for (; j < j_fast; j += NBUF) {
-            step(std::integral_constant<int, 0>{}, j);
-            step(std::integral_constant<int, 1>{}, j + 1);
-            step(std::integral_constant<int, 2>{}, j + 2);
-            step(std::integral_constant<int, 3>{}, j + 3);
+            // tile step j: softmax(j) (with the copies of pair j + 3), then S(j+1) and O += V(j)^T P(j) on pair j + 1
+            auto step = [&](auto u_c, int j) {
+                constexpr int U = decltype(u_c)::value;   // j % NBUF in the unrolled loop, -1 in the general one
+                using CopySlot = std::integral_constant<int, (U >= 0 ? (U + 3) % NBUF : -1)>;
+                using ReadSlot = std::integral_constant<int, (U >= 0 ? (U + 1) % NBUF : -1)>;
+                softmax_tile(s, j, pf, CopySlot{}, j + 3);
+                pin_p(pf);
+                preload(I0{}, ReadSlot{}, (j + 1) & (NBUF - 1), fr);
+                end_phase();
+                __builtin_amdgcn_s_setprio(1);
+                mfma_phase(I0{}, I32{}, ReadSlot{}, (j + 1) & (NBUF - 1), s, pf, fr);
+                __builtin_amdgcn_s_setprio(0);
+                pin_s(s);
+                pin_o();
+                end_phase();
+            };
+            // unrolled loop: while the pair copied in step j (tiles j + 3 and j + 2) is made of full tiles
+            const int j_fast = max(0, min(n_full - 3, n_tiles - 1)) & ~(NBUF - 1);
+            int j = 0;
+            for (; j < j_fast; j += NBUF) {
+                step(std::integral_constant<int, 0>{}, j);
+                step(std::integral_constant<int, 1>{}, j + 1);
+                step(std::integral_constant<int, 2>{}, j + 2);
+                step(std::integral_constant<int, 3>{}, j + 3);
+            }
+            for (; j + 1 < n_tiles; ++j) step(Dyn{}, j);
+            softmax_tile(s, n_tiles - 1, pf, std::integral_constant<int, -2>{}, 0);
+            pin_p(pf);
+            preload(I16{}, Dyn{}, n_tiles & (NBUF - 1), fr);
+            end_phase();
+            mfma_phase(I16{}, I32{}, Dyn{}, n_tiles & (NBUF - 1), s, pf, fr);     // O += V(last)^T P(last) alone
+            end_phase();
+            if (!late) end_phase();  // waves 0..3 idle while waves 4..7 finish
+            // behind this barrier no wave reads LDS any more; the copies past the end of the item that are still on their
+            // way must land before the next item's pairs are sent into the same slots (or the workgroup ends)
+            wait_vmcnt<0>();
+            MI355_TL(tl_w[2] = timeline::wall_clock(); tl_c[1] += timeline::shader_cycles() - tl_c0; tl_tiles += (unsigned long long)n_tiles;)
         }
-        for (; j + 1 < n_tiles; ++j) step(Dyn{}, j);
-        softmax_tile(s, n_tiles - 1, pf, std::integral_constant<int, -2>{}, 0);
-        pin_p(pf);
-        preload(I16{}, Dyn{}, n_tiles & (NBUF - 1), fr);
-        end_phase();
-        mfma_phase(I16{}, I32{}, Dyn{}, n_tiles & (NBUF - 1), s, pf, fr);     // O += V(last)^T P(last) alone
-        end_phase();
-        if (!late) end_phase();  // waves 0..3 idle while waves 4..7 finish
-        wait_vmcnt<0>();   // no copy may still be on its way into LDS when the workgroup gives the memory back
-    }
-    MI355_TL(tl_w[2] = timeline::wall_clock(); tl_c[1] = timeline::shader_cycles();)
 
+        // what the epilogue needs of the item just finished, then on to the next one
+        T* const o_item = Oh;
+        const int q_item0 = q_wave0;
+        float* const lse_item = LSE == nullptr ? nullptr : LSE + ((long)b * Hq + hq) * (long)Sq;
+        const bool more = set_item(++round);
+        if (more) {
+            load_q();
+            if (n_tiles > 0) issue_first_pairs();
+        }
+        // ---- finalize: O / l, LSE: lane holds O[query 16 qb + c][d = 16 db + 4 g + 0..3] --------------------------------
 #pragma unroll
-    for (int qb = 0; qb < QB; ++qb) {
-        const float l_tot = kSumOnMatrixPipe ? l_acc[qb][0] : quad_sum(l_acc[qb][0]);
-        const float inv = (l_tot > 0.f) ? 1.f / l_tot : 0.f;
-        const int qi = q_wave0 + qb * 16 + c16;
-        if (qi < Sq) {
-            T* orow = Oh + qi * sd.o_row + 4 * g;
+        for (int qb = 0; qb < QB; ++qb) {
+            const float l_tot = kSumOnMatrixPipe ? l_acc[qb][0] : quad_sum(l_acc[qb][0]);
+            const float inv = (l_tot > 0.f) ? 1.f / l_tot : 0.f;
+            const int qi = q_item0 + qb * 16 + c16;
+            if (qi < Sq) {
+                T* orow = o_item + qi * sd.o_row + 4 * g;
 #pragma unroll
-            for (int db = 0; db < 8; ++db) {
-                V4 v;
+                for (int db = 0; db < 8; ++db) {
+                    V4 v;
 #pragma unroll
-                for (int e = 0; e < 4; ++e) v[e] = (T)(o[db][qb][e] * inv);
-                *(V4*)(orow + db * 16) = v;
-            }
-            if (LSE != nullptr && g == 0) {
-                const float lse = (l_tot > 0.f) ? (m_run[qb] * scale_log2 + __builtin_log2f(l_tot)) * 0.69314718055994531f : -INFINITY;
-                LSE[((long)b * Hq + hq) * (long)Sq + qi] = lse;
+                    for (int e = 0; e < 4; ++e) v[e] = (T)(o[db][qb][e] * inv);
+                    *(V4*)(orow + db * 16) = v;
+                }
+                if (lse_item != nullptr && g == 0)
+                    lse_item[qi] = (l_tot > 0.f) ? (m_run[qb] * scale_log2 + __builtin_log2f(l_tot)) * 0.69314718055994531f : -INFINITY;
             }
         }
+        if (!more) break;
     }
     MI355_TL(
         wait_vmcnt<0>();   // the stores of this wave have been accepted
@@ -562,8 +610,21 @@ __global__ __launch_bounds__(512, 2) void fmha_fwd_pingpong_kernel(const T* __re
         if (tid == 0 && blockIdx.x < timeline::kMaxWorkgroups) {
             unsigned long long* rec = fmha_fwd_stamps + (long)blockIdx.x * timeline::kSlots;
             rec[0] = tl_w[0]; rec[1] = tl_w[1]; rec[2] = tl_w[2]; rec[3] = tl_w[3];
-            rec[4] = tl_c[0]; rec[5] = tl_c[1]; rec[6] = (unsigned long long)max(n_tiles, 0); rec[7] = 0;
+            rec[4] = 0; rec[5] = tl_c[1]; rec[6] = tl_tiles; rec[7] = 0;
         })
+}
+
+// number of CUs of the current device (asked once per device)
+static hipError_t compute_units(int& cus) {
+    static std::atomic<int> cached[DynamicLdsOnce::kMaxDevices] = {};
+    int dev = 0;
+    if (hipError_t e = hipGetDevice(&dev); e != hipSuccess) return e;
+    const bool tracked = dev >= 0 && dev < DynamicLdsOnce::kMaxDevices;
+    if (tracked && (cus = cached[dev].load(std::memory_order_relaxed)) > 0) return hipSuccess;
+    if (hipError_t e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev); e != hipSuccess) return e;
+    if (cus < 1) return hipErrorInvalidDevice;
+    if (tracked) cached[dev].store(cus, std::memory_order_relaxed);
+    return hipSuccess;
 }
 
 template <typename T, int QB>
@@ -576,8 +637,14 @@ static hipError_t launch_fmha_pingpong(const T* Q, const T* K, const T* V, T* O,
     static DynamicLdsOnce lds_once;
     if (hipError_t e = lds_once.ensure(reinterpret_cast<const void*>(kern), LDS); e != hipSuccess) return e;
     const int q_tiles = (Sq + BM - 1) / BM;
-    const long blocks = (long)q_tiles * Hq * B;
-    if (blocks > 0x7fffffffL) return hipErrorInvalidValue;
+    const long items = (long)q_tiles * Hq * B;
+    if (items > 0x7fffffffL) return hipErrorInvalidValue;
+    // one workgroup per CU at most (128 KiB of LDS each: a CU holds one); a multiple of 8 when the (batch, kv head) groups
+    // divide over the 8 XCDs, so that fmha_work_item can give every XCD whole groups
+    int cus = 0;
+    if (hipError_t e = compute_units(cus); e != hipSuccess) return e;
+    long blocks = items < cus ? items : cus;
+    if (((long)Hkv * B) % 8 == 0 && blocks >= 8) blocks &= ~7L;
     const float scale_log2 = scale * 1.4426950408889634f;
     kern<<<dim3((unsigned)blocks), dim3(512), LDS, stream>>>(Q, K, V, O, LSE, B, Hq, Hkv, Sq, Sk, scale_log2, causal, kv_valid,
                                                              q_tiles, sd);
@@ -597,16 +664,16 @@ static hipError_t fmha_fwd_dispatch_t(const void* Q, const void* K, const void* 
     if (variant == 0 && fmha_decode_applicable(B, Hq, Hkv, Sq, Sk, kv_valid_len))
         return fmha_decode_dispatch<T>(q, k, v, o, LSE, B, Hq, Hkv, Sq, Sk, scale, causal, kv_valid_len, sd, ws, stream);
     if (variant == 0) {
-        // 256-query workgroups (every K / V fragment feeds two MFMAs) once they fill the machine: clearly more of them than
-        // CUs for a causal problem (with about one per CU it runs as long as its heaviest tile, and 128-query workgroups
-        // balance better), one per CU otherwise; never for sequences of a tile or two. Measured (b x heads q/kv x s, 128-
-        // / 256-query workgroups, us): causal 1 x 32/8 x 1024 21 / 31, 1 x 32/8 x 2048 48 / 54, 2 x 32/8 x 1024 31 / 34,
-        // 1 x 16/16 x 4096 84 / 94, 1 x 8/8 x 8192 149 / 173, 32 x 32/8 x 256 71 / 74, but 8 x 32/8 x 512 46 / 45,
-        // 1 x 32/8 x 3000 99 / 83, 2 x 32/8 x 1536 62 / 53, 4 x 32/8 x 1024 62 / 59, 1 x 32/8 x 4096 160 / 134,
-        // 16 x 32/8 x 768 152 / 137, 4 x 32/8 x 2048 189 / 155; not causal 2 x 32/8 x 1024 47 / 38, 1 x 32/8 x 2048 81 / 65,
-        // 4 x 32/32 x 1024 93 / 75.
+        // 256-query workgroups (every K / V fragment feeds two MFMAs) once their work items fill the machine: clearly more
+        // of them than CUs for a causal problem (with about one per CU it runs as long as its heaviest item, and 128-query
+        // items balance better), one per CU otherwise. Measured (b x heads q/kv x s, 128- / 256-query items, us): causal
+        // 1 x 32/8 x 1024 20 / 30, 1 x 32/8 x 2048 45 / 51, 2 x 32/8 x 1024 30 / 32, 1 x 16/16 x 4096 76 / 88,
+        // 1 x 8/8 x 8192 139 / 163, 2 x 8/2 x 4096 76 / 88, but 32 x 32/8 x 256 68 / 64, 8 x 32/8 x 512 42 / 39,
+        // 1 x 32/8 x 3000 92 / 78, 2 x 32/8 x 1536 56 / 50, 4 x 32/8 x 1024 57 / 50, 1 x 32/8 x 4096 149 / 126,
+        // 16 x 32/8 x 768 148 / 128, 4 x 32/8 x 2048 170 / 147; not causal 2 x 32/8 x 1024 42 / 36, 1 x 32/8 x 2048 73 / 62,
+        // 4 x 32/32 x 1024 89 / 71.
         const long wg256 = (long)((Sq + 255) / 256) * Hq * B;
-        variant = (Sq >= 512 && wg256 >= (causal ? 320 : 256)) ? 2 : 1;
+        variant = (Sq >= 256 && wg256 >= (causal ? 320 : 256)) ? 2 : 1;
     }
     if (variant == 2) return launch_fmha_pingpong<T, 2>(q, k, v, o, LSE, B, Hq, Hkv, Sq, Sk, scale, causal, kv_valid_len, sd, stream);
     return launch_fmha_pingpong<T, 1>(q, k, v, o, LSE, B, Hq, Hkv, Sq, Sk, scale, causal, kv_valid_len, sd, stream);
