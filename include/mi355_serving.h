@@ -11,17 +11,21 @@
  *     Hq/Hkv * Sq <= 32 and kv_valid_len >= 512, i.e. generation steps): one buffer per (device, stream), obtained
  *     with hipMalloc at first use (>= 4 MiB; when a later call needs more, a larger buffer is allocated and the old
  *     one is kept, because a HIP graph captured earlier may still hold its address; nothing is freed before the
- *     process ends), so steady-state calls allocate nothing and calls on different streams never share a buffer.
+ *     process ends, and every stream that ever made such a call keeps its buffer), so steady-state calls allocate
+ *     nothing and calls on different streams never share a buffer.
  *     A call that would have to allocate while its stream is being captured fails (hipErrorStreamCaptureUnsupported)
  *     and launches nothing: run the step once on that stream before capturing it, and replay the graph on the stream it
- *     was captured on (or use mi355_fmha_fwd_ws with memory of your own);
+ *     was captured on (or use mi355_fmha_fwd_ws with memory of your own). Only the calling stream's capture state is
+ *     visible to the library: a first (or growing) call made while ANOTHER stream captures in global capture mode is a
+ *     hipMalloc inside that capture and invalidates it, so make such calls before any capture starts;
  *   - `stream` is a hipStream_t passed as void* (NULL = the null stream); calls are asynchronous;
  *   - fp16 data is IEEE binary16 (`_Float16` / `__half` / torch.float16);
  *   - return value 0 = launched; non-zero = a hipError_t value or MI355_ERR_* below, nothing was launched.
  *     mi355_last_error() returns a thread-local description of the last failure.
- *   - calls are re-entrant and thread-safe; the only mutable global state is one-time kernel attribute
- *     initialisation (atomic flags) and the mutex-protected table of those workspaces. Which kernel runs depends on
- *     the arguments alone.
+ *   - calls are re-entrant and thread-safe, with one exception: mi355_fmha_fwd_noalloc, whose calls share one fixed
+ *     array per GPU and must not overlap on a GPU (see there). The only other mutable global state is one-time kernel
+ *     attribute initialisation (atomic flags) and the mutex-protected table of those workspaces. Which kernel runs
+ *     depends on the arguments alone.
  */
 #ifndef MI355_SERVING_H
 #define MI355_SERVING_H
@@ -71,11 +75,11 @@ int mi355_hgemm(const void* A, const void* B, void* C, int M, int N, int K, int6
  * gate and up projections of a Llama MLP computed by one GEMM on an interleaved weight matrix, with the activation
  * applied to the accumulators before the single rounding to fp16. Replaces `self.act_fn(self.gate_proj(x)) * self.up_proj(x)`
  * (benchmarks/flashattn-cuda/modeling_llama.py:227): two GEMMs, a SiLU kernel and a multiply kernel in the reference.
- * Layouts NN and NT. The fused form exists for M <= 16 in layout NT (the generation step: the split-K small-M kernel with
- * the same epilogue) and for the shapes the tiled kernels cover (M > 64, or M > 16 when the product is wide enough for
- * the tiled kernels to beat the small-M kernels); N a multiple of 32, K a multiple of 64, 16-byte aligned operands and
- * leading dimensions. Other shapes return MI355_ERR_UNSUPPORTED and nothing is launched: run
- * mi355_hgemm on the same operands followed by mi355_silu_mul with interleave = 32.
+ * Layouts NN and NT; N a multiple of 32, K a multiple of 64, 16-byte aligned operands and leading dimensions. Every such
+ * shape is one launch: up to 16 rows in layout NT on the split-K small-M kernel, up to 64 rows otherwise on 64x64 tiles
+ * with a deep ring (both stream the weight once), more rows on the 128x128 / 256x256 tiles, all with the same epilogue.
+ * Other shapes (K or N off those multiples, unaligned operands, layout TN) return MI355_ERR_UNSUPPORTED and nothing is
+ * launched: run mi355_hgemm on the same operands followed by mi355_silu_mul with interleave = 32.
  */
 int mi355_hgemm_silu_mul(const void* A, const void* B, void* C, int M, int N, int K, int64_t lda, int64_t ldb, int64_t ldc,
                          int layout, void* stream);
@@ -239,8 +243,12 @@ int mi355_fmha_fwd_ws(const void* Q, const void* K, const void* V, void* O, floa
  * per GPU the library runs on, held until the process ends; its first 64 KiB hold the ticket counters). A call whose partial results do not fit (more than about
  * 7800 = (4 MiB - 64 KiB) / 528 B (workgroup, query column) pairs; a call runs about 256 workgroups, so this means more than ~30 query
  * rows per kv head at small batch; a Llama generation step has 4) returns MI355_ERR_UNSUPPORTED and launches nothing. Every call on a GPU shares that GPU's array: calls through this entry point
- * that overlap on one GPU (different streams, or threads) race; order them on one stream. Shapes outside the split-KV path
- * (prefill) do not touch the array and behave exactly like mi355_fmha_fwd_strided.
+ * that overlap on one GPU (different streams, or threads) race; order them on one stream. The array's ticket counters are
+ * zero when the library is loaded and every completed call leaves them at zero; a call that does not complete (an aborted
+ * kernel, overlapping calls) can leave one that is not, and later calls for that (batch, kv head) then write no output
+ * and report no error until the process ends (mi355_fmha_fwd_ws zeroes its counters on every call and has no such
+ * memory). Shapes outside the split-KV path (prefill) do not touch the array and behave exactly like
+ * mi355_fmha_fwd_strided.
  */
 int mi355_fmha_fwd_noalloc(const void* Q, const void* K, const void* V, void* O, float* LSE, int B, int Hq, int Hkv, int Sq,
                            int Sk, int D, float scale, int causal, int kv_valid_len, const int64_t* strides, void* stream);

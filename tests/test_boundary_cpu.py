@@ -104,7 +104,7 @@ def test_capi_rejects_bad_arguments_without_a_gpu(lib):
     assert cdll.mi355_silu_mul(p, p, 4, 64, 12, 128, 64, None) == 10001                             # interleave % 8
     assert cdll.mi355_hgemm_silu_mul(p, p, p, 256, 128, 64, 64, 64, 128, 2, None) == 10002          # TN has no fused epilogue
     assert cdll.mi355_hgemm_silu_mul(p, p, p, 256, 128, 64, 64, 64, 64, 1, None) == 10001           # ldc < N
-    assert cdll.mi355_hgemm_silu_mul(p, p, p, 32, 128, 64, 64, 64, 128, 1, None) == 10002           # few rows: small-M product + silu_mul
+    assert cdll.mi355_hgemm_silu_mul(p, p, p, 32, 128, 96, 96, 96, 128, 1, None) == 10002           # K not a multiple of 64: product + silu_mul
     assert b"mi355_silu_mul" in cdll.mi355_last_error()
     assert cdll.mi355_hgemm_add(p, p, None, p, 64, 64, 64, 64, 64, 64, 64, 0, None) == 10001            # residual missing
     assert cdll.mi355_hgemm_add(p, p, p2, p, 64, 64, 64, 64, 64, 32, 64, 0, None) == 10001              # ldr < N

@@ -106,6 +106,16 @@ def test_ragged_m_and_n_on_the_tiled_kernels(lib, gpu, variant, layout, M, N, K)
     assert bool((c[M:] == 9.0).all()) and bool((c[:, N:] == 9.0).all())
 
 
+@pytest.mark.parametrize("layout", ["NN", "TN", "NT"])
+@pytest.mark.parametrize("M,N,K", [(512, 384, 1072), (1024, 1024, 1040), (256, 256, 80), (16, 4096, 4112), (8, 512, 2096),
+                                   (48, 2048, 1056), (1000, 520, 4144), (2048, 2048, 176)])
+def test_k_that_is_a_multiple_of_16_but_not_of_the_tile_depth(lib, gpu, layout, M, N, K):
+    # the reference's checked wrapper takes K % 16 == 0 (kernels/gemm/pkg/gemm_unified/csrc/auto/gemm_7.cu:115-135): the
+    # tiled / small-M kernels do the first K - K % 64 columns, the bounds-checked kernel only the last K % 64
+    a, b = operands(M, N, K, layout, seed=M + K, b_std=0.05)
+    check(lib, gpu, a, b, layout, K)
+
+
 @pytest.mark.parametrize("variant", [1, 2])
 @pytest.mark.parametrize("layout", ["NN", "TN", "NT"])
 def test_every_tile_variant(lib, gpu, variant, layout):

@@ -135,10 +135,12 @@ def test_silu_mul(lib, gpu, rows, inter):
                                           (300, 160, 128, "NT"), (1000, 14336, 128, "NT"), (4100, 4096, 64, "NN"),
                                           (32, 14336, 256, "NT"), (64, 14336, 128, "NN"), (24, 7168, 512, "NT"),
                                           (1, 32, 64, "NT"), (8, 14336, 512, "NT"), (16, 2048, 1024, "NT"), (13, 96, 128, "NT"),
-                                          (9, 4096, 4096, "NT"), (16, 512, 256, "NN")])
+                                          (9, 4096, 4096, "NT"), (16, 512, 256, "NN"), (17, 1024, 512, "NT"), (48, 7168, 256, "NT"),
+                                          (33, 512, 1024, "NN"), (64, 2048, 128, "NN"), (40, 96, 64, "NT"), (5, 256, 192, "NN")])
 def test_gemm_with_gate_up_epilogue(lib, gpu, M, F, K, layout):
     # silu(x Wg^T) * (x Wu^T) from one launch on the interleaved weight (tiled shapes; up to 16 rows in layout NT on the
-    # split-K kernel, with and without the second half of the A slab) or from the two-step fallback;
+    # split-K kernel, with and without the second half of the A slab; up to 64 rows otherwise on the 64x64 deep-ring tiles)
+    # or, where K is off the tiles' multiple, from the two-step fallback;
     # compared with the fp32 oracle. One rounding of an fp32 value: |err| <= 2^-10 |ref| + the GEMM's accumulation slack.
     x = so.randn_fp16((M, K), 1)
     wg, wu = so.randn_fp16((F, K), 2, 0.05), so.randn_fp16((F, K), 3, 0.05)
@@ -155,6 +157,40 @@ def test_gemm_with_gate_up_epilogue(lib, gpu, M, F, K, layout):
     # the interleaved silu_mul on the plain product gives the same numbers up to the extra fp16 rounding of the product
     two_step = lib.silu_mul(lib.hgemm(x.to(gpu), w, layout), interleave=32)
     assert (two_step.float() - out.float()).abs().max() <= 2e-2 * ref.abs().max()
+
+
+def test_gate_up_epilogue_is_one_launch_for_every_row_count(lib, gpu):
+    # N a multiple of 32 and K a multiple of 64: the entry point itself never answers "unsupported", whatever M is
+    K, F = 256, 512
+    wg, wu = so.randn_fp16((F, K), 2, 0.05), so.randn_fp16((F, K), 3, 0.05)
+    w = lib.interleave_gate_up(wg.to(gpu), wu.to(gpu), dim=0)
+    for M in (1, 8, 16, 17, 31, 32, 33, 63, 64, 65, 100, 128, 300):
+        x = so.randn_fp16((M, K), 10 + M)
+        out = torch.empty((M, F), dtype=torch.float16, device=gpu)
+        xg = x.to(gpu)
+        rc = lib.load().mi355_hgemm_silu_mul(xg.data_ptr(), w.data_ptr(), out.data_ptr(), M, F, K, K, K, F, lib.GEMM_NT, 0)
+        assert rc == 0, (M, rc)
+        torch.cuda.synchronize()
+        ref = so.silu_mul_ref(torch.cat((so.gemm_ref(x, wg, "NT"), so.gemm_ref(x, wu, "NT")), 1))
+        err = (out.float().cpu() - ref).abs()
+        assert bool((err <= 2.0 ** -10 * ref.abs() + 1e-3).all()), (M, float(err.max()))
+
+
+def test_gate_up_single_row_activation_with_arbitrary_row_stride(lib, gpu):
+    # torch calls a [1, K] tensor contiguous whatever its stride(0): the wrapper passes the logical leading dimension
+    K, F = 256, 128
+    x = so.randn_fp16((1, K), 4)
+    wg, wu = so.randn_fp16((F, K), 5, 0.05), so.randn_fp16((F, K), 6, 0.05)
+    w = lib.interleave_gate_up(wg.to(gpu), wu.to(gpu), dim=0)
+    ref = so.silu_mul_ref(torch.cat((so.gemm_ref(x, wg, "NT"), so.gemm_ref(x, wu, "NT")), 1))
+    base = torch.zeros(4 * K, dtype=torch.float16, device=gpu)
+    base[:K] = x[0].to(gpu)
+    for stride0 in (7, 0, 3 * K):
+        x1 = base.as_strided((1, K), (stride0, 1))
+        assert x1.is_contiguous() and x1.stride(0) == stride0
+        out = lib.hgemm_silu_mul(x1, w, "NT")
+        err = (out.float().cpu() - ref).abs()
+        assert bool((err <= 2.0 ** -10 * ref.abs() + 1e-3).all()), (stride0, float(err.max()))
 
 
 def layer_weights(H, n_q, n_kv, F, seed=0):

@@ -1,6 +1,9 @@
-"""CPU-only check of the one place where loads are issued as inline assembly and waited for later
-(csrc/fmha_decode.hip, the merge of the key ranges: `global_load_dwordx4 ... sc1`, one `s_waitcnt vmcnt(0)` behind up to
-32 of them). To the compiler the result of such a statement exists as soon as it has been issued, so nothing stops it from
+"""CPU-only checks of the generated code of csrc/fmha_decode.hip, whose merge of the key ranges orders its memory
+accesses with instructions instead of fences (a device-scope fence writes back / invalidates a whole L2 and costs 2.5-3 us per
+launch there).
+
+First, the one place where loads are issued as inline assembly and waited for later (`global_load_dwordx4 ... sc1`, one
+`s_waitcnt vmcnt(0)` behind up to 32 of them). To the compiler the result of such a statement exists as soon as it has been issued, so nothing stops it from
 copying or reusing a destination register before the data has landed (it does so, for instance, at the join behind a
 conditional group of loads when the values are carried in a second register set). The generated code is what counts:
 compile the file to assembly and check that no instruction touches a destination register between its load and the
@@ -27,8 +30,12 @@ def vgprs(text):
     return found
 
 
+# a device-coherent load of any width: global_load_dword[x2|x3|x4] dst, address.. with sc0 / sc1 (/ nt) in any order
+COHERENT_LOAD = re.compile(r"global_load_dword(?:x[234])? (v\[\d+:\d+\]|v\d+), (.*?)((?: (?:sc0|sc1|nt))+)$")
+
+
 def violations(asm_text):
-    """Program-order scan: registers that an `sc1` 16-byte load writes stay pending until the next `s_waitcnt vmcnt(0)`;
+    """Program-order scan: registers that a device-coherent load writes stay pending until the next `s_waitcnt vmcnt(0)`;
     any instruction in between that names one of them is reported (a later load may not use one as its address either)."""
     pending, bad, n_loads = set(), [], 0
     for no, line in enumerate(asm_text.split("\n"), 1):
@@ -38,7 +45,7 @@ def violations(asm_text):
         if t.startswith("s_endpgm") or (t.startswith("s_waitcnt") and "vmcnt(0)" in t):
             pending = set()
             continue
-        m = re.match(r"global_load_dwordx4 (v\[\d+:\d+\]), (.*) sc1\b", t)
+        m = COHERENT_LOAD.match(t)
         if m:
             if vgprs(m.group(2)) & pending:
                 bad.append((no, t))
@@ -49,12 +56,44 @@ def violations(asm_text):
     return n_loads, bad
 
 
+def unordered_tickets(asm_text):
+    """Program-order scan for the writers' side of the merge: every device-coherent store of a partial result
+    (`global_store_dword ... sc1`) must be followed by an `s_waitcnt vmcnt(0)` before the ticket is drawn
+    (`global_atomic_add... `). Returns (number of ticket atomics, lines of those that have a store pending)."""
+    pending, tickets, bad = False, 0, []
+    for no, line in enumerate(asm_text.split("\n"), 1):
+        t = line.strip()
+        if not t or t[0] in ";.":
+            continue
+        if t.startswith("s_waitcnt") and "vmcnt(0)" in t:
+            pending = False
+        elif re.match(r"global_store_dword\S* .*\bsc1\b", t):
+            pending = True
+        elif t.startswith("global_atomic_add"):
+            tickets += 1
+            if pending:
+                bad.append((no, t))
+    return tickets, bad
+
+
 def test_checker_flags_a_copy_of_a_register_whose_load_is_in_flight():
     good = "global_load_dwordx4 v[4:7], v[2:3], off sc1\nv_add_u32 v1, v0, v0\ns_waitcnt vmcnt(0)\nv_mov_b32 v8, v4\n"
     bad = "global_load_dwordx4 v[4:7], v[2:3], off sc1\nv_mov_b32 v8, v5\ns_waitcnt vmcnt(0)\n"
     reuse = "global_load_dwordx4 v[4:7], v[2:3], off sc1\nglobal_load_dwordx4 v[8:11], v[4:5], off sc1\ns_waitcnt vmcnt(0)\n"
     assert violations(good) == (1, [])
     assert len(violations(bad)[1]) == 1 and len(violations(reuse)[1]) == 1
+    # other spellings of a coherent load: narrower, flags in another order, an offset in front of the flags
+    for load in ("global_load_dword v4, v[2:3], off sc1", "global_load_dwordx2 v[4:5], v[2:3], off sc1 sc0",
+                 "global_load_dwordx4 v[4:7], v[2:3], off offset:16 sc0 sc1"):
+        assert len(violations(load + "\nv_mov_b32 v8, v4\ns_waitcnt vmcnt(0)\n")[1]) == 1, load
+    assert violations("global_load_dwordx4 v[4:7], v[2:3], off\nv_mov_b32 v8, v4\n") == (0, [])   # an ordinary load: the compiler's business
+
+
+def test_checker_flags_a_ticket_drawn_before_the_partial_results_are_waited_for():
+    good = "global_store_dword v[2:3], v4, off sc1\ns_waitcnt vmcnt(0)\ns_barrier\nglobal_atomic_add_u32 v5, v[0:1], v6, off sc0\n"
+    bad = "global_store_dword v[2:3], v4, off sc1\ns_waitcnt lgkmcnt(0)\ns_barrier\nglobal_atomic_add_u32 v5, v[0:1], v6, off sc0\n"
+    assert unordered_tickets(good) == (1, [])
+    assert len(unordered_tickets(bad)[1]) == 1
 
 
 def test_no_instruction_touches_an_inline_asm_load_before_its_wait(tmp_path):
@@ -66,6 +105,11 @@ def test_no_instruction_touches_an_inline_asm_load_before_its_wait(tmp_path):
     src = "csrc/fmha_decode.hip"
     cmd = [b.HIPCC] + b.DEVICE_FLAGS + b.SOURCE_FLAGS.get(src, []) + ["-I", b.INCLUDE, "-S", "--cuda-device-only", src, "-o", out]
     subprocess.run(cmd, cwd=PKG, check=True, stdout=subprocess.DEVNULL, stderr=subprocess.DEVNULL)
-    n_loads, bad = violations(open(out).read())
+    text = open(out).read()
+    n_loads, bad = violations(text)
     assert n_loads >= 64, n_loads           # fp16 and bf16 instances, 32 loads each at least
     assert bad == [], bad[:5]
+    # the writers' side: partial results are waited for (s_waitcnt vmcnt(0) behind the stores) before the ticket is drawn
+    tickets, unordered = unordered_tickets(text)
+    assert tickets >= 2, tickets            # one ticket per instance of the kernel
+    assert unordered == [], unordered[:5]

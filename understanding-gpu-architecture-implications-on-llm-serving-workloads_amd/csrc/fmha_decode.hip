@@ -316,9 +316,23 @@ __global__ __launch_bounds__(WAVES * 64) void fmha_decode_kernel(
         MI355_TL(wait_vmcnt<0>(); tl[7] = timeline::wall_clock(); tl_dump();)
         return;
     }
-    // Partial results cross XCDs (each has its own L2), so they are written and read with device-scope relaxed atomic
-    // accesses, which go through to memory, instead of plain accesses bracketed by device-scope fences: such a fence
-    // writes back / invalidates a whole L2 and costs microseconds per workgroup here.
+    // Partial results cross XCDs (each has its own L2). The hand-over from the workgroups that write them to the one that
+    // merges them is ordered by instructions, not by a release / acquire pair: a device-scope fence writes back and
+    // invalidates a whole L2 here, and an acquire-release ticket costs 2.5-3 us per launch (b = 1 over 8192 keys: 13.8 us
+    // against 11.0). What takes the fence's place, step by step:
+    //   1. every partial result is stored with a device-scope atomic store, i.e. `global_store_dword .. sc1`: written through
+    //      the XCD's L2 to memory, nothing of it stays dirty in a cache;
+    //   2. `s_waitcnt vmcnt(0)` behind the stores: on gfx9-family parts a store leaves vmcnt only when the memory system has
+    //      acknowledged it at the scope it was issued with. The wait is an assembly statement with a memory clobber, so the
+    //      compiler keeps the stores in front of it;
+    //   3. the workgroup barrier: all threads have passed their wait before thread 0 draws the ticket;
+    //   4. the ticket is a device-scope atomic add, carried out at the memory side: the tickets of one counter are totally
+    //      ordered, and the workgroup that draws the last one knows that every other workgroup of its (batch, kv head) has
+    //      passed step 2;
+    //   5. the merging workgroup reads the partial results with `global_load_dword[x4] .. sc1` (device-coherent: served from
+    //      memory, not from a line its XCD's L2 may still hold from an earlier launch), issued behind the branch on the
+    //      ticket's value, which the hardware cannot pass before the atomic has returned.
+    // tests/test_inline_asm_loads_cpu.py checks 1, 2 and 5 in the generated code.
     float* mypart = part + (long)blockIdx.x * ncols * PART_STRIDE;
     for (int idx = tid; idx < ncols * D; idx += NTHREADS) {
         const int c = idx >> 7, d = idx & (D - 1);
@@ -330,7 +344,7 @@ __global__ __launch_bounds__(WAVES * 64) void fmha_decode_kernel(
         }
     }
     // ---- ticket: the workgroup that completes the set of key ranges of (b, hkv) merges them ----------------------------
-    wait_vmcnt<0>();   // this thread's partial results have reached memory before the ticket is drawn
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // this thread's partial results have reached memory before the ticket is drawn
     MI355_TL(tl[3] = timeline::wall_clock();)
     __syncthreads();
     MI355_LDS unsigned* ticket_sh = (MI355_LDS unsigned*)(cmb + WAVES * wave_floats);
@@ -455,7 +469,9 @@ __global__ __launch_bounds__(WAVES * 64) void fmha_decode_kernel(
         if (LSE != nullptr && d == 0)
             LSE[row0 + c] = (l > 0.f) ? (st_mc[c] * scale_log2 + __builtin_log2f(l)) * 0.69314718055994531f : -INFINITY;
     }
-    if (tid == 0) counters[(long)bh * kCounterStride] = 0u;   // ready for the next call that uses this workspace
+    // ready for the next call that uses this workspace (a device-scope store like the tickets, which are the only other
+    // accesses to the counter; the next launch on the stream starts after this one has ended)
+    if (tid == 0) __hip_atomic_store(&counters[(long)bh * kCounterStride], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     MI355_TL(wait_vmcnt<0>(); tl[7] = timeline::wall_clock(); tl_dump();)
 }
 
@@ -508,11 +524,17 @@ size_t fmha_decode_workspace_bytes(int B, int Hq, int Hkv, int Sq, int Sk, int k
 // The library's own workspace: one buffer per (device, stream), allocated on first use and replaced by a larger one when
 // a call needs more. A buffer that has been handed to a kernel is NEVER freed: a HIP graph captured earlier may hold
 // its address, so replaced buffers stay allocated until the process ends (each replacement is at least 1.5x larger, so
-// together they hold less than three times the largest request). Calls on one stream are ordered, so they can share a
-// buffer; calls on different streams get different ones. Nothing can be allocated while the stream is capturing: such a
-// call fails with hipErrorStreamCaptureUnsupported unless an earlier call on the same stream already made the buffer
-// large enough (run the step once before capturing it, or hand in a workspace of your own).
-static hipError_t decode_workspace(size_t bytes, hipStream_t stream, char** out) {
+// together they hold less than three times the largest request), and so does the buffer of every stream that ever made
+// such a call (at least 4 MiB each: a process that creates streams without end should hand in its own workspace,
+// mi355_fmha_fwd_ws). Calls on one stream are ordered, so they can share a buffer; calls on different streams get
+// different ones. Nothing can be allocated while the stream is capturing: such a call fails with
+// hipErrorStreamCaptureUnsupported unless an earlier call on the same stream already made the buffer large enough (run
+// the step once before capturing it, or hand in a workspace of your own). Only the calling stream's capture state can be
+// seen from here: while ANOTHER stream of the process captures in global capture mode, a first or growing call (a
+// hipMalloc) would invalidate that capture, so make those calls before any capture starts. `fresh_counters` tells the
+// caller that the buffer is new and its ticket counters still have to be set to zero (on the calling stream, in front of
+// the kernel: no synchronous fill of the whole buffer on the null stream).
+static hipError_t decode_workspace(size_t bytes, hipStream_t stream, char** out, bool* fresh_counters) {
     struct Buf {
         void* ptr = nullptr;
         size_t size = 0;
@@ -524,6 +546,7 @@ static hipError_t decode_workspace(size_t bytes, hipStream_t stream, char** out)
     if (e != hipSuccess) return e;
     std::lock_guard<std::mutex> lock(mu);
     Buf& b = bufs[std::make_pair(dev, stream)];
+    *fresh_counters = false;
     if (b.size < bytes) {
         hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
         e = hipStreamIsCapturing(stream, &cap);
@@ -533,18 +556,22 @@ static hipError_t decode_workspace(size_t bytes, hipStream_t stream, char** out)
         void* fresh = nullptr;
         e = hipMalloc(&fresh, want);
         if (e != hipSuccess) return e;
-        e = hipMemset(fresh, 0, want);   // the ticket counters start at zero; every call leaves them at zero
-        if (e != hipSuccess) return e;
         b.ptr = fresh;   // the previous buffer, if any, stays allocated (see above)
         b.size = want;
+        *fresh_counters = true;
     }
     *out = static_cast<char*>(b.ptr);
     return hipSuccess;
 }
 
 // Static scratch for callers that must not allocate (mi355_fmha_fwd_noalloc): a fixed array in device memory, one copy
-// per GPU the library is loaded on, held until the process ends; it starts out zeroed (so do its ticket counters). Host code never uses the symbol's name as an address:
-// the device address is looked up once per device with hipGetSymbolAddress and kept.
+// per GPU the library is loaded on, held until the process ends; it starts out zeroed (so do its ticket counters). Host
+// code never uses the symbol's name as an address: the device address is looked up once per device with
+// hipGetSymbolAddress and kept. Every call on a GPU shares that GPU's array and relies on finding its ticket counters at
+// zero, where every completed call leaves them: calls that overlap on one GPU race, and a call that does not run to its end
+// (a kernel that is aborted, overlapping calls) leaves a counter that is not zero. From then on no workgroup of that
+// (batch, kv head) draws the last ticket, O and LSE of its rows are not written and no error is reported, until the
+// process ends; mi355_fmha_fwd_ws (counters zeroed on every call) is the entry point that does not depend on history.
 constexpr size_t kStaticScratchBytes = size_t(4) << 20;
 static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
 
@@ -593,23 +620,30 @@ hipError_t fmha_decode_dispatch(const T* Q, const T* K, const T* V, T* O, float*
     char* wsp = nullptr;
     hipError_t e = hipSuccess;
     if (plan.bytes > 0) {
+        // Ticket counters must be zero when the kernel starts. The library's buffers and the static array are zeroed once
+        // (a fresh buffer by the fill kernel below, the static array by the loader) and every call leaves its counters at
+        // zero; a caller's memory holds anything, so its counters are zeroed on every call.
+        bool clear_counters = false;
+        long n_counters = (long)B * Hkv * kCounterStride;   // this call's counters
         switch (ws.kind) {
             case FmhaWorkspace::kCaller:
                 if (ws.ptr == nullptr || ws.bytes < plan.bytes || reinterpret_cast<uintptr_t>(ws.ptr) % 16 != 0) return hipErrorInvalidValue;
                 wsp = static_cast<char*>(ws.ptr);
-                // a caller's memory holds anything: zero its counters first (the library's own buffers and the static array
-                // start at zero and every call leaves them at zero)
-                fmha_decode_clear_kernel<<<dim3(1), dim3(256), 0, stream>>>(reinterpret_cast<unsigned*>(wsp),
-                                                                            (int)((long)B * Hkv * kCounterStride));   // this call's counters
-                e = hipGetLastError();
+                clear_counters = true;
                 break;
             case FmhaWorkspace::kStatic:
                 if (plan.bytes > kStaticScratchBytes) return hipErrorOutOfMemory;   // the entry point checks first and says why
                 e = static_scratch_ptr(&wsp);
                 break;
             default:
-                e = decode_workspace(plan.bytes, stream, &wsp);
+                e = decode_workspace(plan.bytes, stream, &wsp, &clear_counters);
+                n_counters = kCounterBytes / (long)sizeof(unsigned);   // a fresh buffer: the whole counter region, once
                 break;
+        }
+        if (e != hipSuccess) return e;
+        if (clear_counters) {
+            fmha_decode_clear_kernel<<<dim3(4), dim3(256), 0, stream>>>(reinterpret_cast<unsigned*>(wsp), (int)n_counters);
+            e = hipGetLastError();
         }
         if (e != hipSuccess) return e;
     }

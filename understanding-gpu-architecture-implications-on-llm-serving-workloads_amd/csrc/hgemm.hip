@@ -388,10 +388,16 @@ void hgemm_main_kernel(const T* __restrict__ A, const T* __restrict__ B,
             __builtin_amdgcn_sched_barrier(0);
         });
     };
+    // the fragment reads that ride in slot m: fragments m, m + NSLOT, .. (a wave with a single row or column of blocks has
+    // more fragments than MFMAs per substep)
+    auto frags_of_slot = [&](MI355_LDS char* st, int kk, auto mc, V8(&afn)[TM], V8(&bfn)[TN]) {
+        constexpr int m = decltype(mc)::value;
+        if constexpr (m < NFRAG) load_frag(st, kk, mc, afn, bfn);
+        if constexpr (m + NSLOT < NFRAG) load_frag(st, kk, std::integral_constant<int, m + NSLOT>{}, afn, bfn);
+        static_assert(NFRAG <= 2 * NSLOT, "at most two fragment reads per slot");
+    };
     auto reads_of = [&](MI355_LDS char* st, int kk, V8(&afn)[TM], V8(&bfn)[TN]) {
-        return [&, st, kk](auto mc) {
-            if constexpr (decltype(mc)::value < NFRAG) load_frag(st, kk, mc, afn, bfn);
-        };
+        return [&, st, kk](auto mc) { frags_of_slot(st, kk, mc, afn, bfn); };
     };
     // copy d of a tile goes out in slot d * kCopySpacing of the substep behind the barrier that frees its stage: every
     // second slot where there are that many (buffer loads are cheap to issue in a row, and the earlier a copy leaves the
@@ -428,8 +434,7 @@ void hgemm_main_kernel(const T* __restrict__ A, const T* __restrict__ B,
         else wait_vmcnt<0>();
         __syncthreads();
         substep(af[1], bf[1], [&](auto mc) {
-            constexpr int m = decltype(mc)::value;
-            if constexpr (m < NFRAG) load_frag(stn, 0, mc, af[0], bf[0]);
+            frags_of_slot(stn, 0, mc, af[0], bf[0]);
             if constexpr (decltype(with_copies)::value) copies_of_slot(stage, mc);   // tile kt + NSTAGE
         });
         if constexpr (decltype(with_copies)::value) advance_copies();
@@ -965,6 +970,20 @@ static hipError_t launch_layout(const T* A, const T* B, T* C, const T* R, int M,
     const bool aligned = (reinterpret_cast<uintptr_t>(A) % 16 == 0) && (reinterpret_cast<uintptr_t>(B) % 16 == 0) &&
                          (reinterpret_cast<uintptr_t>(C) % 16 == 0) && (lda % 8 == 0) && (ldb % 8 == 0) &&
                          (ldc % 8 == 0) && (reinterpret_cast<uintptr_t>(R) % 16 == 0) && (ldr % 8 == 0);
+    // K that is not a multiple of the tiles' depth (the reference's own tiled kernels take K % 16 == 0,
+    // kernels/gemm/pkg/gemm_unified/csrc/auto/gemm_7.cu:115-135): the last K % 64 columns go through the bounds-checked
+    // kernel first, into C, and the tiled kernels then add the product over the first K - K % 64 to it as their residual
+    // (two roundings more than a single pass; a call that brings a residual of its own stays on the bounds-checked kernel,
+    // whose result is bit-identical to the product followed by an elementwise add).
+    if (aligned && R == nullptr && K > 64 && K % 64 != 0 && variant == 0) {
+        const int k_tail = K % 64, k_main = K - k_tail;
+        const T* a_tail = A_KC ? A + k_main : A + (long)k_main * lda;
+        const T* b_tail = B_KC ? B + k_main : B + (long)k_main * ldb;
+        dim3 grid((N + 63) / 64, (M + 63) / 64);
+        hgemm_edge_kernel<T, A_KC, B_KC><<<grid, dim3(256), 0, stream>>>(a_tail, b_tail, C, nullptr, M, N, k_tail, lda, ldb, ldc, 0);
+        if (hipError_t e = hipGetLastError(); e != hipSuccess) return e;
+        return launch_layout<T, A_KC, B_KC>(A, B, C, C, M, N, k_main, lda, ldb, ldc, ldc, variant, stream);
+    }
     // the tiled kernels address a tile with 32-bit byte offsets: up to 256 rows of lda (ldb) elements
     const bool k_ok = aligned && K % 64 == 0 && K >= 64 && lda < (1L << 22) && ldb < (1L << 22);
     const bool fits256 = k_ok && M % 256 == 0 && N % 256 == 0;
@@ -995,8 +1014,8 @@ static hipError_t launch_layout(const T* A, const T* B, T* C, const T* R, int M,
             return launch_main<T, A_KC, B_KC, 128, 64, 2, 2, 0, true>(A, B, C, R, M, N, K, lda, ldb, ldc, ldr, stream);
         }
     }
-    // layout NN: the N-contiguous B tile cannot be narrower than 128 columns, so the tile is halved along M (64x128);
-    // that helps products with several row tiles (1024^3), not the few-row ones
+    // layout NN halves the tile along M (64x128: an N-contiguous B tile of 128 columns keeps its 256-byte rows); that helps
+    // products with several row tiles (1024^3), not the few-row ones, which take the 64x64 tiles above
     if constexpr (A_KC && !B_KC) {
         if (few_tiles && M > 64) {
             if (M % 64 == 0 && N % 128 == 0)
@@ -1011,6 +1030,8 @@ static hipError_t launch_layout(const T* A, const T* B, T* C, const T* R, int M,
     else if (fits128) choice = 2;
     if (variant == 1 && fits256) choice = 1;
     if (variant == 2 && fits128) choice = 2;
+    if (variant == 3 && fits128) return launch_main<T, A_KC, B_KC, 128, 128, 2, 4>(A, B, C, R, M, N, K, lda, ldb, ldc, ldr, stream);
+    if (variant == 4 && fits128) return launch_main<T, A_KC, B_KC, 128, 128, 4, 2>(A, B, C, R, M, N, K, lda, ldb, ldc, ldr, stream);
     switch (choice) {
         case 1: return launch_main<T, A_KC, B_KC, 256, 256, 2, 4>(A, B, C, R, M, N, K, lda, ldb, ldc, ldr, stream);
         case 2: return launch_main<T, A_KC, B_KC, 128, 128, 2, 2>(A, B, C, R, M, N, K, lda, ldb, ldc, ldr, stream);
@@ -1028,8 +1049,9 @@ static hipError_t launch_layout(const T* A, const T* B, T* C, const T* R, int M,
     return hipGetLastError();
 }
 
-// Product with the gate/up epilogue (EPI = 1): N counts the columns of op(B) (twice those of C). Only the tiled kernels
-// have it; other shapes report hipErrorNotSupported and the caller runs the product and mi355_silu_mul separately.
+// Product with the gate/up epilogue (EPI = 1): N counts the columns of op(B) (twice those of C). Operands that are not
+// 16-byte aligned, K that is not a multiple of 64 or N that is not a multiple of 64 report hipErrorNotSupported and the
+// caller runs the product and mi355_silu_mul separately.
 template <typename T, bool A_KC, bool B_KC>
 static hipError_t launch_silu_mul(const T* A, const T* B, T* C, int M, int N, int K, long lda, long ldb,
                                   long ldc, hipStream_t stream) {
@@ -1040,7 +1062,10 @@ static hipError_t launch_silu_mul(const T* A, const T* B, T* C, int M, int N, in
     if constexpr (A_KC && B_KC) {   // generation step: the split-K small-M kernel with the same epilogue
         if (M <= 16) return launch_smallm_nt_gate_up<T>(A, B, C, M, N, K, lda, ldb, ldc, stream);
     }
-    if (M <= 64 && !few_rows_prefer_tiles(M, N, K, false)) return hipErrorNotSupported;   // the small-M product + silu_mul is faster
+    // up to 64 rows (generation steps of a few dozen sequences): 64x64 tiles with an 8-deep ring as for the plain product,
+    // four waves side by side along M so that every wave holds the gate and the up columns of its rows
+    if (M <= 64 && !few_rows_prefer_tiles(M, N, K, false))
+        return launch_main<T, A_KC, B_KC, 64, 64, 4, 1, 1, true>(A, B, C, nullptr, M, N, K, lda, ldb, ldc, 0, stream);
     const bool fits128 = M % 128 == 0 && N % 128 == 0;
     const bool fits256 = M % 256 == 0 && N % 256 == 0;
     const long t256 = (long)((M + 255) / 256) * ((N + 255) / 256);

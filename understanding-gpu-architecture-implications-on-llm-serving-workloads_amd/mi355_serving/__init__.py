@@ -176,8 +176,13 @@ def fmha_workspace_bytes(B, Hq, Hkv, Sq, Sk, kv_valid_len=None):
 def fmha_fwd_noalloc(q, k, v, out, lse=None, causal=False, kv_valid_len=None, scale=None):
     """mi355_fmha_fwd_noalloc on torch's current stream: fp16 [B, H, S, D] tensors or views with a contiguous last
     dimension; `out` (and `lse`, if wanted) are the caller's. Neither this wrapper nor the library allocates."""
+    import torch
+    assert q.dtype == k.dtype == v.dtype == out.dtype == torch.float16, "mi355_fmha_fwd_noalloc is an fp16 entry point"
+    assert q.is_cuda and q.dim() == 4 and k.dim() == 4 and v.shape == k.shape and out.shape == q.shape
+    assert q.stride(3) == 1 and k.stride(3) == 1 and v.stride(3) == 1 and out.stride(3) == 1
     B, Hq, Sq, D = q.shape
     _, Hkv, Sk, _ = k.shape
+    assert lse is None or (lse.dtype == torch.float32 and tuple(lse.shape) == (B, Hq, Sq) and lse.is_contiguous())
     arr = (ctypes.c_int64 * 12)(*(_bhs_strides(q) + _bhs_strides(k) + _bhs_strides(v) + _bhs_strides(out)))
     _check(load().mi355_fmha_fwd_noalloc(_ptr(q), _ptr(k), _ptr(v), _ptr(out), _ptr(lse), B, Hq, Hkv, Sq, Sk, D,
                                          float(1.0 / (D ** 0.5) if scale is None else scale), int(bool(causal)),
@@ -340,8 +345,8 @@ def hgemm_silu_mul(a, w, layout="NT", out=None):
     if out is None:
         out = torch.empty((M, N), dtype=a.dtype, device=a.device)
     entry = load().mi355_gemm_silu_mul_bf16 if a.dtype == torch.bfloat16 else load().mi355_hgemm_silu_mul
-    rc = entry(_ptr(a), _ptr(w), _ptr(out), M, N, K, a.stride(0), w.stride(0), out.stride(0), lay,
-                                     _stream_of(a))
+    # leading dimensions of the logical layout: a contiguous tensor with a single row may carry any stride(0)
+    rc = entry(_ptr(a), _ptr(w), _ptr(out), M, N, K, a.shape[1], w.shape[1], max(out.stride(0), N), lay, _stream_of(a))
     if rc == ERR_UNSUPPORTED:
         return silu_mul(hgemm(a, w, layout), out=out, interleave=GATE_UP_BLOCK)
     _check(rc)
