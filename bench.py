@@ -344,6 +344,13 @@ def main():
         bt = b.t().contiguous()
         ms_vt = time_launches(lambda: torch.matmul(a, bt.t(), out=cv), 20, 3)
         ms_sd = time_launches(lambda: torch.nn.functional.scaled_dot_product_attention(q, k, v, is_causal=True, enable_gqa=True), 20, 3)
+        # this library on the same NT operands (B stored [N, K]), same timing loop: the like-for-like figure next to the vendor's
+        cnt = torch.empty_like(c)
+        ms_nt = time_launches(lambda: lib.hgemm_raw(a.data_ptr(), bt.data_ptr(), cnt.data_ptr(), M, N, K, K, K, N, lib.GEMM_NT, stream), 20, 3)
+        ms_nn = time_launches(gemm, 20, 3)
+        other["hgemm_8192_same_loop_as_vendor"] = {"nn": {"ms": ms_nn, "tflops": gemm_flops / ms_nn / 1e9},
+                                                   "nt": {"ms": ms_nt, "tflops": gemm_flops / ms_nt / 1e9}}
+        del cnt
         other["vendor_libraries_same_box"] = {
             "torch_matmul_hipblaslt_8192_nn": {"ms": ms_v, "tflops": gemm_flops / ms_v / 1e9},
             "torch_matmul_hipblaslt_8192_nt": {"ms": ms_vt, "tflops": gemm_flops / ms_vt / 1e9},
@@ -536,7 +543,7 @@ def main():
     # ---- CPU baseline: the same step with torch fp32 on the host cores -------------------------------------------------
     cpu_baseline = None
     if not args.no_cpu_baseline:
-        cores = torch.get_num_threads()
+        cores = torch.get_num_threads()   # the box's CPU share for one GPU (OMP_NUM_THREADS), not every core of the host
         a32, b32 = a_h.float(), b_h.float()
         so.attention_sdpa_ref(q_h[:, :2], k_h[:, :1], v_h[:, :1], True)  # warm up the SDPA path on a small slice
         t0 = time.perf_counter()
@@ -550,8 +557,61 @@ def main():
                         "sample": "one full step on the host: torch.matmul fp32 8192^3 (%.2f s, %.3f TFLOP/s) + torch SDPA fp32 "
                                   "causal GQA F4 with repeat_kv (%.2f s, %.3f TFLOP/s algorithmic); single run, no warm-up of the GEMM"
                                   % (t_g, gemm_flops / t_g / 1e12, t_f, fmha_flops / t_f / 1e12),
-                        "cpu": _cpu_model()}
+                        "cpu": _cpu_model(), "logical_cpus_visible": os.cpu_count(), "threads_used": cores}
+        del a32, b32
+        if not args.no_other_configs:
+            # the other configurations on the same host cores (reported baselines): median of 3 runs after one warm-up, a
+            # single run for the decoder layer chain
+            def cpu_ms(fn, runs=3, warm=1):
+                for _ in range(warm):
+                    fn()
+                ts = []
+                for _ in range(runs):
+                    t0_ = time.perf_counter()
+                    fn()
+                    ts.append((time.perf_counter() - t0_) * 1e3)
+                return sorted(ts)[len(ts) // 2]
+            for name, (m_, n_, k_) in (("G1_gemm_1024", (1024, 1024, 1024)), ("G2a_gemm_4096", (4096, 4096, 4096)),
+                                       ("G2c_gemm_decode_16x14336x4096", (16, 14336, 4096))):
+                x_c, w_c = so.randn_fp16((m_, k_), 1).float(), so.randn_fp16((k_, n_), 2, 0.02).float()
+                ms_c = cpu_ms(lambda: torch.matmul(x_c, w_c))
+                other[name]["cpu_ms"] = ms_c
+                other[name]["cpu_tflops"] = 2.0 * m_ * n_ * k_ / ms_c / 1e9
+            q3c, k3c, v3c = so.fmha_inputs(4, 32, 32, 1024, 1024, seed=42)
+            ms_c = cpu_ms(lambda: so.attention_sdpa_ref(q3c, k3c, v3c, False))
+            other["F3_fmha_noncausal_b4_h32_s1024"]["cpu_ms"] = ms_c
+            other["F3_fmha_noncausal_b4_h32_s1024"]["cpu_tflops"] = 4.0 * 4 * 32 * 128 * 1024 * 1024 / ms_c / 1e9
+            del q3c, k3c, v3c
+            S5c, H5c, F5c = 8192, 4096, 14336
+            x5c = so.randn_fp16((S5c, H5c), 0)
+            w5c = [so.randn_fp16((H5c, 6144), 1, 0.02), so.randn_fp16((H5c, H5c), 2, 0.02), so.randn_fp16((H5c, 2 * F5c), 3, 0.02),
+                   so.randn_fp16((F5c, H5c), 4, 0.02)]
+            def l5_cpu():
+                # the chain of the decoder layer's matrix stages in fp32 on the host (SDPA for the attention stage)
+                qkv_c = x5c.float() @ w5c[0].float()
+                qc = qkv_c[:, :4096].reshape(S5c, 32, 128).permute(1, 0, 2)[None]
+                kc = qkv_c[:, 4096:5120].reshape(S5c, 8, 128).permute(1, 0, 2)[None]
+                vc = qkv_c[:, 5120:].reshape(S5c, 8, 128).permute(1, 0, 2)[None]
+                oc = so.attention_sdpa_ref(qc, kc, vc, True)
+                oc = (oc[0] if isinstance(oc, tuple) else oc)[0].permute(1, 0, 2).reshape(S5c, H5c)
+                gu_c = (oc @ w5c[1].float()) @ w5c[2].float()
+                return (torch.nn.functional.silu(gu_c[:, :F5c]) * gu_c[:, F5c:]) @ w5c[3].float()
+            t0 = time.perf_counter()
+            l5_cpu()
+            ms_c = (time.perf_counter() - t0) * 1e3
+            fl5 = 2.0 * S5c * H5c * 6144 + 4.0 * 32 * 128 * causal_pairs(S5c, S5c) + 2.0 * S5c * H5c * H5c + 2.0 * S5c * H5c * 2 * F5c + 2.0 * S5c * F5c * H5c
+            other["L5_llama3_8b_layer_s8192"]["cpu_ms"] = ms_c
+            other["L5_llama3_8b_layer_s8192"]["cpu_tflops"] = fl5 / ms_c / 1e9
+            other["cpu_baselines_note"] = ("cpu_ms / cpu_tflops: torch fp32 on %d threads of %s (torch.matmul; SDPA with repeat_kv; L5: the four "
+                                           "products, causal SDPA and the activation chained, one run)" % (cores, _cpu_model()))
+            del x5c, w5c
 
+    step_protocol = ("value / ms_per_step: %d steps (GEMM then attention, back to back on one stream) after %d warm-up steps, host "
+                     "clock between device synchronisations" % (args.steps, args.warmup))
+    kernel_protocol = ("kernels / roofline*: per kernel >= 10 warm-up launches, then untimed launches until ~25 ms of that kernel "
+                       "have run (clocks settle), then >= 50 launches between two HIP events on the launch stream; median / "
+                       "minimum from a second batch with an event after every launch; ms_graph_replay / other_configs GEMMs: "
+                       "the launches replayed from one HIP graph")
     out = {
         "metric": "TFLOP/s + % fp16 MFMA peak: GEMM 8192^3 and causal GQA FMHA s=4096 d=128",
         "value": value, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -559,6 +619,7 @@ def main():
         "dtype": "fp16 (fp32 accumulate)", "data": "synthetic",
         "config": {"workload": "one step = hgemm 8192x8192x8192 NN (G2b) + fmha fwd causal GQA b1 h32/8 s4096 d128 with LSE (F4)",
                    "flops_per_step": gemm_flops + fmha_flops, "pct_of_fp16_mfma_peak": 100 * value / PEAK_FP16_TFLOPS},
+        "step_protocol": step_protocol, "kernel_protocol": kernel_protocol,
         "kernels": kernels, "roofline": roofline, "roofline_fmha": roofline_fmha, "roofline_decode_gemm": roofline_g2c,
         "cpu_baseline": cpu_baseline,
         "other_configs": other, "parity": checks,
@@ -579,10 +640,10 @@ KERNEL_CONFIGS = {
     "gemm_64x14336x4096_nt": ("gemm", 64, 14336, 4096, "NT"),               # 64x64 tiles, 8-deep ring
     "gemm_16x4096x14336_nt": ("gemm", 16, 4096, 14336, "NT"),               # split-K small-M kernel (NT)
     "gemm_1024x4096x4096_nt": ("gemm", 1024, 4096, 4096, "NT"),             # 128x64 tiles
-    "f3_fmha_noncausal_b4_h32_s1024": ("fmha", 4, 32, 32, 1024, 1024, False),   # ping-pong kernel
+    "f3_fmha_noncausal_b4_h32_s1024": ("fmha", 4, 32, 32, 1024, 1024, False),   # ping-pong kernel, 256-query work items
     "f4_fmha_causal_gqa_s4096": ("fmha", 1, 32, 8, 4096, 4096, True),           # ping-pong kernel
     "l5_fmha_causal_gqa_s8192": ("fmha", 1, 32, 8, 8192, 8192, True),           # ping-pong kernel
-    "fmha_causal_gqa_s1024": ("fmha", 1, 32, 8, 1024, 1024, True),              # 4-wave kernel (128 workgroups of 256 queries would not fill the CUs)
+    "fmha_causal_gqa_s1024": ("fmha", 1, 32, 8, 1024, 1024, True),              # ping-pong kernel, 128-query work items (128 items of 256 queries would not fill the CUs)
     "fmha_decode_b1_sk8192": ("fmha", 1, 32, 8, 1, 8192, False),                # split-KV kernel
     "fmha_decode_b8_sk8192": ("fmha", 8, 32, 8, 1, 8192, False),
     "fmha_decode_b64_sk8192": ("fmha", 64, 32, 8, 1, 8192, False),              # one key range per (batch, kv head)
