@@ -34,6 +34,10 @@ DEVICE_FLAGS = [
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
 ]
 KERNEL_SOURCES = ["csrc/hgemm.hip", "csrc/fmha_fwd.hip", "csrc/fmha_decode.hip", "csrc/glue.hip", "csrc/capi.hip"]
+# A source listed here is compiled once per entry, each time with that entry's defines, into objects of its own (side by
+# side with the others): the GEMM source holds every tile shape for two element types and three layouts, and one
+# compiler process per element type halves the time the build waits for it.
+SOURCE_PARTS = {"csrc/hgemm.hip": (("fp16", ["-DMI355_HGEMM_PART=0"]), ("bf16", ["-DMI355_HGEMM_PART=1"]))}
 # Per-source additions. The GEMM keeps its MFMA accumulators in ordinary VGPRs: left to itself the compiler moves part of
 # them to AGPRs in the 4-wave kernels and then shuffles them back and forth inside the K loop.
 SOURCE_FLAGS = {"csrc/hgemm.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"]}
@@ -85,28 +89,31 @@ def build_library(verbose=True):
     check_archs()
     with tempfile.TemporaryDirectory(prefix="mi355_build_") as tmp:
         jobs = []
+        objs, tl_objs = [], []
+
+        def add(src, defines, suffix):
+            made = []
+            for tag, part_defines in SOURCE_PARTS.get(src, (("", []),)):
+                obj = os.path.join(tmp, os.path.basename(src) + (("." + tag) if tag else "") + suffix + ".o")
+                cmd = [HIPCC] + DEVICE_FLAGS + SOURCE_FLAGS.get(src, []) + part_defines + defines + ["-I", INCLUDE, "-c", src, "-o", obj]
+                jobs.append((cmd, obj))
+                made.append(obj)
+            return made
+
         for src in KERNEL_SOURCES:
-            obj = os.path.join(tmp, os.path.basename(src) + ".o")
-            cmd = [HIPCC] + DEVICE_FLAGS + SOURCE_FLAGS.get(src, []) + ["-I", INCLUDE, "-c", src, "-o", obj]
-            jobs.append((cmd, obj))
-        tl_objs = {}
-        for src in TIMELINE_SOURCES:
-            obj = os.path.join(tmp, os.path.basename(src) + ".timeline.o")
-            cmd = [HIPCC] + DEVICE_FLAGS + SOURCE_FLAGS.get(src, []) + ["-DMI355_TIMELINE", "-I", INCLUDE, "-c", src, "-o", obj]
-            jobs.append((cmd, obj))
-            tl_objs[src] = obj
-        tl_extra = []
+            plain = add(src, [], "")
+            objs += plain
+            tl_objs += add(src, ["-DMI355_TIMELINE"], ".timeline") if src in TIMELINE_SOURCES else plain
         for src in TIMELINE_ONLY_SOURCES:
-            obj = os.path.join(tmp, os.path.basename(src) + ".timeline.o")
-            jobs.append(([HIPCC] + DEVICE_FLAGS + ["-DMI355_TIMELINE", "-I", INCLUDE, "-c", src, "-o", obj], obj))
-            tl_extra.append(obj)
+            tl_objs += add(src, ["-DMI355_TIMELINE"], ".timeline")
+        # the longest compilations first, so that they do not start behind the short ones
+        jobs.sort(key=lambda job: 0 if "hgemm" in job[1] else 1 if "fmha_fwd" in job[1] else 2)
         if verbose:
             for cmd, _ in jobs:
                 print("[build] " + " ".join(cmd))
         with ThreadPoolExecutor(max_workers=max_jobs(len(jobs))) as pool:
             list(pool.map(lambda job: _run(job[0]), jobs))
-        objs = [os.path.join(tmp, os.path.basename(src) + ".o") for src in KERNEL_SOURCES]
-        for out, these in ((LIB_PATH, objs), (TIMELINE_LIB_PATH, [tl_objs.get(src, o) for src, o in zip(KERNEL_SOURCES, objs)] + tl_extra)):
+        for out, these in ((LIB_PATH, objs), (TIMELINE_LIB_PATH, tl_objs)):
             link = [HIPCC, "--offload-arch=gfx950", "-fPIC", "-shared"] + these + ["-o", out]
             if verbose:
                 print("[build] " + " ".join(link))

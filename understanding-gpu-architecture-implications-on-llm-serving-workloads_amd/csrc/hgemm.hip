@@ -13,6 +13,13 @@
 //     The copies are buffer loads (scalar tile base + one 32-bit lane offset): a global load with 64-bit lane
 //     addresses takes about twice as much issue time away from the MFMAs it runs beside, and several times as
 //     much when such loads are issued back to back.
+//   * a wave issues an instruction every ~5 cycles at best and every ~10 next to its SIMD partner's MFMAs, whatever the
+//     instruction, so the K loop is kept short: it is unrolled over the ring, which makes every LDS address a
+//     loop-invariant register plus an immediate (A's stages lie one behind the other, then B's, so that one register
+//     reaches all stages of an operand) and every copy destination a scalar plus an immediate; the tile bases advance
+//     inside their buffer resources; every tile issues the same instructions (the copies of the last tiles run on a
+//     resource whose size is set to zero: out of range, nothing is fetched), so the waits never change and the loop has
+//     one body per stage. Per K tile and wave of the 256x256 kernel: 64 MFMAs and ~58 other instructions.
 //   * an operand whose K index is contiguous in memory is read from LDS with ds_read_b128; an operand whose
 //     M/N index is contiguous (B in the NN case) is read with the transposing ds_read_b64_tr_b16, so no
 //     transpose pass over B is ever made.
@@ -145,6 +152,14 @@ struct MainCfg {
     static constexpr int B_INSTS = B_BYTES / (NWAVES * 1024);
     static constexpr int FRAG_SLOTS = TM > TN ? TM : TN;
 };
+
+// x < 0 ? -1 : 0 of a wave-uniform value, computed and kept on the scalar unit (written as a shift or a select, the
+// compiler may carry the result, and every value formed from it, in vector registers)
+__device__ __forceinline__ int sign_mask_scalar(int x) {
+    int r;
+    asm("s_ashr_i32 %0, %1, 31" : "=s"(r) : "s"(x) : "scc");
+    return r;
+}
 
 // f(std::integral_constant<int, I>) for I = BEGIN .. END-1, unrolled at compile time
 template <int BEGIN, int END, class F>
@@ -287,21 +302,39 @@ void hgemm_main_kernel(const T* __restrict__ A, const T* __restrict__ B,
     // A fragments: TM blocks of 16 rows; B fragments: TN blocks of 16 columns; a K tile is two 32-deep substeps.
     constexpr int NSUB = BK / 32;
     static_assert(NSUB == 2, "the pipeline below is written for two substeps per K tile");
-    int a_off[Cfg::FRAG_SLOTS];  // K-contiguous operand: one per k-substep; M/N-contiguous: one per 16-wide block
-    int b_off[Cfg::FRAG_SLOTS];
-    if constexpr (A_KC) {
+    // LDS layout: the NSTAGE stages of A one behind the other, then those of B. A stage index is a compile-time constant
+    // wherever fragments are read (the K loop is unrolled over the ring), so a fragment address is a loop-invariant
+    // register plus an immediate offset and the loop holds no address arithmetic. The immediate field of an LDS read
+    // reaches 64 KiB: where an operand's ring is longer than that (less the largest offset inside a stage), its stages
+    // are grouped into sets within reach, one register per set.
+    constexpr int kAImm = A_KC ? (TM - 1) * 16 * ATK::kRowBytes : 36 * ATM::kRowBytes;   // largest offset inside a stage
+    constexpr int kBImm = B_KC ? (TN - 1) * 16 * BTK::kRowBytes : 36 * BTN::kRowBytes;
+    constexpr int kAPerSet = (65535 - kAImm) / Cfg::A_BYTES + 1, kBPerSet = (65535 - kBImm) / Cfg::B_BYTES + 1;
+    constexpr int kASets = (Cfg::NSTAGE + kAPerSet - 1) / kAPerSet, kBSets = (Cfg::NSTAGE + kBPerSet - 1) / kBPerSet;
+    constexpr int kBRegion = Cfg::NSTAGE * Cfg::A_BYTES;
+    MI355_LDS char* a_ptr[kASets][Cfg::FRAG_SLOTS];  // K-contiguous operand: one per k-substep; M/N-contiguous: one per 16-wide block
+    MI355_LDS char* b_ptr[kBSets][Cfg::FRAG_SLOTS];
 #pragma unroll
-        for (int kk = 0; kk < NSUB; ++kk) a_off[kk] = ATK::frag_offset(wm * TM * 16, kk, lane);
-    } else {
+    for (int s = 0; s < kASets; ++s) {
+        MI355_LDS char* base = smem + s * kAPerSet * Cfg::A_BYTES;
+        if constexpr (A_KC) {
 #pragma unroll
-        for (int i = 0; i < TM; ++i) a_off[i] = ATM::frag_offset(wm * TM * 16 + i * 16, lane);
+            for (int kk = 0; kk < NSUB; ++kk) a_ptr[s][kk] = base + ATK::frag_offset(wm * TM * 16, kk, lane);
+        } else {
+#pragma unroll
+            for (int i = 0; i < TM; ++i) a_ptr[s][i] = base + ATM::frag_offset(wm * TM * 16 + i * 16, lane);
+        }
     }
-    if constexpr (B_KC) {
 #pragma unroll
-        for (int kk = 0; kk < NSUB; ++kk) b_off[kk] = Cfg::A_BYTES + BTK::frag_offset(wn * TN * 16, kk, lane);
-    } else {
+    for (int s = 0; s < kBSets; ++s) {
+        MI355_LDS char* base = smem + kBRegion + s * kBPerSet * Cfg::B_BYTES;
+        if constexpr (B_KC) {
 #pragma unroll
-        for (int j = 0; j < TN; ++j) b_off[j] = Cfg::A_BYTES + BTN::frag_offset(wn * TN * 16 + j * 16, lane);
+            for (int kk = 0; kk < NSUB; ++kk) b_ptr[s][kk] = base + BTK::frag_offset(wn * TN * 16, kk, lane);
+        } else {
+#pragma unroll
+            for (int j = 0; j < TN; ++j) b_ptr[s][j] = base + BTN::frag_offset(wn * TN * 16 + j * 16, lane);
+        }
     }
 
     float4v acc[TM][TN];
@@ -324,53 +357,69 @@ void hgemm_main_kernel(const T* __restrict__ A, const T* __restrict__ B,
     constexpr int NFRAG = TM + TN;
     constexpr int NCOPY = Cfg::A_INSTS + Cfg::B_INSTS;
     // fragment f of substep kk, f in the order of first use: A0, B0 .. B(TN-1), A1 .. A(TM-1)
-    auto load_frag = [&](MI355_LDS char* st, int kk, auto fc, V8(&afn)[TM], V8(&bfn)[TN]) {
-        constexpr int f = decltype(fc)::value;
+    auto load_frag = [&](auto sc, auto kc, auto fc, V8(&afn)[TM], V8(&bfn)[TN]) {
+        constexpr int f = decltype(fc)::value, kk = decltype(kc)::value;
+        constexpr int st = decltype(sc)::value;
+        constexpr int aset = st / kAPerSet, ao = (st % kAPerSet) * Cfg::A_BYTES;   // set, and stage offset inside it
+        constexpr int bset = st / kBPerSet, bo = (st % kBPerSet) * Cfg::B_BYTES;
         if constexpr (f == 0 || f > TN) {
             constexpr int i = f == 0 ? 0 : f - TN;
             if constexpr (A_KC) {
-                afn[i] = Elem<T>::frag(lds_read_b128(st + a_off[kk] + i * 16 * ATK::kRowBytes));
+                afn[i] = Elem<T>::frag(lds_read_b128(a_ptr[aset][kk] + (ao + i * 16 * ATK::kRowBytes)));
             } else {
-                half4 lo = lds_read_tr16_b64(st + a_off[i] + (kk * 32) * ATM::kRowBytes);
-                half4 hi = lds_read_tr16_b64(st + a_off[i] + (kk * 32 + 4) * ATM::kRowBytes);
+                half4 lo = lds_read_tr16_b64(a_ptr[aset][i] + (ao + (kk * 32) * ATM::kRowBytes));
+                half4 hi = lds_read_tr16_b64(a_ptr[aset][i] + (ao + (kk * 32 + 4) * ATM::kRowBytes));
                 afn[i] = Elem<T>::frag(concat(lo, hi));
             }
         } else {
             constexpr int j = f - 1;
             if constexpr (B_KC) {
-                bfn[j] = Elem<T>::frag(lds_read_b128(st + b_off[kk] + j * 16 * BTK::kRowBytes));
+                bfn[j] = Elem<T>::frag(lds_read_b128(b_ptr[bset][kk] + (bo + j * 16 * BTK::kRowBytes)));
             } else {
-                half4 lo = lds_read_tr16_b64(st + b_off[j] + (kk * 32) * BTN::kRowBytes);
-                half4 hi = lds_read_tr16_b64(st + b_off[j] + (kk * 32 + 4) * BTN::kRowBytes);
+                half4 lo = lds_read_tr16_b64(b_ptr[bset][j] + (bo + (kk * 32) * BTN::kRowBytes));
+                half4 hi = lds_read_tr16_b64(b_ptr[bset][j] + (bo + (kk * 32 + 4) * BTN::kRowBytes));
                 bfn[j] = Elem<T>::frag(concat(lo, hi));
             }
         }
     };
-    auto load_frags = [&](MI355_LDS char* st, int kk, V8(&afn)[TM], V8(&bfn)[TN]) {
-        static_for<0, NFRAG>([&](auto fc) { load_frag(st, kk, fc, afn, bfn); });
+    auto load_frags = [&](auto sc, auto kc, V8(&afn)[TM], V8(&bfn)[TN]) {
+        static_for<0, NFRAG>([&](auto fc) { load_frag(sc, kc, fc, afn, bfn); });
     };
-    auto issue_copy = [&](int stage, auto dc) {
-        constexpr int d = decltype(dc)::value;
-        MI355_LDS char* sa = smem + stage * Cfg::STAGE_BYTES;
-        if constexpr (d < Cfg::A_INSTS) {
-            MI355_LDS char* dst = sa + (d * Cfg::NWAVES + wave) * 1024;
-            if constexpr (RAGGED) copy16_buffer_to_lds(a_res, a_voff[d], 0u, dst);
-            else copy16_buffer_to_lds(a_res, a_lane_off, d * a_copy_step, dst);
+    // copy d of a stage lands at (stage, operand, d) + this wave's 1 KiB slice: a scalar register plus an immediate
+    const uint32_t wave_lds = (uint32_t)(uintptr_t)(smem + wave * 1024);
+    // part selects what is issued: 0 = the whole copy, 1 = only the scalar instruction that points M0 at the destination,
+    // 2 = only the load (M0 was set a slot earlier, the matrix instruction in between is the wait state M0 needs)
+    auto issue_copy = [&](auto sc, auto dc, auto part) {
+        constexpr int d = decltype(dc)::value, pt = decltype(part)::value;
+        constexpr int st = decltype(sc)::value;
+        constexpr bool is_a = d < Cfg::A_INSTS;
+        constexpr int e = is_a ? d : d - Cfg::A_INSTS;
+        constexpr int dst = is_a ? st * Cfg::A_BYTES + e * Cfg::NWAVES * 1024 : kBRegion + st * Cfg::B_BYTES + e * Cfg::NWAVES * 1024;
+        if constexpr (pt == 1) {
+            set_m0_at<dst>(wave_lds);
         } else {
-            constexpr int e = d - Cfg::A_INSTS;
-            MI355_LDS char* dst = sa + Cfg::A_BYTES + (e * Cfg::NWAVES + wave) * 1024;
-            if constexpr (RAGGED) copy16_buffer_to_lds(b_res, b_voff[e], 0u, dst);
-            else copy16_buffer_to_lds(b_res, b_lane_off, e * b_copy_step, dst);
+            const int4v& res = is_a ? a_res : b_res;
+            uint32_t voff, soff = 0u;
+            if constexpr (RAGGED && is_a) voff = a_voff[e];
+            else if constexpr (RAGGED) voff = b_voff[e];
+            else { voff = is_a ? a_lane_off : b_lane_off; soff = e * (is_a ? a_copy_step : b_copy_step); }
+            if constexpr (pt == 0) copy16_buffer_to_lds_at<dst>(res, voff, soff, wave_lds);
+            else copy16_buffer_to_lds_m0(res, voff, soff);
         }
     };
-    auto advance_copies = [&]() {   // next K tile: scalar arithmetic on the two bases
-        a_base += a_k_step;
-        b_base += b_k_step;
-        a_res = make_buffer_resource(a_base);
-        b_res = make_buffer_resource(b_base);
+    // next K tile: the two bases advance inside their resource words (two scalar instructions each; the bases are
+    // 48-bit addresses, so the carry into word 1 stays inside its address field)
+    auto advance_base = [](int4v& res, long step) {
+        const uint64_t b = (((uint64_t)(uint32_t)res[1] << 32) | (uint32_t)res[0]) + (uint64_t)step;
+        res[0] = __builtin_amdgcn_readfirstlane((int)(uint32_t)b);
+        res[1] = __builtin_amdgcn_readfirstlane((int)(uint32_t)(b >> 32));
     };
-    auto issue_copies = [&](int stage) {
-        static_for<0, NCOPY>([&](auto dc) { issue_copy(stage, dc); });
+    auto advance_copies = [&]() {
+        advance_base(a_res, a_k_step);
+        advance_base(b_res, b_k_step);
+    };
+    auto issue_copies = [&](auto sc) {
+        static_for<0, NCOPY>([&](auto dc) { issue_copy(sc, dc, std::integral_constant<int, 0>{}); });
         advance_copies();
     };
     // The MFMA is issued with the B fragment as first operand, i.e. it produces the transposed block: lane l ends up
@@ -390,25 +439,37 @@ void hgemm_main_kernel(const T* __restrict__ A, const T* __restrict__ B,
     };
     // the fragment reads that ride in slot m: fragments m, m + NSLOT, .. (a wave with a single row or column of blocks has
     // more fragments than MFMAs per substep)
-    auto frags_of_slot = [&](MI355_LDS char* st, int kk, auto mc, V8(&afn)[TM], V8(&bfn)[TN]) {
+    auto frags_of_slot = [&](auto sc, auto kc, auto mc, V8(&afn)[TM], V8(&bfn)[TN]) {
         constexpr int m = decltype(mc)::value;
-        if constexpr (m < NFRAG) load_frag(st, kk, mc, afn, bfn);
-        if constexpr (m + NSLOT < NFRAG) load_frag(st, kk, std::integral_constant<int, m + NSLOT>{}, afn, bfn);
+        if constexpr (m < NFRAG) load_frag(sc, kc, mc, afn, bfn);
+        if constexpr (m + NSLOT < NFRAG) load_frag(sc, kc, std::integral_constant<int, m + NSLOT>{}, afn, bfn);
         static_assert(NFRAG <= 2 * NSLOT, "at most two fragment reads per slot");
-    };
-    auto reads_of = [&](MI355_LDS char* st, int kk, V8(&afn)[TM], V8(&bfn)[TN]) {
-        return [&, st, kk](auto mc) { frags_of_slot(st, kk, mc, afn, bfn); };
     };
     // copy d of a tile goes out in slot d * kCopySpacing of the substep behind the barrier that frees its stage: every
     // second slot where there are that many (buffer loads are cheap to issue in a row, and the earlier a copy leaves the
     // more time it has to land), evenly over the substep otherwise
     constexpr int kCopySpacingNum = NSLOT >= 2 * NCOPY ? 8 : 4 * NSLOT / NCOPY, kCopySpacingDen = 4;
     static_assert((NCOPY - 1) * kCopySpacingNum / kCopySpacingDen < NSLOT, "copies go out within one substep");
-    auto copies_of_slot = [&](int stage, auto gc) {   // issue the copies whose slot is g
+    // where a substep has a slot to spare, M0 is set one slot ahead of its load
+#ifdef MI355_GEMM_NO_SPLIT_M0
+    constexpr bool kSplitM0 = false;
+#else
+    constexpr bool kSplitM0 = (NCOPY - 1) * kCopySpacingNum / kCopySpacingDen + 1 < NSLOT;
+#endif
+    auto copies_of_slot = [&](auto sc, auto gc) {   // issue the copies whose slot is g
         constexpr int g = decltype(gc)::value;
         static_for<0, NCOPY>([&](auto dc) {
-            if constexpr (decltype(dc)::value * kCopySpacingNum / kCopySpacingDen == g) issue_copy(stage, dc);
+            constexpr int slot = decltype(dc)::value * kCopySpacingNum / kCopySpacingDen;
+            if constexpr (!kSplitM0) {
+                if constexpr (slot == g) issue_copy(sc, dc, std::integral_constant<int, 0>{});
+            } else {
+                if constexpr (slot + 1 == g) issue_copy(sc, dc, std::integral_constant<int, 2>{});
+            }
         });
+        if constexpr (kSplitM0)
+            static_for<0, NCOPY>([&](auto dc) {
+                if constexpr (decltype(dc)::value * kCopySpacingNum / kCopySpacingDen == g) issue_copy(sc, dc, std::integral_constant<int, 1>{});
+            });
     };
     // Ring of NSTAGE stages, tile t in stage t % NSTAGE. The prologue fills every stage; in tile kt, behind the barrier,
     // the copies of tile kt + NSTAGE go into the stage tile kt has just left. At that barrier tile kt+1 must have
@@ -416,39 +477,43 @@ void hgemm_main_kernel(const T* __restrict__ A, const T* __restrict__ B,
     constexpr int NSTAGE = Cfg::NSTAGE;
     const int ktiles = K / BK;
     V8 af[2][TM], bf[2][TN];
-    for (int t = 0; t < NSTAGE && t < ktiles; ++t) issue_copies(t);
-    if (ktiles >= NSTAGE) wait_vmcnt<NCOPY * (NSTAGE - 1)>();
-    else wait_vmcnt<0>();
+    using Sub0 = std::integral_constant<int, 0>;
+    using Sub1 = std::integral_constant<int, 1>;
+    static_for<0, NSTAGE>([&](auto sc) {
+        const int records = sign_mask_scalar(decltype(sc)::value - ktiles);
+        a_res[2] = records;
+        b_res[2] = records;
+        issue_copies(sc);
+    });
+    wait_vmcnt<NCOPY * (NSTAGE - 1)>();
     __syncthreads();
-    load_frags(smem, 0, af[0], bf[0]);
+    load_frags(Sub0{}, Sub0{}, af[0], bf[0]);
 
-    int stage = 0;   // kt % NSTAGE
-    auto tile = [&](auto with_copies) {
-        const int next = stage + 1 == NSTAGE ? 0 : stage + 1;
-        MI355_LDS char* st = smem + stage * Cfg::STAGE_BYTES;
-        MI355_LDS char* stn = smem + next * Cfg::STAGE_BYTES;
-        substep(af[0], bf[0], reads_of(st, 1, af[1], bf[1]));
+    // One K tile in stage sc (a compile-time constant: the loop below is unrolled over the ring). Every tile issues the
+    // same instructions, so the count the waits rely on never changes: once no tile is left to fetch, the copies run on
+    // an empty buffer (num_records = 0: out of range, nothing is fetched).
+    auto tile = [&](auto sc, int kt) {
+        using Next = std::integral_constant<int, (decltype(sc)::value + 1) % NSTAGE>;
+        substep(af[0], bf[0], [&](auto mc) { frags_of_slot(sc, Sub1{}, mc, af[1], bf[1]); });
         // my copies of the next tile have landed and my reads of this stage are complete; after the barrier that holds
         // for every wave, so this stage may be refilled and the next one may be read
-        if constexpr (decltype(with_copies)::value) wait_vmcnt<NCOPY * (NSTAGE - 2)>();
-        else wait_vmcnt<0>();
+        wait_vmcnt<NCOPY * (NSTAGE - 2)>();
         __syncthreads();
+        const int records = sign_mask_scalar(kt + NSTAGE - ktiles);   // -1 while a tile is left to fetch, else 0
+        a_res[2] = records;
+        b_res[2] = records;
         substep(af[1], bf[1], [&](auto mc) {
-            frags_of_slot(stn, 0, mc, af[0], bf[0]);
-            if constexpr (decltype(with_copies)::value) copies_of_slot(stage, mc);   // tile kt + NSTAGE
+            frags_of_slot(Next{}, Sub0{}, mc, af[0], bf[0]);
+            copies_of_slot(sc, mc);   // tile kt + NSTAGE
         });
-        if constexpr (decltype(with_copies)::value) advance_copies();
-        stage = next;
+        advance_copies();
     };
     int kt = 0;
     MI355_TL(tl_w[1] = timeline::wall_clock(); tl_c[0] = timeline::shader_cycles();)
-    for (; kt + NSTAGE < ktiles; ++kt) tile(std::true_type{});
-    for (; kt + 1 < ktiles; ++kt) tile(std::false_type{});
-    {  // last tile: nothing left to fetch
-        MI355_LDS char* st = smem + stage * Cfg::STAGE_BYTES;
-        substep(af[0], bf[0], reads_of(st, 1, af[1], bf[1]));
-        substep(af[1], bf[1], [](auto) {});
-    }
+    for (; kt < ktiles; kt += NSTAGE)
+        static_for<0, NSTAGE>([&](auto sc) {
+            if (kt + decltype(sc)::value < ktiles) tile(sc, kt + decltype(sc)::value);
+        });
     MI355_TL(tl_w[2] = timeline::wall_clock(); tl_c[1] = timeline::shader_cycles();)
 
     // ---- epilogue ------------------------------------------------------------------------------------------------
@@ -466,6 +531,7 @@ void hgemm_main_kernel(const T* __restrict__ A, const T* __restrict__ B,
     constexpr int kRowsPerStore = 64 / kChunksC;  // rows covered by one store instruction
     constexpr int kSwzC = kChunksC < 8 ? kChunksC - 1 : 7;
     static_assert(Cfg::NWAVES * TM * 16 * kRowBytesC <= Cfg::LDS_BYTES, "epilogue staging does not fit in LDS");
+    wait_vmcnt<0>();  // the last tiles' copies (on the empty buffer) have written their zeros
     __syncthreads();  // every wave has finished reading the operand stages
     MI355_LDS char* cst = smem + wave * (TM * 16 * kRowBytesC);
     {
@@ -1030,8 +1096,6 @@ static hipError_t launch_layout(const T* A, const T* B, T* C, const T* R, int M,
     else if (fits128) choice = 2;
     if (variant == 1 && fits256) choice = 1;
     if (variant == 2 && fits128) choice = 2;
-    if (variant == 3 && fits128) return launch_main<T, A_KC, B_KC, 128, 128, 2, 4>(A, B, C, R, M, N, K, lda, ldb, ldc, ldr, stream);
-    if (variant == 4 && fits128) return launch_main<T, A_KC, B_KC, 128, 128, 4, 2>(A, B, C, R, M, N, K, lda, ldb, ldc, ldr, stream);
     switch (choice) {
         case 1: return launch_main<T, A_KC, B_KC, 256, 256, 2, 4>(A, B, C, R, M, N, K, lda, ldb, ldc, ldr, stream);
         case 2: return launch_main<T, A_KC, B_KC, 128, 128, 2, 2>(A, B, C, R, M, N, K, lda, ldb, ldc, ldr, stream);
@@ -1090,11 +1154,26 @@ static hipError_t silu_mul_dispatch_t(const void* A, const void* B, void* C, int
     }
 }
 
+// MI355_HGEMM_PART: undefined = everything in this translation unit; 0 = the fp16 kernels and the two entry points, 1 =
+// only the bf16 kernels behind the two *_bf16 functions (the build compiles the two parts side by side).
+hipError_t hgemm_dispatch_bf16(const void* A, const void* B, void* C, const void* R, int M, int N, int K, long lda, long ldb,
+                               long ldc, long ldr, int layout, int variant, hipStream_t stream);
+hipError_t hgemm_silu_mul_dispatch_bf16(const void* A, const void* B, void* C, int M, int N2, int K, long lda, long ldb,
+                                        long ldc, int layout, hipStream_t stream);
+
+#if !defined(MI355_HGEMM_PART) || MI355_HGEMM_PART == 1
+hipError_t hgemm_silu_mul_dispatch_bf16(const void* A, const void* B, void* C, int M, int N2, int K, long lda, long ldb,
+                                        long ldc, int layout, hipStream_t stream) {
+    return silu_mul_dispatch_t<bf16_t>(A, B, C, M, N2, K, lda, ldb, ldc, layout, stream);
+}
+#endif
+#if !defined(MI355_HGEMM_PART) || MI355_HGEMM_PART == 0
 hipError_t hgemm_silu_mul_dispatch(const void* A, const void* B, void* C, int M, int N2, int K, long lda, long ldb, long ldc,
                                    int layout, int dtype, hipStream_t stream) {
-    if (dtype == MI355_DTYPE_BF16) return silu_mul_dispatch_t<bf16_t>(A, B, C, M, N2, K, lda, ldb, ldc, layout, stream);
+    if (dtype == MI355_DTYPE_BF16) return hgemm_silu_mul_dispatch_bf16(A, B, C, M, N2, K, lda, ldb, ldc, layout, stream);
     return silu_mul_dispatch_t<half_t>(A, B, C, M, N2, K, lda, ldb, ldc, layout, stream);
 }
+#endif
 
 template <typename T>
 static hipError_t gemm_dispatch_t(const void* A, const void* B, void* C, const void* R, int M, int N, int K, long lda,
@@ -1111,16 +1190,24 @@ static hipError_t gemm_dispatch_t(const void* A, const void* B, void* C, const v
     }
 }
 
+#if !defined(MI355_HGEMM_PART) || MI355_HGEMM_PART == 1
+hipError_t hgemm_dispatch_bf16(const void* A, const void* B, void* C, const void* R, int M, int N, int K, long lda, long ldb,
+                               long ldc, long ldr, int layout, int variant, hipStream_t stream) {
+    return gemm_dispatch_t<bf16_t>(A, B, C, R, M, N, K, lda, ldb, ldc, ldr, layout, variant, stream);
+}
+#endif
+#if !defined(MI355_HGEMM_PART) || MI355_HGEMM_PART == 0
 hipError_t hgemm_dispatch(const void* A, const void* B, void* C, const void* R, int M, int N, int K, long lda, long ldb,
                           long ldc, long ldr, int layout, int dtype, int variant, hipStream_t stream) {
-    if (dtype == MI355_DTYPE_BF16) return gemm_dispatch_t<bf16_t>(A, B, C, R, M, N, K, lda, ldb, ldc, ldr, layout, variant, stream);
+    if (dtype == MI355_DTYPE_BF16) return hgemm_dispatch_bf16(A, B, C, R, M, N, K, lda, ldb, ldc, ldr, layout, variant, stream);
     return gemm_dispatch_t<half_t>(A, B, C, R, M, N, K, lda, ldb, ldc, ldr, layout, variant, stream);
 }
+#endif
 
 }  // namespace mi355
 
-#ifdef MI355_TIMELINE
-// profiling build: copies the records of the last tiled GEMM launch (kMaxWorkgroups x kSlots 64-bit values) to the host
+#if defined(MI355_TIMELINE) && (!defined(MI355_HGEMM_PART) || MI355_HGEMM_PART == 0)
+// profiling build: copies the records of the last tiled fp16 GEMM launch (kMaxWorkgroups x kSlots 64-bit values) to the host
 extern "C" int mi355_timeline_read_hgemm(void* dst, size_t bytes) {
     const size_t all = sizeof(unsigned long long) * mi355::timeline::kMaxWorkgroups * mi355::timeline::kSlots;
     return (int)hipMemcpyFromSymbol(dst, HIP_SYMBOL(mi355::hgemm_stamps), bytes < all ? bytes : all);

@@ -99,6 +99,31 @@ __device__ __forceinline__ void copy16_buffer_to_lds(int4v resource, uint32_t la
         : "memory", "m0");
 }
 
+// The same with the LDS destination given as a scalar register plus a compile-time offset: one scalar instruction sets
+// M0 (a copy whose destination is a run-time value needs a second one to form it).
+template <int IMM>
+__device__ __forceinline__ void copy16_buffer_to_lds_at(int4v resource, uint32_t lane_byte_offset, uint32_t uniform_byte_offset,
+                                                        uint32_t lds_wave_base) {
+    asm volatile(
+        "s_add_u32 m0, %3, %4\n\t"
+        "s_nop 0\n\t"
+        "buffer_load_dwordx4 %0, %1, %2 offen lds"
+        :
+        : "v"(lane_byte_offset), "s"(resource), "s"(uniform_byte_offset), "s"(lds_wave_base), "n"(IMM)
+        : "memory", "m0", "scc");
+}
+
+// The two halves of the copy above for code that can place an unrelated instruction between them (M0 needs one wait
+// state between the scalar write and the load that uses it; any instruction serves). Nothing else may write M0 in between:
+// the compiler uses M0 only for instructions this library does not contain (LDS-direct and GWS operations, s_movrel).
+template <int IMM>
+__device__ __forceinline__ void set_m0_at(uint32_t lds_wave_base) {
+    asm volatile("s_add_u32 m0, %0, %1" : : "s"(lds_wave_base), "n"(IMM) : "m0", "scc");
+}
+__device__ __forceinline__ void copy16_buffer_to_lds_m0(int4v resource, uint32_t lane_byte_offset, uint32_t uniform_byte_offset) {
+    asm volatile("buffer_load_dwordx4 %0, %1, %2 offen lds" : : "v"(lane_byte_offset), "s"(resource), "s"(uniform_byte_offset) : "memory");
+}
+
 __device__ __forceinline__ half4 lds_read_tr16_b64(MI355_LDS const void* p) {
     short4v t = __builtin_amdgcn_ds_read_tr16_b64_v4i16((MI355_LDS short4v*)p);
     return __builtin_bit_cast(half4, t);
