@@ -88,7 +88,7 @@ def test_layouts_and_shapes(lib, gpu, layout, M, N, K):
     assert c.shape == (M, N)
 
 
-@pytest.mark.parametrize("variant", [0, 1, 2])
+@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4])
 @pytest.mark.parametrize("layout", ["NN", "TN", "NT"])
 @pytest.mark.parametrize("M,N,K", [(1000, 1000, 1024), (300, 4096, 512), (2056, 1032, 128), (130, 8, 64), (4104, 4096, 256),
                                    (257, 264, 64)])
@@ -116,7 +116,7 @@ def test_k_that_is_a_multiple_of_16_but_not_of_the_tile_depth(lib, gpu, layout, 
     check(lib, gpu, a, b, layout, K)
 
 
-@pytest.mark.parametrize("variant", [1, 2])
+@pytest.mark.parametrize("variant", [1, 2, 3, 4])
 @pytest.mark.parametrize("layout", ["NN", "TN", "NT"])
 def test_every_tile_variant(lib, gpu, variant, layout):
     a, b = operands(512, 768, 448, layout, seed=variant)

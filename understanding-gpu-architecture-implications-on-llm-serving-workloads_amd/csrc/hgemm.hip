@@ -129,7 +129,7 @@ struct MNContigTile {
 // 256x256x64 main kernel
 // ---------------------------------------------------------------------------------------------------------
 
-template <bool A_KC, bool B_KC, int BM_, int BN_, int WM_, int WN_>
+template <bool A_KC, bool B_KC, int BM_, int BN_, int WM_, int WN_, int STAGES = 0>
 struct MainCfg {
     static constexpr int BM = BM_, BN = BN_, BK = 64;
     static constexpr int WM = WM_, WN = WN_, NWAVES = WM_ * WN_, NTHREADS = NWAVES * 64;
@@ -146,7 +146,7 @@ struct MainCfg {
     // K tile of time to land (small problems run few tiles per workgroup and are bound by that latency). The narrow tiles
     // serve products with few rows, which are bound by the stream of the weight matrix from HBM: their ring is as deep
     // as 128 KiB of LDS allow (5 stages of 24 KiB, 8 of 16 KiB), so that a CU keeps ~50 KiB of that stream in flight.
-    static constexpr int NSTAGE = STAGE_BYTES > 48 * 1024 ? 2 : STAGE_BYTES > 24 * 1024 ? 3 : STAGE_BYTES > 16 * 1024 ? 5 : 8;
+    static constexpr int NSTAGE = STAGES > 0 ? STAGES : STAGE_BYTES > 48 * 1024 ? 2 : STAGE_BYTES > 24 * 1024 ? 3 : STAGE_BYTES > 16 * 1024 ? 5 : 8;
     static constexpr int LDS_BYTES = STAGE_BYTES * NSTAGE;
     static constexpr int A_INSTS = A_BYTES / (NWAVES * 1024);  // 16-byte copies per lane per K tile
     static constexpr int B_INSTS = B_BYTES / (NWAVES * 1024);
@@ -191,6 +191,74 @@ __device__ __forceinline__ void tile_of_block(int bid, int tiles_m, int tiles_n,
     tn = in_g / rows;
 }
 
+// Epilogue of the tiled kernels for one wave's sub-tile of TM x TN blocks of 16x16 (first row row0, first stored column
+// col0, of a C with NC columns). A lane holds C[m][n .. n+3] for m = l%16, n = 4*(l/16) of every block. Storing that
+// directly would write 8-byte pieces of 16 different rows per instruction (partial cache lines, read-modify-write in
+// the memory system), so the wave first parks its sub-tile in its own slice of LDS (cst; fp16, 16-byte chunks
+// XOR-swizzled by row) and then stores whole rows: every store instruction writes complete 128-byte lines.
+// EPI == 1: the wave's columns come in groups of [32 gate | 32 up]; output block jo takes its gate from block
+// 4 (jo / 2) + jo % 2 and its up from two blocks further.
+template <typename T, int TM, int TN, int EPI, bool RAGGED>
+__device__ __forceinline__ void store_wave_tile(const float4v (&acc)[TM][TN], MI355_LDS char* cst, T* C, const T* R, long row0,
+                                                long col0, int M, int NC, long ldc, long ldr, int lane) {
+    using V8 = typename Elem<T>::v8;
+    using V4 = typename Elem<T>::v4;
+    static_assert(EPI == 0 || TN % 4 == 0, "the gate/up epilogue pairs column blocks 32 columns apart");
+    constexpr int TNO = EPI == 1 ? TN / 2 : TN;   // column blocks a wave stores
+    constexpr int kRowHalfs = TNO * 16;           // width of the stored wave sub-tile
+    constexpr int kRowBytesC = kRowHalfs * 2;
+    constexpr int kChunksC = kRowBytesC / 16;     // 16-byte chunks per row (4, 8 or 16)
+    constexpr int kRowsPerStore = 64 / kChunksC;  // rows covered by one store instruction
+    constexpr int kSwzC = kChunksC < 8 ? kChunksC - 1 : 7;
+    {
+        const int r = lane & 15;
+        const int g = lane >> 4;
+#pragma unroll
+        for (int i = 0; i < TM; ++i) {
+            const int row = i * 16 + r;
+#pragma unroll
+            for (int jo = 0; jo < TNO; ++jo) {
+                V4 v;
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    if constexpr (EPI == 1) {
+                        const int gj = (jo / 2) * 4 + (jo % 2);
+                        const float gt = acc[i][gj][q];
+                        const float sig = __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(-gt * 1.4426950408889634f));
+                        v[q] = (T)(gt * sig * acc[i][gj + 2][q]);
+                    } else {
+                        v[q] = (T)acc[i][jo][q];
+                    }
+                }
+                const int chunk = (2 * jo + (g >> 1)) ^ (row & kSwzC);
+                *(MI355_LDS V4*)(cst + row * kRowBytesC + chunk * 16 + (g & 1) * 8) = v;
+            }
+        }
+    }
+    // only this wave reads what it wrote: no workgroup barrier needed, the LDS operations of a wave complete in order
+    {
+        const int rr = lane / kChunksC;
+        const int cc = lane % kChunksC;
+        T* cbase = C + row0 * ldc + col0 + cc * 8;
+        const long rows_left = M - row0;   // RAGGED: rows and 8-column chunks that exist
+        const bool col_ok = col0 + cc * 8 < NC;
+        const T* rbase = R + row0 * ldr + col0 + cc * 8;
+#pragma unroll
+        for (int it = 0; it < TM * 16 / kRowsPerStore; ++it) {
+            const int row = it * kRowsPerStore + rr;
+            V8 v = *(MI355_LDS const V8*)(cst + row * kRowBytesC + ((cc ^ (row & kSwzC)) << 4));
+            if (!RAGGED || (row < rows_left && col_ok)) {
+                if (R != nullptr) {
+                    const V8 r = *(const V8*)(rbase + (long)row * ldr);
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) v[j] = (T)((float)v[j] + (float)r[j]);
+                }
+                *(V8*)(cbase + (long)row * ldc) = v;
+            }
+        }
+    }
+}
+
 // EPI selects what is stored: 0 = the product; 1 = silu(g) * u for a B operand whose columns alternate between 32 gate
 // columns and their 32 up columns (`act_fn(gate_proj(x)) * up_proj(x)`, benchmarks/flashattn-cuda/modeling_llama.py:227,
 // with the two projections interleaved in one weight matrix): a wave then holds g and u of the same outputs in its two
@@ -200,15 +268,15 @@ __device__ __forceinline__ void tile_of_block(int bid, int tiles_m, int tiles_n,
 // RAGGED: M (and N) need not be multiples of the tile. Copies of rows past the end are redirected to the last row (or, for
 // an operand whose M/N index is contiguous, to the last 8 columns; that dimension must be a multiple of 8), so every
 // load stays inside the matrices, and the epilogue stores only what exists.
-template <typename T, bool A_KC, bool B_KC, int BM, int BN, int WM, int WN, int EPI = 0, bool RAGGED = false>
-__global__ __launch_bounds__(WM * WN * 64) __attribute__((amdgpu_waves_per_eu(WM * WN / 4, WM * WN / 4)))
+template <typename T, bool A_KC, bool B_KC, int BM, int BN, int WM, int WN, int EPI = 0, bool RAGGED = false, int STAGES = 0, int PER_CU = 1>
+__global__ __launch_bounds__(WM * WN * 64) __attribute__((amdgpu_waves_per_eu(WM * WN / 4, PER_CU * WM * WN / 4)))
 void hgemm_main_kernel(const T* __restrict__ A, const T* __restrict__ B,
                                                          T* C, const T* R, int M, int N, int K, long lda,
                                                          long ldb, long ldc, long ldr) {
     using V8 = typename Elem<T>::v8;
     using V4 = typename Elem<T>::v4;
     using V2 = typename Elem<T>::v2;
-    using Cfg = MainCfg<A_KC, B_KC, BM, BN, WM, WN>;
+    using Cfg = MainCfg<A_KC, B_KC, BM, BN, WM, WN, STAGES>;
     using ATK = typename Cfg::ATileK;
     using ATM = typename Cfg::ATileM;
     using BTK = typename Cfg::BTileK;
@@ -517,70 +585,12 @@ void hgemm_main_kernel(const T* __restrict__ A, const T* __restrict__ B,
     MI355_TL(tl_w[2] = timeline::wall_clock(); tl_c[1] = timeline::shader_cycles();)
 
     // ---- epilogue ------------------------------------------------------------------------------------------------
-    // A lane holds C[m][n .. n+3] for m = l%16, n = 4*(l/16) of every 16x16 block. Storing that directly would write
-    // 8-byte pieces of 16 different rows per instruction (partial cache lines, read-modify-write in the memory
-    // system), so each wave first parks its sub-tile in its own slice of LDS (fp16, 16-byte chunks XOR-swizzled by
-    // row) and then stores whole rows: every store instruction writes complete 128-byte lines.
-    // EPI == 1: the wave's columns come in groups of [32 gate | 32 up]; output block jo takes its gate from block
-    // 4 (jo / 2) + jo % 2 and its up from two blocks further.
-    static_assert(EPI == 0 || TN % 4 == 0, "the gate/up epilogue pairs column blocks 32 columns apart");
     constexpr int TNO = EPI == 1 ? TN / 2 : TN;   // column blocks a wave stores
-    constexpr int kRowHalfs = TNO * 16;           // width of the stored wave sub-tile
-    constexpr int kRowBytesC = kRowHalfs * 2;
-    constexpr int kChunksC = kRowBytesC / 16;     // 16-byte chunks per row (4, 8 or 16)
-    constexpr int kRowsPerStore = 64 / kChunksC;  // rows covered by one store instruction
-    constexpr int kSwzC = kChunksC < 8 ? kChunksC - 1 : 7;
-    static_assert(Cfg::NWAVES * TM * 16 * kRowBytesC <= Cfg::LDS_BYTES, "epilogue staging does not fit in LDS");
+    static_assert(Cfg::NWAVES * TM * 16 * TNO * 32 <= Cfg::LDS_BYTES, "epilogue staging does not fit in LDS");
     wait_vmcnt<0>();  // the last tiles' copies (on the empty buffer) have written their zeros
     __syncthreads();  // every wave has finished reading the operand stages
-    MI355_LDS char* cst = smem + wave * (TM * 16 * kRowBytesC);
-    {
-        const int r = lane & 15;
-        const int g = lane >> 4;
-#pragma unroll
-        for (int i = 0; i < TM; ++i) {
-            const int row = i * 16 + r;
-#pragma unroll
-            for (int jo = 0; jo < TNO; ++jo) {
-                V4 v;
-#pragma unroll
-                for (int q = 0; q < 4; ++q) {
-                    if constexpr (EPI == 1) {
-                        const int gj = (jo / 2) * 4 + (jo % 2);
-                        const float gt = acc[i][gj][q];
-                        const float sig = __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(-gt * 1.4426950408889634f));
-                        v[q] = (T)(gt * sig * acc[i][gj + 2][q]);
-                    } else {
-                        v[q] = (T)acc[i][jo][q];
-                    }
-                }
-                const int chunk = (2 * jo + (g >> 1)) ^ (row & kSwzC);
-                *(MI355_LDS V4*)(cst + row * kRowBytesC + chunk * 16 + (g & 1) * 8) = v;
-            }
-        }
-    }
-    // only this wave reads what it wrote: no workgroup barrier needed, the LDS operations of a wave complete in order
-    {
-        const int rr = lane / kChunksC;
-        const int cc = lane % kChunksC;
-        T* cbase = C + (m0 + wm * TM * 16) * ldc + (EPI == 1 ? n0 / 2 : n0) + wn * TNO * 16 + cc * 8;
-        const long rows_left = M - (m0 + wm * TM * 16);   // RAGGED: rows and 8-column chunks that exist
-        const bool col_ok = (EPI == 1 ? n0 / 2 : n0) + wn * TNO * 16 + cc * 8 < (EPI == 1 ? N / 2 : N);
-        const T* rbase = R + (m0 + wm * TM * 16) * ldr + (EPI == 1 ? n0 / 2 : n0) + wn * TNO * 16 + cc * 8;
-#pragma unroll
-        for (int it = 0; it < TM * 16 / kRowsPerStore; ++it) {
-            const int row = it * kRowsPerStore + rr;
-            V8 v = *(MI355_LDS const V8*)(cst + row * kRowBytesC + ((cc ^ (row & kSwzC)) << 4));
-            if (!RAGGED || (row < rows_left && col_ok)) {
-                if (R != nullptr) {
-                    const V8 r = *(const V8*)(rbase + (long)row * ldr);
-#pragma unroll
-                    for (int j = 0; j < 8; ++j) v[j] = (T)((float)v[j] + (float)r[j]);
-                }
-                *(V8*)(cbase + (long)row * ldc) = v;
-            }
-        }
-    }
+    store_wave_tile<T, TM, TN, EPI, RAGGED>(acc, smem + wave * (TM * 16 * TNO * 32), C, R, m0 + wm * TM * 16,
+                                            (EPI == 1 ? n0 / 2 : n0) + wn * TNO * 16, M, EPI == 1 ? N / 2 : N, ldc, ldr, lane);
     MI355_TL(
         wait_vmcnt<0>();   // the stores of this wave have been accepted
         tl_w[3] = timeline::wall_clock();
@@ -979,11 +989,11 @@ static hipError_t launch_smallm_nt_gate_up(const T* A, const T* B, T* C, int M, 
     return hipGetLastError();
 }
 
-template <typename T, bool A_KC, bool B_KC, int BM, int BN, int WM, int WN, int EPI = 0, bool RAGGED = false>
+template <typename T, bool A_KC, bool B_KC, int BM, int BN, int WM, int WN, int EPI = 0, bool RAGGED = false, int STAGES = 0, int PER_CU = 1>
 static hipError_t launch_main(const T* A, const T* B, T* C, const T* R, int M, int N, int K, long lda, long ldb,
                               long ldc, long ldr, hipStream_t stream) {
-    using Cfg = MainCfg<A_KC, B_KC, BM, BN, WM, WN>;
-    auto kern = hgemm_main_kernel<T, A_KC, B_KC, BM, BN, WM, WN, EPI, RAGGED>;
+    using Cfg = MainCfg<A_KC, B_KC, BM, BN, WM, WN, STAGES>;
+    auto kern = hgemm_main_kernel<T, A_KC, B_KC, BM, BN, WM, WN, EPI, RAGGED, STAGES, PER_CU>;
     static DynamicLdsOnce lds_once;
     if (hipError_t e = lds_once.ensure(reinterpret_cast<const void*>(kern), Cfg::LDS_BYTES); e != hipSuccess) return e;
     const long nblocks = (long)((M + BM - 1) / BM) * ((N + BN - 1) / BN);
@@ -1012,6 +1022,33 @@ static bool few_rows_prefer_tiles(int M, int N, int K, bool nt) {
     if (M <= 16) return false;
     return few_row_tiles_us(M, N, K, nt) < small_m_us(M, N, K, false) - 4.0;
 }
+// Which tile shape is expected to finish a product of more than 64 rows first (1 = 256x256, 2 = 128x128, 3 = 64x128 or
+// 128x64, 4 = 64x64 two to a CU). A CU takes in 64 bytes per cycle from the memory system and its LDS serves the
+// direct-to-LDS writes and the fragment reads one after the other, so the time of a K tile is set by the tile's bytes
+// as much as by its matrix instructions: measured cycles per K tile of 64 of one workgroup alone on its CU are 2470
+// (256x256; matrix pipes 2048), 770 (128x128; pipes 512, LDS 768), 576 (half tile) and 384 (64x64). A workgroup spends
+// another 5000-12000 cycles outside its K loop (first tiles in flight, epilogue). The workgroups run in rounds of one
+// per CU (two for the 64x64 tiles); the last round may be a partial one. The model reproduces the measured times of
+// 1024^3 .. 8192^3, 2048 x 4096 x 4096 and 1536 x 1536 x 8192 within ~10 %. The 128x128 figure used below is 840: on
+// N(0,1) operands, under the board's power limit, the 256x256 tiles do better against the smaller ones than on zeros
+// (3072 x 3072 x 4096: 75 us against 87 where zeros give 70 against 71).
+static int cheapest_tile_shape(int M, int N, int K) {
+    struct Cand { int shape, bm, bn, per_cu; double step, fixed; };
+    static const Cand cands[] = {{1, 256, 256, 1, 2470., 12000.}, {2, 128, 128, 1, 840., 7000.}, {3, 64, 128, 1, 576., 6000.},
+                                 {4, 64, 64, 2, 384., 5000.}};
+    const double ktiles = (double)(K / 64);
+    int best = 2;
+    double best_t = 0.;
+    for (const Cand& c : cands) {
+        const long tiles = (long)((M + c.bm - 1) / c.bm) * ((N + c.bn - 1) / c.bn);
+        const long cap = 256L * c.per_cu, full = tiles / cap, rem = tiles % cap;
+        double t = (double)full * (c.per_cu * ktiles * c.step + c.fixed);
+        if (rem) t += (double)((rem + 255) / 256) * ktiles * c.step + c.fixed;
+        if (best_t == 0. || t < best_t) { best_t = t; best = c.shape; }
+    }
+    return best;
+}
+
 // Up to 64 rows on 64x64 tiles with an 8-deep ring: the second operand is streamed once whatever M is, by N / 64
 // workgroups that each sustain ~38 GB/s until HBM saturates (~6.3 TB/s); layout NN pays ~10 % for its 128-byte row
 // segments. True when that is expected to beat both alternatives above (measured at Llama projection shapes:
@@ -1052,8 +1089,6 @@ static hipError_t launch_layout(const T* A, const T* B, T* C, const T* R, int M,
     }
     // the tiled kernels address a tile with 32-bit byte offsets: up to 256 rows of lda (ldb) elements
     const bool k_ok = aligned && K % 64 == 0 && K >= 64 && lda < (1L << 22) && ldb < (1L << 22);
-    const bool fits256 = k_ok && M % 256 == 0 && N % 256 == 0;
-    const bool fits128 = k_ok && M % 128 == 0 && N % 128 == 0;
     const bool ragged_ok = k_ok && N % 8 == 0 && N >= 8 && (A_KC || (M % 8 == 0 && M >= 8));
     const bool small_m = M <= 64 && !(ragged_ok && few_rows_prefer_tiles(M, N, K, A_KC && B_KC));
     // Up to 64 rows (generation-step projections): 64x64 tiles with an 8-deep ring stream the second operand once, on
@@ -1069,44 +1104,34 @@ static hipError_t launch_layout(const T* A, const T* B, T* C, const T* R, int M,
     if constexpr (A_KC && B_KC) {
         if (aligned && small_m && K % 64 == 0 && K >= 64) return launch_smallm_nt<T>(A, B, C, R, M, N, K, lda, ldb, ldc, ldr, stream);
     }
-    // Fewer than ~3/4 x 256 tiles of 128x128 cannot occupy the CUs: halve the tile so that twice as many workgroups pull
-    // on the memory system (64 x 14336 x 4096 NT: 22 us instead of 27.5; 1024^3: 7 us instead of 9.5). Layout NT halves
-    // the tile along N (128x64).
-    const bool few_tiles = ragged_ok && (long)((M + 127) / 128) * ((N + 127) / 128) < 192 && variant == 0;
-    if constexpr (A_KC && B_KC) {
-        if (few_tiles) {
-            if (M % 128 == 0 && N % 64 == 0)
-                return launch_main<T, A_KC, B_KC, 128, 64, 2, 2>(A, B, C, R, M, N, K, lda, ldb, ldc, ldr, stream);
-            return launch_main<T, A_KC, B_KC, 128, 64, 2, 2, 0, true>(A, B, C, R, M, N, K, lda, ldb, ldc, ldr, stream);
-        }
-    }
-    // layout NN halves the tile along M (64x128: an N-contiguous B tile of 128 columns keeps its 256-byte rows); that helps
-    // products with several row tiles (1024^3), not the few-row ones, which take the 64x64 tiles above
-    if constexpr (A_KC && !B_KC) {
-        if (few_tiles && M > 64) {
-            if (M % 64 == 0 && N % 128 == 0)
-                return launch_main<T, A_KC, B_KC, 64, 128, 1, 4>(A, B, C, R, M, N, K, lda, ldb, ldc, ldr, stream);
-            return launch_main<T, A_KC, B_KC, 64, 128, 1, 4, 0, true>(A, B, C, R, M, N, K, lda, ldb, ldc, ldr, stream);
-        }
-    }
-    // 256x256 tiles when they fill the machine (>= ~3/4 of the 256 CUs), 128x128 tiles for smaller problems
-    const long tiles256 = fits256 ? (long)(M / 256) * (N / 256) : 0;
-    int choice = 0;
-    if (fits256 && (tiles256 >= 192 || !fits128)) choice = 1;
-    else if (fits128) choice = 2;
-    if (variant == 1 && fits256) choice = 1;
-    if (variant == 2 && fits128) choice = 2;
-    switch (choice) {
-        case 1: return launch_main<T, A_KC, B_KC, 256, 256, 2, 4>(A, B, C, R, M, N, K, lda, ldb, ldc, ldr, stream);
-        case 2: return launch_main<T, A_KC, B_KC, 128, 128, 2, 2>(A, B, C, R, M, N, K, lda, ldb, ldc, ldr, stream);
-        default: break;
-    }
-    // ragged M / N on the same tiles: N (and M for layout TN) a multiple of 8, so 16-byte chunks never straddle the end
+    // Tiled kernels: N (and M for layout TN) a multiple of 8, so that 16-byte chunks never straddle the end; M and N need
+    // not be multiples of the tile. Shapes: 1 = 256x256 (8 waves, ring of 2), 2 = 128x128 (4 waves, ring of 3), 3 = half
+    // of that (64x128, for layout NT 128x64, which keeps the 128-byte rows of both K-contiguous operands; ring of 5),
+    // 4 = 64x64 with a ring of 4 (64 KiB: two workgroups fit on a CU). More than 64 rows: the shape with the least
+    // estimated time. Up to 64 rows (products that few_rows_prefer_tiles sends here): half tiles for layout NT, which
+    // put twice as many workgroups on the stream of the second operand, 128x128 otherwise.
     if (ragged_ok) {
-        const long t256 = (long)((M + 255) / 256) * ((N + 255) / 256);
-        if ((t256 >= 192 && variant != 2) || variant == 1)
-            return launch_main<T, A_KC, B_KC, 256, 256, 2, 4, 0, true>(A, B, C, R, M, N, K, lda, ldb, ldc, ldr, stream);
-        return launch_main<T, A_KC, B_KC, 128, 128, 2, 2, 0, true>(A, B, C, R, M, N, K, lda, ldb, ldc, ldr, stream);
+        int shape = variant >= 1 && variant <= 4 ? variant : M <= 64 ? ((A_KC && B_KC) ? 3 : 2) : cheapest_tile_shape(M, N, K);
+        const auto whole = [&](int bm, int bn) { return M % bm == 0 && N % bn == 0; };
+        switch (shape) {
+            case 1:
+                if (whole(256, 256)) return launch_main<T, A_KC, B_KC, 256, 256, 2, 4>(A, B, C, R, M, N, K, lda, ldb, ldc, ldr, stream);
+                return launch_main<T, A_KC, B_KC, 256, 256, 2, 4, 0, true>(A, B, C, R, M, N, K, lda, ldb, ldc, ldr, stream);
+            case 3:
+                if constexpr (A_KC && B_KC) {
+                    if (whole(128, 64)) return launch_main<T, A_KC, B_KC, 128, 64, 2, 2>(A, B, C, R, M, N, K, lda, ldb, ldc, ldr, stream);
+                    return launch_main<T, A_KC, B_KC, 128, 64, 2, 2, 0, true>(A, B, C, R, M, N, K, lda, ldb, ldc, ldr, stream);
+                } else {
+                    if (whole(64, 128)) return launch_main<T, A_KC, B_KC, 64, 128, 1, 4>(A, B, C, R, M, N, K, lda, ldb, ldc, ldr, stream);
+                    return launch_main<T, A_KC, B_KC, 64, 128, 1, 4, 0, true>(A, B, C, R, M, N, K, lda, ldb, ldc, ldr, stream);
+                }
+            case 4:
+                if (whole(64, 64)) return launch_main<T, A_KC, B_KC, 64, 64, 2, 2, 0, false, 4, 2>(A, B, C, R, M, N, K, lda, ldb, ldc, ldr, stream);
+                return launch_main<T, A_KC, B_KC, 64, 64, 2, 2, 0, true, 4, 2>(A, B, C, R, M, N, K, lda, ldb, ldc, ldr, stream);
+            default:
+                if (whole(128, 128)) return launch_main<T, A_KC, B_KC, 128, 128, 2, 2>(A, B, C, R, M, N, K, lda, ldb, ldc, ldr, stream);
+                return launch_main<T, A_KC, B_KC, 128, 128, 2, 2, 0, true>(A, B, C, R, M, N, K, lda, ldb, ldc, ldr, stream);
+        }
     }
     dim3 grid((N + 63) / 64, (M + 63) / 64);
     hgemm_edge_kernel<T, A_KC, B_KC><<<grid, dim3(256), 0, stream>>>(A, B, C, R, M, N, K, lda, ldb, ldc, ldr);
