@@ -175,6 +175,25 @@ __device__ __forceinline__ void static_for(F&& f) {
 __device__ __forceinline__ void tile_of_block(int bid, int tiles_m, int tiles_n, int& tm, int& tn) {
     const int total = tiles_m * tiles_n;
     constexpr int kXcd = 8;
+#ifndef MI355_GEMM_NO_SUPERBLOCKS
+    // Large grids: the 256 workgroups that run at the same time (ids 256 s .. 256 s + 255, one per CU) take one
+    // super-block of 256 tiles, each XCD an 8 x 4 piece of it, and the super-blocks follow one another in serpentine
+    // order, so that consecutive ones share their row panels of A or their column panels of B. A super-block reads
+    // (16 + 16) or (32 + 8) panels where the same 256 tiles taken as 8 stripes of 8 x 4 from all over the matrix read
+    // all 32 row panels: fewer bytes pass through the memory-side cache, and half of them were there a step earlier.
+    const int sb_n = tiles_n % 16 == 0 ? 16 : tiles_n % 8 == 0 ? 8 : 0;   // super-block: sb_m x sb_n tiles
+    const int sb_m = sb_n ? 256 / sb_n : 0;
+    if (sb_n && tiles_m % sb_m == 0 && total >= 512) {
+        const int step = bid >> 8, x = bid & 7, j = (bid >> 3) & 31;    // j: this XCD's 32 workgroups of the step
+        const int blocks_n = tiles_n / sb_n;
+        const int brow = step / blocks_n;
+        const int bcol = (brow & 1) ? blocks_n - 1 - step % blocks_n : step % blocks_n;
+        const int xcd_cols = sb_n / 4;                                   // XCD pieces side by side in a super-block
+        tm = brow * sb_m + (x / xcd_cols) * 8 + (j & 7);
+        tn = bcol * sb_n + (x % xcd_cols) * 4 + (j >> 3);
+        return;
+    }
+#endif
     int t = bid;
     if (total % kXcd == 0) {
         int per = total / kXcd;
