@@ -31,11 +31,11 @@ PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 
 # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (KiB per dispatch), each scaled by what the same
 # counter reads for a 1 GiB device-to-device copy (FETCH_SIZE x2.0, WRITE_SIZE x1.0); see profiles/.
-MEASURED_TRAFFIC_BYTES = (786975 * 2.0 + 131072 * 1.0) * 1024        # hgemm_main_kernel, 8192^3 NN
+MEASURED_TRAFFIC_BYTES = (795037 * 2.0 + 131072 * 1.0) * 1024        # hgemm_main_kernel, 8192^3 NN
 MEASURED_TRAFFIC_BYTES_G2C = (57882 * 2.0 + 448 * 1.0) * 1024          # hgemm_smallm_nn_kernel, 16 x 14336 x 4096
-MEASURED_TRAFFIC_BYTES_FMHA = (26705 * 2.0 + 33280 * 1.0) * 1024     # fmha_fwd_pingpong_kernel, F4
+MEASURED_TRAFFIC_BYTES_FMHA = (26670 * 2.0 + 33280 * 1.0) * 1024     # fmha_fwd_pingpong_kernel, F4
 # the figures above are constants copied from these counter summaries (they are not read at run time)
-TRAFFIC_SOURCE = {"gemm": "constant from profiles/hgemm_main_kernel_8192_nn.md (rocprofv3 --pmc FETCH_SIZE, WRITE_SIZE)",
+TRAFFIC_SOURCE = {"gemm": "constant from profiles/hgemm_main_kernel_256x256_8192_nn.md (rocprofv3 --pmc FETCH_SIZE, WRITE_SIZE)",
                   "g2c": "constant from profiles/hgemm_smallm_nn_kernel_g2c_16x14336x4096_nn.md",
                   "fmha": "constant from profiles/fmha_fwd_pingpong_kernel_f4_causal_gqa.md"}
 
