@@ -116,6 +116,20 @@ def test_k_that_is_a_multiple_of_16_but_not_of_the_tile_depth(lib, gpu, layout, 
     check(lib, gpu, a, b, layout, K)
 
 
+@pytest.mark.parametrize("variant,tile_m,tile_n", [(1, 256, 256), (2, 128, 128), (3, 64, 128), (4, 64, 64)])
+@pytest.mark.parametrize("layout", ["NN", "NT"])
+@pytest.mark.parametrize("tiles_m,tiles_n,ragged", [(16, 32, 0), (32, 24, 0), (32, 16, 8), (48, 16, 0)])
+def test_grids_walked_in_super_blocks(lib, gpu, variant, tile_m, tile_n, layout, tiles_m, tiles_n, ragged):
+    # grids of >= 512 tiles whose dimensions are multiples of a 16x16 or 32x8 block of tiles are walked block by block in
+    # serpentine order (hgemm.hip: tile_of_block): every tile must still be computed exactly once, also when the last tile
+    # row / column is ragged. K = 64 keeps the host product cheap.
+    if layout == "NT" and variant == 3:
+        tile_m, tile_n = 128, 64
+    M, N, K = tiles_m * tile_m - ragged, tiles_n * tile_n - ragged, 64
+    a, b = operands(M, N, K, layout, seed=tiles_m + tiles_n + variant)
+    check(lib, gpu, a, b, layout, K, variant=variant)
+
+
 @pytest.mark.parametrize("variant", [1, 2, 3, 4])
 @pytest.mark.parametrize("layout", ["NN", "TN", "NT"])
 def test_every_tile_variant(lib, gpu, variant, layout):
