@@ -130,6 +130,34 @@ def test_grids_walked_in_super_blocks(lib, gpu, variant, tile_m, tile_n, layout,
     check(lib, gpu, a, b, layout, K, variant=variant)
 
 
+def _seeded_shapes(n, seed):
+    """n products drawn with a fixed seed: row counts from one to a few thousand, widths and depths on and off the tile grid
+    (multiples of 8, sometimes odd), every layout. The library picks the kernel (variant 0): small-M, one of the four tile
+    shapes, the K tail through the bounds-checked kernel, or that kernel alone."""
+    rng = np.random.default_rng(seed)
+    out = []
+    for _ in range(n):
+        layout = ["NN", "NT", "TN"][int(rng.integers(3))]
+        m = int(rng.choice([1, 7, 16, 24, 64, 100, 128, 200, 384, 520, 1000, 1536, 2048, 3000]))
+        nn = int(rng.choice([8, 64, 136, 512, 1000, 1024, 2048, 4096, 5120])) + int(rng.choice([0, 0, 0, 8, 24, 3]))
+        k = int(rng.choice([64, 128, 192, 448, 1024, 2048, 4096])) + int(rng.choice([0, 0, 0, 16, 32, 8, 5]))
+        if m * nn > 6e6:
+            k = min(k, 1100)
+        out.append((layout, m, nn, k))
+    return out
+
+
+@pytest.mark.parametrize("layout,M,N,K", _seeded_shapes(40, 20260417))
+def test_seeded_random_products_choose_their_own_kernel(lib, gpu, layout, M, N, K):
+    a, b = operands(M, N, K, layout, seed=M + 3 * N + 7 * K, b_std=0.05)
+    c = torch.full((M + 1, N + 3), 7.0, dtype=torch.float16, device=gpu)
+    lib.hgemm(a.to(gpu), b.to(gpu), layout, out=c[:M, :N])
+    torch.cuda.synchronize()
+    ok, st = so.gemm_tolerance_ok(c[:M, :N].cpu(), so.gemm_ref(a, b, layout), K)
+    assert ok, (layout, M, N, K, st)
+    assert bool((c[M:] == 7.0).all()) and bool((c[:, N:] == 7.0).all())
+
+
 @pytest.mark.parametrize("variant", [1, 2, 3, 4])
 @pytest.mark.parametrize("layout", ["NN", "TN", "NT"])
 def test_every_tile_variant(lib, gpu, variant, layout):
