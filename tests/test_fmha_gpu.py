@@ -113,6 +113,33 @@ def test_ragged_shapes_and_masks(lib, gpu, B, Hq, Hkv, Sq, Sk, causal, kvv):
         assert bool((o[:, :, :n] == 0).all()) and bool(torch.isinf(lse[:, :, :n]).all()) and bool((lse[:, :, :n] < 0).all())
 
 
+def _seeded_attention_shapes(n, seed):
+    """n prefill shapes drawn with a fixed seed: a few to a few thousand work items (one workgroup per CU walks them in
+    rounds), ragged query and key counts, GQA groups of 1..8, causal or not, sometimes a valid length short of Sk."""
+    rng = np.random.default_rng(seed)
+    out = []
+    while len(out) < n:
+        b = int(rng.choice([1, 2, 3, 5]))
+        hkv = int(rng.choice([1, 2, 4, 8]))
+        hq = hkv * int(rng.choice([1, 2, 4, 8]))
+        sq = int(rng.choice([33, 128, 200, 256, 384, 640, 1000, 1024, 1500]))
+        sk = sq if rng.random() < 0.5 else int(rng.choice([64, 191, 256, 700, 1024, 2048]))
+        causal = bool(rng.random() < 0.6)
+        kvv = None if rng.random() < 0.7 else max(1, sk - int(rng.integers(1, 70)))
+        if b * hq * sq * sk > 1.6e8:
+            continue
+        out.append((b, hq, hkv, sq, sk, causal, kvv))
+    return out
+
+
+@pytest.mark.parametrize("variant", [0, 1, 2])
+@pytest.mark.parametrize("B,Hq,Hkv,Sq,Sk,causal,kvv", _seeded_attention_shapes(16, 4242) + [
+    (8, 32, 8, 512, 512, True, None), (4, 40, 8, 384, 384, False, None), (16, 24, 8, 130, 130, True, None)])   # many short items: several rounds per workgroup
+def test_seeded_random_prefill_shapes(lib, gpu, variant, B, Hq, Hkv, Sq, Sk, causal, kvv):
+    q, k, v = so.fmha_inputs(B, Hq, Hkv, Sq, Sk, seed=B + Hq + Sq + Sk)
+    check(lib, gpu, q, k, v, causal, kvv, variant=variant)
+
+
 @pytest.mark.parametrize("variant", [1, 2])
 @pytest.mark.parametrize("B,Hq,Hkv,Sq,Sk,causal,kvv", [
     (1, 4, 1, 128, 128, True, None), (2, 4, 2, 100, 177, True, None), (1, 2, 1, 300, 300, True, 290),
