@@ -172,6 +172,23 @@ def test_decode_shaped_small_m(lib, gpu, layout, M, N, K):
     check(lib, gpu, a, b, layout, K)
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("M,N,K", [(16, 6144, 4096), (8, 14336, 4096), (13, 14336, 4096), (1, 12288, 4096), (3, 6144, 4096),
+                                   (16, 28672, 4096), (16, 6160, 4096)])
+def test_generation_step_projections_with_the_activation_rows_kept_in_registers(lib, gpu, dtype, M, N, K):
+    # layout NT, K = 4096, up to 16 rows, a few hundred row tiles or more: a workgroup takes two or four row tiles and copies
+    # the activation rows only for the first (hgemm_smallm_nt_rega_kernel); 6160 = 385 tiles is not divisible and keeps one
+    # tile per workgroup
+    a, b = operands(M, N, K, "NT", seed=M + N, b_std=0.05)
+    if dtype == torch.bfloat16:
+        a, b = a.float().bfloat16(), b.float().bfloat16()
+        c = lib.hgemm(a.to(gpu), b.to(gpu), "NT").cpu()
+        ok, worst = bf16_close(c, so.gemm_ref(a, b, "NT"), K)
+        assert ok, worst
+    else:
+        check(lib, gpu, a, b, "NT", K)
+
+
 @pytest.mark.parametrize("layout", ["NN", "NT", "TN"])
 @pytest.mark.parametrize("M,N,K", [(24, 14336, 512), (64, 14336, 256), (32, 28672, 128), (40, 4096, 1024), (17, 12800, 192)])
 def test_17_to_64_rows_small_m_or_tiles(lib, gpu, layout, M, N, K):
@@ -339,6 +356,7 @@ def test_bfloat16_gemm_exact_cases_and_torch_operator(lib, gpu):
                                    (4096, 4096, 128),    # 256x256 tiles
                                    (1000, 264, 128),     # ragged tiles
                                    (16, 4096, 1024),     # small-M kernels (NN, NT)
+                                   (12, 6144, 4096),     # NT: several row tiles per workgroup, A kept in registers
                                    (8, 72, 192),
                                    (100, 70, 50)])       # bounds-checked kernel
 def test_residual_epilogue_equals_product_then_add(lib, gpu, dtype, layout, M, N, K):

@@ -135,7 +135,8 @@ def test_silu_mul(lib, gpu, rows, inter):
                                           (300, 160, 128, "NT"), (1000, 14336, 128, "NT"), (4100, 4096, 64, "NN"),
                                           (32, 14336, 256, "NT"), (64, 14336, 128, "NN"), (24, 7168, 512, "NT"),
                                           (1, 32, 64, "NT"), (8, 14336, 512, "NT"), (16, 2048, 1024, "NT"), (13, 96, 128, "NT"),
-                                          (9, 4096, 4096, "NT"), (16, 512, 256, "NN"), (17, 1024, 512, "NT"), (48, 7168, 256, "NT"),
+                                          (9, 4096, 4096, "NT"), (16, 14336, 4096, "NT"), (8, 7168, 4096, "NT"), (4, 3072, 4096, "NT"),
+                                          (16, 512, 256, "NN"), (17, 1024, 512, "NT"), (48, 7168, 256, "NT"),
                                           (33, 512, 1024, "NN"), (64, 2048, 128, "NN"), (40, 96, 64, "NT"), (5, 256, 192, "NN")])
 def test_gemm_with_gate_up_epilogue(lib, gpu, M, F, K, layout):
     # silu(x Wg^T) * (x Wu^T) from one launch on the interleaved weight (tiled shapes; up to 16 rows in layout NT on the

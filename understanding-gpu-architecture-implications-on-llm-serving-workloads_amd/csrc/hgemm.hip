@@ -974,11 +974,161 @@ __global__ __launch_bounds__(kSmallMNtWaves * 64) void hgemm_smallm_nt_kernel(co
     }
 }
 
+// The same product for wide weights (at least a few hundred row tiles) and K = 256 STEPS: a workgroup takes TPW
+// consecutive row tiles and keeps its slice of A in registers after the first of them (a wave's K / 4 columns of the 16
+// rows: 2 STEPS fragments, 128 registers at K = 4096), so from the second tile on only the weights are copied: the
+// activation rows are then fetched from L2 once per TPW tiles instead of once per tile (they are as many bytes through
+// the CU's memory pipeline as the weights themselves). The stream over (tile, k-step) is unrolled completely: every LDS
+// offset, copy destination and wait count is an immediate, a k-step is ~18 instructions. The partial
+// tiles of the four waves meet in LDS once, behind the stream (no barrier inside it).
+template <typename T, bool HALF_A, bool GATE_UP, int STEPS, int TPW>
+__global__ __launch_bounds__(kSmallMNtWaves * 64) void hgemm_smallm_nt_rega_kernel(const T* __restrict__ A, const T* __restrict__ B,
+                                                                   T* C, const T* R, int M, int N, long lda, long ldb,
+                                                                   long ldc, long ldr, int n_groups) {
+    using V8 = typename Elem<T>::v8;
+    constexpr int NST = kSmallMNtStages, TOTAL = TPW * STEPS;
+    constexpr int kCopiesA = HALF_A ? 1 : 2;
+    extern __shared__ __attribute__((aligned(1024))) char smem_raw[];
+    MI355_LDS char* smem = (MI355_LDS char*)smem_raw;
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+
+    int group = blockIdx.x;
+    if (n_groups % 8 == 0) group = (blockIdx.x % 8) * (n_groups / 8) + blockIdx.x / 8;
+    const int tile0 = group * TPW;
+    const long kbase = (long)wave * STEPS * 64;
+
+    // slab = 16 rows x 128 bytes; a copy instruction covers 8 rows (row lane/8, chunk position lane%8); chunk c of row r is
+    // stored at position c ^ (r & 7). Lane offsets are relative to the tile's first row and the wave's first column.
+    const int c_row = lane >> 3;
+    const int c_chunk = (lane & 7) ^ (c_row & 7);
+    const uint32_t b_voff0 = (uint32_t)((long)c_row * ldb * 2 + c_chunk * 16);
+    const uint32_t b_voff1 = (uint32_t)((long)(c_row + (GATE_UP ? 32 : 8)) * ldb * 2 + c_chunk * 16);
+    const uint32_t a_voff0 = (uint32_t)((long)min(c_row, M - 1) * lda * 2 + c_chunk * 16);
+    const uint32_t a_voff1 = (uint32_t)((long)min(c_row + 8, M - 1) * lda * 2 + c_chunk * 16);
+    const T* a_base = A + kbase;
+    // first weight row of tile t (GATE_UP: 8 gate rows there, their 8 up rows 32 further on)
+    const T* b_base[TPW];
+#pragma unroll
+    for (int i = 0; i < TPW; ++i) {
+        const int t = tile0 + i;
+        b_base[i] = B + (long)(GATE_UP ? 64 * (t >> 2) + 8 * (t & 3) : t * 16) * ldb + kbase;
+    }
+    const uint32_t wave_lds = (uint32_t)(uintptr_t)(smem + wave * kSmallMNtWaveBytes);
+
+    // fragment of k-substep sub (32 deep): lane holds X[row = lane%16][k = 32*sub + 8*(lane/16) .. +7]
+    const int f_row = lane & 15;
+    MI355_LDS char* f_ptr[2];
+#pragma unroll
+    for (int sub = 0; sub < 2; ++sub)
+        f_ptr[sub] = smem + wave * kSmallMNtWaveBytes + f_row * 128 + (((4 * sub + (lane >> 4)) ^ (f_row & 7)) << 4);
+    MI355_LDS float* red = (MI355_LDS float*)(smem + kSmallMNtLdsBytes);   // [TPW][waves][256]
+
+    V8 areg[STEPS][2];
+    float4v acc = float4v{0.f, 0.f, 0.f, 0.f};
+
+    auto copies_of = [](int u) { return u >= TOTAL ? 0 : u < STEPS ? 2 + kCopiesA : 2; };
+    auto issue = [&](auto uc) {
+        constexpr int u = decltype(uc)::value, i = u / STEPS, st = u % STEPS, slot = u % NST;
+        const T* bb = b_base[i] + st * 64;   // scalar pointer arithmetic
+        copy16_global_to_lds_imm<slot * kSmallMNtStageBytes>(bb, b_voff0, wave_lds);
+        copy16_global_to_lds_imm<slot * kSmallMNtStageBytes + 1024>(bb, b_voff1, wave_lds);
+        if constexpr (i == 0) {
+            const T* ab = a_base + st * 64;
+            copy16_global_to_lds_imm<slot * kSmallMNtStageBytes + 2048>(ab, a_voff0, wave_lds);
+            if constexpr (!HALF_A) copy16_global_to_lds_imm<slot * kSmallMNtStageBytes + 3072>(ab, a_voff1, wave_lds);
+        }
+    };
+    static_for<0, NST - 1>([&](auto uc) { issue(uc); });
+    static_for<0, TOTAL>([&](auto uc) {
+        constexpr int u = decltype(uc)::value, i = u / STEPS, st = u % STEPS, slot = u % NST;
+        if constexpr (u + NST - 1 < TOTAL) issue(std::integral_constant<int, u + NST - 1>{});
+        wait_vmcnt<copies_of(u + 1) + copies_of(u + 2) + copies_of(u + 3)>();   // everything up to step u has landed
+        static_assert(NST == 4, "the wait above counts the three steps in flight behind step u");
+#pragma unroll
+        for (int sub = 0; sub < 2; ++sub) {
+            V8 bf = Elem<T>::frag(lds_read_b128(f_ptr[sub] + slot * kSmallMNtStageBytes));
+            if constexpr (i == 0) areg[st][sub] = Elem<T>::frag(lds_read_b128(f_ptr[sub] + (slot * kSmallMNtStageBytes + 2048)));
+            acc = Elem<T>::mfma16(areg[st][sub], bf, acc);
+        }
+        wait_lgkmcnt<0>();  // the reads of this slot are complete before a later copy refills it
+        if constexpr (st == STEPS - 1) {   // acc[q] is D[m = 4*(lane/16) + q][n = lane%16] of tile i
+#pragma unroll
+            for (int q = 0; q < 4; ++q) red[(i * kSmallMNtWaves + wave) * 256 + (4 * (lane >> 4) + q) * 16 + (lane & 15)] = acc[q];
+            acc = float4v{0.f, 0.f, 0.f, 0.f};
+        }
+    });
+
+    __syncthreads();
+    for (int o = tid; o < TPW * 256; o += kSmallMNtWaves * 64) {
+        const int i = o >> 8, e = o & 255, tile = tile0 + i;
+        const MI355_LDS float* rt = red + i * kSmallMNtWaves * 256;
+        float sum = 0.f;
+#pragma unroll
+        for (int w = 0; w < kSmallMNtWaves; ++w) sum += rt[w * 256 + e];
+        const int m = e >> 4;
+        if constexpr (GATE_UP) {
+            if ((e & 15) < 8 && m < M) {   // column e % 16 is a gate, the one 8 further on its up
+                float up = 0.f;
+#pragma unroll
+                for (int w = 0; w < kSmallMNtWaves; ++w) up += rt[w * 256 + e + 8];
+                const float sig = __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(-sum * 1.4426950408889634f));
+                C[(long)m * ldc + 32 * (tile >> 2) + 8 * (tile & 3) + (e & 15)] = (T)(sum * sig * up);
+            }
+        } else {
+            const int n = tile * 16 + (e & 15);
+            if (m < M && n < N) {
+                T v = (T)sum;
+                if (R != nullptr) v = (T)((float)v + (float)R[(long)m * ldr + n]);
+                C[(long)m * ldc + n] = v;
+            }
+        }
+    }
+}
+
+// Tiles per workgroup for the kernel above, or 0 when it does not apply: K = 4096, at most 16 rows, whole tiles, and at
+// least 192 workgroups left to keep the memory system busy. Measured on weights that come from HBM (a different weight
+// matrix on every launch), against one tile per workgroup: 16 x 14336 x 4096 24.5 -> 21.7 us with four tiles (22.1 with
+// two), 16 x 6144 x 4096 13.1 -> 11.4 (two), 16 x 28672 x 4096 43.2 -> 40.5 (four; 42.2 with two). Up to 8 rows, where
+// the activation slab is half as large to begin with: 8 x 14336 x 4096 22.3 -> 20.5 us with two tiles (21.2 with four),
+// 8 x 28672 x 4096 39.1 -> 39.4-39.9 either way, so the widest products keep one tile per workgroup there.
+static int smallm_nt_rega_tpw(int M, int n_tiles, int K) {
+    if (M > 16 || K != 4096) return 0;
+    if (M <= 8) return n_tiles % 2 == 0 && n_tiles / 2 >= 192 && n_tiles / 2 <= 512 ? 2 : 0;
+    for (int tpw : {4, 2})
+        if (n_tiles % tpw == 0 && n_tiles / tpw >= 192) return tpw;
+    return 0;
+}
+
+template <typename T, bool HALF_A, bool GATE_UP>
+static hipError_t launch_smallm_nt_rega(const T* A, const T* B, T* C, const T* R, int M, int N, long lda, long ldb, long ldc,
+                                        long ldr, int n_tiles, int tpw, hipStream_t stream) {
+    static DynamicLdsOnce once4, once2;
+    const int groups = n_tiles / tpw;
+    if (tpw == 4) {
+        constexpr int lds = kSmallMNtLdsBytes + 4 * kSmallMNtWaves * 1024;
+        auto kern = hgemm_smallm_nt_rega_kernel<T, HALF_A, GATE_UP, 16, 4>;
+        if (hipError_t e = once4.ensure(reinterpret_cast<const void*>(kern), lds); e != hipSuccess) return e;
+        kern<<<dim3(groups), dim3(kSmallMNtWaves * 64), lds, stream>>>(A, B, C, R, M, N, lda, ldb, ldc, ldr, groups);
+    } else {
+        constexpr int lds = kSmallMNtLdsBytes + 2 * kSmallMNtWaves * 1024;
+        auto kern = hgemm_smallm_nt_rega_kernel<T, HALF_A, GATE_UP, 16, 2>;
+        if (hipError_t e = once2.ensure(reinterpret_cast<const void*>(kern), lds); e != hipSuccess) return e;
+        kern<<<dim3(groups), dim3(kSmallMNtWaves * 64), lds, stream>>>(A, B, C, R, M, N, lda, ldb, ldc, ldr, groups);
+    }
+    return hipGetLastError();
+}
+
 template <typename T>
 static hipError_t launch_smallm_nt(const T* A, const T* B, T* C, const T* R, int M, int N, int K, long lda, long ldb,
                                    long ldc, long ldr, hipStream_t stream) {
     static DynamicLdsOnce lds_once, lds_once_half;
     const int n_tiles = (N + 15) / 16;
+    if (const int tpw = N % 16 == 0 ? smallm_nt_rega_tpw(M, n_tiles, K) : 0; tpw > 0) {
+        if (M <= 8) return launch_smallm_nt_rega<T, true, false>(A, B, C, R, M, N, lda, ldb, ldc, ldr, n_tiles, tpw, stream);
+        return launch_smallm_nt_rega<T, false, false>(A, B, C, R, M, N, lda, ldb, ldc, ldr, n_tiles, tpw, stream);
+    }
     dim3 grid(n_tiles, (M + 15) / 16);
     if (M <= 8) {
         if (hipError_t e = lds_once_half.ensure(reinterpret_cast<const void*>(hgemm_smallm_nt_kernel<T, true, false>), kSmallMNtLdsBytes); e != hipSuccess) return e;
@@ -997,6 +1147,10 @@ static hipError_t launch_smallm_nt_gate_up(const T* A, const T* B, T* C, int M, 
                                            hipStream_t stream) {
     static DynamicLdsOnce lds_once, lds_once_half;
     const int n_tiles = N / 16;
+    if (const int tpw = smallm_nt_rega_tpw(M, n_tiles, K); tpw > 0) {
+        if (M <= 8) return launch_smallm_nt_rega<T, true, true>(A, B, C, nullptr, M, N, lda, ldb, ldc, 0, n_tiles, tpw, stream);
+        return launch_smallm_nt_rega<T, false, true>(A, B, C, nullptr, M, N, lda, ldb, ldc, 0, n_tiles, tpw, stream);
+    }
     dim3 grid(n_tiles, 1);
     if (M <= 8) {
         if (hipError_t e = lds_once_half.ensure(reinterpret_cast<const void*>(hgemm_smallm_nt_kernel<T, true, true>), kSmallMNtLdsBytes); e != hipSuccess) return e;

@@ -72,6 +72,19 @@ __device__ __forceinline__ void copy16_global_to_lds(const void* uniform_base, u
         : "memory", "m0");
 }
 
+// The same with the LDS destination as a scalar register plus a compile-time constant (one scalar instruction into M0).
+// The instruction's own offset field is not used: the hardware adds it to the LDS address as well as to the global one.
+template <int LDS_IMM>
+__device__ __forceinline__ void copy16_global_to_lds_imm(const void* uniform_base, uint32_t lane_byte_offset, uint32_t lds_wave_base) {
+    asm volatile(
+        "s_add_u32 m0, %2, %3\n\t"
+        "s_nop 0\n\t"
+        "global_load_lds_dwordx4 %0, %1"
+        :
+        : "v"(lane_byte_offset), "s"(uniform_base), "s"(lds_wave_base), "n"(LDS_IMM)
+        : "memory", "m0", "scc");
+}
+
 // Buffer resource (V#) over a whole address range: 48-bit base, no stride, no swizzle, the largest record count, raw
 // 32-bit data format. The four words must sit in scalar registers, so every word is made wave-uniform explicitly.
 __device__ __forceinline__ int4v make_buffer_resource(const void* base) {
