@@ -1093,8 +1093,8 @@ __global__ __launch_bounds__(kSmallMNtWaves * 64) void hgemm_smallm_nt_rega_kern
 // two), 16 x 6144 x 4096 13.1 -> 11.4 (two), 16 x 28672 x 4096 43.2 -> 40.5 (four; 42.2 with two). Up to 8 rows, where
 // the activation slab is half as large to begin with: 8 x 14336 x 4096 22.3 -> 20.5 us with two tiles (21.2 with four),
 // 8 x 28672 x 4096 39.1 -> 39.4-39.9 either way, so the widest products keep one tile per workgroup there.
-static int smallm_nt_rega_tpw(int M, int n_tiles, int K) {
-    if (M > 16 || K != 4096) return 0;
+static int smallm_nt_rega_tpw(int M, int n_tiles, int K, long lda, long ldb) {
+    if (M > 16 || K != 4096 || lda >= (1L << 22) || ldb >= (1L << 22)) return 0;   // lane offsets of up to 40 rows in 32 bits
     if (M <= 8) return n_tiles % 2 == 0 && n_tiles / 2 >= 192 && n_tiles / 2 <= 512 ? 2 : 0;
     for (int tpw : {4, 2})
         if (n_tiles % tpw == 0 && n_tiles / tpw >= 192) return tpw;
@@ -1125,7 +1125,7 @@ static hipError_t launch_smallm_nt(const T* A, const T* B, T* C, const T* R, int
                                    long ldc, long ldr, hipStream_t stream) {
     static DynamicLdsOnce lds_once, lds_once_half;
     const int n_tiles = (N + 15) / 16;
-    if (const int tpw = N % 16 == 0 ? smallm_nt_rega_tpw(M, n_tiles, K) : 0; tpw > 0) {
+    if (const int tpw = N % 16 == 0 ? smallm_nt_rega_tpw(M, n_tiles, K, lda, ldb) : 0; tpw > 0) {
         if (M <= 8) return launch_smallm_nt_rega<T, true, false>(A, B, C, R, M, N, lda, ldb, ldc, ldr, n_tiles, tpw, stream);
         return launch_smallm_nt_rega<T, false, false>(A, B, C, R, M, N, lda, ldb, ldc, ldr, n_tiles, tpw, stream);
     }
@@ -1147,7 +1147,7 @@ static hipError_t launch_smallm_nt_gate_up(const T* A, const T* B, T* C, int M, 
                                            hipStream_t stream) {
     static DynamicLdsOnce lds_once, lds_once_half;
     const int n_tiles = N / 16;
-    if (const int tpw = smallm_nt_rega_tpw(M, n_tiles, K); tpw > 0) {
+    if (const int tpw = smallm_nt_rega_tpw(M, n_tiles, K, lda, ldb); tpw > 0) {
         if (M <= 8) return launch_smallm_nt_rega<T, true, true>(A, B, C, nullptr, M, N, lda, ldb, ldc, 0, n_tiles, tpw, stream);
         return launch_smallm_nt_rega<T, false, true>(A, B, C, nullptr, M, N, lda, ldb, ldc, 0, n_tiles, tpw, stream);
     }
