@@ -8,8 +8,9 @@
 //
 // Main kernel: one workgroup of 8 waves computes a 256x256 tile of C, K is walked in steps of 64.
 //   * global -> LDS staging uses 16-byte direct-to-LDS copies (no VGPR bounce) into a ring of stages (two 64 KiB
-//     stages for the 256x256 tile, three stages for the 128x128 and 128x64 tiles); every wave-instruction writes 1 KiB
-//     of contiguous LDS, the XOR swizzle is applied on the global-address side.
+//     stages for the 256x256 tile, three for 128x128, five for 64x128 / 128x64, eight - or four, with two workgroups
+//     on a CU - for 64x64); every wave-instruction writes 1 KiB of contiguous LDS, the XOR swizzle is applied on the
+//     global-address side.
 //     The copies are buffer loads (scalar tile base + one 32-bit lane offset): a global load with 64-bit lane
 //     addresses takes about twice as much issue time away from the MFMAs it runs beside, and several times as
 //     much when such loads are issued back to back.
@@ -146,6 +147,7 @@ struct MainCfg {
     // K tile of time to land (small problems run few tiles per workgroup and are bound by that latency). The narrow tiles
     // serve products with few rows, which are bound by the stream of the weight matrix from HBM: their ring is as deep
     // as 128 KiB of LDS allow (5 stages of 24 KiB, 8 of 16 KiB), so that a CU keeps ~50 KiB of that stream in flight.
+    // STAGES > 0 sets the depth (the 64x64 tiles of small products run with four stages, two workgroups to a CU).
     static constexpr int NSTAGE = STAGES > 0 ? STAGES : STAGE_BYTES > 48 * 1024 ? 2 : STAGE_BYTES > 24 * 1024 ? 3 : STAGE_BYTES > 16 * 1024 ? 5 : 8;
     static constexpr int LDS_BYTES = STAGE_BYTES * NSTAGE;
     static constexpr int A_INSTS = A_BYTES / (NWAVES * 1024);  // 16-byte copies per lane per K tile
