@@ -63,8 +63,9 @@ extern "C" {
  *   layout NT  <- finegemm_13..15 (manual/gemm_13_amd.cpp:248-270, gemm_14_amd.cpp:268-290,
  *                                  gemm_15_amd.cpp:291-313)
  * lda/ldb/ldc are in elements and refer to the stored matrices (e.g. lda >= M for layout TN).
- * Any M, N, K >= 1 is accepted. The fast paths need 16-byte aligned operands and leading dimensions, K % 64 == 0 and
- * N % 8 == 0 (M % 8 == 0 for layout TN); M is otherwise free (ragged tile edges are handled inside the kernels).
+ * Any M, N, K >= 1 is accepted. The fast paths need 16-byte aligned operands and leading dimensions, N % 8 == 0 and
+ * K % 64 == 0 (other K > 64: one more launch for the last K % 64 columns); M is free (ragged tile edges are handled inside the kernels; layout TN reads up to 7 columns of the padding
+ * that lda, a multiple of 8, leaves behind M).
  */
 int mi355_hgemm(const void* A, const void* B, void* C, int M, int N, int K, int64_t lda, int64_t ldb,
                 int64_t ldc, int layout, void* stream);

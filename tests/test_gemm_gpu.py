@@ -158,6 +158,26 @@ def test_seeded_random_products_choose_their_own_kernel(lib, gpu, layout, M, N, 
     assert bool((c[M:] == 7.0).all()) and bool((c[:, N:] == 7.0).all())
 
 
+@pytest.mark.parametrize("M,N,K", [(5, 512, 256), (13, 4096, 1024), (33, 136, 192), (100, 1024, 512), (300, 2048, 256),
+                                   (1001, 1000, 1024), (2050, 512, 128), (12, 4096, 4160)])
+def test_layout_tn_with_any_row_count_in_padded_rows(lib, gpu, M, N, K):
+    # A stored [K, M] in rows of lda = M rounded up to a multiple of 8 (16-byte aligned rows): the small-M and tiled
+    # kernels read whole 16-byte chunks, so up to 7 columns of the padding, which holds NaNs here, and must keep them out
+    # of the M rows they store; nothing outside C[:M, :N] may change
+    a, b = so.gemm_inputs(M, N, K, seed=M + N, b_std=0.05)
+    lda = (M + 7) // 8 * 8
+    a_pad = torch.full((K, lda), float("nan"), dtype=torch.float16)
+    a_pad[:, :M] = a.t()
+    ag, bg = a_pad.to(gpu), b.to(gpu)
+    c = torch.full((M + 2, N + 8), 5.0, dtype=torch.float16, device=gpu)
+    lib.hgemm_raw(ag.data_ptr(), bg.data_ptr(), c.data_ptr(), M, N, K, lda, N, N + 8, lib.GEMM_TN,
+                  torch.cuda.current_stream(gpu).cuda_stream)
+    torch.cuda.synchronize()
+    ok, st = so.gemm_tolerance_ok(c[:M, :N].cpu(), so.gemm_ref(a, b, "NN"), K)
+    assert ok, (M, N, K, st)
+    assert bool((c[M:] == 5.0).all()) and bool((c[:, N:] == 5.0).all())
+
+
 @pytest.mark.parametrize("variant", [1, 2, 3, 4])
 @pytest.mark.parametrize("layout", ["NN", "TN", "NT"])
 def test_every_tile_variant(lib, gpu, variant, layout):

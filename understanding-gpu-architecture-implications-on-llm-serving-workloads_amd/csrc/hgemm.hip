@@ -287,8 +287,9 @@ __device__ __forceinline__ void store_wave_tile(const float4v (&acc)[TM][TN], MI
 // R (may be null, may be C itself): a residual of C's shape added to the rounded product, `residual + proj(x)` of
 // modeling_llama.py:776,781 with the rounding of the unfused sequence (product to T, then the sum to T).
 // RAGGED: M (and N) need not be multiples of the tile. Copies of rows past the end are redirected to the last row (or, for
-// an operand whose M/N index is contiguous, to the last 8 columns; that dimension must be a multiple of 8), so every
-// load stays inside the matrices, and the epilogue stores only what exists.
+// an operand whose M/N index is contiguous, to the last 8 columns: N must be a multiple of 8; M of layout TN is rounded
+// up to one, the columns in between lie in the padding of A's rows because lda is a multiple of 8), so every load stays
+// inside the matrices' rows, and the epilogue stores only what exists.
 template <typename T, bool A_KC, bool B_KC, int BM, int BN, int WM, int WN, int EPI = 0, bool RAGGED = false, int STAGES = 0, int PER_CU = 1>
 __global__ __launch_bounds__(WM * WN * 64) __attribute__((amdgpu_waves_per_eu(WM * WN / 4, PER_CU * WM * WN / 4)))
 void hgemm_main_kernel(const T* __restrict__ A, const T* __restrict__ B,
@@ -370,7 +371,7 @@ void hgemm_main_kernel(const T* __restrict__ A, const T* __restrict__ B,
                 a_voff[i] = clamped(lda, true, ATK::kRowsPerInst, ATK::kChunksPerRow, ATK::kRowsPerPass, i, m0, M, ATK::swz(row));
             } else {
                 const int row = wave * ATM::kRowsPerInst + lane / ATM::kChunksPerRow + i * ATM::kRowsPerPass;
-                a_voff[i] = clamped(lda, false, ATM::kRowsPerInst, ATM::kChunksPerRow, ATM::kRowsPerPass, i, m0, M, ATM::swz(row));
+                a_voff[i] = clamped(lda, false, ATM::kRowsPerInst, ATM::kChunksPerRow, ATM::kRowsPerPass, i, m0, (M + 7) & ~7, ATM::swz(row));
             }
         }
 #pragma unroll
@@ -679,7 +680,9 @@ __global__ __launch_bounds__(256) void hgemm_edge_kernel(const T* __restrict__ A
 //     keeps kSmallMStages-1 steps in flight, and waits for the oldest with s_waitcnt vmcnt;
 //   * B fragments are read with the transposing LDS read, the product is MFMA 16x16x32;
 //   * layout TN (A stored [K,M], A_KC = false): the A slab of a k-step is 32 rows (k) x 16 m, copied as it lies and read
-//     with the transposing read like B; M must be a multiple of 8.
+//     with the transposing read like B. Its 16-byte chunks hold 8 rows of the product: the chunks of the rows M .. M
+//     rounded up to 8 lie in the padding of A's rows (lda is a multiple of 8 and at least M), their rows of the product
+//     are never stored; chunks past that fold back onto the last one.
 // ---------------------------------------------------------------------------------------------------------
 constexpr int kSmallMWaves = 8;
 constexpr int kSmallMStages = 3;
@@ -731,7 +734,7 @@ __global__ __launch_bounds__(kSmallMWaves * 64) void hgemm_smallm_nn_kernel(cons
     const int at_slot = lane >> 1;
     const int at_k = (at_slot & ~12) | ((at_slot & 4) << 1) | ((at_slot & 8) >> 1);
     const T* a_src = A_KC ? A + (long)min(m0 + a_row, M - 1) * lda + (long)s_begin * 32 + a_chunk * 8
-                          : A + (long)(s_begin * 32 + at_k) * lda + min(m0 + 8 * (lane & 1), M - 8);
+                          : A + (long)(s_begin * 32 + at_k) * lda + min(m0 + 8 * (lane & 1), ((M + 7) & ~7) - 8);
 
     auto issue_stage = [&](int slot) {
         MI355_LDS char* st = wbase + slot * kSmallMStageBytes;
@@ -1264,7 +1267,7 @@ static hipError_t launch_layout(const T* A, const T* B, T* C, const T* R, int M,
     }
     // the tiled kernels address a tile with 32-bit byte offsets: up to 256 rows of lda (ldb) elements
     const bool k_ok = aligned && K % 64 == 0 && K >= 64 && lda < (1L << 22) && ldb < (1L << 22);
-    const bool ragged_ok = k_ok && N % 8 == 0 && N >= 8 && (A_KC || (M % 8 == 0 && M >= 8));
+    const bool ragged_ok = k_ok && N % 8 == 0 && N >= 8;
     const bool small_m = M <= 64 && !(ragged_ok && few_rows_prefer_tiles(M, N, K, A_KC && B_KC));
     // Up to 64 rows (generation-step projections): 64x64 tiles with an 8-deep ring stream the second operand once, on
     // N / 64 workgroups with ~50 KiB each in flight, where the split-K small-M kernels below stream it once per 16 rows.
@@ -1272,8 +1275,8 @@ static hipError_t launch_layout(const T* A, const T* B, T* C, const T* R, int M,
         if (M == 64 && N % 64 == 0) return launch_main<T, A_KC, B_KC, 64, 64, 2, 2>(A, B, C, R, M, N, K, lda, ldb, ldc, ldr, stream);
         return launch_main<T, A_KC, B_KC, 64, 64, 2, 2, 0, true>(A, B, C, R, M, N, K, lda, ldb, ldc, ldr, stream);
     }
-    if constexpr (!B_KC) {   // NN, and TN with M a multiple of 8 (its A slab is copied in 8-row chunks)
-        if (aligned && small_m && K % 32 == 0 && K >= 32 && N % 8 == 0 && ldc % 2 == 0 && (A_KC || M % 8 == 0))
+    if constexpr (!B_KC) {   // NN and TN
+        if (aligned && small_m && K % 32 == 0 && K >= 32 && N % 8 == 0 && ldc % 2 == 0)
             return launch_smallm_nn<T, A_KC>(A, B, C, R, M, N, K, lda, ldb, ldc, ldr, stream);
     }
     if constexpr (A_KC && B_KC) {
