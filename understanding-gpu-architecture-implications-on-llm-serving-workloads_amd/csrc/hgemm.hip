@@ -177,7 +177,6 @@ __device__ __forceinline__ void static_for(F&& f) {
 __device__ __forceinline__ void tile_of_block(int bid, int tiles_m, int tiles_n, int& tm, int& tn) {
     const int total = tiles_m * tiles_n;
     constexpr int kXcd = 8;
-#ifndef MI355_GEMM_NO_SUPERBLOCKS
     // Large grids: the 256 workgroups that run at the same time (ids 256 s .. 256 s + 255, one per CU) take one
     // super-block of 256 tiles, each XCD an 8 x 4 piece of it, and the super-blocks follow one another in serpentine
     // order, so that consecutive ones share their row panels of A or their column panels of B. A super-block reads
@@ -195,7 +194,6 @@ __device__ __forceinline__ void tile_of_block(int bid, int tiles_m, int tiles_n,
         tn = bcol * sb_n + (x % xcd_cols) * 4 + (j >> 3);
         return;
     }
-#endif
     int t = bid;
     if (total % kXcd == 0) {
         int per = total / kXcd;
@@ -541,11 +539,7 @@ void hgemm_main_kernel(const T* __restrict__ A, const T* __restrict__ B,
     constexpr int kCopySpacingNum = NSLOT >= 2 * NCOPY ? 8 : 4 * NSLOT / NCOPY, kCopySpacingDen = 4;
     static_assert((NCOPY - 1) * kCopySpacingNum / kCopySpacingDen < NSLOT, "copies go out within one substep");
     // where a substep has a slot to spare, M0 is set one slot ahead of its load
-#ifdef MI355_GEMM_NO_SPLIT_M0
-    constexpr bool kSplitM0 = false;
-#else
     constexpr bool kSplitM0 = (NCOPY - 1) * kCopySpacingNum / kCopySpacingDen + 1 < NSLOT;
-#endif
     auto copies_of_slot = [&](auto sc, auto gc) {   // issue the copies whose slot is g
         constexpr int g = decltype(gc)::value;
         static_for<0, NCOPY>([&](auto dc) {

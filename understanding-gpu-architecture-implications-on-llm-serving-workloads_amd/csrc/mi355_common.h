@@ -100,20 +100,8 @@ __device__ __forceinline__ int4v make_buffer_resource(const void* base) {
 // The same 16-byte global -> LDS copy through a buffer resource: lane address = resource base + lane_byte_offset (one
 // 32-bit VGPR) + uniform_byte_offset (a scalar register). A wave instruction that reads one address VGPR instead of a
 // 64-bit pair takes about half as much issue time away from the MFMAs it runs beside, and all per-tile address
-// arithmetic (advancing the base) runs on the scalar unit.
-__device__ __forceinline__ void copy16_buffer_to_lds(int4v resource, uint32_t lane_byte_offset, uint32_t uniform_byte_offset,
-                                                     MI355_LDS void* lds_wave_base) {
-    asm volatile(
-        "s_mov_b32 m0, %3\n\t"
-        "s_nop 0\n\t"
-        "buffer_load_dwordx4 %0, %1, %2 offen lds"
-        :
-        : "v"(lane_byte_offset), "s"(resource), "s"(uniform_byte_offset), "s"((uint32_t)(uintptr_t)lds_wave_base)
-        : "memory", "m0");
-}
-
-// The same with the LDS destination given as a scalar register plus a compile-time offset: one scalar instruction sets
-// M0 (a copy whose destination is a run-time value needs a second one to form it).
+// arithmetic (advancing the base) runs on the scalar unit. The LDS destination is a scalar register plus a compile-time
+// offset: one scalar instruction sets M0 (a destination that is a run-time value needs a second one to form it).
 template <int IMM>
 __device__ __forceinline__ void copy16_buffer_to_lds_at(int4v resource, uint32_t lane_byte_offset, uint32_t uniform_byte_offset,
                                                         uint32_t lds_wave_base) {
