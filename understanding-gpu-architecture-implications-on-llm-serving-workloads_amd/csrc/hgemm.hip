@@ -1195,10 +1195,10 @@ static bool few_rows_prefer_tiles(int M, int N, int K, bool nt) {
     return few_row_tiles_us(M, N, K, nt) < small_m_us(M, N, K, false) - 4.0;
 }
 // Which tile shape is expected to finish a product of more than 64 rows first (1 = 256x256, 2 = 128x128, 3 = 64x128 or
-// 128x64, 4 = 64x64 two to a CU). A CU takes in 64 bytes per cycle from the memory system and its LDS serves the
-// direct-to-LDS writes and the fragment reads one after the other, so the time of a K tile is set by the tile's bytes
-// as much as by its matrix instructions: measured cycles per K tile of 64 of one workgroup alone on its CU are 2470
-// (256x256; matrix pipes 2048), 770 (128x128; pipes 512, LDS 768), 576 (half tile) and 384 (64x64). A workgroup spends
+// 128x64, 4 = 64x64 two to a CU). A CU takes in 64 bytes per cycle from the memory system, so the time of a K tile is
+// set by the tile's bytes as much as by its matrix instructions (the operands of a 128x128 tile need the same 512 cycles
+// to arrive that its matrix instructions take): measured cycles per K tile of 64 of one workgroup alone on its CU are
+// 2470 (256x256; matrix pipes 2048), 770 (128x128; pipes 512), 576 (half tile) and 384 (64x64). A workgroup spends
 // another 5000-12000 cycles outside its K loop (first tiles in flight, epilogue). The workgroups run in rounds of one
 // per CU (two for the 64x64 tiles); the last round may be a partial one. The model reproduces the measured times of
 // 1024^3 .. 8192^3, 2048 x 4096 x 4096 and 1536 x 1536 x 8192 within ~10 %. The 128x128 figure used below is 840: on
