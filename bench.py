@@ -629,7 +629,7 @@ def main():
 
 # name -> ("gemm", M, N, K, layout) or ("fmha", B, Hq, Hkv, Sq, Sk, causal); each runs one kernel of the library
 KERNEL_CONFIGS = {
-    "g1_gemm_1024_nn": ("gemm", 1024, 1024, 1024, "NN"),                    # 64x128 tiles
+    "g1_gemm_1024_nn": ("gemm", 1024, 1024, 1024, "NN"),                    # 64x64 tiles, two workgroups to a CU
     "g2a_gemm_4096_nn": ("gemm", 4096, 4096, 4096, "NN"),                   # 256x256 tiles, one per CU
     "g2b_gemm_8192_nn": ("gemm", 8192, 8192, 8192, "NN"),                   # 256x256 tiles
     "g2b_gemm_8192_nt": ("gemm", 8192, 8192, 8192, "NT"),
