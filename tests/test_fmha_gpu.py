@@ -174,6 +174,62 @@ def test_generation_step_workspace_shared_by_calls_of_different_shapes(lib, gpu)
         check(lib, gpu, q, k, v, False, None)
 
 
+def _seeded_mixed_cases(n, seed):
+    """n cases drawn with a fixed seed over everything a caller can vary at once: prefill, generation-step and very short
+    shapes; fp16 or bf16; contiguous [B,H,S,D] tensors or [B,S,H,D] tensors viewed as [B,H,S,D]; a valid length short of
+    Sk (with NaNs behind it); the entry point that allocates nothing."""
+    rng = np.random.default_rng(seed)
+    out = []
+    while len(out) < n:
+        mode = str(rng.choice(["prefill", "prefill", "step", "short"]))
+        hkv = int(rng.choice([1, 2, 4, 8]))
+        hq = hkv * int(rng.choice([1, 1, 2, 4, 8]))
+        if mode == "prefill":
+            b = int(rng.choice([1, 2, 3])); sq = int(rng.choice([100, 129, 255, 256, 257, 511, 777, 1024])); sk = sq + int(rng.choice([0, 0, 1, 63, 200]))
+        elif mode == "step":
+            b = int(rng.choice([1, 2, 4, 9])); sq = int(rng.choice([1, 1, 2, 4])); sk = int(rng.choice([512, 513, 1000, 2048, 5000]))
+        else:
+            b = int(rng.choice([1, 2, 7])); sq = int(rng.choice([1, 2, 5, 16, 33, 64])); sk = int(rng.choice([1, 3, 17, 63, 64, 65, 130, 400]))
+        if b * hq * sq * sk > 4e7:
+            continue
+        causal = bool(rng.random() < 0.5)
+        if causal and sq > sk:
+            sk = sq
+        kvv = sk if rng.random() < 0.6 else int(rng.integers(1, sk + 1))
+        bf16 = bool(rng.random() < 0.25)
+        out.append((b, hq, hkv, sq, sk, causal, kvv, bf16, bool(rng.random() < 0.4), (not bf16) and bool(rng.random() < 0.3)))
+    return out
+
+
+@pytest.mark.parametrize("B,Hq,Hkv,Sq,Sk,causal,kvv,bf16,strided,noalloc", _seeded_mixed_cases(48, 777))
+def test_seeded_random_cases_across_dtypes_views_and_entry_points(lib, gpu, B, Hq, Hkv, Sq, Sk, causal, kvv, bf16, strided, noalloc):
+    q, k, v = (bf16_inputs if bf16 else so.fmha_inputs)(B, Hq, Hkv, Sq, Sk, seed=B + 3 * Hq + 5 * Sq + 7 * Sk)
+    o_ref, lse_ref = so.attention_ref(q, k, v, causal=causal, kv_valid_len=kvv)
+    k, v = k.clone(), v.clone()
+    k[:, :, kvv:] = float("nan")   # keys behind the valid length must not be read into the result
+    v[:, :, kvv:] = float("nan")
+    if strided:
+        qg, kg, vg = (t.transpose(1, 2).contiguous().to(gpu).transpose(1, 2) for t in (q, k, v))
+        o = torch.full((B, Sq, Hq, 128), 7.0, dtype=q.dtype, device=gpu).transpose(1, 2)
+    else:
+        qg, kg, vg = q.to(gpu), k.to(gpu), v.to(gpu)
+        o = torch.full((B, Hq, Sq, 128), 7.0, dtype=q.dtype, device=gpu)
+    lse = None
+    if noalloc:
+        lse = torch.full((B, Hq, Sq), 7.0, dtype=torch.float32, device=gpu)
+        try:
+            lib.fmha_fwd_noalloc(qg, kg, vg, o, lse, causal=causal, kv_valid_len=kvv)
+        except lib.Mi355Error as e:   # more partial results than the static scratch holds: refused, nothing written
+            assert "static scratch" in str(e)
+            lse = None
+    if lse is None:
+        o, lse = lib.fmha_fwd(qg, kg, vg, causal=causal, kv_valid_len=kvv, out=o)
+    torch.cuda.synchronize()
+    err_o = float((o.float().cpu() - o_ref).abs().max())
+    err_l = float((lse.cpu() - lse_ref).abs().max())
+    assert err_o <= (1.6e-2 if bf16 else 2e-3) and err_l <= 1e-3, (err_o, err_l)
+
+
 def test_generation_step_on_two_streams(lib, gpu):
     # the split-KV workspace is per stream: interleaved calls on two streams must not disturb each other
     qa, ka, va = (t.to(gpu) for t in so.fmha_inputs(1, 32, 8, 1, 4096, seed=1))

@@ -178,6 +178,44 @@ def test_layout_tn_with_any_row_count_in_padded_rows(lib, gpu, M, N, K):
     assert bool((c[M:] == 5.0).all()) and bool((c[:, N:] == 5.0).all())
 
 
+def _seeded_padded_products(n, seed):
+    """n products drawn with a fixed seed whose three matrices all live in wider allocations: leading dimensions rounded
+    up to a multiple of 8 plus 0, 8 or 64 elements, in every layout, row counts from 1 to 3000, K on and off the tiles'
+    depth."""
+    rng = np.random.default_rng(seed)
+    out = []
+    for _ in range(n):
+        layout = ["NN", "NT", "TN"][int(rng.integers(3))]
+        m = int(rng.choice([1, 2, 5, 8, 9, 15, 16, 17, 31, 32, 48, 63, 64, 65, 100, 127, 128, 129, 200, 255, 256, 257, 384, 500, 512, 1000, 1500, 3000]))
+        nn = int(rng.choice([8, 16, 24, 64, 72, 128, 136, 256, 512, 1000, 1024, 2048, 3072, 4096])) + int(rng.choice([0, 0, 0, 8, 16]))
+        k = int(rng.choice([32, 64, 96, 128, 192, 256, 448, 512, 1024, 2048, 4096])) + int(rng.choice([0, 0, 0, 0, 16, 32, 8]))
+        if m * nn * k > 4e9:
+            k = 256
+        out.append((layout, m, nn, k, int(rng.choice([0, 0, 8, 64])), int(rng.choice([0, 0, 8, 64])), int(rng.choice([0, 8]))))
+    return out
+
+
+@pytest.mark.parametrize("layout,M,N,K,pad_a,pad_b,pad_c", _seeded_padded_products(48, 1234))
+def test_seeded_random_products_in_padded_allocations(lib, gpu, layout, M, N, K, pad_a, pad_b, pad_c):
+    # the padding of A and B holds NaNs: whatever a kernel reads of it must stay out of the product; C's padding and
+    # the row behind C must come back untouched
+    a, b = operands(M, N, K, layout, seed=M + 3 * N + 7 * K + pad_a, b_std=0.05)
+    lda = (a.shape[1] + 7) // 8 * 8 + pad_a
+    ldb = (b.shape[1] + 7) // 8 * 8 + pad_b
+    ldc = N + pad_c
+    ag = torch.full((a.shape[0], lda), float("nan"), dtype=torch.float16, device=gpu)
+    bg = torch.full((b.shape[0], ldb), float("nan"), dtype=torch.float16, device=gpu)
+    ag[:, :a.shape[1]] = a.to(gpu)
+    bg[:, :b.shape[1]] = b.to(gpu)
+    c = torch.full((M + 1, ldc), 3.0, dtype=torch.float16, device=gpu)
+    lib.hgemm_raw(ag.data_ptr(), bg.data_ptr(), c.data_ptr(), M, N, K, lda, ldb, ldc, lib.LAYOUTS[layout],
+                  torch.cuda.current_stream(gpu).cuda_stream)
+    torch.cuda.synchronize()
+    ok, st = so.gemm_tolerance_ok(c[:M, :N].cpu(), so.gemm_ref(a, b, layout), K)
+    assert ok, (layout, M, N, K, lda, ldb, ldc, st)
+    assert bool((c[M:] == 3.0).all()) and bool((c[:, N:] == 3.0).all())
+
+
 @pytest.mark.parametrize("variant", [1, 2, 3, 4])
 @pytest.mark.parametrize("layout", ["NN", "TN", "NT"])
 def test_every_tile_variant(lib, gpu, variant, layout):
