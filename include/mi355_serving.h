@@ -64,7 +64,7 @@ extern "C" {
  *                                  gemm_15_amd.cpp:291-313)
  * lda/ldb/ldc are in elements and refer to the stored matrices (e.g. lda >= M for layout TN).
  * Any M, N, K >= 1 is accepted. The fast paths need 16-byte aligned operands and leading dimensions, N % 8 == 0 and
- * K % 64 == 0 (other K > 64: one more launch for the last K % 64 columns); M is free (ragged tile edges are handled inside the kernels; layout TN reads up to 7 columns of the padding
+ * K % 8 == 0 (K % 64 != 0 with M <= 64 and no residual: one more launch for the last K % 64 columns); M is free (ragged tile edges are handled inside the kernels; layout TN reads up to 7 columns of the padding
  * that lda, a multiple of 8, leaves behind M).
  */
 int mi355_hgemm(const void* A, const void* B, void* C, int M, int N, int K, int64_t lda, int64_t ldb,
@@ -90,7 +90,8 @@ int mi355_hgemm_silu_mul(const void* A, const void* B, void* C, int M, int N, in
  * projections of a decoder layer whose result is added to the residual stream (`hidden_states = residual + hidden_states`
  * after o_proj and after down_proj, benchmarks/flashattn-cuda/modeling_llama.py:776,781; an elementwise kernel of its own
  * in the reference). The product is rounded to fp16 first and the sum once more, so the result equals that of the two
- * separate operations bit for bit. R may be C (in place; then ldr must equal ldc), otherwise R and C must not overlap;
+ * separate operations bit for bit (one exception: with K % 64 != 0 and M <= 64, mi355_hgemm forms its product in two
+ * passes and this entry point in one, so the two may differ in the last bit of the product). R may be C (in place; then ldr must equal ldc), otherwise R and C must not overlap;
  * ldr >= N. Layouts, shapes and fast-path conditions as mi355_hgemm (R and ldr aligned like C and ldc).
  */
 int mi355_hgemm_add(const void* A, const void* B, const void* R, void* C, int M, int N, int K, int64_t lda, int64_t ldb,

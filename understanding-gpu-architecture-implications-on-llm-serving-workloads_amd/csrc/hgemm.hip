@@ -383,8 +383,13 @@ void hgemm_main_kernel(const T* __restrict__ A, const T* __restrict__ B,
             }
         }
     }
-    int4v a_res = make_buffer_resource(a_base);
-    int4v b_res = make_buffer_resource(b_base);
+    // K need not be a multiple of the tile depth: the last K tile, which then holds K % 64 columns (rows) of the
+    // operands, is taken FIRST, by the prologue, with copies of its own (below); the loop never sees it.
+    const int ktiles = (K + BK - 1) / BK;
+    const int k_first = K - (ktiles - 1) * BK;   // depth of that tile: 8 .. 64
+    const long first_tile = k_first < BK ? ktiles - 1 : 0;   // position along K, in tiles, of the tile taken first
+    int4v a_res = make_buffer_resource(a_base + first_tile * a_k_step);
+    int4v b_res = make_buffer_resource(b_base + first_tile * b_k_step);
 
     // ---- LDS fragment read offsets (bytes inside one stage) -------------------------------------------
     // A fragments: TM blocks of 16 rows; B fragments: TN blocks of 16 columns; a K tile is two 32-deep substeps.
@@ -559,11 +564,42 @@ void hgemm_main_kernel(const T* __restrict__ A, const T* __restrict__ B,
     // the copies of tile kt + NSTAGE go into the stage tile kt has just left. At that barrier tile kt+1 must have
     // landed: all but the copies of the NSTAGE-2 tiles issued after it.
     constexpr int NSTAGE = Cfg::NSTAGE;
-    const int ktiles = K / BK;
     V8 af[2][TM], bf[2][TN];
     using Sub0 = std::integral_constant<int, 0>;
     using Sub1 = std::integral_constant<int, 1>;
-    static_for<0, NSTAGE>([&](auto sc) {
+    // The first tile is the one at the end of K. Its copies fetch nothing for k >= K: such a lane's offset is moved out
+    // of the range of the resource (2 GiB for these copies; offsets inside a tile stay below that), and a copy that is
+    // out of range writes zeros to LDS. Then the bases go back to k = 0 (with K a multiple of 64 the first tile is the
+    // one at k = 0 and the bases move on to the next: the tiles are then walked in memory order).
+    {
+        constexpr uint32_t kOutOfRange = 0x80000000u;   // with any uniform offset added it stays at or above the range, without wrapping
+        a_res[2] = (int)0x80000000u;
+        b_res[2] = (int)0x80000000u;
+        static_for<0, NCOPY>([&](auto dc) {
+            constexpr int d = decltype(dc)::value;
+            constexpr bool is_a = d < Cfg::A_INSTS;
+            constexpr int e = is_a ? d : d - Cfg::A_INSTS;
+            constexpr int dst = is_a ? e * Cfg::NWAVES * 1024 : kBRegion + e * Cfg::NWAVES * 1024;
+            uint32_t voff, soff = 0u;
+            if constexpr (RAGGED && is_a) voff = a_voff[e];
+            else if constexpr (RAGGED) voff = b_voff[e];
+            else { voff = is_a ? a_lane_off : b_lane_off; soff = e * (is_a ? a_copy_step : b_copy_step); }
+            int k_of_lane;   // first k (inside the tile) of the 16 bytes this lane copies
+            if constexpr (is_a ? A_KC : B_KC) {
+                using TK = std::conditional_t<is_a, ATK, BTK>;
+                const int row = wave * TK::kRowsPerInst + lane / TK::kChunksPerRow;
+                k_of_lane = ((lane % TK::kChunksPerRow) ^ TK::swz(row)) * 8;
+            } else {
+                using TC = std::conditional_t<is_a, ATM, BTN>;
+                k_of_lane = wave * TC::kRowsPerInst + lane / TC::kChunksPerRow + e * TC::kRowsPerPass;
+            }
+            if (k_of_lane >= k_first) voff = kOutOfRange;
+            copy16_buffer_to_lds_at<dst>(is_a ? a_res : b_res, voff, soff, wave_lds);
+        });
+        advance_base(a_res, k_first < BK ? -first_tile * a_k_step : a_k_step);
+        advance_base(b_res, k_first < BK ? -first_tile * b_k_step : b_k_step);
+    }
+    static_for<1, NSTAGE>([&](auto sc) {
         const int records = sign_mask_scalar(decltype(sc)::value - ktiles);
         a_res[2] = records;
         b_res[2] = records;
@@ -1208,7 +1244,7 @@ static int cheapest_tile_shape(int M, int N, int K) {
     struct Cand { int shape, bm, bn, per_cu; double step, fixed; };
     static const Cand cands[] = {{1, 256, 256, 1, 2470., 12000.}, {2, 128, 128, 1, 840., 7000.}, {3, 64, 128, 1, 576., 6000.},
                                  {4, 64, 64, 2, 384., 5000.}};
-    const double ktiles = (double)(K / 64);
+    const double ktiles = (double)((K + 63) / 64);
     int best = 2;
     double best_t = 0.;
     for (const Cand& c : cands) {
@@ -1246,11 +1282,12 @@ static hipError_t launch_layout(const T* A, const T* B, T* C, const T* R, int M,
                          (reinterpret_cast<uintptr_t>(C) % 16 == 0) && (lda % 8 == 0) && (ldb % 8 == 0) &&
                          (ldc % 8 == 0) && (reinterpret_cast<uintptr_t>(R) % 16 == 0) && (ldr % 8 == 0);
     // K that is not a multiple of the tiles' depth (the reference's own tiled kernels take K % 16 == 0,
-    // kernels/gemm/pkg/gemm_unified/csrc/auto/gemm_7.cu:115-135): the last K % 64 columns go through the bounds-checked
-    // kernel first, into C, and the tiled kernels then add the product over the first K - K % 64 to it as their residual
-    // (two roundings more than a single pass; a call that brings a residual of its own stays on the bounds-checked kernel,
-    // whose result is bit-identical to the product followed by an elementwise add).
-    if (aligned && R == nullptr && K > 64 && K % 64 != 0 && variant == 0) {
+    // kernels/gemm/pkg/gemm_unified/csrc/auto/gemm_7.cu:115-135): the tiled kernels take any multiple of 8, their
+    // prologue handles the K % 64 columns at the end. Up to 64 rows are better served by the small-M kernels, which
+    // need whole k-steps: there the last K % 64 columns go through the bounds-checked kernel first, into C, and the
+    // product over the first K - K % 64 is added to it as a residual (two roundings more than a single pass; 16 x 4096 x
+    // 4104 NT: 10 us, against 16 on tiles). A call that brings a residual of its own takes the tiles.
+    if (aligned && R == nullptr && M <= 64 && K > 64 && K % 64 != 0 && variant == 0) {
         const int k_tail = K % 64, k_main = K - k_tail;
         const T* a_tail = A_KC ? A + k_main : A + (long)k_main * lda;
         const T* b_tail = B_KC ? B + k_main : B + (long)k_main * ldb;
@@ -1260,7 +1297,7 @@ static hipError_t launch_layout(const T* A, const T* B, T* C, const T* R, int M,
         return launch_layout<T, A_KC, B_KC>(A, B, C, C, M, N, k_main, lda, ldb, ldc, ldc, variant, stream);
     }
     // the tiled kernels address a tile with 32-bit byte offsets: up to 256 rows of lda (ldb) elements
-    const bool k_ok = aligned && K % 64 == 0 && K >= 64 && lda < (1L << 22) && ldb < (1L << 22);
+    const bool k_ok = aligned && K % 8 == 0 && K >= 8 && lda < (1L << 22) && ldb < (1L << 22);
     const bool ragged_ok = k_ok && N % 8 == 0 && N >= 8;
     const bool small_m = M <= 64 && !(ragged_ok && few_rows_prefer_tiles(M, N, K, A_KC && B_KC));
     // Up to 64 rows (generation-step projections): 64x64 tiles with an 8-deep ring stream the second operand once, on
