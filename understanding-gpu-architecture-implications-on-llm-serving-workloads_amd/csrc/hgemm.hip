@@ -21,6 +21,9 @@
 //     inside their buffer resources; every tile issues the same instructions (the copies of the last tiles run on a
 //     resource whose size is set to zero: out of range, nothing is fetched), so the waits never change and the loop has
 //     one body per stage. Per K tile and wave of the 256x256 kernel: 64 MFMAs and ~58 other instructions.
+//   * K is any multiple of 8: the tile that holds the last K % 64 columns is taken first, by the prologue, whose copies
+//     point the lanes at k >= K out of the resource's range (such a copy writes zeros to LDS); the loop is the same code
+//     for every K.
 //   * an operand whose K index is contiguous in memory is read from LDS with ds_read_b128; an operand whose
 //     M/N index is contiguous (B in the NN case) is read with the transposing ds_read_b64_tr_b16, so no
 //     transpose pass over B is ever made.
