@@ -63,9 +63,12 @@ extern "C" {
  *   layout NT  <- finegemm_13..15 (manual/gemm_13_amd.cpp:248-270, gemm_14_amd.cpp:268-290,
  *                                  gemm_15_amd.cpp:291-313)
  * lda/ldb/ldc are in elements and refer to the stored matrices (e.g. lda >= M for layout TN).
- * Any M, N, K >= 1 is accepted. The fast paths need 16-byte aligned operands and leading dimensions, N % 8 == 0 and
- * K % 8 == 0 (K % 64 != 0 with M <= 64 and no residual: one more launch for the last K % 64 columns); M is free (ragged tile edges are handled inside the kernels; layout TN reads up to 7 columns of the padding
- * that lda, a multiple of 8, leaves behind M).
+ * Any M, N, K >= 1 is accepted. The fast paths need A and B 16-byte aligned with lda and ldb multiples of 8, and
+ * K % 8 == 0 (K % 64 != 0 with M <= 64 and no residual: one more launch for the last K % 64 columns); M and N are free
+ * (ragged tile edges are handled inside the kernels; an operand whose M or N index is contiguous is read in 16-byte
+ * chunks, up to 7 elements into the padding that its leading dimension, a multiple of 8, leaves behind M or N). C (and
+ * a residual) may have any row stride and alignment: rows that are not 16-byte aligned, or whose width is not a multiple
+ * of 8, are stored element by element.
  */
 int mi355_hgemm(const void* A, const void* B, void* C, int M, int N, int K, int64_t lda, int64_t ldb,
                 int64_t ldc, int layout, void* stream);

@@ -145,6 +145,45 @@ def test_k_tail_with_a_residual(lib, gpu, layout, M, N, K):
     assert bool((err <= bound).all()), (float(err.max()), int((err > bound).sum()))
 
 
+@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4])
+@pytest.mark.parametrize("layout", ["NN", "TN", "NT"])
+@pytest.mark.parametrize("M,N,K,ldc_pad", [(300, 1001, 256, 0), (512, 515, 136, 5), (1000, 77, 64, 3), (130, 3, 512, 0),
+                                           (16, 1001, 1024, 0), (48, 2049, 256, 1), (256, 256, 128, 1)])
+def test_widths_that_are_no_multiple_of_8_and_unaligned_rows_of_c(lib, gpu, variant, layout, M, N, K, ldc_pad):
+    # N need not be a multiple of 8 and C's rows need not be 16-byte aligned (a vocabulary of 50257 or 32001 entries): the
+    # tiled kernels (layout NT also the small-M kernel) store such a C element by element. An operand stored [K,N] is
+    # still copied in 16-byte chunks, so its rows must be aligned: ldb is N rounded up to 8, the padding holds NaNs and
+    # must stay out of the product. The residual has C's row stride. Nothing outside C[:M, :N] may change.
+    a, b = operands(M, N, K, layout, seed=M + N + K, b_std=0.05)
+    ldb = (b.shape[1] + 7) // 8 * 8
+    lda = (a.shape[1] + 7) // 8 * 8
+    ag = torch.full((a.shape[0], lda), float("nan"), dtype=torch.float16, device=gpu)
+    bg = torch.full((b.shape[0], ldb), float("nan"), dtype=torch.float16, device=gpu)
+    ag[:, :a.shape[1]] = a.to(gpu)
+    bg[:, :b.shape[1]] = b.to(gpu)
+    ldc = N + ldc_pad
+    c = torch.full((M + 1, ldc), 3.0, dtype=torch.float16, device=gpu)
+    st = torch.cuda.current_stream(gpu).cuda_stream
+    L = lib.load()
+    rc = L.mi355_internal_hgemm_variant(ag.data_ptr(), bg.data_ptr(), c.data_ptr(), M, N, K, lda, ldb, ldc, lib.LAYOUTS[layout], 0,
+                                        variant, st)
+    assert rc == 0
+    torch.cuda.synchronize()
+    ref = so.gemm_ref(a, b, layout)
+    ok, stt = so.gemm_tolerance_ok(c[:M, :N].cpu(), ref, K)
+    assert ok, (layout, M, N, K, ldc, stt)
+    assert bool((c[M:] == 3.0).all()) and bool((c[:, N:] == 3.0).all())
+    if variant == 0:   # with a residual of the same row stride, in place: bit for bit the product plus the residual
+        r = (torch.randn(M, N, generator=torch.Generator().manual_seed(1)) * 2).half().to(gpu)
+        want = c[:M, :N] + r
+        c[:M, :N] = r
+        assert L.mi355_hgemm_add(ag.data_ptr(), bg.data_ptr(), c.data_ptr(), c.data_ptr(), M, N, K, lda, ldb, ldc, ldc,
+                                 lib.LAYOUTS[layout], st) == 0
+        torch.cuda.synchronize()
+        assert torch.equal(c[:M, :N], want)
+        assert bool((c[M:] == 3.0).all()) and bool((c[:, N:] == 3.0).all())
+
+
 @pytest.mark.parametrize("variant,tile_m,tile_n", [(1, 256, 256), (2, 128, 128), (3, 64, 128), (4, 64, 64)])
 @pytest.mark.parametrize("layout", ["NN", "NT"])
 @pytest.mark.parametrize("tiles_m,tiles_n,ragged", [(16, 32, 0), (32, 24, 0), (32, 16, 8), (48, 16, 0)])

@@ -222,7 +222,7 @@ __device__ __forceinline__ void tile_of_block(int bid, int tiles_m, int tiles_n,
 // 4 (jo / 2) + jo % 2 and its up from two blocks further.
 template <typename T, int TM, int TN, int EPI, bool RAGGED>
 __device__ __forceinline__ void store_wave_tile(const float4v (&acc)[TM][TN], MI355_LDS char* cst, T* C, const T* R, long row0,
-                                                long col0, int M, int NC, long ldc, long ldr, int lane) {
+                                                long col0, int M, int NC, long ldc, long ldr, int lane, bool c_vec = true) {
     using V8 = typename Elem<T>::v8;
     using V4 = typename Elem<T>::v4;
     static_assert(EPI == 0 || TN % 4 == 0, "the gate/up epilogue pairs column blocks 32 columns apart");
@@ -262,20 +262,30 @@ __device__ __forceinline__ void store_wave_tile(const float4v (&acc)[TM][TN], MI
         const int rr = lane / kChunksC;
         const int cc = lane % kChunksC;
         T* cbase = C + row0 * ldc + col0 + cc * 8;
-        const long rows_left = M - row0;   // RAGGED: rows and 8-column chunks that exist
-        const bool col_ok = col0 + cc * 8 < NC;
+        const long rows_left = M - row0;   // RAGGED: rows and columns that exist
+        const long cols_left = NC - (col0 + cc * 8);   // of this lane's 8
         const T* rbase = R + row0 * ldr + col0 + cc * 8;
 #pragma unroll
         for (int it = 0; it < TM * 16 / kRowsPerStore; ++it) {
             const int row = it * kRowsPerStore + rr;
             V8 v = *(MI355_LDS const V8*)(cst + row * kRowBytesC + ((cc ^ (row & kSwzC)) << 4));
-            if (!RAGGED || (row < rows_left && col_ok)) {
+            if (!RAGGED || (row < rows_left && cols_left >= 8 && c_vec)) {
                 if (R != nullptr) {
                     const V8 r = *(const V8*)(rbase + (long)row * ldr);
 #pragma unroll
                     for (int j = 0; j < 8; ++j) v[j] = (T)((float)v[j] + (float)r[j]);
                 }
                 *(V8*)(cbase + (long)row * ldc) = v;
+            } else if (row < rows_left) {
+                // the last columns of a C whose width is not a multiple of 8, or a C (or residual) whose rows are not
+                // 16-byte aligned: element by element
+#pragma unroll
+                for (int j = 0; j < 8; ++j)
+                    if (j < cols_left) {
+                        T x = v[j];
+                        if (R != nullptr) x = (T)((float)x + (float)rbase[(long)row * ldr + j]);
+                        cbase[(long)row * ldc + j] = x;
+                    }
             }
         }
     }
@@ -287,10 +297,12 @@ __device__ __forceinline__ void store_wave_tile(const float4v (&acc)[TM][TN], MI
 // column blocks, at the same accumulator positions, and C has N / 2 columns.
 // R (may be null, may be C itself): a residual of C's shape added to the rounded product, `residual + proj(x)` of
 // modeling_llama.py:776,781 with the rounding of the unfused sequence (product to T, then the sum to T).
-// RAGGED: M (and N) need not be multiples of the tile. Copies of rows past the end are redirected to the last row (or, for
-// an operand whose M/N index is contiguous, to the last 8 columns: N must be a multiple of 8; M of layout TN is rounded
-// up to one, the columns in between lie in the padding of A's rows because lda is a multiple of 8), so every load stays
-// inside the matrices' rows, and the epilogue stores only what exists.
+// RAGGED: M and N need not be multiples of the tile, nor of 8. Copies of rows past the end are redirected to the last row
+// (or, for an operand whose M/N index is contiguous, to the last 8 columns of its extent rounded up to a multiple of 8: the
+// columns between the extent and that multiple lie in the padding of the operand's rows, because its leading dimension is
+// a multiple of 8, and what they hold only reaches rows / columns of the product that are never stored), so every load
+// stays inside the matrices' rows; the epilogue stores only what exists, element by element where a 16-byte piece would
+// cross the end of a row of C or where C's rows are not 16-byte aligned.
 template <typename T, bool A_KC, bool B_KC, int BM, int BN, int WM, int WN, int EPI = 0, bool RAGGED = false, int STAGES = 0, int PER_CU = 1>
 __global__ __launch_bounds__(WM * WN * 64) __attribute__((amdgpu_waves_per_eu(WM * WN / 4, PER_CU * WM * WN / 4)))
 void hgemm_main_kernel(const T* __restrict__ A, const T* __restrict__ B,
@@ -382,7 +394,7 @@ void hgemm_main_kernel(const T* __restrict__ A, const T* __restrict__ B,
                 b_voff[i] = clamped(ldb, true, BTK::kRowsPerInst, BTK::kChunksPerRow, BTK::kRowsPerPass, i, n0, N, BTK::swz(row));
             } else {
                 const int row = wave * BTN::kRowsPerInst + lane / BTN::kChunksPerRow + i * BTN::kRowsPerPass;
-                b_voff[i] = clamped(ldb, false, BTN::kRowsPerInst, BTN::kChunksPerRow, BTN::kRowsPerPass, i, n0, N, BTN::swz(row));
+                b_voff[i] = clamped(ldb, false, BTN::kRowsPerInst, BTN::kChunksPerRow, BTN::kRowsPerPass, i, n0, (N + 7) & ~7, BTN::swz(row));
             }
         }
     }
@@ -644,8 +656,10 @@ void hgemm_main_kernel(const T* __restrict__ A, const T* __restrict__ B,
     static_assert(Cfg::NWAVES * TM * 16 * TNO * 32 <= Cfg::LDS_BYTES, "epilogue staging does not fit in LDS");
     wait_vmcnt<0>();  // the last tiles' copies (on the empty buffer) have written their zeros
     __syncthreads();  // every wave has finished reading the operand stages
+    // whole 16-byte pieces of C (and of the residual) can be stored (read) where their rows are 16-byte aligned
+    const bool c_vec = !RAGGED || ((((uintptr_t)C | (uintptr_t)R) & 15) == 0 && ((ldc | ldr) & 7) == 0);
     store_wave_tile<T, TM, TN, EPI, RAGGED>(acc, smem + wave * (TM * 16 * TNO * 32), C, R, m0 + wm * TM * 16,
-                                            (EPI == 1 ? n0 / 2 : n0) + wn * TNO * 16, M, EPI == 1 ? N / 2 : N, ldc, ldr, lane);
+                                            (EPI == 1 ? n0 / 2 : n0) + wn * TNO * 16, M, EPI == 1 ? N / 2 : N, ldc, ldr, lane, c_vec);
     MI355_TL(
         wait_vmcnt<0>();   // the stores of this wave have been accepted
         tl_w[3] = timeline::wall_clock();
@@ -1281,9 +1295,13 @@ static bool few_rows_prefer_deep_ring(int M, int N, int K, bool nn, bool nt) {
 template <typename T, bool A_KC, bool B_KC>
 static hipError_t launch_layout(const T* A, const T* B, T* C, const T* R, int M, int N, int K, long lda, long ldb,
                                 long ldc, long ldr, int variant, hipStream_t stream) {
-    const bool aligned = (reinterpret_cast<uintptr_t>(A) % 16 == 0) && (reinterpret_cast<uintptr_t>(B) % 16 == 0) &&
-                         (reinterpret_cast<uintptr_t>(C) % 16 == 0) && (lda % 8 == 0) && (ldb % 8 == 0) &&
-                         (ldc % 8 == 0) && (reinterpret_cast<uintptr_t>(R) % 16 == 0) && (ldr % 8 == 0);
+    // the copies of the fast kernels move 16 bytes: the operands' rows must be 16-byte aligned. C and the residual are
+    // stored (read) in 16-byte pieces where their rows are aligned too, element by element otherwise.
+    const bool ab_aligned = (reinterpret_cast<uintptr_t>(A) % 16 == 0) && (reinterpret_cast<uintptr_t>(B) % 16 == 0) &&
+                            (lda % 8 == 0) && (ldb % 8 == 0);
+    const bool c_aligned = (reinterpret_cast<uintptr_t>(C) % 16 == 0) && (ldc % 8 == 0) &&
+                           (reinterpret_cast<uintptr_t>(R) % 16 == 0) && (ldr % 8 == 0);
+    const bool aligned = ab_aligned && c_aligned;
     // K that is not a multiple of the tiles' depth (the reference's own tiled kernels take K % 16 == 0,
     // kernels/gemm/pkg/gemm_unified/csrc/auto/gemm_7.cu:115-135): the tiled kernels take any multiple of 8, their
     // prologue handles the K % 64 columns at the end. Up to 64 rows are better served by the small-M kernels, which
@@ -1300,13 +1318,14 @@ static hipError_t launch_layout(const T* A, const T* B, T* C, const T* R, int M,
         return launch_layout<T, A_KC, B_KC>(A, B, C, C, M, N, k_main, lda, ldb, ldc, ldc, variant, stream);
     }
     // the tiled kernels address a tile with 32-bit byte offsets: up to 256 rows of lda (ldb) elements
-    const bool k_ok = aligned && K % 8 == 0 && K >= 8 && lda < (1L << 22) && ldb < (1L << 22);
-    const bool ragged_ok = k_ok && N % 8 == 0 && N >= 8;
+    // Any N: an operand stored [K,N] is copied in 16-byte chunks of its rows, and the chunk that straddles N ends in the
+    // padding a leading dimension of a multiple of 8 leaves (what it holds only reaches columns that are never stored).
+    const bool ragged_ok = ab_aligned && K % 8 == 0 && K >= 8 && lda < (1L << 22) && ldb < (1L << 22);
     const bool small_m = M <= 64 && !(ragged_ok && few_rows_prefer_tiles(M, N, K, A_KC && B_KC));
     // Up to 64 rows (generation-step projections): 64x64 tiles with an 8-deep ring stream the second operand once, on
     // N / 64 workgroups with ~50 KiB each in flight, where the split-K small-M kernels below stream it once per 16 rows.
     if (ragged_ok && M <= 64 && variant == 0 && few_rows_prefer_deep_ring(M, N, K, A_KC && !B_KC, A_KC && B_KC)) {
-        if (M == 64 && N % 64 == 0) return launch_main<T, A_KC, B_KC, 64, 64, 2, 2>(A, B, C, R, M, N, K, lda, ldb, ldc, ldr, stream);
+        if (M == 64 && N % 64 == 0 && c_aligned) return launch_main<T, A_KC, B_KC, 64, 64, 2, 2>(A, B, C, R, M, N, K, lda, ldb, ldc, ldr, stream);
         return launch_main<T, A_KC, B_KC, 64, 64, 2, 2, 0, true>(A, B, C, R, M, N, K, lda, ldb, ldc, ldr, stream);
     }
     if constexpr (!B_KC) {   // NN and TN
@@ -1314,17 +1333,17 @@ static hipError_t launch_layout(const T* A, const T* B, T* C, const T* R, int M,
             return launch_smallm_nn<T, A_KC>(A, B, C, R, M, N, K, lda, ldb, ldc, ldr, stream);
     }
     if constexpr (A_KC && B_KC) {
-        if (aligned && small_m && K % 64 == 0 && K >= 64) return launch_smallm_nt<T>(A, B, C, R, M, N, K, lda, ldb, ldc, ldr, stream);
+        // (this kernel stores element by element: C and the residual may lie anywhere)
+        if (ab_aligned && small_m && K % 64 == 0 && K >= 64) return launch_smallm_nt<T>(A, B, C, R, M, N, K, lda, ldb, ldc, ldr, stream);
     }
-    // Tiled kernels: N (and M for layout TN) a multiple of 8, so that 16-byte chunks never straddle the end; M and N need
-    // not be multiples of the tile. Shapes: 1 = 256x256 (8 waves, ring of 2), 2 = 128x128 (4 waves, ring of 3), 3 = half
+    // Tiled kernels: M and N need not be multiples of the tile, nor of 8. Shapes: 1 = 256x256 (8 waves, ring of 2), 2 = 128x128 (4 waves, ring of 3), 3 = half
     // of that (64x128, for layout NT 128x64, which keeps the 128-byte rows of both K-contiguous operands; ring of 5),
     // 4 = 64x64 with a ring of 4 (64 KiB: two workgroups fit on a CU). More than 64 rows: the shape with the least
     // estimated time. Up to 64 rows (products that few_rows_prefer_tiles sends here): half tiles for layout NT, which
     // put twice as many workgroups on the stream of the second operand, 128x128 otherwise.
     if (ragged_ok) {
         int shape = variant >= 1 && variant <= 4 ? variant : M <= 64 ? ((A_KC && B_KC) ? 3 : 2) : cheapest_tile_shape(M, N, K);
-        const auto whole = [&](int bm, int bn) { return M % bm == 0 && N % bn == 0; };
+        const auto whole = [&](int bm, int bn) { return c_aligned && M % bm == 0 && N % bn == 0; };
         switch (shape) {
             case 1:
                 if (whole(256, 256)) return launch_main<T, A_KC, B_KC, 256, 256, 2, 4>(A, B, C, R, M, N, K, lda, ldb, ldc, ldr, stream);
