@@ -665,6 +665,10 @@ KERNEL_CONFIGS = {
     # the vendor library on the same box, same operands and timing loop (torch.matmul = hipBLASLt); not this code
     "vendor_gemm_8192_nn": ("vendor_gemm", 8192, 8192, 8192, "NN"),
     "vendor_gemm_8192_nt": ("vendor_gemm", 8192, 8192, 8192, "NT"),
+    "vendor_gemm_4096_nn": ("vendor_gemm", 4096, 4096, 4096, "NN"),
+    "vendor_gemm_2048x2048x4096_nn": ("vendor_gemm", 2048, 2048, 4096, "NN"),
+    "vendor_gemm_1024x4096x4096_nt": ("vendor_gemm", 1024, 4096, 4096, "NT"),
+    "vendor_gemm_1024_nn": ("vendor_gemm", 1024, 1024, 1024, "NN"),
 }
 
 
@@ -802,7 +806,7 @@ def run_kernel_config(args, torch, lib, so, dev):
         flops = 2.0 * M * N * K
         print(json.dumps(dict(t, kernel_config=args.kernel_config, zero_inputs=bool(args.zero_inputs), tflops=flops / t["ms"] / 1e9,
                               pct_of_fp16_mfma_peak=100 * flops / t["ms"] / 1e9 / PEAK_FP16_TFLOPS,
-                              note="torch.matmul (hipBLASLt) on the operands of the g2b configuration; the vendor library, not this code")))
+                              note="torch.matmul (hipBLASLt) on the operands of the configuration of that shape; the vendor library, not this code")))
         return
     if cfg[0] == "gemm":
         _, M, N, K, lay = cfg
