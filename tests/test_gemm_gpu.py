@@ -125,6 +125,10 @@ def test_k_tail_on_every_tile_shape(lib, gpu, variant, layout, M, N, K):
     # every tiled kernel takes its K % 64 columns in its prologue (out-of-range copies write zeros); K below one tile's
     # depth is all tail
     a, b = operands(M, N, K, layout, seed=M + K + variant, b_std=0.05)
+    # LDS keeps what the last kernel left there: a product of NaNs on the same tile shape first, over enough tiles to
+    # reach every CU, so that a tail lane whose copy wrote nothing would leave a NaN in the tile
+    nan_a = torch.full((4096, 128), float("nan"), dtype=torch.float16, device=gpu)
+    lib.hgemm(nan_a, nan_a.t().contiguous() if layout == "NN" else nan_a, "NN" if layout == "NN" else "NT", variant=variant)
     check(lib, gpu, a, b, layout, K, variant=variant)
 
 
