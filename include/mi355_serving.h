@@ -67,8 +67,8 @@ extern "C" {
  * K % 8 == 0 (K % 64 != 0 with M <= 64 and no residual: one more launch for the last K % 64 columns); M and N are free
  * (ragged tile edges are handled inside the kernels; an operand whose M or N index is contiguous is read in 16-byte
  * chunks, up to 7 elements into the padding that its leading dimension, a multiple of 8, leaves behind M or N). C (and
- * a residual) may have any row stride and alignment: rows that are not 16-byte aligned, or whose width is not a multiple
- * of 8, are stored element by element.
+ * a residual) may have any row stride and alignment (global memory takes 16-byte accesses at any element; only the
+ * last N % 8 columns of a row are stored element by element).
  */
 int mi355_hgemm(const void* A, const void* B, void* C, int M, int N, int K, int64_t lda, int64_t ldb,
                 int64_t ldc, int layout, void* stream);

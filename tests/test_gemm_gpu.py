@@ -155,7 +155,8 @@ def test_k_tail_with_a_residual(lib, gpu, layout, M, N, K):
                                            (16, 1001, 1024, 0), (48, 2049, 256, 1), (256, 256, 128, 1)])
 def test_widths_that_are_no_multiple_of_8_and_unaligned_rows_of_c(lib, gpu, variant, layout, M, N, K, ldc_pad):
     # N need not be a multiple of 8 and C's rows need not be 16-byte aligned (a vocabulary of 50257 or 32001 entries): the
-    # tiled kernels (layout NT also the small-M kernel) store such a C element by element. An operand stored [K,N] is
+    # tiled kernels store such a C in 16-byte pieces of no stated alignment and the last N % 8 columns element by element
+    # (the small-M kernel of layout NT element by element). An operand stored [K,N] is
     # still copied in 16-byte chunks, so its rows must be aligned: ldb is N rounded up to 8, the padding holds NaNs and
     # must stay out of the product. The residual has C's row stride. Nothing outside C[:M, :N] may change.
     a, b = operands(M, N, K, layout, seed=M + N + K, b_std=0.05)

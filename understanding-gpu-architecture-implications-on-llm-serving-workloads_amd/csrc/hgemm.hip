@@ -222,7 +222,7 @@ __device__ __forceinline__ void tile_of_block(int bid, int tiles_m, int tiles_n,
 // 4 (jo / 2) + jo % 2 and its up from two blocks further.
 template <typename T, int TM, int TN, int EPI, bool RAGGED>
 __device__ __forceinline__ void store_wave_tile(const float4v (&acc)[TM][TN], MI355_LDS char* cst, T* C, const T* R, long row0,
-                                                long col0, int M, int NC, long ldc, long ldr, int lane, bool c_vec = true) {
+                                                long col0, int M, int NC, long ldc, long ldr, int lane) {
     using V8 = typename Elem<T>::v8;
     using V4 = typename Elem<T>::v4;
     static_assert(EPI == 0 || TN % 4 == 0, "the gate/up epilogue pairs column blocks 32 columns apart");
@@ -269,16 +269,25 @@ __device__ __forceinline__ void store_wave_tile(const float4v (&acc)[TM][TN], MI
         for (int it = 0; it < TM * 16 / kRowsPerStore; ++it) {
             const int row = it * kRowsPerStore + rr;
             V8 v = *(MI355_LDS const V8*)(cst + row * kRowBytesC + ((cc ^ (row & kSwzC)) << 4));
-            if (!RAGGED || (row < rows_left && cols_left >= 8 && c_vec)) {
+            if constexpr (!RAGGED) {
                 if (R != nullptr) {
                     const V8 r = *(const V8*)(rbase + (long)row * ldr);
 #pragma unroll
                     for (int j = 0; j < 8; ++j) v[j] = (T)((float)v[j] + (float)r[j]);
                 }
                 *(V8*)(cbase + (long)row * ldc) = v;
+            } else if (row < rows_left && cols_left >= 8) {
+                // C's rows (and the residual's) may start at any element: the 16 bytes move as a copy of no stated
+                // alignment, for which the compiler still issues one 16-byte access (global memory takes unaligned ones)
+                if (R != nullptr) {
+                    V8 r;
+                    __builtin_memcpy(&r, rbase + (long)row * ldr, 16);
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) v[j] = (T)((float)v[j] + (float)r[j]);
+                }
+                __builtin_memcpy(cbase + (long)row * ldc, &v, 16);
             } else if (row < rows_left) {
-                // the last columns of a C whose width is not a multiple of 8, or a C (or residual) whose rows are not
-                // 16-byte aligned: element by element
+                // the last columns of a C whose width is not a multiple of 8: element by element
 #pragma unroll
                 for (int j = 0; j < 8; ++j)
                     if (j < cols_left) {
@@ -301,8 +310,8 @@ __device__ __forceinline__ void store_wave_tile(const float4v (&acc)[TM][TN], MI
 // (or, for an operand whose M/N index is contiguous, to the last 8 columns of its extent rounded up to a multiple of 8: the
 // columns between the extent and that multiple lie in the padding of the operand's rows, because its leading dimension is
 // a multiple of 8, and what they hold only reaches rows / columns of the product that are never stored), so every load
-// stays inside the matrices' rows; the epilogue stores only what exists, element by element where a 16-byte piece would
-// cross the end of a row of C or where C's rows are not 16-byte aligned.
+// stays inside the matrices' rows; the epilogue stores only what exists: whole 16-byte pieces wherever a row of C starts
+// (global memory takes such an access at any element), the last N % 8 columns of a row element by element.
 template <typename T, bool A_KC, bool B_KC, int BM, int BN, int WM, int WN, int EPI = 0, bool RAGGED = false, int STAGES = 0, int PER_CU = 1>
 __global__ __launch_bounds__(WM * WN * 64) __attribute__((amdgpu_waves_per_eu(WM * WN / 4, PER_CU * WM * WN / 4)))
 void hgemm_main_kernel(const T* __restrict__ A, const T* __restrict__ B,
@@ -656,10 +665,8 @@ void hgemm_main_kernel(const T* __restrict__ A, const T* __restrict__ B,
     static_assert(Cfg::NWAVES * TM * 16 * TNO * 32 <= Cfg::LDS_BYTES, "epilogue staging does not fit in LDS");
     wait_vmcnt<0>();  // the last tiles' copies (on the empty buffer) have written their zeros
     __syncthreads();  // every wave has finished reading the operand stages
-    // whole 16-byte pieces of C (and of the residual) can be stored (read) where their rows are 16-byte aligned
-    const bool c_vec = !RAGGED || ((((uintptr_t)C | (uintptr_t)R) & 15) == 0 && ((ldc | ldr) & 7) == 0);
     store_wave_tile<T, TM, TN, EPI, RAGGED>(acc, smem + wave * (TM * 16 * TNO * 32), C, R, m0 + wm * TM * 16,
-                                            (EPI == 1 ? n0 / 2 : n0) + wn * TNO * 16, M, EPI == 1 ? N / 2 : N, ldc, ldr, lane, c_vec);
+                                            (EPI == 1 ? n0 / 2 : n0) + wn * TNO * 16, M, EPI == 1 ? N / 2 : N, ldc, ldr, lane);
     MI355_TL(
         wait_vmcnt<0>();   // the stores of this wave have been accepted
         tl_w[3] = timeline::wall_clock();
@@ -1295,8 +1302,8 @@ static bool few_rows_prefer_deep_ring(int M, int N, int K, bool nn, bool nt) {
 template <typename T, bool A_KC, bool B_KC>
 static hipError_t launch_layout(const T* A, const T* B, T* C, const T* R, int M, int N, int K, long lda, long ldb,
                                 long ldc, long ldr, int variant, hipStream_t stream) {
-    // the copies of the fast kernels move 16 bytes: the operands' rows must be 16-byte aligned. C and the residual are
-    // stored (read) in 16-byte pieces where their rows are aligned too, element by element otherwise.
+    // the copies of the fast kernels move 16 bytes into LDS: the operands' rows must be 16-byte aligned. C and the residual
+    // may lie anywhere; the kernels that assume whole tiles also assume aligned rows of C (c_aligned).
     const bool ab_aligned = (reinterpret_cast<uintptr_t>(A) % 16 == 0) && (reinterpret_cast<uintptr_t>(B) % 16 == 0) &&
                             (lda % 8 == 0) && (ldb % 8 == 0);
     const bool c_aligned = (reinterpret_cast<uintptr_t>(C) % 16 == 0) && (ldc % 8 == 0) &&
