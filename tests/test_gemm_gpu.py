@@ -454,7 +454,8 @@ def bf16_close(c, ref, K):
 
 @pytest.mark.parametrize("layout", ["NN", "NT", "TN"])
 @pytest.mark.parametrize("M,N,K", [(1024, 1024, 1024), (512, 768, 320), (1000, 264, 128), (16, 4096, 1024), (7, 72, 96),
-                                   (100, 70, 50)])
+                                   (100, 70, 50),
+                                   (1000, 520, 4144), (2048, 2048, 72), (300, 1001, 264), (16, 515, 1096)])   # K tails, odd widths
 def test_bfloat16_gemm(lib, gpu, layout, M, N, K):
     a, b = operands(M, N, K, layout, seed=K, b_std=0.05)
     a, b = a.float().bfloat16(), b.float().bfloat16()
