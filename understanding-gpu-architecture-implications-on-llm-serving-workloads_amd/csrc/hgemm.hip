@@ -146,8 +146,8 @@ struct MainCfg {
     static constexpr int A_BYTES = BM * BK * 2;
     static constexpr int B_BYTES = BN * BK * 2;
     static constexpr int STAGE_BYTES = A_BYTES + B_BYTES;
-    // 64 KiB stages: two of them fit; the 32 KiB stages of the 128x128 tile get a third, which gives every copy one more
-    // K tile of time to land (small problems run few tiles per workgroup and are bound by that latency). The narrow tiles
+    // 64 KiB stages: two of them fit; the 48 KiB stages of the 128x256 tiles and the 32 KiB stages of the 128x128 tile
+    // get a third, which gives every copy one more K tile of time to land (small problems run few tiles per workgroup and are bound by that latency). The narrow tiles
     // serve products with few rows, which are bound by the stream of the weight matrix from HBM: their ring is as deep
     // as 128 KiB of LDS allow (5 stages of 24 KiB, 8 of 16 KiB), so that a CU keeps ~50 KiB of that stream in flight.
     // STAGES > 0 sets the depth (the 64x64 tiles of small products run with four stages, two workgroups to a CU).
@@ -1255,19 +1255,23 @@ static bool few_rows_prefer_tiles(int M, int N, int K, bool nt) {
     return few_row_tiles_us(M, N, K, nt) < small_m_us(M, N, K, false) - 4.0;
 }
 // Which tile shape is expected to finish a product of more than 64 rows first (1 = 256x256, 2 = 128x128, 3 = 64x128 or
-// 128x64, 4 = 64x64 two to a CU). A CU takes in 64 bytes per cycle from the memory system, so the time of a K tile is
-// set by the tile's bytes as much as by its matrix instructions (the operands of a 128x128 tile need the same 512 cycles
-// to arrive that its matrix instructions take): measured cycles per K tile of 64 of one workgroup alone on its CU are
-// 2470 (256x256; matrix pipes 2048), 770 (128x128; pipes 512), 576 (half tile) and 384 (64x64). A workgroup spends
-// another 5000-12000 cycles outside its K loop (first tiles in flight, epilogue). The workgroups run in rounds of one
-// per CU (two for the 64x64 tiles); the last round may be a partial one. The model reproduces the measured times of
-// 1024^3 .. 8192^3, 2048 x 4096 x 4096 and 1536 x 1536 x 8192 within ~10 %. The 128x128 figure used below is 840: on
-// N(0,1) operands, under the board's power limit, the 256x256 tiles do better against the smaller ones than on zeros
-// (3072 x 3072 x 4096: 75 us against 87 where zeros give 70 against 71).
+// 128x64, 4 = 64x64 two to a CU, 5 = 128x256, 6 = 256x128). A CU takes in 64 bytes per cycle from the memory system, so
+// the time of a K tile is set by the tile's bytes as much as by its matrix instructions (the operands of a 128x128 tile
+// need the same 512 cycles to arrive that its matrix instructions take): measured cycles per K tile of 64 of one
+// workgroup alone on its CU are 2470 (256x256; matrix pipes 2048), 1340 (128x256 and 256x128 on a ring of three stages;
+// pipes 1024), 770 (128x128; pipes 512), 576 (half tile) and 384 (64x64). A workgroup spends another 5000-12000 cycles
+// outside its K loop (first tiles in flight, epilogue). The workgroups run in rounds of one per CU (two for the 64x64
+// tiles); the last round may be a partial one. The model reproduces the measured times of 1024^3 .. 8192^3,
+// 2048 x 4096 x 4096 and 1536 x 1536 x 8192 within ~10 %. The 128x128 figure used below is 840, that of the 128x256
+// tiles 1400: on N(0,1) operands, under the board's power limit, the larger tiles do better against the smaller ones
+// than on zeros (3072 x 3072 x 4096: 75 us against 87 where zeros give 70 against 71). The 128x256 tiles are for the
+// products that fill the chip once with them, where 256x256 tiles leave CUs idle and 128x128 tiles need two rounds
+// (2048 x 4096 x 4096: 59 us against 66 on 128x128 tiles and 89 on 256x256; 2048 x 4096 x 14336: 186 against 216); of
+// the two orientations the one with fewer rounds, the long side along the longer dimension of C if they tie.
 static int cheapest_tile_shape(int M, int N, int K) {
     struct Cand { int shape, bm, bn, per_cu; double step, fixed; };
     static const Cand cands[] = {{1, 256, 256, 1, 2470., 12000.}, {2, 128, 128, 1, 840., 7000.}, {3, 64, 128, 1, 576., 6000.},
-                                 {4, 64, 64, 2, 384., 5000.}};
+                                 {4, 64, 64, 2, 384., 5000.}, {5, 128, 256, 1, 1400., 9000.}, {6, 256, 128, 1, 1400., 9000.}};
     const double ktiles = (double)((K + 63) / 64);
     int best = 2;
     double best_t = 0.;
@@ -1276,6 +1280,7 @@ static int cheapest_tile_shape(int M, int N, int K) {
         const long cap = 256L * c.per_cu, full = tiles / cap, rem = tiles % cap;
         double t = (double)full * (c.per_cu * ktiles * c.step + c.fixed);
         if (rem) t += (double)((rem + 255) / 256) * ktiles * c.step + c.fixed;
+        if (c.shape == 6 && M > N) t -= 1.;   // a tie between the two orientations
         if (best_t == 0. || t < best_t) { best_t = t; best = c.shape; }
     }
     return best;
@@ -1343,13 +1348,14 @@ static hipError_t launch_layout(const T* A, const T* B, T* C, const T* R, int M,
         // (this kernel stores element by element: C and the residual may lie anywhere)
         if (ab_aligned && small_m && K % 64 == 0 && K >= 64) return launch_smallm_nt<T>(A, B, C, R, M, N, K, lda, ldb, ldc, ldr, stream);
     }
-    // Tiled kernels: M and N need not be multiples of the tile, nor of 8. Shapes: 1 = 256x256 (8 waves, ring of 2), 2 = 128x128 (4 waves, ring of 3), 3 = half
-    // of that (64x128, for layout NT 128x64, which keeps the 128-byte rows of both K-contiguous operands; ring of 5),
-    // 4 = 64x64 with a ring of 4 (64 KiB: two workgroups fit on a CU). More than 64 rows: the shape with the least
+    // Tiled kernels: M and N need not be multiples of the tile, nor of 8. Shapes: 1 = 256x256 (8 waves, ring of 2),
+    // 2 = 128x128 (4 waves, ring of 3), 3 = half of that (64x128, for layout NT 128x64, which keeps the 128-byte rows of
+    // both K-contiguous operands; ring of 5), 4 = 64x64 with a ring of 4 (64 KiB: two workgroups fit on a CU), 5 = 128x256
+    // and 6 = 256x128 (8 waves of 64x64, ring of 3). More than 64 rows: the shape with the least
     // estimated time. Up to 64 rows (products that few_rows_prefer_tiles sends here): half tiles for layout NT, which
     // put twice as many workgroups on the stream of the second operand, 128x128 otherwise.
     if (ragged_ok) {
-        int shape = variant >= 1 && variant <= 4 ? variant : M <= 64 ? ((A_KC && B_KC) ? 3 : 2) : cheapest_tile_shape(M, N, K);
+        int shape = variant >= 1 && variant <= 6 ? variant : M <= 64 ? ((A_KC && B_KC) ? 3 : 2) : cheapest_tile_shape(M, N, K);
         const auto whole = [&](int bm, int bn) { return c_aligned && M % bm == 0 && N % bn == 0; };
         switch (shape) {
             case 1:
@@ -1363,6 +1369,12 @@ static hipError_t launch_layout(const T* A, const T* B, T* C, const T* R, int M,
                     if (whole(64, 128)) return launch_main<T, A_KC, B_KC, 64, 128, 1, 4>(A, B, C, R, M, N, K, lda, ldb, ldc, ldr, stream);
                     return launch_main<T, A_KC, B_KC, 64, 128, 1, 4, 0, true>(A, B, C, R, M, N, K, lda, ldb, ldc, ldr, stream);
                 }
+            case 5:
+                if (whole(128, 256)) return launch_main<T, A_KC, B_KC, 128, 256, 2, 4>(A, B, C, R, M, N, K, lda, ldb, ldc, ldr, stream);
+                return launch_main<T, A_KC, B_KC, 128, 256, 2, 4, 0, true>(A, B, C, R, M, N, K, lda, ldb, ldc, ldr, stream);
+            case 6:
+                if (whole(256, 128)) return launch_main<T, A_KC, B_KC, 256, 128, 4, 2>(A, B, C, R, M, N, K, lda, ldb, ldc, ldr, stream);
+                return launch_main<T, A_KC, B_KC, 256, 128, 4, 2, 0, true>(A, B, C, R, M, N, K, lda, ldb, ldc, ldr, stream);
             case 4:
                 if (whole(64, 64)) return launch_main<T, A_KC, B_KC, 64, 64, 2, 2, 0, false, 4, 2>(A, B, C, R, M, N, K, lda, ldb, ldc, ldr, stream);
                 return launch_main<T, A_KC, B_KC, 64, 64, 2, 2, 0, true, 4, 2>(A, B, C, R, M, N, K, lda, ldb, ldc, ldr, stream);
