@@ -634,6 +634,7 @@ KERNEL_CONFIGS = {
     "g2b_gemm_8192_nn": ("gemm", 8192, 8192, 8192, "NN"),                   # 256x256 tiles
     "g2b_gemm_8192_nt": ("gemm", 8192, 8192, 8192, "NT"),
     "gemm_2048x2048x4096_nn": ("gemm", 2048, 2048, 4096, "NN"),             # 128x128 tiles
+    "gemm_2048x4096x4096_nn": ("gemm", 2048, 4096, 4096, "NN"),             # 128x256 tiles, one per CU
     "g2c_gemm_16x14336x4096_nn": ("gemm", 16, 14336, 4096, "NN"),           # split-K small-M kernel
     "gemm_16x14336x4096_nt": ("gemm", 16, 14336, 4096, "NT"),               # split-K small-M kernel (NT)
     "gemm_8x28672x4096_nt": ("gemm", 8, 28672, 4096, "NT"),                 # split-K small-M kernel (NT), A rows 0..7 only
@@ -667,6 +668,7 @@ KERNEL_CONFIGS = {
     "vendor_gemm_8192_nt": ("vendor_gemm", 8192, 8192, 8192, "NT"),
     "vendor_gemm_4096_nn": ("vendor_gemm", 4096, 4096, 4096, "NN"),
     "vendor_gemm_2048x2048x4096_nn": ("vendor_gemm", 2048, 2048, 4096, "NN"),
+    "vendor_gemm_2048x4096x4096_nn": ("vendor_gemm", 2048, 4096, 4096, "NN"),
     "vendor_gemm_1024x4096x4096_nt": ("vendor_gemm", 1024, 4096, 4096, "NT"),
     "vendor_gemm_1024_nn": ("vendor_gemm", 1024, 1024, 1024, "NN"),
 }
