@@ -671,9 +671,13 @@ static hipError_t fmha_fwd_dispatch_t(const void* Q, const void* K, const void* 
         // 1 x 8/8 x 8192 139 / 163, 2 x 8/2 x 4096 76 / 88, but 32 x 32/8 x 256 68 / 64, 8 x 32/8 x 512 42 / 39,
         // 1 x 32/8 x 3000 92 / 78, 2 x 32/8 x 1536 56 / 50, 4 x 32/8 x 1024 57 / 50, 1 x 32/8 x 4096 149 / 126,
         // 16 x 32/8 x 768 148 / 128, 4 x 32/8 x 2048 170 / 147; not causal 2 x 32/8 x 1024 42 / 36, 1 x 32/8 x 2048 73 / 62,
-        // 4 x 32/32 x 1024 89 / 71.
+        // 4 x 32/32 x 1024 89 / 71. A problem that is not causal and has a few more 256-query items than CUs runs as long
+        // as two of them, on a quarter of the machine at the end; twice as many 128-query items are three to a CU then,
+        // each a little more than half as long (1 x H/1 x 2048 with H = 33 .. 44, i.e. 264 .. 352 items: 94.5 - 97.6 us
+        // against 99.9; 368 items 99.6 / 100.0; 384 items 102.6 / 100.1).
         const long wg256 = (long)((Sq + 255) / 256) * Hq * B;
         variant = (Sq >= 256 && wg256 >= (causal ? 320 : 256)) ? 2 : 1;
+        if (!causal && wg256 > 256 && wg256 <= 352) variant = 1;
     }
     if (variant == 2) return launch_fmha_pingpong<T, 2>(q, k, v, o, LSE, B, Hq, Hkv, Sq, Sk, scale, causal, kv_valid_len, sd, stream);
     return launch_fmha_pingpong<T, 1>(q, k, v, o, LSE, B, Hq, Hkv, Sq, Sk, scale, causal, kv_valid_len, sd, stream);
