@@ -1267,7 +1267,8 @@ static bool few_rows_prefer_tiles(int M, int N, int K, bool nt) {
 // than on zeros (3072 x 3072 x 4096: 75 us against 87 where zeros give 70 against 71). The 128x256 tiles are for the
 // products that fill the chip once with them, where 256x256 tiles leave CUs idle and 128x128 tiles need two rounds
 // (2048 x 4096 x 4096: 59 us against 66 on 128x128 tiles and 89 on 256x256; 2048 x 4096 x 14336: 186 against 216); of
-// the two orientations the one with fewer rounds, the long side along the longer dimension of C if they tie.
+// the two orientations the one with fewer rounds, 256x128 if they tie (768 x 28672 x 4096: 163 us against 168,
+// 1536 x 4096 x 14336: 157 against 161, 768 x 6144 x 4096: 40.7 against 42.1; 2048 x 4096 x 4096 the same either way).
 static int cheapest_tile_shape(int M, int N, int K) {
     struct Cand { int shape, bm, bn, per_cu; double step, fixed; };
     static const Cand cands[] = {{1, 256, 256, 1, 2470., 12000.}, {2, 128, 128, 1, 840., 7000.}, {3, 64, 128, 1, 576., 6000.},
@@ -1280,7 +1281,7 @@ static int cheapest_tile_shape(int M, int N, int K) {
         const long cap = 256L * c.per_cu, full = tiles / cap, rem = tiles % cap;
         double t = (double)full * (c.per_cu * ktiles * c.step + c.fixed);
         if (rem) t += (double)((rem + 255) / 256) * ktiles * c.step + c.fixed;
-        if (c.shape == 6 && M > N) t -= 1.;   // a tie between the two orientations
+        if (c.shape == 6) t -= 1.;   // a tie between the two orientations
         if (best_t == 0. || t < best_t) { best_t = t; best = c.shape; }
     }
     return best;
