@@ -88,7 +88,7 @@ def test_layouts_and_shapes(lib, gpu, layout, M, N, K):
     assert c.shape == (M, N)
 
 
-@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4, 5, 6])
+@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4, 5, 6, 7])
 @pytest.mark.parametrize("layout", ["NN", "TN", "NT"])
 @pytest.mark.parametrize("M,N,K", [(1000, 1000, 1024), (300, 4096, 512), (2056, 1032, 128), (130, 8, 64), (4104, 4096, 256),
                                    (257, 264, 64)])
@@ -117,7 +117,7 @@ def test_k_that_is_a_multiple_of_16_but_not_of_the_tile_depth(lib, gpu, layout, 
     check(lib, gpu, a, b, layout, K)
 
 
-@pytest.mark.parametrize("variant", [1, 2, 3, 4, 5, 6])
+@pytest.mark.parametrize("variant", [1, 2, 3, 4, 5, 6, 7])
 @pytest.mark.parametrize("layout", ["NN", "TN", "NT"])
 @pytest.mark.parametrize("M,N,K", [(512, 512, 72), (300, 520, 200), (256, 256, 40), (1000, 264, 1048), (64, 128, 8),
                                    (257, 72, 136)])
@@ -149,7 +149,7 @@ def test_k_tail_with_a_residual(lib, gpu, layout, M, N, K):
     assert bool((err <= bound).all()), (float(err.max()), int((err > bound).sum()))
 
 
-@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4, 5, 6])
+@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4, 5, 6, 7])
 @pytest.mark.parametrize("layout", ["NN", "TN", "NT"])
 @pytest.mark.parametrize("M,N,K,ldc_pad", [(300, 1001, 256, 0), (512, 515, 136, 5), (1000, 77, 64, 3), (130, 3, 512, 0),
                                            (16, 1001, 1024, 0), (48, 2049, 256, 1), (256, 256, 128, 1)])
@@ -189,7 +189,7 @@ def test_widths_that_are_no_multiple_of_8_and_unaligned_rows_of_c(lib, gpu, vari
         assert bool((c[M:] == 3.0).all()) and bool((c[:, N:] == 3.0).all())
 
 
-@pytest.mark.parametrize("variant,tile_m,tile_n", [(1, 256, 256), (2, 128, 128), (3, 64, 128), (4, 64, 64), (5, 128, 256), (6, 256, 128)])
+@pytest.mark.parametrize("variant,tile_m,tile_n", [(1, 256, 256), (2, 128, 128), (3, 64, 128), (4, 64, 64), (5, 128, 256), (6, 256, 128), (7, 32, 64)])
 @pytest.mark.parametrize("layout", ["NN", "NT"])
 @pytest.mark.parametrize("tiles_m,tiles_n,ragged", [(16, 32, 0), (32, 24, 0), (32, 16, 8), (48, 16, 0)])
 def test_grids_walked_in_super_blocks(lib, gpu, variant, tile_m, tile_n, layout, tiles_m, tiles_n, ragged):
@@ -289,7 +289,7 @@ def test_seeded_random_products_in_padded_allocations(lib, gpu, layout, M, N, K,
     assert bool((c[M:] == 3.0).all()) and bool((c[:, N:] == 3.0).all())
 
 
-@pytest.mark.parametrize("variant", [1, 2, 3, 4, 5, 6])
+@pytest.mark.parametrize("variant", [1, 2, 3, 4, 5, 6, 7])
 @pytest.mark.parametrize("layout", ["NN", "TN", "NT"])
 def test_every_tile_variant(lib, gpu, variant, layout):
     a, b = operands(512, 768, 448, layout, seed=variant)

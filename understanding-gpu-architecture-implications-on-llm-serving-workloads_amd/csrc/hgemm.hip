@@ -139,10 +139,11 @@ struct MainCfg {
     static constexpr int WM = WM_, WN = WN_, NWAVES = WM_ * WN_, NTHREADS = NWAVES * 64;
     static constexpr int TM = BM / WM / 16;  // MFMA 16x16 blocks along M per wave
     static constexpr int TN = BN / WN / 16;  // along N
-    using ATileK = KContigTile<BM, BK, NWAVES>;
-    using ATileM = MNContigTile<BM, BK, NWAVES>;
-    using BTileK = KContigTile<BN, BK, NWAVES>;
-    using BTileN = MNContigTile<BN, BK, NWAVES>;
+    // (the description of the layout an operand does not have is never used: it is formed with an extent that exists)
+    using ATileK = KContigTile<A_KC ? BM : 256, BK, NWAVES>;
+    using ATileM = MNContigTile<A_KC ? 64 : BM, BK, NWAVES>;
+    using BTileK = KContigTile<B_KC ? BN : 256, BK, NWAVES>;
+    using BTileN = MNContigTile<B_KC ? 64 : BN, BK, NWAVES>;
     static constexpr int A_BYTES = BM * BK * 2;
     static constexpr int B_BYTES = BN * BK * 2;
     static constexpr int STAGE_BYTES = A_BYTES + B_BYTES;
@@ -1255,7 +1256,7 @@ static bool few_rows_prefer_tiles(int M, int N, int K, bool nt) {
     return few_row_tiles_us(M, N, K, nt) < small_m_us(M, N, K, false) - 4.0;
 }
 // Which tile shape is expected to finish a product of more than 64 rows first (1 = 256x256, 2 = 128x128, 3 = 64x128 or
-// 128x64, 4 = 64x64 two to a CU, 5 = 128x256, 6 = 256x128). A CU takes in 64 bytes per cycle from the memory system, so
+// 128x64, 4 = 64x64 two to a CU, 5 = 128x256, 6 = 256x128, 7 = 32x64). A CU takes in 64 bytes per cycle from the memory system, so
 // the time of a K tile is set by the tile's bytes as much as by its matrix instructions (the operands of a 128x128 tile
 // need the same 512 cycles to arrive that its matrix instructions take): measured cycles per K tile of 64 of one
 // workgroup alone on its CU are 2470 (256x256; matrix pipes 2048), 1340 (128x256 and 256x128 on a ring of three stages;
@@ -1269,14 +1270,20 @@ static bool few_rows_prefer_tiles(int M, int N, int K, bool nt) {
 // (2048 x 4096 x 4096: 59 us against 66 on 128x128 tiles and 89 on 256x256; 2048 x 4096 x 14336: 186 against 216); of
 // the two orientations the one with fewer rounds, 256x128 if they tie (768 x 28672 x 4096: 163 us against 168,
 // 1536 x 4096 x 14336: 157 against 161, 768 x 6144 x 4096: 40.7 against 42.1; 2048 x 4096 x 4096 the same either way).
-static int cheapest_tile_shape(int M, int N, int K) {
+// The 32x64 tiles (ring of 8 stages of 12 KiB, 335 cycles per K tile) are for 65 .. 128 rows against a narrow second
+// operand (generation steps of that many sequences through the O and down projections), where 64x64 tiles are only
+// half as many as CUs: 128 x 4096 x 14336 NT 41 -> 33 us, 128 x 4096 x 4096 13.2 -> 11.2, 96 x 4096 x 14336 40 -> 32
+// (with 256 rows, or 6144 columns, they would need two rounds and lose: 63 us against 45, 20 against 14).
+static int cheapest_tile_shape(int M, int N, int K, bool a_k_contiguous) {
     struct Cand { int shape, bm, bn, per_cu; double step, fixed; };
     static const Cand cands[] = {{1, 256, 256, 1, 2470., 12000.}, {2, 128, 128, 1, 840., 7000.}, {3, 64, 128, 1, 576., 6000.},
-                                 {4, 64, 64, 2, 384., 5000.}, {5, 128, 256, 1, 1400., 9000.}, {6, 256, 128, 1, 1400., 9000.}};
+                                 {4, 64, 64, 2, 384., 5000.}, {5, 128, 256, 1, 1400., 9000.}, {6, 256, 128, 1, 1400., 9000.},
+                                 {7, 32, 64, 1, 335., 5000.}};
     const double ktiles = (double)((K + 63) / 64);
     int best = 2;
     double best_t = 0.;
     for (const Cand& c : cands) {
+        if (c.shape == 7 && !a_k_contiguous) continue;   // 32-row tiles exist for a K-contiguous A only
         const long tiles = (long)((M + c.bm - 1) / c.bm) * ((N + c.bn - 1) / c.bn);
         const long cap = 256L * c.per_cu, full = tiles / cap, rem = tiles % cap;
         double t = (double)full * (c.per_cu * ktiles * c.step + c.fixed);
@@ -1352,11 +1359,12 @@ static hipError_t launch_layout(const T* A, const T* B, T* C, const T* R, int M,
     // Tiled kernels: M and N need not be multiples of the tile, nor of 8. Shapes: 1 = 256x256 (8 waves, ring of 2),
     // 2 = 128x128 (4 waves, ring of 3), 3 = half of that (64x128, for layout NT 128x64, which keeps the 128-byte rows of
     // both K-contiguous operands; ring of 5), 4 = 64x64 with a ring of 4 (64 KiB: two workgroups fit on a CU), 5 = 128x256
-    // and 6 = 256x128 (8 waves of 64x64, ring of 3). More than 64 rows: the shape with the least
+    // and 6 = 256x128 (8 waves of 64x64, ring of 3), 7 = 32x64 (4 waves of 16x32, ring of 8; layouts with a K-contiguous
+    // A). More than 64 rows: the shape with the least
     // estimated time. Up to 64 rows (products that few_rows_prefer_tiles sends here): half tiles for layout NT, which
     // put twice as many workgroups on the stream of the second operand, 128x128 otherwise.
     if (ragged_ok) {
-        int shape = variant >= 1 && variant <= 6 ? variant : M <= 64 ? ((A_KC && B_KC) ? 3 : 2) : cheapest_tile_shape(M, N, K);
+        int shape = variant >= 1 && variant <= (A_KC ? 7 : 6) ? variant : M <= 64 ? ((A_KC && B_KC) ? 3 : 2) : cheapest_tile_shape(M, N, K, A_KC);
         const auto whole = [&](int bm, int bn) { return c_aligned && M % bm == 0 && N % bn == 0; };
         switch (shape) {
             case 1:
@@ -1376,6 +1384,9 @@ static hipError_t launch_layout(const T* A, const T* B, T* C, const T* R, int M,
             case 6:
                 if (whole(256, 128)) return launch_main<T, A_KC, B_KC, 256, 128, 4, 2>(A, B, C, R, M, N, K, lda, ldb, ldc, ldr, stream);
                 return launch_main<T, A_KC, B_KC, 256, 128, 4, 2, 0, true>(A, B, C, R, M, N, K, lda, ldb, ldc, ldr, stream);
+            case 7:
+                if constexpr (A_KC) return launch_main<T, A_KC, B_KC, 32, 64, 2, 2, 0, true, 8>(A, B, C, R, M, N, K, lda, ldb, ldc, ldr, stream);
+                [[fallthrough]];
             case 4:
                 if (whole(64, 64)) return launch_main<T, A_KC, B_KC, 64, 64, 2, 2, 0, false, 4, 2>(A, B, C, R, M, N, K, lda, ldb, ldc, ldr, stream);
                 return launch_main<T, A_KC, B_KC, 64, 64, 2, 2, 0, true, 4, 2>(A, B, C, R, M, N, K, lda, ldb, ldc, ldr, stream);

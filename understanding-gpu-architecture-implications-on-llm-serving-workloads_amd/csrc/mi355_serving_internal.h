@@ -82,7 +82,7 @@ hipError_t silu_mul_dispatch(const void* in, void* out, long rows, int inter, in
 // Test and tuning hooks: exported from the shared library but not part of its public header. They take the kernel
 // variant as an argument (no process-wide state): variants that do not fit the shape fall back to the choice by shape.
 //   gemm: 0 = by shape; 1 = 256x256 tiles, 2 = 128x128, 3 = 64x128 (layout NT: 128x64), 4 = 64x64 with a ring of four
-//         stages, 5 = 128x256, 6 = 256x128: the tiled kernel of that shape for any product the tiled kernels take (M and N need not be multiples
+//         stages, 5 = 128x256, 6 = 256x128, 7 = 32x64 (layouts NN and NT): the tiled kernel of that shape for any product the tiled kernels take (M and N need not be multiples
 //         of the tile); products of up to 64 rows that the small-M kernels take stay on those
 //   fmha: 0 = by shape, 1 = 128-query workgroups, 2 = 256-query workgroups (1 and 2 also keep generation-step shapes off
 //         the split-KV path)

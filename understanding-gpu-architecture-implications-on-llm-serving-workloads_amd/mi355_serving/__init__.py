@@ -120,7 +120,7 @@ def hgemm(a, b, layout="NN", out=None, residual=None, variant=0):
     """C = op(a) op(b) (+ residual) through the C ABI on torch's current stream. a, b: contiguous fp16 or bf16 GPU
     tensors; `residual`: [M, N] rows with a contiguous last dimension, added in the GEMM's epilogue (mi355_hgemm_add);
     it may be `out` itself. `variant` != 0 pins a tile shape through the library's internal test hook (1 = 256x256,
-    2 = 128x128, 3 = 64x128 or, for layout NT, 128x64, 4 = 64x64, 5 = 128x256, 6 = 256x128) instead of the choice by shape."""
+    2 = 128x128, 3 = 64x128 or, for layout NT, 128x64, 4 = 64x64, 5 = 128x256, 6 = 256x128, 7 = 32x64 for layouts NN and NT) instead of the choice by shape."""
     import torch
     lay = LAYOUTS[layout] if isinstance(layout, str) else int(layout)
     assert a.dtype in (torch.float16, torch.bfloat16) and b.dtype == a.dtype and a.is_cuda and b.is_cuda
