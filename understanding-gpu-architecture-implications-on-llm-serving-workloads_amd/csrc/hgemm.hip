@@ -1342,6 +1342,16 @@ static hipError_t launch_layout(const T* A, const T* B, T* C, const T* R, int M,
     // padding a leading dimension of a multiple of 8 leaves (what it holds only reaches columns that are never stored).
     const bool ragged_ok = ab_aligned && K % 8 == 0 && K >= 8 && lda < (1L << 22) && ldb < (1L << 22);
     const bool small_m = M <= 64 && !(ragged_ok && few_rows_prefer_tiles(M, N, K, A_KC && B_KC));
+    // 33 .. 64 rows against a second operand of up to 8192 columns (generation steps of that many sequences through the
+    // QKV, O and down projections): 32x64 tiles, two rows of up to 128 workgroups. The 64x64 tiles below put half as many
+    // workgroups on the stream of the second operand, the small-M kernels stream it once per 16 rows; with weights that
+    // come from HBM (us, 64x64 tiles with the 8-deep ring / 32x64 tiles): NT 64 x 4096 x 14336 71 / 55, 48 x 4096 x 4096
+    // 19.9 / 15.8, 40 x 6144 x 4096 19.8 / 15.6; NN 64 x 4096 x 14336 84 / 69, 33 x 4096 x 4096 23.5 / 19.5. Up to 32 rows
+    // are one row of such tiles, and the small-M kernels stay ahead (NT 32 x 4096 x 14336 37 / 56).
+    if constexpr (A_KC) {
+        if (ragged_ok && variant == 0 && M > 32 && M <= 64 && (N + 63) / 64 <= 128)
+            return launch_main<T, A_KC, B_KC, 32, 64, 2, 2, 0, true, 8>(A, B, C, R, M, N, K, lda, ldb, ldc, ldr, stream);
+    }
     // Up to 64 rows (generation-step projections): 64x64 tiles with an 8-deep ring stream the second operand once, on
     // N / 64 workgroups with ~50 KiB each in flight, where the split-K small-M kernels below stream it once per 16 rows.
     if (ragged_ok && M <= 64 && variant == 0 && few_rows_prefer_deep_ring(M, N, K, A_KC && !B_KC, A_KC && B_KC)) {
@@ -1361,10 +1371,11 @@ static hipError_t launch_layout(const T* A, const T* B, T* C, const T* R, int M,
     // both K-contiguous operands; ring of 5), 4 = 64x64 with a ring of 4 (64 KiB: two workgroups fit on a CU), 5 = 128x256
     // and 6 = 256x128 (8 waves of 64x64, ring of 3), 7 = 32x64 (4 waves of 16x32, ring of 8; layouts with a K-contiguous
     // A). More than 64 rows: the shape with the least
-    // estimated time. Up to 64 rows (products that few_rows_prefer_tiles sends here): half tiles for layout NT, which
-    // put twice as many workgroups on the stream of the second operand, 128x128 otherwise.
+    // estimated time. Up to 64 rows (products that few_rows_prefer_tiles sends here): 64x64 tiles, two to a CU, for layout
+    // NT (17 .. 64 x 28672 x 4096 with weights from HBM: 45 - 52 us against 53 - 57 on 128x64 tiles and 51 on 128x128),
+    // 128x128 otherwise (layout NN: 42 - 47 us against 52 - 64).
     if (ragged_ok) {
-        int shape = variant >= 1 && variant <= (A_KC ? 7 : 6) ? variant : M <= 64 ? ((A_KC && B_KC) ? 3 : 2) : cheapest_tile_shape(M, N, K, A_KC);
+        int shape = variant >= 1 && variant <= (A_KC ? 7 : 6) ? variant : M <= 64 ? ((A_KC && B_KC) ? 4 : 2) : cheapest_tile_shape(M, N, K, A_KC);
         const auto whole = [&](int bm, int bn) { return c_aligned && M % bm == 0 && N % bn == 0; };
         switch (shape) {
             case 1:
