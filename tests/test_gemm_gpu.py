@@ -189,6 +189,92 @@ def test_widths_that_are_no_multiple_of_8_and_unaligned_rows_of_c(lib, gpu, vari
         assert bool((c[M:] == 3.0).all()) and bool((c[:, N:] == 3.0).all())
 
 
+# ---- split-K: 17 .. 256 rows against a narrow second operand --------------------------------------------------------
+SPLIT_K_SHAPES = [(64, 4096, 14336), (17, 4096, 8192), (100, 2048, 4096), (128, 4096, 4096), (48, 1000, 2048), (33, 6144, 4096),
+                  (250, 1024, 8192), (40, 72, 16384)]
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("layout", ["NN", "NT", "TN"])
+@pytest.mark.parametrize("M,N,K", SPLIT_K_SHAPES)
+def test_split_k_products(lib, gpu, dtype, layout, M, N, K):
+    # the ranges of K of a tile run on different workgroups and meet in the library's workspace; the workgroup that
+    # arrives last adds them in the order of the ranges, so the result does not depend on the order of arrival: five
+    # launches give the same bits, also with launches of other shapes (other tile and range counts, a workspace that
+    # grows) in between
+    a, b = operands(M, N, K, layout, seed=M + N + K, b_std=0.05)
+    a, b = a.to(dtype), b.to(dtype)
+    ag, bg = a.to(gpu), b.to(gpu)
+    first = lib.hgemm(ag, bg, layout)
+    torch.cuda.synchronize()
+    ref = so.gemm_ref(a, b, layout)
+    if dtype == torch.float16:
+        ok, st = so.gemm_tolerance_ok(first.cpu(), ref, K)
+        assert ok, (layout, M, N, K, st)
+    else:
+        assert bf16_close(first, ref, K)[0]
+    other_a, other_b = operands(96, 512, 1024, "NT", seed=1)
+    for _ in range(4):
+        lib.hgemm(other_a.to(gpu), other_b.to(gpu), "NT")
+        assert torch.equal(lib.hgemm(ag, bg, layout), first)
+
+
+def test_split_k_with_residual_in_place_and_unaligned_c(lib, gpu):
+    M, N, K = 72, 1001, 8192
+    a, b = operands(M, N, K, "NT", seed=3, b_std=0.05)
+    ag, bg = a.to(gpu), b.to(gpu)
+    c = torch.full((M + 1, N + 3), 3.0, dtype=torch.float16, device=gpu)      # rows of 1004 elements: not 16-byte aligned
+    st = torch.cuda.current_stream(gpu).cuda_stream
+    lib.hgemm_raw(ag.data_ptr(), bg.data_ptr(), c.data_ptr(), M, N, K, K, K, N + 3, lib.GEMM_NT, st)
+    torch.cuda.synchronize()
+    ok, stt = so.gemm_tolerance_ok(c[:M, :N].cpu(), so.gemm_ref(a, b, "NT"), K)
+    assert ok, stt
+    assert bool((c[M:] == 3.0).all()) and bool((c[:, N:] == 3.0).all())
+    r = (torch.randn(M, N, generator=torch.Generator().manual_seed(1)) * 2).half().to(gpu)
+    want = c[:M, :N] + r
+    c[:M, :N] = r
+    assert lib.load().mi355_hgemm_add(ag.data_ptr(), bg.data_ptr(), c.data_ptr(), c.data_ptr(), M, N, K, K, K, N + 3, N + 3,
+                                      lib.GEMM_NT, st) == 0
+    torch.cuda.synchronize()
+    assert torch.equal(c[:M, :N], want)
+    assert bool((c[M:] == 3.0).all()) and bool((c[:, N:] == 3.0).all())
+
+
+def test_split_k_on_two_streams_and_under_graph_capture(lib, gpu):
+    # every stream has a workspace of its own: interleaved calls on two streams do not disturb each other. A call made
+    # while its stream is being captured and has no workspace yet takes the kernels without split-K instead of failing;
+    # once the stream has a workspace, the captured call uses it, and replays give the eager result.
+    M, N, K = 64, 2048, 8192
+    a, b = operands(M, N, K, "NT", seed=5, b_std=0.05)
+    ag, bg = a.to(gpu), b.to(gpu)
+    ref = lib.hgemm(ag, bg, "NT").clone()
+    a2, b2 = operands(120, 1024, 4096, "NT", seed=6, b_std=0.05)
+    a2g, b2g = a2.to(gpu), b2.to(gpu)
+    ref2 = lib.hgemm(a2g, b2g, "NT").clone()
+    torch.cuda.synchronize()
+    s1, s2 = torch.cuda.Stream(gpu), torch.cuda.Stream(gpu)
+    outs1, outs2 = [], []
+    for _ in range(6):
+        with torch.cuda.stream(s1):
+            outs1.append(lib.hgemm(ag, bg, "NT"))
+        with torch.cuda.stream(s2):
+            outs2.append(lib.hgemm(a2g, b2g, "NT"))
+    torch.cuda.synchronize()
+    assert all(torch.equal(o, ref) for o in outs1) and all(torch.equal(o, ref2) for o in outs2)
+    s3 = torch.cuda.Stream(gpu)                       # a stream that has never made such a call
+    out = torch.empty((M, N), dtype=torch.float16, device=gpu)
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(s3):
+        with torch.cuda.graph(g, stream=s3):
+            lib.hgemm(ag, bg, "NT", out=out)          # no workspace yet: the kernels without split-K
+    for _ in range(3):
+        out.zero_()
+        g.replay()
+        torch.cuda.synchronize()
+        ok, stt = so.gemm_tolerance_ok(out.cpu(), so.gemm_ref(a, b, "NT"), K)
+        assert ok, stt
+
+
 @pytest.mark.parametrize("variant,tile_m,tile_n", [(1, 256, 256), (2, 128, 128), (3, 64, 128), (4, 64, 64), (5, 128, 256), (6, 256, 128), (7, 32, 64)])
 @pytest.mark.parametrize("layout", ["NN", "NT"])
 @pytest.mark.parametrize("tiles_m,tiles_n,ragged", [(16, 32, 0), (32, 24, 0), (32, 16, 8), (48, 16, 0)])

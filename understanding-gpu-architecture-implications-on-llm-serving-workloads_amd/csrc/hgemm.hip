@@ -32,7 +32,10 @@
 //     The MFMA is issued with the B fragment as first operand, i.e. it produces the transposed block, so a
 //     lane ends up with 4 consecutive N of one row of C; the epilogue parks the sub-tile in LDS and stores whole
 //     128-byte lines.
+#include <map>
+#include <mutex>
 #include <type_traits>
+#include <utility>
 #include "mi355_common.h"
 #include "mi355_serving_internal.h"
 #include "mi355_timeline.h"
@@ -313,11 +316,20 @@ __device__ __forceinline__ void store_wave_tile(const float4v (&acc)[TM][TN], MI
 // a multiple of 8, and what they hold only reaches rows / columns of the product that are never stored), so every load
 // stays inside the matrices' rows; the epilogue stores only what exists: whole 16-byte pieces wherever a row of C starts
 // (global memory takes such an access at any element), the last N % 8 columns of a row element by element.
-template <typename T, bool A_KC, bool B_KC, int BM, int BN, int WM, int WN, int EPI = 0, bool RAGGED = false, int STAGES = 0, int PER_CU = 1>
+// SPLIT_K: the grid's y index selects one of `splits` equal ranges of K (K a multiple of 64 * splits). A workgroup
+// stores its partial tile (fp32, each lane its own accumulators) to `part`, draws a ticket from the tile's counter, and
+// the workgroup that draws the last one adds the partial tiles of all ranges, in the order of the ranges (so the sum does
+// not depend on which workgroup arrives last), and runs the epilogue. Ordering without a fence, as in the split-KV
+// attention kernel: the partial tiles are stored device-coherently (`sc1`), every lane waits for its stores to be
+// acknowledged (`s_waitcnt vmcnt(0)`), a workgroup barrier, then one thread draws the ticket with a relaxed device-scope
+// atomic (carried out at the memory side); the last workgroup reads the partial tiles with `sc1` loads behind the branch
+// on the ticket's value, and sets the counter back to zero for the next launch.
+template <typename T, bool A_KC, bool B_KC, int BM, int BN, int WM, int WN, int EPI = 0, bool RAGGED = false, int STAGES = 0, int PER_CU = 1,
+          bool SPLIT_K = false>
 __global__ __launch_bounds__(WM * WN * 64) __attribute__((amdgpu_waves_per_eu(WM * WN / 4, PER_CU * WM * WN / 4)))
 void hgemm_main_kernel(const T* __restrict__ A, const T* __restrict__ B,
                                                          T* C, const T* R, int M, int N, int K, long lda,
-                                                         long ldb, long ldc, long ldr) {
+                                                         long ldb, long ldc, long ldr, float* part, unsigned* counters, int splits) {
     using V8 = typename Elem<T>::v8;
     using V4 = typename Elem<T>::v4;
     using V2 = typename Elem<T>::v2;
@@ -342,6 +354,12 @@ void hgemm_main_kernel(const T* __restrict__ A, const T* __restrict__ B,
     tile_of_block(blockIdx.x, (M + Cfg::BM - 1) / Cfg::BM, (N + Cfg::BN - 1) / Cfg::BN, tile_m, tile_n);
     const long m0 = (long)tile_m * Cfg::BM;
     const long n0 = (long)tile_n * Cfg::BN;
+    if constexpr (SPLIT_K) {   // this workgroup's range of K
+        K /= splits;
+        const long k0 = (long)blockIdx.y * K;
+        A += A_KC ? k0 : k0 * lda;
+        B += B_KC ? k0 : k0 * ldb;
+    }
 
     // ---- global -> LDS copy descriptors --------------------------------------------------------------
     // A copy reads (tile base, kept in scalar registers and advanced per K tile) + (this lane's byte offset inside the
@@ -666,6 +684,51 @@ void hgemm_main_kernel(const T* __restrict__ A, const T* __restrict__ B,
     static_assert(Cfg::NWAVES * TM * 16 * TNO * 32 <= Cfg::LDS_BYTES, "epilogue staging does not fit in LDS");
     wait_vmcnt<0>();  // the last tiles' copies (on the empty buffer) have written their zeros
     __syncthreads();  // every wave has finished reading the operand stages
+    if constexpr (SPLIT_K) {
+        // partial tile (block, range): element q of lane t's accumulator block b at float (b * 4 + q) * NTHREADS + t, so
+        // that every store and load instruction of a wave covers 256 contiguous bytes
+        const long tile_floats = (long)Cfg::NTHREADS * TM * TN * 4;
+        float* tile_part = part + (long)blockIdx.x * splits * tile_floats;
+        float* mine = tile_part + (long)blockIdx.y * tile_floats + tid;
+        // (device-scope atomic stores, i.e. `global_store_dword .. sc1`, written as such so that the compiler places the
+        // wait states between the last matrix instructions and the first memory instruction that reads their result: a
+        // wave that arrives last at the barrier above is only a few cycles behind its last MFMA)
+#pragma unroll
+        for (int b = 0; b < TM * TN; ++b)
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+                __hip_atomic_store(mine + (long)(b * 4 + q) * Cfg::NTHREADS, acc[b / TN][b % TN][q], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // this lane's part has reached memory before the ticket is drawn
+        __syncthreads();
+        MI355_LDS unsigned* ticket_sh = (MI355_LDS unsigned*)smem;
+        if (tid == 0) *ticket_sh = __hip_atomic_fetch_add(&counters[blockIdx.x], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __syncthreads();
+        const unsigned ticket = *ticket_sh;
+        __syncthreads();   // the epilogue below reuses that LDS
+        if (ticket != (unsigned)(splits - 1)) return;
+        // the last one: every other workgroup of this tile drew its ticket after its part had reached memory. The parts
+        // are read with device-coherent loads (sc1), 16 in flight per lane, and added in the order of the ranges.
+#pragma unroll
+        for (int b = 0; b < TM * TN; ++b) {
+            float4v sum = float4v{0.f, 0.f, 0.f, 0.f};
+            for (int r0 = 0; r0 < splits; r0 += 4) {
+                float4v v[4];
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    const float* pa = tile_part + (long)min(r0 + u, splits - 1) * tile_floats + (long)(b * 4) * Cfg::NTHREADS + tid;
+#pragma unroll
+                    for (int q = 0; q < 4; ++q)
+                        asm volatile("global_load_dword %0, %1, off sc1" : "=v"(v[u][q]) : "v"(pa + (long)q * Cfg::NTHREADS) : "memory");
+                }
+                asm volatile("s_waitcnt vmcnt(0)" : "+v"(v[0]), "+v"(v[1]), "+v"(v[2]), "+v"(v[3]) :: "memory");
+#pragma unroll
+                for (int u = 0; u < 4; ++u)
+                    if (r0 + u < splits) sum += v[u];
+            }
+            acc[b / TN][b % TN] = sum;
+        }
+        if (tid == 0) __hip_atomic_store(&counters[blockIdx.x], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
     store_wave_tile<T, TM, TN, EPI, RAGGED>(acc, smem + wave * (TM * 16 * TNO * 32), C, R, m0 + wm * TM * 16,
                                             (EPI == 1 ? n0 / 2 : n0) + wn * TNO * 16, M, EPI == 1 ? N / 2 : N, ldc, ldr, lane);
     MI355_TL(
@@ -1232,7 +1295,93 @@ static hipError_t launch_main(const T* A, const T* B, T* C, const T* R, int M, i
     const long nblocks = (long)((M + BM - 1) / BM) * ((N + BN - 1) / BN);
     if (nblocks > 0x7fffffffL) return hipErrorInvalidValue;
     int blocks = (int)nblocks;
-    kern<<<dim3(blocks), dim3(Cfg::NTHREADS), Cfg::LDS_BYTES, stream>>>(A, B, C, R, M, N, K, lda, ldb, ldc, ldr);
+    kern<<<dim3(blocks), dim3(Cfg::NTHREADS), Cfg::LDS_BYTES, stream>>>(A, B, C, R, M, N, K, lda, ldb, ldc, ldr, nullptr, nullptr, 1);
+    return hipGetLastError();
+}
+
+// ---------------------------------------------------------------------------------------------------------
+// Split-K on 64x64 tiles, for 17 .. 256 rows against a second operand that is too narrow to give every CU a tile: the
+// ranges of K of a tile run on different workgroups (see SPLIT_K of hgemm_main_kernel) and meet in a workspace of the
+// library's own: one buffer per (device, stream), allocated at first use and replaced by a larger one when a call needs
+// more; a buffer that has been handed to a kernel is never freed (a HIP graph captured earlier may hold its address).
+// Nothing can be allocated while the stream is capturing: such a call (no buffer yet, or too small a one) takes the
+// kernels without split-K instead. The ticket counters, in front of the partial tiles, are zeroed when a buffer is new
+// (a fill kernel on the calling stream) and left at zero by every launch.
+// ---------------------------------------------------------------------------------------------------------
+constexpr size_t kSplitKCounterBytes = 16 * 1024;   // one counter per tile: up to 4096 tiles
+
+static __global__ void hgemm_clear_kernel(unsigned* p, int n) {
+    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < n; i += gridDim.x * blockDim.x) p[i] = 0u;
+}
+
+static hipError_t split_k_workspace(size_t bytes, hipStream_t stream, char** out, bool* fresh) {
+    struct Buf {
+        void* ptr = nullptr;
+        size_t size = 0;
+    };
+    static std::mutex mu;
+    static std::map<std::pair<int, hipStream_t>, Buf> bufs;
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    std::lock_guard<std::mutex> lock(mu);
+    Buf& b = bufs[std::make_pair(dev, stream)];
+    *fresh = false;
+    if (b.size < bytes) {
+        hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+        e = hipStreamIsCapturing(stream, &cap);
+        if (e != hipSuccess) return e;
+        if (cap != hipStreamCaptureStatusNone) return hipErrorStreamCaptureUnsupported;
+        const size_t want = bytes < (size_t(8) << 20) ? (size_t(8) << 20) : bytes + bytes / 2;
+        void* fresh_buf = nullptr;
+        e = hipMalloc(&fresh_buf, want);
+        if (e != hipSuccess) return e;
+        b.ptr = fresh_buf;   // the previous buffer, if any, stays allocated (see above)
+        b.size = want;
+        *fresh = true;
+    }
+    *out = static_cast<char*>(b.ptr);
+    return hipSuccess;
+}
+
+// Number of ranges K is cut into, or 0 where split-K does not apply: 17 .. 256 rows, K a multiple of 64, few enough
+// 64x64 tiles for at least four ranges at about two workgroups per CU, at least eight K tiles per range, ranges of equal
+// length. Measured with weights that come from HBM, layout NT (us, without / with split-K): 64 x 4096 x 14336 55 / 32,
+// 17 x 4096 x 14336 35 / 29, 128 x 4096 x 14336 54 / 44, 64 x 4096 x 4096 17.4 / 15.7, 96 x 4096 x 4096 17.3 / 15.5,
+// 48 x 6144 x 4096 16.6 / 17.4; two ranges only lose (96 x 6144 x 4096 20 / 24, 192 x 4096 x 4096 21 / 25), and so do up to
+// 32 rows with a short K, where the small-M kernels are at their best (32 x 4096 x 4096 11 / 15).
+static int split_k_ranges(int M, int N, int K) {
+    if (M < 17 || M > 256 || K % 64 != 0) return 0;
+    if (M <= 32 && K < 8192) return 0;
+    const long tiles = (long)((M + 63) / 64) * ((N + 63) / 64);
+    if (tiles > 128) return 0;
+    const int ktiles = K / 64;
+    int s = (int)(512 / tiles);
+    if (s > 16) s = 16;
+    while (s >= 4 && (ktiles % s != 0 || ktiles / s < 8)) --s;
+    return s >= 4 ? s : 0;
+}
+
+// hipErrorStreamCaptureUnsupported / hipErrorOutOfMemory: no workspace to be had, the caller takes another kernel
+template <typename T, bool A_KC, bool B_KC>
+static hipError_t launch_split_k(const T* A, const T* B, T* C, const T* R, int M, int N, int K, long lda, long ldb, long ldc,
+                                 long ldr, int splits, hipStream_t stream) {
+    using Cfg = MainCfg<A_KC, B_KC, 64, 64, 2, 2, 4>;
+    auto kern = hgemm_main_kernel<T, A_KC, B_KC, 64, 64, 2, 2, 0, true, 4, 2, true>;
+    static DynamicLdsOnce lds_once;
+    if (hipError_t e = lds_once.ensure(reinterpret_cast<const void*>(kern), Cfg::LDS_BYTES); e != hipSuccess) return e;
+    const long tiles = (long)((M + 63) / 64) * ((N + 63) / 64);
+    if (tiles * sizeof(unsigned) > kSplitKCounterBytes) return hipErrorOutOfMemory;
+    const size_t bytes = kSplitKCounterBytes + (size_t)tiles * splits * Cfg::NTHREADS * Cfg::TM * Cfg::TN * 16;
+    char* ws = nullptr;
+    bool fresh = false;
+    if (hipError_t e = split_k_workspace(bytes, stream, &ws, &fresh); e != hipSuccess) return e;
+    if (fresh) {
+        hgemm_clear_kernel<<<dim3(4), dim3(256), 0, stream>>>(reinterpret_cast<unsigned*>(ws), (int)(kSplitKCounterBytes / sizeof(unsigned)));
+        if (hipError_t e = hipGetLastError(); e != hipSuccess) return e;
+    }
+    kern<<<dim3((unsigned)tiles, (unsigned)splits), dim3(Cfg::NTHREADS), Cfg::LDS_BYTES, stream>>>(
+        A, B, C, R, M, N, K, lda, ldb, ldc, ldr, reinterpret_cast<float*>(ws + kSplitKCounterBytes), reinterpret_cast<unsigned*>(ws), splits);
     return hipGetLastError();
 }
 
@@ -1342,6 +1491,14 @@ static hipError_t launch_layout(const T* A, const T* B, T* C, const T* R, int M,
     // padding a leading dimension of a multiple of 8 leaves (what it holds only reaches columns that are never stored).
     const bool ragged_ok = ab_aligned && K % 8 == 0 && K >= 8 && lda < (1L << 22) && ldb < (1L << 22);
     const bool small_m = M <= 64 && !(ragged_ok && few_rows_prefer_tiles(M, N, K, A_KC && B_KC));
+    // 17 .. 256 rows against a narrow second operand: split-K, where a workspace is to be had (variant 8 asks for it)
+    if (ragged_ok && (variant == 0 || variant == 8)) {
+        if (const int splits = split_k_ranges(M, N, K); splits > 0) {
+            const hipError_t e = launch_split_k<T, A_KC, B_KC>(A, B, C, R, M, N, K, lda, ldb, ldc, ldr, splits, stream);
+            if (e != hipErrorStreamCaptureUnsupported && e != hipErrorOutOfMemory) return e;
+            (void)hipGetLastError();
+        }
+    }
     // 33 .. 64 rows against a second operand of up to 8192 columns (generation steps of that many sequences through the
     // QKV, O and down projections): 32x64 tiles, two rows of up to 128 workgroups. The 64x64 tiles below put half as many
     // workgroups on the stream of the second operand, the small-M kernels stream it once per 16 rows; with weights that
