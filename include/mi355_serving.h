@@ -7,7 +7,7 @@
  *
  * Conventions
  *   - every pointer is a DEVICE pointer owned by the caller; none is retained. The only memory the library ever
- *     allocates is a workspace for the partial results of the split-KV attention path (taken when
+ *     allocates are two kinds of workspace. One holds the partial results of the split-KV attention path (taken when
  *     Hq/Hkv * Sq <= 32 and kv_valid_len >= 512, i.e. generation steps): one buffer per (device, stream), obtained
  *     with hipMalloc at first use (>= 4 MiB; when a later call needs more, a larger buffer is allocated and the old
  *     one is kept, because a HIP graph captured earlier may still hold its address; nothing is freed before the
@@ -17,7 +17,11 @@
  *     and launches nothing: run the step once on that stream before capturing it, and replay the graph on the stream it
  *     was captured on (or use mi355_fmha_fwd_ws with memory of your own). Only the calling stream's capture state is
  *     visible to the library: a first (or growing) call made while ANOTHER stream captures in global capture mode is a
- *     hipMalloc inside that capture and invalidates it, so make such calls before any capture starts;
+ *     hipMalloc inside that capture and invalidates it, so make such calls before any capture starts.
+ *     The GEMM entry points keep a second buffer of the same kind per (device, stream) for the partial tiles of their
+ *     split-K path (17 .. 256 rows against a second operand of up to 8192 columns, K a multiple of 256; >= 8 MiB); a
+ *     GEMM call that cannot get it (its stream is being captured and has none yet, or hipMalloc fails) does not fail: it
+ *     runs the kernels without split-K, so a captured call is faster when the step ran once on that stream before;
  *   - `stream` is a hipStream_t passed as void* (NULL = the null stream); calls are asynchronous;
  *   - fp16 data is IEEE binary16 (`_Float16` / `__half` / torch.float16);
  *   - return value 0 = launched; non-zero = a hipError_t value or MI355_ERR_* below, nothing was launched.

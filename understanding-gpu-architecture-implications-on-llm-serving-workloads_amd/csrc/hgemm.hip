@@ -1491,8 +1491,8 @@ static hipError_t launch_layout(const T* A, const T* B, T* C, const T* R, int M,
     // padding a leading dimension of a multiple of 8 leaves (what it holds only reaches columns that are never stored).
     const bool ragged_ok = ab_aligned && K % 8 == 0 && K >= 8 && lda < (1L << 22) && ldb < (1L << 22);
     const bool small_m = M <= 64 && !(ragged_ok && few_rows_prefer_tiles(M, N, K, A_KC && B_KC));
-    // 17 .. 256 rows against a narrow second operand: split-K, where a workspace is to be had (variant 8 asks for it)
-    if (ragged_ok && (variant == 0 || variant == 8)) {
+    // 17 .. 256 rows against a narrow second operand: split-K, where a workspace is to be had
+    if (ragged_ok && variant == 0) {
         if (const int splits = split_k_ranges(M, N, K); splits > 0) {
             const hipError_t e = launch_split_k<T, A_KC, B_KC>(A, B, C, R, M, N, K, lda, ldb, ldc, ldr, splits, stream);
             if (e != hipErrorStreamCaptureUnsupported && e != hipErrorOutOfMemory) return e;
