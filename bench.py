@@ -387,6 +387,20 @@ def main():
                                                  "ms_weights_not_cached": ms64_cold, "gbs_weights_not_cached": by64 / ms64_cold / 1e6,
                                                  "pct_of_hbm_peak_weights_not_cached": 100 * by64 / ms64_cold / 1e6 / PEAK_HBM_GBS}
         del x64, o64, wd_sets
+        # a down projection at batch 64 (4096 rows of a [N, K] weight with K = 14336): 64 tiles of 64x64, split-K over 8 ranges
+        xk = so.randn_fp16((64, 14336), 4).to(dev)
+        wk = so.randn_fp16((4096, 14336), 5, 0.02).to(dev)
+        ok_ = torch.empty((64, 4096), dtype=torch.float16, device=dev)
+        wk_sets = [wk] + [wk.clone() for _ in range(copies_to_defeat_cache(wk.numel() * 2) - 1)]
+        msk = time_launches(lambda: lib.hgemm_raw(xk.data_ptr(), wk.data_ptr(), ok_.data_ptr(), 64, 4096, 14336, 14336, 14336,
+                                                  4096, lib.GEMM_NT, stream), 20, 3)
+        msk_cold = time_launches(rotating(lambda j: lib.hgemm_raw(xk.data_ptr(), wk_sets[j].data_ptr(), ok_.data_ptr(), 64, 4096, 14336,
+                                                                  14336, 14336, 4096, lib.GEMM_NT, stream), len(wk_sets)), 40, 3)
+        byk = 2.0 * (64 * 14336 + 4096 * 14336 + 64 * 4096)
+        other["gemm_decode_nt_64x4096x14336_split_k"] = {"ms": msk, "gbs": byk / msk / 1e6, "pct_of_hbm_peak": 100 * byk / msk / 1e6 / PEAK_HBM_GBS,
+                                                        "ms_weights_not_cached": msk_cold, "gbs_weights_not_cached": byk / msk_cold / 1e6,
+                                                        "pct_of_hbm_peak_weights_not_cached": 100 * byk / msk_cold / 1e6 / PEAK_HBM_GBS}
+        del xk, wk, ok_, wk_sets
         ab, bb = a.to(torch.bfloat16), b.to(torch.bfloat16)
         cb = torch.empty((M, N), dtype=torch.bfloat16, device=dev)
         msb = time_launches(lambda: lib.hgemm(ab, bb, "NN", out=cb), 10, 2)
@@ -639,6 +653,7 @@ KERNEL_CONFIGS = {
     "gemm_16x14336x4096_nt": ("gemm", 16, 14336, 4096, "NT"),               # split-K small-M kernel (NT)
     "gemm_8x28672x4096_nt": ("gemm", 8, 28672, 4096, "NT"),                 # split-K small-M kernel (NT), A rows 0..7 only
     "gemm_64x14336x4096_nt": ("gemm", 64, 14336, 4096, "NT"),               # 64x64 tiles, 8-deep ring
+    "gemm_64x4096x14336_nt": ("gemm", 64, 4096, 14336, "NT"),               # 64x64 tiles, split-K over 8 ranges
     "gemm_16x4096x14336_nt": ("gemm", 16, 4096, 14336, "NT"),               # split-K small-M kernel (NT)
     "gemm_1024x4096x4096_nt": ("gemm", 1024, 4096, 4096, "NT"),             # 128x64 tiles
     "f3_fmha_noncausal_b4_h32_s1024": ("fmha", 4, 32, 32, 1024, 1024, False),   # ping-pong kernel, 256-query work items
