@@ -191,7 +191,7 @@ def test_widths_that_are_no_multiple_of_8_and_unaligned_rows_of_c(lib, gpu, vari
 
 # ---- split-K: 17 .. 256 rows against a narrow second operand --------------------------------------------------------
 SPLIT_K_SHAPES = [(64, 4096, 14336), (17, 4096, 8192), (100, 2048, 4096), (128, 4096, 4096), (48, 1000, 2048), (33, 6144, 4096),
-                  (250, 1024, 8192), (40, 72, 16384)]
+                  (250, 1024, 8192), (40, 72, 16384), (160, 4096, 8192), (192, 4000, 14336)]
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])

@@ -1345,18 +1345,20 @@ static hipError_t split_k_workspace(size_t bytes, hipStream_t stream, char** out
 }
 
 // Number of ranges K is cut into, or 0 where split-K does not apply: 17 .. 256 rows, K a multiple of 64, few enough
-// 64x64 tiles for at least four ranges at about two workgroups per CU, at least eight K tiles per range, ranges of equal
-// length. Measured with weights that come from HBM, layout NT (us, without / with split-K): 64 x 4096 x 14336 55 / 32,
+// 64x64 tiles for at least four ranges at about two workgroups per CU (up to 128 tiles; up to 192 with a long K), at
+// least eight K tiles per range, ranges of equal length. Measured with weights that come from HBM, layout NT (us, without / with split-K): 64 x 4096 x 14336 55 / 32,
 // 17 x 4096 x 14336 35 / 29, 128 x 4096 x 14336 54 / 44, 64 x 4096 x 4096 17.4 / 15.7, 96 x 4096 x 4096 17.3 / 15.5,
 // 48 x 6144 x 4096 16.6 / 17.4; two ranges only lose (96 x 6144 x 4096 20 / 24, 192 x 4096 x 4096 21 / 25), and so do up to
-// 32 rows with a short K, where the small-M kernels are at their best (32 x 4096 x 4096 11 / 15).
+// 32 rows with a short K, where the small-M kernels are at their best (32 x 4096 x 4096 11 / 15). 129 .. 192 tiles get
+// four ranges where K is long (192 x 4096 x 14336 70 / 58, NN 81 / 59; with K = 4096 22 against 21 without; 256 tiles:
+// 69 / 73).
 static int split_k_ranges(int M, int N, int K) {
     if (M < 17 || M > 256 || K % 64 != 0) return 0;
     if (M <= 32 && K < 8192) return 0;
     const long tiles = (long)((M + 63) / 64) * ((N + 63) / 64);
-    if (tiles > 128) return 0;
+    if (tiles > 192 || (tiles > 128 && K < 8192)) return 0;
     const int ktiles = K / 64;
-    int s = (int)(512 / tiles);
+    int s = tiles > 128 ? 4 : (int)(512 / tiles);
     if (s > 16) s = 16;
     while (s >= 4 && (ktiles % s != 0 || ktiles / s < 8)) --s;
     return s >= 4 ? s : 0;
