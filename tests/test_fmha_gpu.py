@@ -478,6 +478,115 @@ def test_torch_operator_reads_transposed_views_in_place(gpu):
 # ---- bfloat16 -----------------------------------------------------------------------------------------------------------
 # Tolerance for bfloat16 outputs (8 significand bits; the fp16 bound of 2e-3 is below half a bf16 ulp of values near 1):
 # max|O - O_ref| <= 1.6e-2 against fp32 attention over the same bf16-rounded inputs; LSE (fp32 from fp32 scores) keeps 1e-3.
+# ---- a chunk of queries against a long cache: keys cut into ranges, merged by a second kernel --------------------
+@pytest.mark.parametrize("B,Hq,Hkv,Sq,Sk,causal,kvv", [
+    (1, 32, 8, 128, 8192, True, None),     # 8 ranges of 1024 keys
+    (1, 32, 8, 64, 8192, True, 8000),      # half-filled q tile, last range shorter
+    (1, 16, 4, 300, 4500, True, 4097),     # 3 q tiles, ranges that are no multiple of the tile, one valid key in the last
+    (2, 8, 2, 200, 5000, False, None),     # 4 ranges of 1280 keys
+    (1, 32, 8, 512, 8192, False, 5000),    # 128 items: two ranges
+    (3, 4, 1, 100, 4096, True, None),
+    (1, 4, 4, 4096, 4096, True, None),     # causal square: the second range is invisible to the early q tiles
+    (1, 8, 1, 5, 12000, True, 11000),      # 40 query rows per kv head: more than the generation-step kernels take
+])
+def test_chunk_against_long_cache_key_ranges(lib, gpu, B, Hq, Hkv, Sq, Sk, causal, kvv):
+    q, k, v = so.fmha_inputs(B, Hq, Hkv, Sq, Sk, seed=Sq + Sk + Hq)
+    o, lse = check(lib, gpu, q, k, v, causal, kvv, variant=3)     # variant 3: key ranges, or an error where they do not apply
+    if kvv is not None:     # keys past the valid length may hold anything
+        k, v = k.clone(), v.clone()
+        k[:, :, kvv:] = float("nan")
+        v[:, :, kvv:] = float("inf")
+        o_p, lse_p = run(lib, gpu, q, k, v, causal, kvv, variant=3)
+        assert torch.equal(o, o_p) and torch.equal(lse, lse_p)
+    o0, lse0 = run(lib, gpu, q, k, v, causal, kvv)                # the choice by shape takes the same path
+    assert torch.equal(o, o0) and torch.equal(lse, lse0)
+    o1, lse1 = run(lib, gpu, q, k, v, causal, kvv, variant=1)     # the same kernel over all keys at once
+    assert (o.float() - o1.float()).abs().max() <= 2e-3 and (lse - lse1).abs().max() <= 1e-3
+
+
+def test_key_ranges_only_where_they_pay(lib, gpu):
+    # enough work items for the machine, a short cache, or a generation step: no ranges (variant 3 reports it)
+    for B, Hq, Hkv, Sq, Sk in ((1, 32, 8, 1024, 8192), (1, 32, 8, 128, 1024), (1, 32, 8, 512, 2048)):
+        q, k, v = (t.to(gpu) for t in so.fmha_inputs(B, Hq, Hkv, Sq, Sk, seed=3))
+        with pytest.raises(lib.Mi355Error):
+            lib.fmha_fwd(q, k, v, causal=True, variant=3)
+
+
+def test_key_ranges_bfloat16_and_transposed_views(lib, gpu):
+    B, Hq, Hkv, Sq, Sk = 2, 8, 2, 150, 6000
+    q, k, v = so.fmha_inputs(B, Hq, Hkv, Sq, Sk, seed=77)
+    qb, kb, vb = q.float().bfloat16(), k.float().bfloat16(), v.float().bfloat16()
+    o, lse = lib.fmha_fwd(qb.to(gpu), kb.to(gpu), vb.to(gpu), causal=True, kv_valid_len=5555)
+    o_ref, lse_ref = so.attention_ref(qb, kb, vb, causal=True, kv_valid_len=5555)
+    assert (o.float().cpu() - o_ref).abs().max() <= 1.6e-2 and (lse.cpu() - lse_ref).abs().max() <= 1e-3
+    # [B, S, H, D] storage viewed as [B, H, S, D]: inputs and output
+    qt = q.transpose(1, 2).contiguous().to(gpu).transpose(1, 2)
+    kt = k.transpose(1, 2).contiguous().to(gpu).transpose(1, 2)
+    vt = v.transpose(1, 2).contiguous().to(gpu).transpose(1, 2)
+    out = torch.full((B, Sq, Hq, 128), 7.0, dtype=torch.float16, device=gpu).transpose(1, 2)
+    lib.fmha_fwd(qt, kt, vt, causal=True, return_lse=False, out=out)
+    o_ref, _ = so.attention_ref(q, k, v, causal=True)
+    assert (out.float().cpu() - o_ref).abs().max() <= 2e-3
+
+
+def test_key_ranges_workspace_per_stream_growing_and_reused(lib, gpu):
+    # one workspace per stream, replaced by a larger one when a call needs more; results are reproducible bit for bit
+    small = [t.to(gpu) for t in so.fmha_inputs(1, 8, 2, 128, 4096, seed=5)]        # 4 MB of partial results
+    large = [t.to(gpu) for t in so.fmha_inputs(1, 32, 8, 512, 8192, seed=6)]       # 17 MB
+    ref_s = lib.fmha_fwd(*small, causal=True)
+    ref_l = lib.fmha_fwd(*large, causal=True)
+    torch.cuda.synchronize()
+    s1, s2 = torch.cuda.Stream(), torch.cuda.Stream()
+    got = []
+    for _ in range(3):
+        with torch.cuda.stream(s1):
+            got.append((lib.fmha_fwd(*small, causal=True), ref_s))
+            got.append((lib.fmha_fwd(*large, causal=True), ref_l))
+        with torch.cuda.stream(s2):
+            got.append((lib.fmha_fwd(*large, causal=True), ref_l))
+            got.append((lib.fmha_fwd(*small, causal=True), ref_s))
+    torch.cuda.synchronize()
+    for (o, lse), (o_ref, lse_ref) in got:
+        assert torch.equal(o, o_ref) and torch.equal(lse, lse_ref)
+
+
+def test_key_ranges_fall_back_to_one_walk_when_capture_forbids_allocation(lib, gpu):
+    # A stream the library has never seen has no workspace for the partial results; under capture none may be allocated,
+    # so the call runs the kernel over all keys at once (same result as that variant, bit for bit) instead of failing.
+    import ctypes
+    hip = ctypes.CDLL("libamdhip64.so")
+    raw = ctypes.c_void_p()
+    assert hip.hipStreamCreate(ctypes.byref(raw)) == 0
+    fresh = torch.cuda.ExternalStream(raw.value)
+    q, k, v = (t.to(gpu) for t in so.fmha_inputs(1, 32, 8, 128, 4096, seed=41))
+    ranges = lib.fmha_fwd(q, k, v, causal=True)[0].clone()
+    whole = lib.fmha_fwd(q, k, v, causal=True, variant=1)[0].clone()
+    out_g = torch.zeros_like(q)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=fresh):
+        lib.fmha_fwd(q, k, v, causal=True, return_lse=False, out=out_g)
+    for _ in range(2):
+        out_g.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out_g, whole)
+    del graph
+    # with a workspace in place (first eager call on the stream) a capture records the ranges and the merge
+    with torch.cuda.stream(fresh):
+        lib.fmha_fwd(q, k, v, causal=True, return_lse=False, out=out_g)
+    fresh.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=fresh):
+        lib.fmha_fwd(q, k, v, causal=True, return_lse=False, out=out_g)
+    for _ in range(2):
+        out_g.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out_g, ranges)
+    del graph
+
+
 def bf16_inputs(B, Hq, Hkv, Sq, Sk, seed):
     q, k, v = so.fmha_inputs(B, Hq, Hkv, Sq, Sk, seed=seed)
     return q.float().bfloat16(), k.float().bfloat16(), v.float().bfloat16()

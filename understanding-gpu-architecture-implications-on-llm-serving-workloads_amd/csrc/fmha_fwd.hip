@@ -17,7 +17,10 @@
 //                      ds_read_b64_tr_b16 in that same key order.
 // K and V tiles (64 keys x 128 d) are copied global -> LDS with 16-byte direct-to-LDS copies into a ring of four slots
 // per operand, 16-byte chunks XOR-swizzled so that both the b128 reads (K) and the transposing reads (V) are conflict free.
+#include <map>
+#include <mutex>
 #include <type_traits>
+#include <utility>
 #include "mi355_common.h"
 #include "mi355_serving_internal.h"
 #include "mi355_timeline.h"
@@ -151,12 +154,17 @@ __device__ __forceinline__ void copy16_global_to_lds_at(const void* uniform_base
         : "memory", "m0", "scc");
 }
 
-template <typename T, int QB>
+// SEG: the keys are cut into `segments` ranges of seg_len keys (a multiple of 64) and a work item is (batch, range, head, q
+// tile): it attends to its range only (K and V start seg * seg_len rows further on, the valid length and the causal limit
+// are counted from there) and writes its O, normalised over its range, and its LSE to the partial buffers
+// O [segments][B][Hq][Sq][128] and LSE [segments][B][Hq][Sq]; fmha_merge_segments_kernel combines them. For a few queries
+// against a long cache, where one item per (head, q tile) would leave most CUs idle behind a long walk over the keys.
+template <typename T, int QB, bool SEG = false>
 __global__ __launch_bounds__(512, 2) void fmha_fwd_pingpong_kernel(const T* __restrict__ Q, const T* __restrict__ K,
                                                                const T* __restrict__ V, T* __restrict__ O,
                                                                float* __restrict__ LSE, int B, int Hq, int Hkv, int Sq,
                                                                int Sk, float scale_log2, int causal, int kv_valid,
-                                                               int q_tiles, FmhaStrides sd) {
+                                                               int q_tiles, FmhaStrides sd, int segments, int seg_len) {
     using namespace fmha;
     using V8 = typename Elem<T>::v8;
     using V4 = typename Elem<T>::v4;
@@ -180,7 +188,9 @@ __global__ __launch_bounds__(512, 2) void fmha_fwd_pingpong_kernel(const T* __re
 
     // ---- the work item this workgroup is on (set_item) --------------------------------------------------------------
     const int group = Hq / Hkv;
-    const int shift = Sk - Sq;
+    int shift = Sk - Sq;
+    const int kv_valid_all = kv_valid;
+    long o_row = sd.o_row;
     int b = 0, hq = 0, q_wave0 = 0, n_tiles = 0, n_full = 0, last_tile = 0;
     const T* Qh = Q;
     const T* Kh = K;
@@ -188,14 +198,28 @@ __global__ __launch_bounds__(512, 2) void fmha_fwd_pingpong_kernel(const T* __re
     T* Oh = O;
     auto set_item = [&](int round) -> bool {
         int q_tile;
-        if (!fmha_work_item(blockIdx.x, gridDim.x, round, q_tiles, group, Hkv, B, b, hq, q_tile)) return false;
+        if (!fmha_work_item(blockIdx.x, gridDim.x, round, q_tiles, group, Hkv, SEG ? B * segments : B, b, hq, q_tile)) return false;
         const int hkv = hq / group;
         const int q_block0 = q_tile * BM;
         q_wave0 = q_block0 + wave * WQ;
+        if constexpr (SEG) {   // b counts (batch, range) pairs
+            const int seg = b % segments;
+            b /= segments;
+            const long k0 = (long)seg * seg_len;
+            Qh = Q + b * sd.q_batch + hq * sd.q_head;
+            Kh = K + b * sd.k_batch + hkv * sd.k_head + k0 * sd.k_row;
+            Vh = V + b * sd.v_batch + hkv * sd.v_head + k0 * sd.v_row;
+            Oh = O + (((long)seg * B + b) * Hq + hq) * (long)Sq * D;
+            o_row = D;
+            kv_valid = min(max(kv_valid_all - (int)k0, 0), seg_len);
+            shift = Sk - Sq - (int)k0;
+            b = seg * B + b;   // the LSE row of this item, below
+        } else {
         Qh = Q + b * sd.q_batch + hq * sd.q_head;
         Kh = K + b * sd.k_batch + hkv * sd.k_head;
         Vh = V + b * sd.v_batch + hkv * sd.v_head;
         Oh = O + b * sd.o_batch + hq * sd.o_head;
+        }
         int k_end = kv_valid;
         if (causal) k_end = min(k_end, min(q_block0 + BM, Sq) - 1 + shift + 1);
         n_tiles = (k_end + BN - 1) / BN;            // may be <= 0: no visible key for the whole work item
@@ -590,7 +614,7 @@ __global__ __launch_bounds__(512, 2) void fmha_fwd_pingpong_kernel(const T* __re
             const float inv = (l_tot > 0.f) ? 1.f / l_tot : 0.f;
             const int qi = q_item0 + qb * 16 + c16;
             if (qi < Sq) {
-                T* orow = o_item + qi * sd.o_row + 4 * g;
+                T* orow = o_item + qi * o_row + 4 * g;
 #pragma unroll
                 for (int db = 0; db < 8; ++db) {
                     V4 v;
@@ -647,7 +671,122 @@ static hipError_t launch_fmha_pingpong(const T* Q, const T* K, const T* V, T* O,
     if (((long)Hkv * B) % 8 == 0 && blocks >= 8) blocks &= ~7L;
     const float scale_log2 = scale * 1.4426950408889634f;
     kern<<<dim3((unsigned)blocks), dim3(512), LDS, stream>>>(Q, K, V, O, LSE, B, Hq, Hkv, Sq, Sk, scale_log2, causal, kv_valid,
-                                                             q_tiles, sd);
+                                                             q_tiles, sd, 1, 0);
+    return hipGetLastError();
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// A few queries against a long cache (a chunk of a prompt appended to earlier chunks): one work item per (head, q tile)
+// would leave most CUs idle behind a walk over all keys, so the keys are cut into ranges, every (range, head, q tile) is
+// a work item of the same kernel (SEG) and a second kernel merges the ranges:
+//   O = sum_s w_s O_s / sum_s w_s,  w_s = exp(LSE_s - max_s LSE_s),  LSE = max_s LSE_s + log(sum_s w_s)
+// (a range without a visible key has LSE_s = -inf and weight 0; a row without any visible key gets O = 0, LSE = -inf).
+// The partial results live in a workspace of the library's own, one buffer per (device, stream), allocated at first use
+// and replaced by a larger one when a call needs more (never freed: a captured graph may hold its address). A call that
+// cannot get it (its stream is being captured and has none yet) runs the kernel without ranges instead.
+// ---------------------------------------------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void fmha_merge_segments_kernel(const T* __restrict__ Opart, const float* __restrict__ LSEpart,
+                                                                  T* __restrict__ O, float* __restrict__ LSE, int B, int Hq, int Sq,
+                                                                  int segments, FmhaStrides sd) {
+    using V2 = typename Elem<T>::v2;
+    const int lane = threadIdx.x & 63;
+    const long row = (long)blockIdx.x * 4 + (threadIdx.x >> 6);   // one wave per (batch, head, query)
+    const long rows = (long)B * Hq * Sq;
+    if (row >= rows) return;
+    const int q = (int)(row % Sq);
+    const long bh = row / Sq;
+    const int h = (int)(bh % Hq), b = (int)(bh / Hq);
+    float m = -INFINITY;
+    for (int s = 0; s < segments; ++s) m = fmaxf(m, LSEpart[(long)s * rows + row]);
+    float acc0 = 0.f, acc1 = 0.f, denom = 0.f;
+    if (m > -INFINITY) {
+        for (int s = 0; s < segments; ++s) {
+            const float w = __expf(LSEpart[(long)s * rows + row] - m);   // exp(-inf) = 0
+            const V2 v = *(const V2*)(Opart + ((long)s * rows + row) * fmha::D + 2 * lane);
+            acc0 += w * (float)v[0];
+            acc1 += w * (float)v[1];
+            denom += w;
+        }
+    }
+    const float inv = denom > 0.f ? 1.f / denom : 0.f;
+    V2 out;
+    out[0] = (T)(acc0 * inv);
+    out[1] = (T)(acc1 * inv);
+    *(V2*)(O + b * sd.o_batch + h * sd.o_head + q * sd.o_row + 2 * lane) = out;
+    if (LSE != nullptr && lane == 0) LSE[row] = denom > 0.f ? m + __logf(denom) : -INFINITY;
+}
+
+static hipError_t segment_workspace(size_t bytes, hipStream_t stream, char** out) {
+    struct Buf {
+        void* ptr = nullptr;
+        size_t size = 0;
+    };
+    static std::mutex mu;
+    static std::map<std::pair<int, hipStream_t>, Buf> bufs;
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    std::lock_guard<std::mutex> lock(mu);
+    Buf& b = bufs[std::make_pair(dev, stream)];
+    if (b.size < bytes) {
+        hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+        e = hipStreamIsCapturing(stream, &cap);
+        if (e != hipSuccess) return e;
+        if (cap != hipStreamCaptureStatusNone) return hipErrorStreamCaptureUnsupported;
+        const size_t want = bytes < (size_t(8) << 20) ? (size_t(8) << 20) : bytes + bytes / 2;
+        void* fresh = nullptr;
+        e = hipMalloc(&fresh, want);
+        if (e != hipSuccess) return e;
+        b.ptr = fresh;   // the previous buffer, if any, stays allocated (see above)
+        b.size = want;
+    }
+    *out = static_cast<char*>(b.ptr);
+    return hipSuccess;
+}
+
+// Number of key ranges, or 0 where the keys are not cut: at most 128 work items of 128 queries; about one item per CU, at
+// least 1024 keys per range (2048 where only two ranges fit), at most 8 ranges. Measured, 32/8 heads, causal, without /
+// with ranges (us): 64 queries over 8192 keys 90 / 29, 128 over 8192 92 / 33, 256 over 8192 92 / 46, 512 over 8192
+// 93 / 79, 128 over 32768 343 / 80, 512 over 32768 350 / 273, 2 x 128 over 4096 50 / 31, 4 x 128 over 8192 94 / 81; two
+// ranges of 1024 keys lose (512 over 2048: 29 / 33).
+static int key_segments(int B, int Hq, int Sq, int kv_valid) {
+    const long items = (long)((Sq + 127) / 128) * Hq * B;
+    if (items > 128 || kv_valid < 2048) return 0;
+    long s = 256 / items;
+    if (s > 8) s = 8;
+    if (s > kv_valid / 1024) s = kv_valid / 1024;
+    if (s == 2 && kv_valid < 4096) return 0;
+    return s >= 2 ? (int)s : 0;
+}
+
+template <typename T>
+static hipError_t launch_fmha_segmented(const T* Q, const T* K, const T* V, T* O, float* LSE, int B, int Hq, int Hkv, int Sq,
+                                        int Sk, float scale, int causal, int kv_valid, const FmhaStrides& sd, int segments,
+                                        hipStream_t stream) {
+    constexpr int LDS = 8 * fmha::TILE_BYTES;
+    auto kern = fmha_fwd_pingpong_kernel<T, 1, true>;
+    static DynamicLdsOnce lds_once;
+    if (hipError_t e = lds_once.ensure(reinterpret_cast<const void*>(kern), LDS); e != hipSuccess) return e;
+    const int seg_len = ((kv_valid + segments - 1) / segments + 63) & ~63;
+    const long rows = (long)B * Hq * Sq;
+    const size_t o_bytes = (size_t)segments * rows * fmha::D * sizeof(T);
+    const size_t bytes = o_bytes + (size_t)segments * rows * sizeof(float);
+    char* ws = nullptr;
+    if (hipError_t e = segment_workspace(bytes, stream, &ws); e != hipSuccess) return e;
+    T* o_part = reinterpret_cast<T*>(ws);
+    float* lse_part = reinterpret_cast<float*>(ws + o_bytes);
+    const int q_tiles = (Sq + 127) / 128;
+    const long items = (long)q_tiles * Hq * B * segments;
+    int cus = 0;
+    if (hipError_t e = compute_units(cus); e != hipSuccess) return e;
+    long blocks = items < cus ? items : cus;
+    if (((long)Hkv * B * segments) % 8 == 0 && blocks >= 8) blocks &= ~7L;
+    const float scale_log2 = scale * 1.4426950408889634f;
+    kern<<<dim3((unsigned)blocks), dim3(512), LDS, stream>>>(Q, K, V, o_part, lse_part, B, Hq, Hkv, Sq, Sk, scale_log2, causal, kv_valid,
+                                                             q_tiles, sd, segments, seg_len);
+    if (hipError_t e = hipGetLastError(); e != hipSuccess) return e;
+    fmha_merge_segments_kernel<T><<<dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, stream>>>(o_part, lse_part, O, LSE, B, Hq, Sq, segments, sd);
     return hipGetLastError();
 }
 
@@ -663,6 +802,15 @@ static hipError_t fmha_fwd_dispatch_t(const void* Q, const void* K, const void* 
     if (sd.k_row >= (1L << 24) || sd.v_row >= (1L << 24)) return hipErrorNotSupported;
     if (variant == 0 && fmha_decode_applicable(B, Hq, Hkv, Sq, Sk, kv_valid_len))
         return fmha_decode_dispatch<T>(q, k, v, o, LSE, B, Hq, Hkv, Sq, Sk, scale, causal, kv_valid_len, sd, ws, stream);
+    if ((variant == 0 || variant == 3) && ws.kind == FmhaWorkspace::kLibrary && !fmha_decode_applicable(B, Hq, Hkv, Sq, Sk, kv_valid_len)) {
+        if (const int segments = key_segments(B, Hq, Sq, kv_valid_len); segments > 0) {
+            const hipError_t e = launch_fmha_segmented<T>(q, k, v, o, LSE, B, Hq, Hkv, Sq, Sk, scale, causal, kv_valid_len, sd, segments, stream);
+            // without the workspace (none yet on a stream that is being captured, or no memory) the keys are walked in one go
+            if (variant == 3 || (e != hipErrorStreamCaptureUnsupported && e != hipErrorOutOfMemory)) return e;
+            (void)hipGetLastError();
+        }
+    }
+    if (variant == 3) return hipErrorInvalidConfiguration;   // the test hook asked for key ranges where they do not apply
     if (variant == 0) {
         // 256-query workgroups (every K / V fragment feeds two MFMAs) once their work items fill the machine: clearly more
         // of them than CUs for a causal problem (with about one per CU it runs as long as its heaviest item, and 128-query
@@ -675,8 +823,12 @@ static hipError_t fmha_fwd_dispatch_t(const void* Q, const void* K, const void* 
         // as two of them, on a quarter of the machine at the end; twice as many 128-query items are three to a CU then,
         // each a little more than half as long (1 x H/1 x 2048 with H = 33 .. 44, i.e. 264 .. 352 items: 94.5 - 97.6 us
         // against 99.9; 368 items 99.6 / 100.0; 384 items 102.6 / 100.1).
+        // (A causal problem whose queries are the last of at least twice as many keys - a chunk of new tokens against a
+        // cache - has items of nearly equal length, like a problem that is not causal: 1 x 32/8 x 2048 queries over 8192
+        // keys 223 / 200.)
         const long wg256 = (long)((Sq + 255) / 256) * Hq * B;
-        variant = (Sq >= 256 && wg256 >= (causal ? 320 : 256)) ? 2 : 1;
+        const bool uneven = causal && Sk < 2 * (long)Sq;
+        variant = (Sq >= 256 && wg256 >= (uneven ? 320 : 256)) ? 2 : 1;
         if (!causal && wg256 > 256 && wg256 <= 352) variant = 1;
     }
     if (variant == 2) return launch_fmha_pingpong<T, 2>(q, k, v, o, LSE, B, Hq, Hkv, Sq, Sk, scale, causal, kv_valid_len, sd, stream);

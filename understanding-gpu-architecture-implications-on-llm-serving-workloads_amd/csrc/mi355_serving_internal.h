@@ -85,7 +85,7 @@ hipError_t silu_mul_dispatch(const void* in, void* out, long rows, int inter, in
 //         stages, 5 = 128x256, 6 = 256x128, 7 = 32x64 (layouts NN and NT): the tiled kernel of that shape for any product the tiled kernels take (M and N need not be multiples
 //         of the tile); products of up to 64 rows that the small-M kernels take stay on those
 //   fmha: 0 = by shape, 1 = 128-query workgroups, 2 = 256-query workgroups (1 and 2 also keep generation-step shapes off
-//         the split-KV path)
+//         the split-KV path), 3 = keys cut into ranges and merged (an error where the choice by shape would not do that)
 extern "C" {
 int mi355_internal_hgemm_variant(const void* A, const void* B, void* C, int M, int N, int K, int64_t lda, int64_t ldb,
                                  int64_t ldc, int layout, int dtype, int variant, void* stream);
