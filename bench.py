@@ -427,6 +427,17 @@ def main():
                                                                "kv_copies": len(kv_sets)}
             del kv_sets
         del xd, wd_nt, od, qd, kd, vd, o_d
+        # a chunk of new tokens against a cache (causal, 32/8 heads): keys cut into ranges and merged, beside the same kernel
+        # walking all keys at once (the library's variant hook)
+        for sqc, skc in ((128, 8192), (512, 8192), (128, 32768)):
+            qc, kc, vc = (t.to(dev) for t in so.fmha_inputs(1, 32, 8, sqc, skc, seed=9))
+            o_c = torch.empty_like(qc)
+            ms_r = time_launches(lambda: lib.fmha_fwd(qc, kc, vc, causal=True, return_lse=False, out=o_c), 20, 3)
+            ms_w = time_launches(lambda: lib.fmha_fwd(qc, kc, vc, causal=True, return_lse=False, out=o_c, variant=1), 20, 3)
+            fl_c = 4.0 * 32 * 128 * causal_pairs(sqc, skc)
+            other["fmha_chunk_q%d_over_%d_causal_gqa" % (sqc, skc)] = {"ms": ms_r, "tflops": fl_c / ms_r / 1e9,
+                                                                       "ms_one_walk_over_all_keys": ms_w}
+        del qc, kc, vc, o_c
         # L5: Llama-3-8B-shaped prefill layer at s = 8192, per stage; every stage is checked on sampled token rows against
         # the oracle fed the GPU's own previous-stage output, and the chain's end against the pure fp32 chain
         S5, H5, F5 = 8192, 4096, 14336
@@ -660,6 +671,8 @@ KERNEL_CONFIGS = {
     "f4_fmha_causal_gqa_s4096": ("fmha", 1, 32, 8, 4096, 4096, True),           # ping-pong kernel
     "l5_fmha_causal_gqa_s8192": ("fmha", 1, 32, 8, 8192, 8192, True),           # ping-pong kernel
     "fmha_causal_gqa_s1024": ("fmha", 1, 32, 8, 1024, 1024, True),              # ping-pong kernel, 128-query work items (128 items of 256 queries would not fill the CUs)
+    "fmha_chunk_q128_over_8192": ("fmha", 1, 32, 8, 128, 8192, True),           # key ranges + merge kernel
+    "fmha_chunk_q512_over_32768": ("fmha", 1, 32, 8, 512, 32768, True),
     "fmha_decode_b1_sk8192": ("fmha", 1, 32, 8, 1, 8192, False),                # split-KV kernel
     "fmha_decode_b8_sk8192": ("fmha", 8, 32, 8, 1, 8192, False),
     "fmha_decode_b64_sk8192": ("fmha", 64, 32, 8, 1, 8192, False),              # one key range per (batch, kv head)

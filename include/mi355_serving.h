@@ -7,7 +7,7 @@
  *
  * Conventions
  *   - every pointer is a DEVICE pointer owned by the caller; none is retained. The only memory the library ever
- *     allocates are two kinds of workspace. One holds the partial results of the split-KV attention path (taken when
+ *     allocates are three kinds of workspace. One holds the partial results of the split-KV attention path (taken when
  *     Hq/Hkv * Sq <= 32 and kv_valid_len >= 512, i.e. generation steps): one buffer per (device, stream), obtained
  *     with hipMalloc at first use (>= 4 MiB; when a later call needs more, a larger buffer is allocated and the old
  *     one is kept, because a HIP graph captured earlier may still hold its address; nothing is freed before the
@@ -21,7 +21,11 @@
  *     The GEMM entry points keep a second buffer of the same kind per (device, stream) for the partial tiles of their
  *     split-K path (17 .. 256 rows against a second operand of up to 8192 columns, K a multiple of 256; >= 8 MiB); a
  *     GEMM call that cannot get it (its stream is being captured and has none yet, or hipMalloc fails) does not fail: it
- *     runs the kernels without split-K, so a captured call is faster when the step ran once on that stream before;
+ *     runs the kernels without split-K, so a captured call is faster when the step ran once on that stream before.
+ *     The attention entry points other than mi355_fmha_fwd_ws and mi355_fmha_fwd_noalloc keep a third buffer of that kind
+ *     for a chunk of queries against a long cache (at most 128 work items of 128 queries, kv_valid_len >= 2048: the keys
+ *     are cut into up to 8 ranges and a second kernel merges the partial outputs, which take ranges * B * Hq * Sq * 260
+ *     bytes; >= 8 MiB); a call that cannot get it walks all keys in one kernel instead of failing, like the GEMM;
  *   - `stream` is a hipStream_t passed as void* (NULL = the null stream); calls are asynchronous;
  *   - fp16 data is IEEE binary16 (`_Float16` / `__half` / torch.float16);
  *   - return value 0 = launched; non-zero = a hipError_t value or MI355_ERR_* below, nothing was launched.

@@ -685,6 +685,8 @@ static hipError_t launch_fmha_pingpong(const T* Q, const T* K, const T* V, T* O,
 // and replaced by a larger one when a call needs more (never freed: a captured graph may hold its address). A call that
 // cannot get it (its stream is being captured and has none yet) runs the kernel without ranges instead.
 // ---------------------------------------------------------------------------------------------------------------
+constexpr int kMaxSegments = 8;
+
 template <typename T>
 __global__ __launch_bounds__(256) void fmha_merge_segments_kernel(const T* __restrict__ Opart, const float* __restrict__ LSEpart,
                                                                   T* __restrict__ O, float* __restrict__ LSE, int B, int Hq, int Sq,
@@ -697,15 +699,26 @@ __global__ __launch_bounds__(256) void fmha_merge_segments_kernel(const T* __res
     const int q = (int)(row % Sq);
     const long bh = row / Sq;
     const int h = (int)(bh % Hq), b = (int)(bh / Hq);
+    // at most kMaxSegments ranges: every load of the row is issued before the first use
+    float ls[kMaxSegments];
+    V2 vs[kMaxSegments];
+#pragma unroll
+    for (int s = 0; s < kMaxSegments; ++s) {
+        const int sc = s < segments ? s : 0;
+        ls[s] = LSEpart[(long)sc * rows + row];
+        vs[s] = *(const V2*)(Opart + ((long)sc * rows + row) * fmha::D + 2 * lane);
+        if (s >= segments) ls[s] = -INFINITY;
+    }
     float m = -INFINITY;
-    for (int s = 0; s < segments; ++s) m = fmaxf(m, LSEpart[(long)s * rows + row]);
+#pragma unroll
+    for (int s = 0; s < kMaxSegments; ++s) m = fmaxf(m, ls[s]);
     float acc0 = 0.f, acc1 = 0.f, denom = 0.f;
     if (m > -INFINITY) {
-        for (int s = 0; s < segments; ++s) {
-            const float w = __expf(LSEpart[(long)s * rows + row] - m);   // exp(-inf) = 0
-            const V2 v = *(const V2*)(Opart + ((long)s * rows + row) * fmha::D + 2 * lane);
-            acc0 += w * (float)v[0];
-            acc1 += w * (float)v[1];
+#pragma unroll
+        for (int s = 0; s < kMaxSegments; ++s) {
+            const float w = __expf(ls[s] - m);   // exp(-inf) = 0: a range without a visible key, or beyond `segments`
+            acc0 += w * (float)vs[s][0];
+            acc1 += w * (float)vs[s][1];
             denom += w;
         }
     }
@@ -754,7 +767,7 @@ static int key_segments(int B, int Hq, int Sq, int kv_valid) {
     const long items = (long)((Sq + 127) / 128) * Hq * B;
     if (items > 128 || kv_valid < 2048) return 0;
     long s = 256 / items;
-    if (s > 8) s = 8;
+    if (s > kMaxSegments) s = kMaxSegments;
     if (s > kv_valid / 1024) s = kv_valid / 1024;
     if (s == 2 && kv_valid < 4096) return 0;
     return s >= 2 ? (int)s : 0;
