@@ -22,7 +22,8 @@
  *     split-K path (17 .. 256 rows against a second operand of up to 8192 columns, K a multiple of 256; >= 8 MiB); a
  *     GEMM call that cannot get it (its stream is being captured and has none yet, or hipMalloc fails) does not fail: it
  *     runs the kernels without split-K, so a captured call is faster when the step ran once on that stream before.
- *     The attention entry points other than mi355_fmha_fwd_ws and mi355_fmha_fwd_noalloc keep a third buffer of that kind
+ *     The attention entry points other than mi355_fmha_fwd_ws (which takes the caller's) and mi355_fmha_fwd_noalloc
+ *     (which walks all keys in one kernel) keep a third buffer of that kind
  *     for a chunk of queries against a long cache (at most 128 work items of 128 queries, kv_valid_len >= 2048: the keys
  *     are cut into up to 8 ranges and a second kernel merges the partial outputs, which take ranges * B * Hq * Sq * 260
  *     bytes; >= 8 MiB); a call that cannot get it walks all keys in one kernel instead of failing, like the GEMM;
@@ -236,8 +237,11 @@ int mi355_silu_mul_bf16(const void* gate_up, void* out, int64_t rows, int inter,
 /*
  * The attention forward with a workspace owned by the caller, for callers that manage all device memory themselves
  * (HIP graph capture, arena allocators). mi355_fmha_fwd_workspace_bytes returns how many bytes a call with these sizes
- * needs: 0 for every shape outside the split-KV path and when B * Hkv is large enough for one key range per (batch, kv
- * head) (then `workspace` may be NULL), otherwise 64 KiB of ticket counters plus the size of its partial results (at most ~9 MiB). mi355_fmha_fwd_ws is mi355_fmha_fwd_strided (strides == NULL:
+ * needs: on the split-KV path 64 KiB of ticket counters plus the size of its partial results (at most ~9 MiB; 0 when
+ * B * Hkv is large enough for one key range per (batch, kv head)); for a chunk of queries against a long cache (see the
+ * conventions above) ranges * B * Hq * Sq * 260 bytes, which the call uses if `workspace_bytes` covers them and otherwise
+ * does without (it then walks all keys in one kernel; a split-KV call with too small a workspace fails); 0 for every
+ * other shape (then `workspace` may be NULL). mi355_fmha_fwd_ws is mi355_fmha_fwd_strided (strides == NULL:
  * contiguous [B, H, S, D] operands) for dtype MI355_DTYPE_FP16 or MI355_DTYPE_BF16 that keeps those partial results in
  * `workspace` (16-byte aligned, at least that many bytes, contents irrelevant before and after the call: a small kernel
  * clears the part that must start at zero) and never allocates. Calls that share a workspace must be ordered on one stream. No counterpart in the reference, whose

@@ -333,6 +333,41 @@ def test_caller_owned_workspace_entry_point(lib, gpu, dtype):
     assert torch.equal(o, lib.fmha_fwd(q, k, v, causal=True)[0])
 
 
+def test_caller_owned_workspace_serves_key_ranges_also_under_capture(lib, gpu):
+    # a chunk against a long cache: the size query reports the partial outputs of the key ranges; with that much memory of
+    # the caller's the call takes the ranges (bit-identical to the library-owned path) and never allocates, so it can be
+    # captured on a stream the library has never seen; with less it walks all keys in one kernel instead of failing
+    import ctypes
+    B, Hq, Hkv, Sq, Sk = 1, 32, 8, 128, 8192
+    q, k, v = (t.to(gpu) for t in so.fmha_inputs(B, Hq, Hkv, Sq, Sk, seed=8))
+    need = lib.fmha_workspace_bytes(B, Hq, Hkv, Sq, Sk)
+    assert need == 8 * B * Hq * Sq * (128 * 2 + 4)
+    assert lib.fmha_workspace_bytes(1, 32, 8, 1024, 8192) == 0 and lib.fmha_workspace_bytes(1, 32, 8, 128, 1024) == 0
+    ranges, lse_r = lib.fmha_fwd(q, k, v, causal=True)
+    whole, lse_w = lib.fmha_fwd(q, k, v, causal=True, variant=1)
+    ws = torch.full((need,), 0xFF, dtype=torch.uint8, device=gpu)
+    o, lse = lib.fmha_fwd(q, k, v, causal=True, workspace=ws)
+    assert torch.equal(o, ranges) and torch.equal(lse, lse_r)
+    o, lse = lib.fmha_fwd(q, k, v, causal=True, workspace=ws[:need - 16])
+    assert torch.equal(o, whole) and torch.equal(lse, lse_w)
+    hip = ctypes.CDLL("libamdhip64.so")
+    raw = ctypes.c_void_p()
+    assert hip.hipStreamCreate(ctypes.byref(raw)) == 0
+    fresh = torch.cuda.ExternalStream(raw.value)
+    out_g = torch.zeros_like(q)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=fresh):
+        lib.fmha_fwd(q, k, v, causal=True, return_lse=False, out=out_g, workspace=ws)
+    for _ in range(2):
+        out_g.zero_()
+        ws.fill_(0x7F)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out_g, ranges)
+    del graph
+
+
 # ---- operands read in place from other layouts ------------------------------------------------------------------------
 @pytest.mark.parametrize("B,Hq,Hkv,Sq,Sk,causal", [
     (2, 8, 2, 300, 300, True),      # prefill, 128-query workgroups

@@ -167,7 +167,7 @@ int mi355_fmha_fwd_bf16(const void* Q, const void* K, const void* V, void* O, fl
 
 size_t mi355_fmha_fwd_workspace_bytes(int B, int Hq, int Hkv, int Sq, int Sk, int kv_valid_len) {
     if (B < 1 || Hq < 1 || Hkv < 1 || Sq < 1 || Sk < 1 || Hq % Hkv != 0 || kv_valid_len < 1 || kv_valid_len > Sk) return 0;
-    return mi355::fmha_decode_workspace_bytes(B, Hq, Hkv, Sq, Sk, kv_valid_len);
+    return mi355::fmha_workspace_bytes(B, Hq, Hkv, Sq, Sk, kv_valid_len);
 }
 
 int mi355_fmha_fwd_ws(const void* Q, const void* K, const void* V, void* O, float* LSE, int B, int Hq, int Hkv, int Sq,

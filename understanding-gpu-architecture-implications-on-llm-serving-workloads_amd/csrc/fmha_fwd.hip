@@ -773,10 +773,21 @@ static int key_segments(int B, int Hq, int Sq, int kv_valid) {
     return s >= 2 ? (int)s : 0;
 }
 
+size_t fmha_key_range_workspace_bytes(int B, int Hq, int Hkv, int Sq, int Sk, int kv_valid_len) {
+    if (fmha_decode_applicable(B, Hq, Hkv, Sq, Sk, kv_valid_len)) return 0;
+    const int segments = key_segments(B, Hq, Sq, kv_valid_len);
+    return (size_t)segments * B * Hq * Sq * (fmha::D * 2 + sizeof(float));   // fp16 / bf16 partial outputs, fp32 LSE
+}
+
+size_t fmha_workspace_bytes(int B, int Hq, int Hkv, int Sq, int Sk, int kv_valid_len) {
+    const size_t decode = fmha_decode_workspace_bytes(B, Hq, Hkv, Sq, Sk, kv_valid_len);
+    return decode > 0 ? decode : fmha_key_range_workspace_bytes(B, Hq, Hkv, Sq, Sk, kv_valid_len);
+}
+
 template <typename T>
 static hipError_t launch_fmha_segmented(const T* Q, const T* K, const T* V, T* O, float* LSE, int B, int Hq, int Hkv, int Sq,
                                         int Sk, float scale, int causal, int kv_valid, const FmhaStrides& sd, int segments,
-                                        hipStream_t stream) {
+                                        char* caller_ws, hipStream_t stream) {
     constexpr int LDS = 8 * fmha::TILE_BYTES;
     auto kern = fmha_fwd_pingpong_kernel<T, 1, true>;
     static DynamicLdsOnce lds_once;
@@ -785,8 +796,9 @@ static hipError_t launch_fmha_segmented(const T* Q, const T* K, const T* V, T* O
     const long rows = (long)B * Hq * Sq;
     const size_t o_bytes = (size_t)segments * rows * fmha::D * sizeof(T);
     const size_t bytes = o_bytes + (size_t)segments * rows * sizeof(float);
-    char* ws = nullptr;
-    if (hipError_t e = segment_workspace(bytes, stream, &ws); e != hipSuccess) return e;
+    char* ws = caller_ws;   // memory of the caller (large enough: see fmha_fwd_dispatch), or the library's own
+    if (ws == nullptr)
+        if (hipError_t e = segment_workspace(bytes, stream, &ws); e != hipSuccess) return e;
     T* o_part = reinterpret_cast<T*>(ws);
     float* lse_part = reinterpret_cast<float*>(ws + o_bytes);
     const int q_tiles = (Sq + 127) / 128;
@@ -815,9 +827,13 @@ static hipError_t fmha_fwd_dispatch_t(const void* Q, const void* K, const void* 
     if (sd.k_row >= (1L << 24) || sd.v_row >= (1L << 24)) return hipErrorNotSupported;
     if (variant == 0 && fmha_decode_applicable(B, Hq, Hkv, Sq, Sk, kv_valid_len))
         return fmha_decode_dispatch<T>(q, k, v, o, LSE, B, Hq, Hkv, Sq, Sk, scale, causal, kv_valid_len, sd, ws, stream);
-    if ((variant == 0 || variant == 3) && ws.kind == FmhaWorkspace::kLibrary && !fmha_decode_applicable(B, Hq, Hkv, Sq, Sk, kv_valid_len)) {
+    const size_t range_bytes = (variant == 0 || variant == 3) ? fmha_key_range_workspace_bytes(B, Hq, Hkv, Sq, Sk, kv_valid_len) : 0;
+    const bool caller_ws = ws.kind == FmhaWorkspace::kCaller && ws.ptr != nullptr && ws.bytes >= range_bytes &&
+                           reinterpret_cast<uintptr_t>(ws.ptr) % 16 == 0;
+    if (range_bytes > 0 && (ws.kind == FmhaWorkspace::kLibrary || caller_ws)) {
         if (const int segments = key_segments(B, Hq, Sq, kv_valid_len); segments > 0) {
-            const hipError_t e = launch_fmha_segmented<T>(q, k, v, o, LSE, B, Hq, Hkv, Sq, Sk, scale, causal, kv_valid_len, sd, segments, stream);
+            const hipError_t e = launch_fmha_segmented<T>(q, k, v, o, LSE, B, Hq, Hkv, Sq, Sk, scale, causal, kv_valid_len, sd, segments,
+                                                          caller_ws ? static_cast<char*>(ws.ptr) : nullptr, stream);
             // without the workspace (none yet on a stream that is being captured, or no memory) the keys are walked in one go
             if (variant == 3 || (e != hipErrorStreamCaptureUnsupported && e != hipErrorOutOfMemory)) return e;
             (void)hipGetLastError();

@@ -41,7 +41,7 @@ struct FmhaStrides {
 hipError_t hgemm_silu_mul_dispatch(const void* A, const void* B, void* C, int M, int N2, int K, long lda, long ldb, long ldc,
                                    int layout, int dtype, hipStream_t stream);
 
-// Where the split-KV attention path keeps its partial results.
+// Where the split-KV and key-range attention paths keep their partial results.
 struct FmhaWorkspace {
     enum Kind { kLibrary, kCaller, kStatic };
     Kind kind = kLibrary;     // kLibrary: the library's own grow-only buffer of (device, stream)
@@ -59,6 +59,10 @@ hipError_t fmha_fwd_dispatch(const void* Q, const void* K, const void* V, void* 
 bool fmha_decode_applicable(int B, int Hq, int Hkv, int Sq, int Sk, int kv_valid_len);
 // Bytes of workspace a call with these sizes uses (0 when it does not take the split-KV path).
 size_t fmha_decode_workspace_bytes(int B, int Hq, int Hkv, int Sq, int Sk, int kv_valid_len);
+// Bytes of workspace the key-range path of fmha_fwd.hip uses for a call with these sizes (0 when it does not take it), and
+// the bytes a call uses on whichever of the two paths it takes.
+size_t fmha_key_range_workspace_bytes(int B, int Hq, int Hkv, int Sq, int Sk, int kv_valid_len);
+size_t fmha_workspace_bytes(int B, int Hq, int Hkv, int Sq, int Sk, int kv_valid_len);
 // Size of the static scratch array behind FmhaWorkspace::kStatic.
 size_t fmha_decode_static_scratch_bytes();
 template <typename T>
