@@ -24,7 +24,7 @@
  *     runs the kernels without split-K, so a captured call is faster when the step ran once on that stream before.
  *     The attention entry points other than mi355_fmha_fwd_ws (which takes the caller's) and mi355_fmha_fwd_noalloc
  *     (which walks all keys in one kernel) keep a third buffer of that kind
- *     for a chunk of queries against a long cache (at most 128 work items of 128 queries, kv_valid_len >= 2048: the keys
+ *     for a chunk of queries against a long cache (at most 128 work items of 128 or 256 queries, kv_valid_len >= 2048: the keys
  *     are cut into up to 8 ranges and a second kernel merges the partial outputs, which take ranges * B * Hq * Sq * 260
  *     bytes; >= 8 MiB); a call that cannot get it walks all keys in one kernel instead of failing, like the GEMM;
  *   - `stream` is a hipStream_t passed as void* (NULL = the null stream); calls are asynchronous;

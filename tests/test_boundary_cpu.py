@@ -79,7 +79,7 @@ def test_capi_rejects_bad_arguments_without_a_gpu(lib):
     need = wsb(1, 32, 8, 1, 8192, 8192)
     assert 0 < need <= 16 << 20 and need % 16 == 0
     assert wsb(8, 32, 8, 1, 8192, 8192) > 0 and wsb(1, 32, 8, 1, 8192, 9000) == 0         # invalid sizes report 0
-    assert wsb(1, 32, 8, 128, 8192, 8192) == 8 * 32 * 128 * 260 and wsb(1, 32, 8, 512, 8192, 8192) == 2 * 32 * 512 * 260   # key ranges
+    assert wsb(1, 32, 8, 128, 8192, 8192) == 8 * 32 * 128 * 260 and wsb(1, 32, 8, 512, 8192, 8192) == 4 * 32 * 512 * 260   # key ranges
     assert wsb(1, 32, 8, 512, 2048, 2048) == 0 and wsb(1, 32, 8, 128, 8192, 2047) == 0
     ws_call = lambda ptr, nbytes, dtype=0: cdll.mi355_fmha_fwd_ws(p, p, p, p, None, 1, 32, 8, 1, 8192, 128, 0.1, 0, 8192, None,
                                                                   dtype, ptr, nbytes, None)

@@ -342,7 +342,8 @@ def test_caller_owned_workspace_serves_key_ranges_also_under_capture(lib, gpu):
     q, k, v = (t.to(gpu) for t in so.fmha_inputs(B, Hq, Hkv, Sq, Sk, seed=8))
     need = lib.fmha_workspace_bytes(B, Hq, Hkv, Sq, Sk)
     assert need == 8 * B * Hq * Sq * (128 * 2 + 4)
-    assert lib.fmha_workspace_bytes(1, 32, 8, 1024, 8192) == 0 and lib.fmha_workspace_bytes(1, 32, 8, 128, 1024) == 0
+    assert lib.fmha_workspace_bytes(1, 32, 8, 2048, 8192) == 0 and lib.fmha_workspace_bytes(1, 32, 8, 128, 1024) == 0
+    assert lib.fmha_workspace_bytes(1, 32, 8, 512, 8192) == 4 * 32 * 512 * (128 * 2 + 4)      # 256-query items, 4 ranges
     ranges, lse_r = lib.fmha_fwd(q, k, v, causal=True)
     whole, lse_w = lib.fmha_fwd(q, k, v, causal=True, variant=1)
     ws = torch.full((need,), 0xFF, dtype=torch.uint8, device=gpu)
@@ -523,6 +524,10 @@ def test_torch_operator_reads_transposed_views_in_place(gpu):
     (3, 4, 1, 100, 4096, True, None),
     (1, 4, 4, 4096, 4096, True, None),     # causal square: the second range is invisible to the early q tiles
     (1, 8, 1, 5, 12000, True, 11000),      # 40 query rows per kv head: more than the generation-step kernels take
+    (1, 32, 8, 512, 8192, True, None),     # 256-query items over 4 ranges
+    (1, 32, 8, 1024, 4500, False, 4200),   # 256-query items over 2 ranges of 2112 keys
+    (1, 64, 8, 480, 9000, True, 8200),     # 256-query items, second q tile ragged
+    (2, 16, 4, 256, 6200, True, 6150),     # too few 256-query items for the machine: 128-query items over 4 ranges
 ])
 def test_chunk_against_long_cache_key_ranges(lib, gpu, B, Hq, Hkv, Sq, Sk, causal, kvv):
     q, k, v = so.fmha_inputs(B, Hq, Hkv, Sq, Sk, seed=Sq + Sk + Hq)
@@ -541,7 +546,7 @@ def test_chunk_against_long_cache_key_ranges(lib, gpu, B, Hq, Hkv, Sq, Sk, causa
 
 def test_key_ranges_only_where_they_pay(lib, gpu):
     # enough work items for the machine, a short cache, or a generation step: no ranges (variant 3 reports it)
-    for B, Hq, Hkv, Sq, Sk in ((1, 32, 8, 1024, 8192), (1, 32, 8, 128, 1024), (1, 32, 8, 512, 2048)):
+    for B, Hq, Hkv, Sq, Sk in ((1, 32, 8, 2048, 8192), (1, 32, 8, 128, 1024), (1, 32, 8, 512, 2048)):
         q, k, v = (t.to(gpu) for t in so.fmha_inputs(B, Hq, Hkv, Sq, Sk, seed=3))
         with pytest.raises(lib.Mi355Error):
             lib.fmha_fwd(q, k, v, causal=True, variant=3)
@@ -553,6 +558,10 @@ def test_key_ranges_bfloat16_and_transposed_views(lib, gpu):
     qb, kb, vb = q.float().bfloat16(), k.float().bfloat16(), v.float().bfloat16()
     o, lse = lib.fmha_fwd(qb.to(gpu), kb.to(gpu), vb.to(gpu), causal=True, kv_valid_len=5555)
     o_ref, lse_ref = so.attention_ref(qb, kb, vb, causal=True, kv_valid_len=5555)
+    assert (o.float().cpu() - o_ref).abs().max() <= 1.6e-2 and (lse.cpu() - lse_ref).abs().max() <= 1e-3
+    q2, k2, v2 = (t.float().bfloat16() for t in so.fmha_inputs(1, 32, 8, 512, 8192, seed=78))      # 256-query items
+    o, lse = lib.fmha_fwd(q2.to(gpu), k2.to(gpu), v2.to(gpu), causal=True)
+    o_ref, lse_ref = so.attention_ref(q2, k2, v2, causal=True)
     assert (o.float().cpu() - o_ref).abs().max() <= 1.6e-2 and (lse.cpu() - lse_ref).abs().max() <= 1e-3
     # [B, S, H, D] storage viewed as [B, H, S, D]: inputs and output
     qt = q.transpose(1, 2).contiguous().to(gpu).transpose(1, 2)

@@ -758,25 +758,49 @@ static hipError_t segment_workspace(size_t bytes, hipStream_t stream, char** out
     return hipSuccess;
 }
 
-// Number of key ranges, or 0 where the keys are not cut: at most 128 work items of 128 queries; about one item per CU, at
-// least 1024 keys per range (2048 where only two ranges fit), at most 8 ranges. Measured, 32/8 heads, causal, without /
-// with ranges (us): 64 queries over 8192 keys 90 / 29, 128 over 8192 92 / 33, 256 over 8192 92 / 46, 512 over 8192
-// 93 / 79, 128 over 32768 343 / 80, 512 over 32768 350 / 273, 2 x 128 over 4096 50 / 31, 4 x 128 over 8192 94 / 81; two
+// How a call cuts its keys: `segments` ranges (0: not cut) walked by work items of 128 `qb` queries.
+// 128-query items: at most 128 of them; about one item per CU, at least 1024 keys per range (2048 where only two ranges
+// fit), at most 8 ranges. Measured, 32/8 heads, causal, one walk / ranges (us): 64 queries over 8192 keys 90 / 25, 128 over
+// 8192 92 / 28, 256 over 8192 92 / 44, 128 over 32768 343 / 75, 2 x 128 over 4096 50 / 29, 4 x 128 over 8192 94 / 79; two
 // ranges of 1024 keys lose (512 over 2048: 29 / 33).
-static int key_segments(int B, int Hq, int Sq, int kv_valid) {
+// 256-query items (every K / V fragment feeds two MFMAs) where they fill the machine with ranges of at least 2048 keys: at
+// most 128 items, at least 192 (item, range) pairs, at most an eighth of the q tiles empty. Measured, 128- / 256-query
+// items over ranges (us): 512 over 8192 81 / 69, 768 over 8192 105 (one walk) / 102, 1024 over 8192 127 (one walk) / 124,
+// 256 over 32768 138 / 120, 512 over 32768 262 / 220, 1024 over 32768 493 (one walk) / 423, 2 x 256 over 8192 78 / 71,
+// 64/8 heads 256 over 16384 139 / 120; but 256 over 8192 (8 ranges of 1024 keys) 44 / 45, 384 over 8192 65 / 67.
+struct KeyRangePlan {
+    int segments = 0;
+    int qb = 1;
+};
+
+static KeyRangePlan key_range_plan(int B, int Hq, int Sq, int kv_valid) {
+    KeyRangePlan plan;
+    if (kv_valid < 2048) return plan;
+    const long q256 = (Sq + 255) / 256, items256 = q256 * Hq * B;
+    if (Sq >= 256 && q256 * 256 - Sq <= Sq / 8 && items256 <= 128) {
+        long s = 256 / items256;
+        if (s > kMaxSegments) s = kMaxSegments;
+        if (s > kv_valid / 2048) s = kv_valid / 2048;
+        if (s >= 2 && items256 * s >= 192) {
+            plan.segments = (int)s;
+            plan.qb = 2;
+            return plan;
+        }
+    }
     const long items = (long)((Sq + 127) / 128) * Hq * B;
-    if (items > 128 || kv_valid < 2048) return 0;
+    if (items > 128) return plan;
     long s = 256 / items;
     if (s > kMaxSegments) s = kMaxSegments;
     if (s > kv_valid / 1024) s = kv_valid / 1024;
-    if (s == 2 && kv_valid < 4096) return 0;
-    return s >= 2 ? (int)s : 0;
+    if (s == 2 && kv_valid < 4096) return plan;
+    if (s >= 2) plan.segments = (int)s;
+    return plan;
 }
 
 size_t fmha_key_range_workspace_bytes(int B, int Hq, int Hkv, int Sq, int Sk, int kv_valid_len) {
     if (fmha_decode_applicable(B, Hq, Hkv, Sq, Sk, kv_valid_len)) return 0;
-    const int segments = key_segments(B, Hq, Sq, kv_valid_len);
-    return (size_t)segments * B * Hq * Sq * (fmha::D * 2 + sizeof(float));   // fp16 / bf16 partial outputs, fp32 LSE
+    const KeyRangePlan plan = key_range_plan(B, Hq, Sq, kv_valid_len);
+    return (size_t)plan.segments * B * Hq * Sq * (fmha::D * 2 + sizeof(float));   // fp16 / bf16 partial outputs, fp32 LSE
 }
 
 size_t fmha_workspace_bytes(int B, int Hq, int Hkv, int Sq, int Sk, int kv_valid_len) {
@@ -784,12 +808,12 @@ size_t fmha_workspace_bytes(int B, int Hq, int Hkv, int Sq, int Sk, int kv_valid
     return decode > 0 ? decode : fmha_key_range_workspace_bytes(B, Hq, Hkv, Sq, Sk, kv_valid_len);
 }
 
-template <typename T>
+template <typename T, int QB>
 static hipError_t launch_fmha_segmented(const T* Q, const T* K, const T* V, T* O, float* LSE, int B, int Hq, int Hkv, int Sq,
                                         int Sk, float scale, int causal, int kv_valid, const FmhaStrides& sd, int segments,
                                         char* caller_ws, hipStream_t stream) {
     constexpr int LDS = 8 * fmha::TILE_BYTES;
-    auto kern = fmha_fwd_pingpong_kernel<T, 1, true>;
+    auto kern = fmha_fwd_pingpong_kernel<T, QB, true>;
     static DynamicLdsOnce lds_once;
     if (hipError_t e = lds_once.ensure(reinterpret_cast<const void*>(kern), LDS); e != hipSuccess) return e;
     const int seg_len = ((kv_valid + segments - 1) / segments + 63) & ~63;
@@ -801,7 +825,7 @@ static hipError_t launch_fmha_segmented(const T* Q, const T* K, const T* V, T* O
         if (hipError_t e = segment_workspace(bytes, stream, &ws); e != hipSuccess) return e;
     T* o_part = reinterpret_cast<T*>(ws);
     float* lse_part = reinterpret_cast<float*>(ws + o_bytes);
-    const int q_tiles = (Sq + 127) / 128;
+    const int q_tiles = (Sq + 128 * QB - 1) / (128 * QB);
     const long items = (long)q_tiles * Hq * B * segments;
     int cus = 0;
     if (hipError_t e = compute_units(cus); e != hipSuccess) return e;
@@ -831,13 +855,14 @@ static hipError_t fmha_fwd_dispatch_t(const void* Q, const void* K, const void* 
     const bool caller_ws = ws.kind == FmhaWorkspace::kCaller && ws.ptr != nullptr && ws.bytes >= range_bytes &&
                            reinterpret_cast<uintptr_t>(ws.ptr) % 16 == 0;
     if (range_bytes > 0 && (ws.kind == FmhaWorkspace::kLibrary || caller_ws)) {
-        if (const int segments = key_segments(B, Hq, Sq, kv_valid_len); segments > 0) {
-            const hipError_t e = launch_fmha_segmented<T>(q, k, v, o, LSE, B, Hq, Hkv, Sq, Sk, scale, causal, kv_valid_len, sd, segments,
-                                                          caller_ws ? static_cast<char*>(ws.ptr) : nullptr, stream);
-            // without the workspace (none yet on a stream that is being captured, or no memory) the keys are walked in one go
-            if (variant == 3 || (e != hipErrorStreamCaptureUnsupported && e != hipErrorOutOfMemory)) return e;
-            (void)hipGetLastError();
-        }
+        const KeyRangePlan plan = key_range_plan(B, Hq, Sq, kv_valid_len);
+        char* const mem = caller_ws ? static_cast<char*>(ws.ptr) : nullptr;
+        const hipError_t e =
+            plan.qb == 2 ? launch_fmha_segmented<T, 2>(q, k, v, o, LSE, B, Hq, Hkv, Sq, Sk, scale, causal, kv_valid_len, sd, plan.segments, mem, stream)
+                         : launch_fmha_segmented<T, 1>(q, k, v, o, LSE, B, Hq, Hkv, Sq, Sk, scale, causal, kv_valid_len, sd, plan.segments, mem, stream);
+        // without the workspace (none yet on a stream that is being captured, or no memory) the keys are walked in one go
+        if (variant == 3 || (e != hipErrorStreamCaptureUnsupported && e != hipErrorOutOfMemory)) return e;
+        (void)hipGetLastError();
     }
     if (variant == 3) return hipErrorInvalidConfiguration;   // the test hook asked for key ranges where they do not apply
     if (variant == 0) {
