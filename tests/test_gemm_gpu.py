@@ -191,7 +191,9 @@ def test_widths_that_are_no_multiple_of_8_and_unaligned_rows_of_c(lib, gpu, vari
 
 # ---- split-K: 17 .. 256 rows against a narrow second operand --------------------------------------------------------
 SPLIT_K_SHAPES = [(64, 4096, 14336), (17, 4096, 8192), (100, 2048, 4096), (128, 4096, 4096), (48, 1000, 2048), (33, 6144, 4096),
-                  (250, 1024, 8192), (40, 72, 16384), (160, 4096, 8192), (192, 4000, 14336)]
+                  (250, 1024, 8192), (40, 72, 16384), (160, 4096, 8192), (192, 4000, 14336),
+                  # 193 .. 512 rows, long K: ranges of K on 128x128 tiles (four ranges, two ranges, ragged M and N)
+                  (256, 4096, 14336), (384, 2048, 16384), (500, 4000, 12288), (300, 4096, 8192)]
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
@@ -219,8 +221,8 @@ def test_split_k_products(lib, gpu, dtype, layout, M, N, K):
         assert torch.equal(lib.hgemm(ag, bg, layout), first)
 
 
-def test_split_k_with_residual_in_place_and_unaligned_c(lib, gpu):
-    M, N, K = 72, 1001, 8192
+@pytest.mark.parametrize("M,N,K", [(72, 1001, 8192), (300, 1001, 12288)])      # 64x64 tiles, 128x128 tiles
+def test_split_k_with_residual_in_place_and_unaligned_c(lib, gpu, M, N, K):
     a, b = operands(M, N, K, "NT", seed=3, b_std=0.05)
     ag, bg = a.to(gpu), b.to(gpu)
     c = torch.full((M + 1, N + 3), 3.0, dtype=torch.float16, device=gpu)      # rows of 1004 elements: not 16-byte aligned

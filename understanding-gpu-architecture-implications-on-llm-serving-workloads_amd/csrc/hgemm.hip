@@ -1300,7 +1300,7 @@ static hipError_t launch_main(const T* A, const T* B, T* C, const T* R, int M, i
 }
 
 // ---------------------------------------------------------------------------------------------------------
-// Split-K on 64x64 tiles, for 17 .. 256 rows against a second operand that is too narrow to give every CU a tile: the
+// Split-K on 64x64 tiles (and, further down, on 128x128 tiles), for 17 .. 256 rows against a second operand that is too narrow to give every CU a tile: the
 // ranges of K of a tile run on different workgroups (see SPLIT_K of hgemm_main_kernel) and meet in a workspace of the
 // library's own: one buffer per (device, stream), allocated at first use and replaced by a larger one when a call needs
 // more; a buffer that has been handed to a kernel is never freed (a HIP graph captured earlier may hold its address).
@@ -1364,15 +1364,32 @@ static int split_k_ranges(int M, int N, int K) {
     return s >= 4 ? s : 0;
 }
 
+// The same on 128x128 tiles (64 KiB of partial tile per workgroup), for 193 .. 512 rows against a long K (the down
+// projection): at most 128 tiles, two to four ranges so that about every CU has a workgroup. Measured, weights from HBM
+// (us, best tile shape without / with split-K): NT 256 x 4096 x 14336 70 / 54, 384 rows 99 / 83, 512 rows 100 / 86,
+// 320 x 2048 x 16384 68 / 47; NN 256 x 4096 x 8192 47 / 38, 384 rows 61 / 54, 512 x 4096 x 14336 108 / 85. Layout NT with
+// K = 8192 loses to its 128x64 tiles (384 x 4096 x 8192: 49 / 52), so it needs a longer K; 640 rows (160 tiles) and every
+// product with K = 4096 lose 10-60 %.
+static int split_k_ranges_128(int M, int N, int K, bool nt) {
+    if (M < 193 || M > 512 || K < (nt ? 12288 : 8192) || K % 64 != 0) return 0;
+    const long tiles = (long)((M + 127) / 128) * ((N + 127) / 128);
+    if (tiles > 128) return 0;
+    const int ktiles = K / 64;
+    int s = (int)(256 / tiles);
+    if (s > 4) s = 4;
+    while (s >= 2 && (ktiles % s != 0 || ktiles / s < 8)) --s;
+    return s >= 2 ? s : 0;
+}
+
 // hipErrorStreamCaptureUnsupported / hipErrorOutOfMemory: no workspace to be had, the caller takes another kernel
-template <typename T, bool A_KC, bool B_KC>
+template <typename T, bool A_KC, bool B_KC, int BT = 64, int STAGES = 4, int PER_CU = 2>
 static hipError_t launch_split_k(const T* A, const T* B, T* C, const T* R, int M, int N, int K, long lda, long ldb, long ldc,
                                  long ldr, int splits, hipStream_t stream) {
-    using Cfg = MainCfg<A_KC, B_KC, 64, 64, 2, 2, 4>;
-    auto kern = hgemm_main_kernel<T, A_KC, B_KC, 64, 64, 2, 2, 0, true, 4, 2, true>;
+    using Cfg = MainCfg<A_KC, B_KC, BT, BT, 2, 2, STAGES>;
+    auto kern = hgemm_main_kernel<T, A_KC, B_KC, BT, BT, 2, 2, 0, true, STAGES, PER_CU, true>;
     static DynamicLdsOnce lds_once;
     if (hipError_t e = lds_once.ensure(reinterpret_cast<const void*>(kern), Cfg::LDS_BYTES); e != hipSuccess) return e;
-    const long tiles = (long)((M + 63) / 64) * ((N + 63) / 64);
+    const long tiles = (long)((M + BT - 1) / BT) * ((N + BT - 1) / BT);
     if (tiles * sizeof(unsigned) > kSplitKCounterBytes) return hipErrorOutOfMemory;
     const size_t bytes = kSplitKCounterBytes + (size_t)tiles * splits * Cfg::NTHREADS * Cfg::TM * Cfg::TN * 16;
     char* ws = nullptr;
@@ -1425,7 +1442,7 @@ static bool few_rows_prefer_tiles(int M, int N, int K, bool nt) {
 // operand (generation steps of that many sequences through the O and down projections), where 64x64 tiles are only
 // half as many as CUs: 128 x 4096 x 14336 NT 41 -> 33 us, 128 x 4096 x 4096 13.2 -> 11.2, 96 x 4096 x 14336 40 -> 32
 // (with 256 rows, or 6144 columns, they would need two rounds and lose: 63 us against 45, 20 against 14).
-static int cheapest_tile_shape(int M, int N, int K, bool a_k_contiguous) {
+static int cheapest_tile_shape(int M, int N, int K, bool a_k_contiguous, bool nt) {
     struct Cand { int shape, bm, bn, per_cu; double step, fixed; };
     static const Cand cands[] = {{1, 256, 256, 1, 2470., 12000.}, {2, 128, 128, 1, 840., 7000.}, {3, 64, 128, 1, 576., 6000.},
                                  {4, 64, 64, 2, 384., 5000.}, {5, 128, 256, 1, 1400., 9000.}, {6, 256, 128, 1, 1400., 9000.},
@@ -1435,7 +1452,8 @@ static int cheapest_tile_shape(int M, int N, int K, bool a_k_contiguous) {
     double best_t = 0.;
     for (const Cand& c : cands) {
         if (c.shape == 7 && !a_k_contiguous) continue;   // 32-row tiles exist for a K-contiguous A only
-        const long tiles = (long)((M + c.bm - 1) / c.bm) * ((N + c.bn - 1) / c.bn);
+        const int bm = (c.shape == 3 && nt) ? c.bn : c.bm, bn = (c.shape == 3 && nt) ? c.bm : c.bn;   // layout NT: 128x64
+        const long tiles = (long)((M + bm - 1) / bm) * ((N + bn - 1) / bn);
         const long cap = 256L * c.per_cu, full = tiles / cap, rem = tiles % cap;
         double t = (double)full * (c.per_cu * ktiles * c.step + c.fixed);
         if (rem) t += (double)((rem + 255) / 256) * ktiles * c.step + c.fixed;
@@ -1499,6 +1517,10 @@ static hipError_t launch_layout(const T* A, const T* B, T* C, const T* R, int M,
             const hipError_t e = launch_split_k<T, A_KC, B_KC>(A, B, C, R, M, N, K, lda, ldb, ldc, ldr, splits, stream);
             if (e != hipErrorStreamCaptureUnsupported && e != hipErrorOutOfMemory) return e;
             (void)hipGetLastError();
+        } else if (const int splits128 = split_k_ranges_128(M, N, K, A_KC && B_KC); splits128 > 0) {
+            const hipError_t e = launch_split_k<T, A_KC, B_KC, 128, 0, 1>(A, B, C, R, M, N, K, lda, ldb, ldc, ldr, splits128, stream);
+            if (e != hipErrorStreamCaptureUnsupported && e != hipErrorOutOfMemory) return e;
+            (void)hipGetLastError();
         }
     }
     // 33 .. 64 rows against a second operand of up to 8192 columns (generation steps of that many sequences through the
@@ -1534,7 +1556,7 @@ static hipError_t launch_layout(const T* A, const T* B, T* C, const T* R, int M,
     // NT (17 .. 64 x 28672 x 4096 with weights from HBM: 45 - 52 us against 53 - 57 on 128x64 tiles and 51 on 128x128),
     // 128x128 otherwise (layout NN: 42 - 47 us against 52 - 64).
     if (ragged_ok) {
-        int shape = variant >= 1 && variant <= (A_KC ? 7 : 6) ? variant : M <= 64 ? ((A_KC && B_KC) ? 4 : 2) : cheapest_tile_shape(M, N, K, A_KC);
+        int shape = variant >= 1 && variant <= (A_KC ? 7 : 6) ? variant : M <= 64 ? ((A_KC && B_KC) ? 4 : 2) : cheapest_tile_shape(M, N, K, A_KC, A_KC && B_KC);
         const auto whole = [&](int bm, int bn) { return c_aligned && M % bm == 0 && N % bn == 0; };
         switch (shape) {
             case 1:
