@@ -400,7 +400,16 @@ def main():
         other["gemm_decode_nt_64x4096x14336_split_k"] = {"ms": msk, "gbs": byk / msk / 1e6, "pct_of_hbm_peak": 100 * byk / msk / 1e6 / PEAK_HBM_GBS,
                                                         "ms_weights_not_cached": msk_cold, "gbs_weights_not_cached": byk / msk_cold / 1e6,
                                                         "pct_of_hbm_peak_weights_not_cached": 100 * byk / msk_cold / 1e6 / PEAK_HBM_GBS}
-        del xk, wk, ok_, wk_sets
+        # the same weight against a chunk of 512 tokens: 128 tiles of 128x128, split-K over 2 ranges
+        xc = so.randn_fp16((512, 14336), 6).to(dev)
+        oc_ = torch.empty((512, 4096), dtype=torch.float16, device=dev)
+        msc_cold = time_launches(rotating(lambda j: lib.hgemm_raw(xc.data_ptr(), wk_sets[j].data_ptr(), oc_.data_ptr(), 512, 4096, 14336,
+                                                                  14336, 14336, 4096, lib.GEMM_NT, stream), len(wk_sets)), 40, 3)
+        msc_v = time_launches(rotating(lambda j: torch.matmul(xc, wk_sets[j].t(), out=oc_), len(wk_sets)), 40, 3)
+        other["gemm_chunk_nt_512x4096x14336_split_k"] = {"ms_weights_not_cached": msc_cold,
+                                                        "tflops_weights_not_cached": 2.0 * 512 * 4096 * 14336 / msc_cold / 1e9,
+                                                        "ms_vendor_weights_not_cached": msc_v}
+        del xk, wk, ok_, wk_sets, xc, oc_
         ab, bb = a.to(torch.bfloat16), b.to(torch.bfloat16)
         cb = torch.empty((M, N), dtype=torch.bfloat16, device=dev)
         msb = time_launches(lambda: lib.hgemm(ab, bb, "NN", out=cb), 10, 2)
@@ -666,6 +675,8 @@ KERNEL_CONFIGS = {
     "gemm_64x14336x4096_nt": ("gemm", 64, 14336, 4096, "NT"),               # 64x64 tiles, 8-deep ring
     "gemm_64x4096x14336_nt": ("gemm", 64, 4096, 14336, "NT"),               # 64x64 tiles, split-K over 8 ranges
     "gemm_16x4096x14336_nt": ("gemm", 16, 4096, 14336, "NT"),               # split-K small-M kernel (NT)
+    "gemm_512x4096x14336_nt": ("gemm", 512, 4096, 14336, "NT"),             # 128x128 tiles, split-K over 2 ranges
+    "vendor_gemm_512x4096x14336_nt": ("vendor_gemm", 512, 4096, 14336, "NT"),
     "gemm_1024x4096x4096_nt": ("gemm", 1024, 4096, 4096, "NT"),             # 128x64 tiles
     "f3_fmha_noncausal_b4_h32_s1024": ("fmha", 4, 32, 32, 1024, 1024, False),   # ping-pong kernel, 256-query work items
     "f4_fmha_causal_gqa_s4096": ("fmha", 1, 32, 8, 4096, 4096, True),           # ping-pong kernel
