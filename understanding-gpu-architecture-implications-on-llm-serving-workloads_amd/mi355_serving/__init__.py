@@ -169,7 +169,9 @@ def _bhs_strides(t):
 
 
 def fmha_workspace_bytes(B, Hq, Hkv, Sq, Sk, kv_valid_len=None):
-    """Bytes of caller workspace mi355_fmha_fwd_ws needs for these sizes (0 outside the split-KV path)."""
+    """Bytes of caller workspace mi355_fmha_fwd_ws uses for these sizes: the partial results of the split-KV path
+    (generation steps; required) or of the key ranges of a chunk of queries against a long cache (optional: with less the
+    call walks all keys in one kernel); 0 for every other shape."""
     return int(load().mi355_fmha_fwd_workspace_bytes(B, Hq, Hkv, Sq, Sk, Sk if kv_valid_len is None else kv_valid_len))
 
 
