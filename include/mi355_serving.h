@@ -19,8 +19,8 @@
  *     visible to the library: a first (or growing) call made while ANOTHER stream captures in global capture mode is a
  *     hipMalloc inside that capture and invalidates it, so make such calls before any capture starts.
  *     The GEMM entry points keep a second buffer of the same kind per (device, stream) for the partial tiles of their
- *     split-K path (17 .. 512 rows against a second operand of up to 8192 columns, K a multiple of 128; >= 8 MiB, up to
- *     24 MiB); a GEMM call that cannot get it (its stream is being captured and has none yet, or hipMalloc fails) does not fail: it
+ *     split-K path (17 .. 1024 rows against a second operand of up to 8192 columns, K a multiple of 128; >= 8 MiB, up to
+ *     72 MiB); a GEMM call that cannot get it (its stream is being captured and has none yet, or hipMalloc fails) does not fail: it
  *     runs the kernels without split-K, so a captured call is faster when the step ran once on that stream before.
  *     The attention entry points other than mi355_fmha_fwd_ws (which takes the caller's) and mi355_fmha_fwd_noalloc
  *     (which walks all keys in one kernel) keep a third buffer of that kind

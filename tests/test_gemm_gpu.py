@@ -192,8 +192,10 @@ def test_widths_that_are_no_multiple_of_8_and_unaligned_rows_of_c(lib, gpu, vari
 # ---- split-K: 17 .. 256 rows against a narrow second operand --------------------------------------------------------
 SPLIT_K_SHAPES = [(64, 4096, 14336), (17, 4096, 8192), (100, 2048, 4096), (128, 4096, 4096), (48, 1000, 2048), (33, 6144, 4096),
                   (250, 1024, 8192), (40, 72, 16384), (160, 4096, 8192), (192, 4000, 14336),
-                  # 193 .. 512 rows, long K: ranges of K on 128x128 tiles (four ranges, two ranges, ragged M and N)
-                  (256, 4096, 14336), (384, 2048, 16384), (500, 4000, 12288), (300, 4096, 8192)]
+                  # 193 .. 1024 rows, long K: ranges of K on 128x128 tiles (four ranges, two ranges, ragged M and N)
+                  (256, 4096, 14336), (384, 2048, 16384), (500, 4000, 12288), (300, 4096, 8192),
+                  # up to 1024 rows: 120 tiles in two ranges, 168 tiles in three, 192 tiles in four
+                  (640, 3072, 12288), (896, 3072, 12288), (768, 4096, 14336)]
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])

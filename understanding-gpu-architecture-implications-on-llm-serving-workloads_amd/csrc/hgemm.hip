@@ -1364,17 +1364,30 @@ static int split_k_ranges(int M, int N, int K) {
     return s >= 4 ? s : 0;
 }
 
-// The same on 128x128 tiles (64 KiB of partial tile per workgroup), for 193 .. 512 rows against a long K (the down
-// projection): at most 128 tiles, two to four ranges so that about every CU has a workgroup. Measured, weights from HBM
+// The same on 128x128 tiles (64 KiB of partial tile per workgroup), for 193 .. 1024 rows against a long K (the down
+// projection): at most 128 tiles, two to four ranges so that about every CU has a workgroup (640 x 3072 x 12288 NT:
+// 96 / 76). Measured, weights from HBM
 // (us, best tile shape without / with split-K): NT 256 x 4096 x 14336 70 / 54, 384 rows 99 / 83, 512 rows 100 / 86,
 // 320 x 2048 x 16384 68 / 47; NN 256 x 4096 x 8192 47 / 38, 384 rows 61 / 54, 512 x 4096 x 14336 108 / 85. Layout NT with
 // K = 8192 loses to its 128x64 tiles (384 x 4096 x 8192: 49 / 52), so it needs a longer K; 640 rows (160 tiles) and every
 // product with K = 4096 lose 10-60 %.
 static int split_k_ranges_128(int M, int N, int K, bool nt) {
-    if (M < 193 || M > 512 || K < (nt ? 12288 : 8192) || K % 64 != 0) return 0;
+    if (M < 193 || M > 1024 || K < (nt ? 12288 : 8192) || K % 64 != 0) return 0;
     const long tiles = (long)((M + 127) / 128) * ((N + 127) / 128);
-    if (tiles > 128) return 0;
     const int ktiles = K / 64;
+    if (tiles > 128) {
+        // 129 .. 255 tiles leave CUs idle for a whole walk over K: the smallest number of ranges, up to four, that makes
+        // whole rounds of 256 workgroups (at least 95 % of the last one), where K is long enough to pay for the partial
+        // tiles (us, without / with: NT 896 x 3072 x 12288 124 / 102 with three ranges, 768 x 4096 x 14336 136 / 129 and
+        // 1024 x 3072 x 12288 124 / 117 with four; eight ranges lose: 896 x 4096 x 14336 138 / 176, 513 rows 102 / 117)
+        if (tiles >= 256 || K < 12288) return 0;
+        for (int s = 2; s <= 4; ++s) {
+            if (ktiles % s != 0 || ktiles / s < 16) continue;
+            const long wgs = tiles * s, rounds = (wgs + 255) / 256;
+            if (wgs * 100 >= rounds * 256 * 95) return s;
+        }
+        return 0;
+    }
     int s = (int)(256 / tiles);
     if (s > 4) s = 4;
     while (s >= 2 && (ktiles % s != 0 || ktiles / s < 8)) --s;
