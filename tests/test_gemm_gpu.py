@@ -194,8 +194,8 @@ SPLIT_K_SHAPES = [(64, 4096, 14336), (17, 4096, 8192), (100, 2048, 4096), (128, 
                   (250, 1024, 8192), (40, 72, 16384), (160, 4096, 8192), (192, 4000, 14336),
                   # 193 .. 1024 rows, long K: ranges of K on 128x128 tiles (four ranges, two ranges, ragged M and N)
                   (256, 4096, 14336), (384, 2048, 16384), (500, 4000, 12288), (300, 4096, 8192),
-                  # up to 1024 rows: 120 tiles in two ranges, 168 tiles in three, 192 tiles in four
-                  (640, 3072, 12288), (896, 3072, 12288), (768, 4096, 14336)]
+                  # up to 1024 rows: 120 tiles in two ranges, 168 tiles in three, 192 tiles in four, 160 tiles in three
+                  (640, 3072, 12288), (896, 3072, 12288), (768, 4096, 14336), (640, 4096, 12288)]
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])

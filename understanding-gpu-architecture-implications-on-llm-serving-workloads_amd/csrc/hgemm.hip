@@ -1376,17 +1376,23 @@ static int split_k_ranges_128(int M, int N, int K, bool nt) {
     const long tiles = (long)((M + 127) / 128) * ((N + 127) / 128);
     const int ktiles = K / 64;
     if (tiles > 128) {
-        // 129 .. 255 tiles leave CUs idle for a whole walk over K: the smallest number of ranges, up to four, that makes
-        // whole rounds of 256 workgroups (at least 95 % of the last one), where K is long enough to pay for the partial
-        // tiles (us, without / with: NT 896 x 3072 x 12288 124 / 102 with three ranges, 768 x 4096 x 14336 136 / 129 and
-        // 1024 x 3072 x 12288 124 / 117 with four; eight ranges lose: 896 x 4096 x 14336 138 / 176, 513 rows 102 / 117)
+        // 129 .. 255 tiles leave CUs idle for a whole walk over K. With s ranges the walk takes rounds(s) / s of that time,
+        // rounds(s) = ceil(tiles * s / 256), plus about 0.05 s of it for the partial tiles (measured, us without / with: NT
+        // 896 x 3072 x 12288, 168 tiles, three ranges 124 / 102; 768 x 4096 x 14336, 192 tiles, four ranges 136 / 130;
+        // 768 x 3072 x 12288, 144 tiles, three ranges 123 / 98; 640 x 4096 x 12288, 160 tiles, three ranges 124 / 102;
+        // eight ranges lose: 896 x 4096 x 14336 138 / 176, 513 rows 102 / 117): the best s up to four, if it saves 4 %; a
+        // saving below 10 % only with a last row of tiles that is at least three quarters full (700 x 4096 x 12288, 192
+        // tiles with 60 rows in the last six of every column: 102 / 107)
         if (tiles >= 256 || K < 12288) return 0;
+        int best = 0;
+        double best_cost = 0.96;
         for (int s = 2; s <= 4; ++s) {
             if (ktiles % s != 0 || ktiles / s < 16) continue;
-            const long wgs = tiles * s, rounds = (wgs + 255) / 256;
-            if (wgs * 100 >= rounds * 256 * 95) return s;
+            const double cost = (double)((tiles * s + 255) / 256) / s + 0.05 * s;
+            if (cost < best_cost) { best_cost = cost; best = s; }
         }
-        return 0;
+        if (best_cost > 0.9 && M % 128 != 0 && M % 128 < 96) return 0;
+        return best;
     }
     int s = (int)(256 / tiles);
     if (s > 4) s = 4;
