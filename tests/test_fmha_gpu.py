@@ -544,6 +544,19 @@ def test_chunk_against_long_cache_key_ranges(lib, gpu, B, Hq, Hkv, Sq, Sk, causa
     assert (o.float() - o1.float()).abs().max() <= 2e-3 and (lse - lse1).abs().max() <= 1e-3
 
 
+def test_key_ranges_with_query_rows_that_see_no_key(lib, gpu):
+    # causal with more queries than keys: the first Sq - Sk rows see nothing (O = 0, LSE = -inf), also after the merge
+    B, Hq, Hkv, Sq, Sk = 1, 2, 1, 5000, 4100
+    q, k, v = (t.to(gpu) for t in so.fmha_inputs(B, Hq, Hkv, Sq, Sk, seed=12))
+    o1, l1 = lib.fmha_fwd(q, k, v, causal=True, variant=1)
+    o3, l3 = lib.fmha_fwd(q, k, v, causal=True, variant=3)
+    torch.cuda.synchronize()
+    empty = torch.isinf(l1)
+    assert int(empty.sum()) == B * Hq * (Sq - Sk) and torch.equal(empty, torch.isinf(l3)) and bool((l3[empty] < 0).all())
+    assert bool((o3[empty] == 0).all())
+    assert (o1.float() - o3.float()).abs().max() <= 2e-3 and (l1[~empty] - l3[~empty]).abs().max() <= 1e-3
+
+
 def test_key_ranges_only_where_they_pay(lib, gpu):
     # enough work items for the machine, a short cache, or a generation step: no ranges (variant 3 reports it)
     for B, Hq, Hkv, Sq, Sk in ((1, 32, 8, 2048, 8192), (1, 32, 8, 128, 1024), (1, 32, 8, 512, 2048)):
